@@ -1,0 +1,180 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) row kernels.
+//
+// Row layout used by every kernel here ("L4"): a wave owns a row (or a 128/256-value head / block); lane p holds the four
+// consecutive elements 256 j + 4 p + k (k = 0..3) of each 256-element slab j, so every global access is one 128-bit
+// load per lane and a wave instruction covers 1 KiB of contiguous memory.
+//
+// The reference's reductions are stated for 256 logical threads in 32-lane groups (thread t owns elements t, t + 256, ..;
+// xor butterfly 16, 8, 4, 2, 1 inside each group of 32; the 8 group sums added in order). In L4, logical thread
+// t = 4 p + k, so a group of 32 logical threads is 8 consecutive lanes x 4 registers, and the butterfly becomes
+// lane xor 4, lane xor 2, lane xor 1, then register pairs (k, k ^ 2) and (k, k ^ 1): the same pairs in the same order,
+// hence the same bits. The group sums are then read with v_readlane from lanes 0, 8, .., 56 and added in order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+#define CAMX_DEV __device__ __forceinline__
+
+// ---- lane permutes (all 64 lanes must be active) ----------------------------------------------------------------------
+CAMX_DEV float lane_xor1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)); }   // quad_perm [1,0,3,2]
+CAMX_DEV float lane_xor2(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)); }   // quad_perm [2,3,0,1]
+CAMX_DEV float lane_xor4(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x101f)); }               // swizzle SWAP,4
+CAMX_DEV float lane_xor8(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false)); }  // row_ror:8
+CAMX_DEV float lane_xor16(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401f)); }              // swizzle SWAP,16
+CAMX_DEV float lane_read(float v, int lane) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane)); }
+
+// ---- the 32-value butterfly in L4 (8 lanes x 4 registers): every lane of the 8 gets the group's sum / max ----------------
+CAMX_DEV float group32_sum(f32x4 v) {
+    float a0 = v.x, a1 = v.y, a2 = v.z, a3 = v.w;
+    a0 += lane_xor4(a0); a1 += lane_xor4(a1); a2 += lane_xor4(a2); a3 += lane_xor4(a3);   // logical xor 16
+    a0 += lane_xor2(a0); a1 += lane_xor2(a1); a2 += lane_xor2(a2); a3 += lane_xor2(a3);   // logical xor 8
+    a0 += lane_xor1(a0); a1 += lane_xor1(a1); a2 += lane_xor1(a2); a3 += lane_xor1(a3);   // logical xor 4
+    const float w0 = a0 + a2, w1 = a1 + a3;                                               // logical xor 2
+    return w0 + w1;                                                                       // logical xor 1
+}
+CAMX_DEV float group8_max(float a) {   // max over the 8 lanes of a group (order-free)
+    a = fmaxf(a, lane_xor4(a)); a = fmaxf(a, lane_xor2(a)); a = fmaxf(a, lane_xor1(a));
+    return a;
+}
+CAMX_DEV float group8_sum(float a) {   // xor 4, 2, 1 butterfly over 8 lanes (the MMQ quantizer's 8-thread sum)
+    a += lane_xor4(a); a += lane_xor2(a); a += lane_xor1(a);
+    return a;
+}
+CAMX_DEV float absmax4(f32x4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
+
+// the 8 group sums of a wave added in order from 0.0f (0 + p0 is p0 for the non-negative sums used here)
+CAMX_DEV float wave_groups_in_order(float g) {
+    float tot = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; q++) tot += lane_read(g, 8 * q);
+    return tot;
+}
+// only the first ng groups (a 128-wide head: 4)
+template <int NG> CAMX_DEV float half_groups_in_order(float g, int base_lane) {
+    float tot = 0.0f;
+#pragma unroll
+    for (int q = 0; q < NG; q++) tot += __shfl(g, base_lane + 8 * q, 64);
+    return tot;
+}
+
+CAMX_DEV float rsqrt_exact(float v) { return 1.0f / sqrtf(v); }   // correctly rounded sqrt then divide (the contract)
+
+// ---- conversions -----------------------------------------------------------------------------------------------------------
+CAMX_DEV float bf2f(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
+CAMX_DEV uint16_t f2bf(float f) {          // round to nearest even; any NaN -> 0x7fc0
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+CAMX_DEV uint16_t to_bf16(float f) {       // the same rounding without the NaN case
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+CAMX_DEV float rbf(float f) { return bf2f(f2bf(f)); }
+CAMX_DEV uint16_t f2h_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+CAMX_DEV float h2f_bits(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+// fp32 -> fp16 -> fp32 of a value that is already rounded to fp32: the opaque copy keeps the backend from folding the
+// producing fma and the convert into one mixed-precision instruction (one rounding instead of two)
+CAMX_DEV float f16r(float x) { asm volatile("" : "+v"(x)); return (float)(_Float16)x; }
+
+CAMX_DEV u32x2 pack_bf16x4_rne(f32x4 v) {  // to_bf16 of four values, packed little-endian
+    u32x2 r;
+    r.x = (uint32_t)to_bf16(v.x) | ((uint32_t)to_bf16(v.y) << 16);
+    r.y = (uint32_t)to_bf16(v.z) | ((uint32_t)to_bf16(v.w) << 16);
+    return r;
+}
+CAMX_DEV u32x2 pack_f2bf_x4(f32x4 v) {
+    u32x2 r;
+    r.x = (uint32_t)f2bf(v.x) | ((uint32_t)f2bf(v.y) << 16);
+    r.y = (uint32_t)f2bf(v.z) | ((uint32_t)f2bf(v.w) << 16);
+    return r;
+}
+CAMX_DEV u32x2 pack_f16x4(f32x4 v) {
+    u32x2 r;
+    r.x = (uint32_t)f2h_bits(v.x) | ((uint32_t)f2h_bits(v.y) << 16);
+    r.y = (uint32_t)f2h_bits(v.z) | ((uint32_t)f2h_bits(v.w) << 16);
+    return r;
+}
+CAMX_DEV f32x4 unpack_bf16x4(u32x2 w) {
+    f32x4 r;
+    r.x = __builtin_bit_cast(float, w.x << 16); r.y = __builtin_bit_cast(float, w.x & 0xffff0000u);
+    r.z = __builtin_bit_cast(float, w.y << 16); r.w = __builtin_bit_cast(float, w.y & 0xffff0000u);
+    return r;
+}
+
+// roundf (half away from zero) of a value known to fit int8 after rounding, as a signed byte in the low 8 bits
+CAMX_DEV uint32_t round_i8(float v) { return (uint32_t)(int)roundf(v) & 0xffu; }
+CAMX_DEV uint32_t pack_round_i8x4(f32x4 v) {
+    return round_i8(v.x) | (round_i8(v.y) << 8) | (round_i8(v.z) << 16) | (round_i8(v.w) << 24);
+}
+
+// ---- q8_1 (ggml 36-byte block) of 32 values held by 8 lanes x 4 registers; sub = lane & 7 -------------------------------
+// d = amax / 127, q = amax == 0 ? 0 : roundf(x / d), header half2(d, sum) with the butterfly sum. blk: the block's base.
+CAMX_DEV void q8_1_emit(f32x4 v, uint8_t * blk, int sub) {
+    const float amax = group8_max(absmax4(v));
+    const float sum = group32_sum(v);
+    const float d = amax / 127.0f;
+    uint32_t q = 0;
+    if (amax != 0.0f) { f32x4 t; t.x = v.x / d; t.y = v.y / d; t.z = v.z / d; t.w = v.w / d; q = pack_round_i8x4(t); }
+    *(uint32_t *)(blk + 4 + 4 * sub) = q;
+    if (sub == 0) *(uint32_t *)blk = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
+}
+
+// ---- Q8 KV wire block (34 bytes) of 32 values held by 8 lanes x 4 registers ----------------------------------------------
+// amax / 127, its fp32 reciprocal, roundf(x * inv), only the stored scale rounded to half. A refused block (non-finite
+// input; nonzero block whose scale underflows, whose reciprocal overflows or whose half scale is not finite) keeps its
+// bytes and ORs 2 into *err. blk is 2-byte aligned. Returns true when the block was written.
+CAMX_DEV bool kv_q8_emit(f32x4 v, uint8_t * blk, int sub, int * err, bool active) {
+    const bool fin = __builtin_isfinite(v.x) && __builtin_isfinite(v.y) && __builtin_isfinite(v.z) && __builtin_isfinite(v.w);
+    const float amax = group8_max(fin ? absmax4(v) : INFINITY);
+    const float d = amax / 127.0f;
+    const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+    const _Float16 stored = (_Float16)d;
+    const bool refuse = !__builtin_isfinite(amax) ||
+                        (amax != 0.0f && (d == 0.0f || !__builtin_isfinite(d) || !__builtin_isfinite(inv) || !__builtin_isfinite((float)stored)));
+    if (!active) return false;
+    if (refuse) { if (sub == 0) atomicOr(err, 2); return false; }
+    f32x4 t; t.x = v.x * inv; t.y = v.y * inv; t.z = v.z * inv; t.w = v.w * inv;
+    const uint32_t q = pack_round_i8x4(t);
+    uint16_t * o = (uint16_t *)(blk + 2 + 4 * sub);
+    o[0] = (uint16_t)q; o[1] = (uint16_t)(q >> 16);
+    if (sub == 0) *(uint16_t *)blk = __builtin_bit_cast(uint16_t, stored);
+    return true;
+}
+
+// ---- the orthonormal 128-point Walsh-Hadamard transform of a head held by 32 lanes x 4 registers (element 4 l + k) ------
+// stages h = 1, 2 pair registers, h = 4 .. 64 pair lanes l ^ 1 .. l ^ 16; pair (i, i + h) -> (a + b, a - b); then times
+// 0x1.6a09e6p-4f. lane: the lane's index inside its 32-lane half.
+CAMX_DEV f32x4 hadamard128_l4(f32x4 v, int lane, bool scale) {
+    float a, b;
+    a = v.x; b = v.y; v.x = a + b; v.y = a - b;
+    a = v.z; b = v.w; v.z = a + b; v.w = a - b;
+    a = v.x; b = v.z; v.x = a + b; v.z = a - b;
+    a = v.y; b = v.w; v.y = a + b; v.w = a - b;
+#define CAMX_HSTAGE(BIT, XOR)                                                                         \
+    {                                                                                                 \
+        const bool hi = (lane & BIT) != 0;                                                            \
+        const float p0 = XOR(v.x), p1 = XOR(v.y), p2 = XOR(v.z), p3 = XOR(v.w);                        \
+        v.x = hi ? p0 - v.x : v.x + p0; v.y = hi ? p1 - v.y : v.y + p1;                               \
+        v.z = hi ? p2 - v.z : v.z + p2; v.w = hi ? p3 - v.w : v.w + p3;                               \
+    }
+    CAMX_HSTAGE(1, lane_xor1) CAMX_HSTAGE(2, lane_xor2) CAMX_HSTAGE(4, lane_xor4) CAMX_HSTAGE(8, lane_xor8) CAMX_HSTAGE(16, lane_xor16)
+#undef CAMX_HSTAGE
+    if (scale) { v.x *= 0x1.6a09e6p-4f; v.y *= 0x1.6a09e6p-4f; v.z *= 0x1.6a09e6p-4f; v.w *= 0x1.6a09e6p-4f; }
+    return v;
+}
+
+// ---- host-side helpers -------------------------------------------------------------------------------------------------------
+#define CAMX_OK 0
+#define CAMX_EINVAL 1     // hipErrorInvalidValue
+#define CAMX_LAUNCH_RET() return (int)hipGetLastError()

@@ -1,0 +1,226 @@
+// Residual add + RMSNorm family for gfx950: one wave64 per row, the row held in registers (128-bit loads, no LDS, no
+// barrier), every copy the callers need (fp32, fp16, bf16, q8_1, row scale) written from the same registers so a row
+// crosses HBM once. Replaces the reference's q3p_add_rms16 / OP_OWN_ADD_RMS16 (kernels/q3m_prefill.hip:385-415,
+// kernels/k3_own_ops.h:326-383), q35p_add_rms16 (kernels/q35_prefill.hip:636-660), pf_rms_mul / OP_RMS_MUL
+// (kernels/prefill_glue.hip:94-124, kernels/k3_gguf_ops.h:1233-1268), rmsnorm_f32 and residual3 (kernels/core.hip:30-61).
+//
+// Numeric contract: sum of squares = fmaf chain per logical thread t over elements t + 256 j, the 32-lane butterfly, the
+// 8 group sums in order; scale = 1 / sqrt(tot / N + eps) with IEEE sqrt and divide; h = (x * scale) * w.
+#include "common.cuh"
+
+enum { ADD_NONE = 0, ADD_F32_SLOTS = 1, ADD_BF16 = 2, ADD_F32_DIRECT = 3 };   // DIRECT: x = x + d (no 0 + d first)
+
+struct NormArgs {
+    float * x;               // [rows][N] residual, updated in place when an addend is given
+    const void * d;          // ADD_F32_SLOTS: fp32 [rows][S][N]; ADD_BF16: bf16 [rows][N]
+    const float * w;         // slot weights [rows][S] or null (weights 1: acc + d)
+    int S;
+    const float * nw;        // gamma [wr][N]; row r uses nw[(r % wr) * N ..]
+    int wr;
+    float eps;
+    float * h;               // optional fp32 [rows][N] (may alias x for the no-addend forms)
+    uint16_t * h16;          // optional fp16 bits
+    int ld16;                // h16 row stride in elements
+    uint16_t * hbf;          // optional bf16 bits (to_bf16 rounding)
+    uint8_t * q8;            // optional q8_1 blocks [rows][N / 32][36]
+    float * scl;             // optional row scale [rows]
+    int N, rows;
+};
+
+template <int NI_MAX, int ADD>
+__global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (row >= a.rows) return;
+    const int N = a.N, ni = N >> 8;
+    float * xr = a.x + (size_t)row * N;
+    f32x4 xv[NI_MAX];
+#pragma unroll
+    for (int j = 0; j < NI_MAX; j++)
+        if (j < ni) xv[j] = *(const f32x4 *)(xr + 256 * j + 4 * lane);
+    if (ADD == ADD_F32_SLOTS && a.S > 0) {
+        const float * dr = (const float *)a.d + (size_t)row * a.S * N;
+        const float * wr = a.w ? a.w + (size_t)row * a.S : nullptr;
+        f32x4 acc[NI_MAX];
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++) acc[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s = 0; s < a.S; s++) {
+            const float ws = wr ? wr[s] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < NI_MAX; j++)
+                if (j < ni) {
+                    const f32x4 dv = *(const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane);
+                    if (wr) {
+                        acc[j].x = __builtin_fmaf(ws, dv.x, acc[j].x); acc[j].y = __builtin_fmaf(ws, dv.y, acc[j].y);
+                        acc[j].z = __builtin_fmaf(ws, dv.z, acc[j].z); acc[j].w = __builtin_fmaf(ws, dv.w, acc[j].w);
+                    } else acc[j] = acc[j] + dv;
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) { xv[j] = xv[j] + acc[j]; *(f32x4 *)(xr + 256 * j + 4 * lane) = xv[j]; }
+    }
+    if (ADD == ADD_F32_DIRECT && a.d) {
+        const float * dr = (const float *)a.d + (size_t)row * N;
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) {
+                xv[j] = xv[j] + *(const f32x4 *)(dr + 256 * j + 4 * lane);
+                *(f32x4 *)(xr + 256 * j + 4 * lane) = xv[j];
+            }
+    }
+    if (ADD == ADD_BF16 && a.d) {
+        const uint16_t * dr = (const uint16_t *)a.d + (size_t)row * N;
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) {
+                const f32x4 dv = unpack_bf16x4(*(const u32x2 *)(dr + 256 * j + 4 * lane));
+                xv[j] = xv[j] + dv;
+                *(f32x4 *)(xr + 256 * j + 4 * lane) = xv[j];
+            }
+    }
+    // sum of squares: logical thread 4 lane + k chains its elements in j order
+    f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NI_MAX; j++)
+        if (j < ni) {
+            ss.x = __builtin_fmaf(xv[j].x, xv[j].x, ss.x); ss.y = __builtin_fmaf(xv[j].y, xv[j].y, ss.y);
+            ss.z = __builtin_fmaf(xv[j].z, xv[j].z, ss.z); ss.w = __builtin_fmaf(xv[j].w, xv[j].w, ss.w);
+        }
+    const float tot = wave_groups_in_order(group32_sum(ss));
+    const float scale = rsqrt_exact(tot / (float)N + a.eps);
+    if (a.scl && lane == 0) a.scl[row] = scale;
+    const float * gw = a.nw + (size_t)(row % a.wr) * N;
+#pragma unroll
+    for (int j = 0; j < NI_MAX; j++)
+        if (j < ni) {
+            const f32x4 g = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+            f32x4 v;
+            v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
+            const size_t o = (size_t)row * N + 256 * j + 4 * lane;
+            if (a.h) *(f32x4 *)(a.h + o) = v;
+            if (a.h16) *(u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane) = pack_f16x4(v);
+            if (a.hbf) *(u32x2 *)(a.hbf + o) = pack_bf16x4_rne(v);
+            if (a.q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
+        }
+}
+
+// Any row length (N not a multiple of 256, or longer than the register forms hold): the same tree with scalar accesses,
+// x re-read for the second walk. One wave per row.
+template <int ADD>
+__global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (row >= a.rows) return;
+    const int N = a.N;
+    float * xr = a.x + (size_t)row * N;
+    float ssk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int base = 0; base < N; base += 256) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = base + 4 * lane + k;
+            if (i < N) {
+                float xv = xr[i];
+                if (ADD == ADD_F32_SLOTS && a.S > 0) {
+                    const float * dr = (const float *)a.d + (size_t)row * a.S * N;
+                    const float * wr = a.w ? a.w + (size_t)row * a.S : nullptr;
+                    float acc = 0.0f;
+                    for (int s = 0; s < a.S; s++) acc = wr ? __builtin_fmaf(wr[s], dr[(size_t)s * N + i], acc) : acc + dr[(size_t)s * N + i];
+                    xv += acc; xr[i] = xv;
+                }
+                if (ADD == ADD_F32_DIRECT && a.d) { xv = xv + ((const float *)a.d)[(size_t)row * N + i]; xr[i] = xv; }
+                if (ADD == ADD_BF16 && a.d) { xv = xv + bf2f(((const uint16_t *)a.d)[(size_t)row * N + i]); xr[i] = xv; }
+                ssk[k] = __builtin_fmaf(xv, xv, ssk[k]);
+            }
+        }
+    }
+    const f32x4 ss = {ssk[0], ssk[1], ssk[2], ssk[3]};
+    const float tot = wave_groups_in_order(group32_sum(ss));
+    const float scale = rsqrt_exact(tot / (float)N + a.eps);
+    if (a.scl && lane == 0) a.scl[row] = scale;
+    const float * gw = a.nw + (size_t)(row % a.wr) * N;
+    // (a lane re-reads only elements it stored itself: program order covers it)
+    for (int base = 0; base < N; base += 256) {
+        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        float vk[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = base + 4 * lane + k;
+            vk[k] = 0.0f;
+            if (i < N) {
+                vk[k] = (xr[i] * scale) * gw[i];
+                const size_t o = (size_t)row * N + i;
+                if (a.h) a.h[o] = vk[k];
+                if (a.h16) a.h16[(size_t)row * a.ld16 + i] = f2h_bits(vk[k]);
+                if (a.hbf) a.hbf[o] = to_bf16(vk[k]);
+            }
+        }
+        v.x = vk[0]; v.y = vk[1]; v.z = vk[2]; v.w = vk[3];
+        if (a.q8 && base + 4 * (lane & ~7) < N)    // N % 32 == 0 is checked on the host when a q8 copy is asked for
+            q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + (base >> 5) + (lane >> 3)) * 36, lane & 7);
+    }
+}
+
+template <int ADD>
+static int launch_norm(const NormArgs & a, hipStream_t st) {
+    if (a.rows <= 0) return CAMX_OK;
+    const dim3 grid((a.rows + 3) / 4), block(256);
+    const int ni = a.N >> 8;
+    const bool vec = (a.N & 255) == 0 && ni <= 32 && (a.ld16 & 3) == 0 &&
+                     ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.nw & 15) == 0 && ((uintptr_t)a.d & 15) == 0 && ((uintptr_t)a.h & 15) == 0 &&
+                     ((uintptr_t)a.h16 & 7) == 0 && ((uintptr_t)a.hbf & 7) == 0 && ((uintptr_t)a.q8 & 3) == 0;
+    if (!vec) add_rms_rows_any<ADD><<<grid, block, 0, st>>>(a);
+    else if (ni <= 8) add_rms_rows<8, ADD><<<grid, block, 0, st>>>(a);
+    else if (ni <= 16) add_rms_rows<16, ADD><<<grid, block, 0, st>>>(a);
+    else if (ni <= 24) add_rms_rows<24, ADD><<<grid, block, 0, st>>>(a);
+    else add_rms_rows<32, ADD><<<grid, block, 0, st>>>(a);
+    CAMX_LAUNCH_RET();
+}
+
+extern "C" {
+
+int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
+                       uint16_t * h16, int N, int n, hipStream_t st) {
+    if (N < 256 || N % 256 || N > 2048 || S < 0 || S > 8 || n < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
+    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n};
+    return launch_norm<ADD_F32_SLOTS>(a, st);
+}
+
+int camx_q35p_add_rms16(float * x, const float * d, const float * nw, float eps, float * h, uint16_t * h16, int N, int n, hipStream_t st) {
+    if (N < 256 || N % 256 || N > 65536 || n < 0 || !x || !nw || !h || !h16) return CAMX_EINVAL;
+    NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n};
+    return launch_norm<ADD_F32_DIRECT>(a, st);
+}
+
+int camx_add_rms_q8_1(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
+                      uint16_t * h16, uint8_t * q8, int N, int n, hipStream_t st) {
+    if (N < 32 || N % 32 || S < 0 || S > 8 || n < 0 || !x || !nw || (S > 0 && !d)) return CAMX_EINVAL;
+    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, q8, nullptr, N, n};
+    return launch_norm<ADD_F32_SLOTS>(a, st);
+}
+
+int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps, float * h, uint16_t * hbf, int N, int n, hipStream_t st) {
+    if (N < 1 || n < 0 || !x || !nw) return CAMX_EINVAL;
+    NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, nullptr, N, hbf, nullptr, nullptr, N, n};
+    return launch_norm<ADD_BF16>(a, st);
+}
+
+int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf, float * scl, int R, int wr, float eps, int K, hipStream_t st) {
+    if (K < 1 || R < 0 || wr < 1 || !x || !w) return CAMX_EINVAL;
+    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, ybf, nullptr, scl, K, R};
+    return launch_norm<ADD_NONE>(a, st);
+}
+
+int camx_op_rms_mul(const float * x, const float * w, float * y, uint8_t * q8, int R, int wr, int K, float eps, hipStream_t st) {
+    if (K < 1 || R < 0 || wr < 1 || !x || !w || (q8 && K % 32)) return CAMX_EINVAL;
+    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, nullptr, q8, nullptr, K, R};
+    return launch_norm<ADD_NONE>(a, st);
+}
+
+int camx_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows, hipStream_t st) {
+    if (D < 1 || rows < 0 || !x || !w || !out) return CAMX_EINVAL;
+    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, 1, eps, out, nullptr, D, nullptr, nullptr, nullptr, D, rows};
+    return launch_norm<ADD_NONE>(a, st);
+}
+
+}   // extern "C"

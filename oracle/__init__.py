@@ -1,0 +1,338 @@
+"""numpy front end of the CPU oracle (oracle/camx_oracle.c). TEST INFRASTRUCTURE ONLY: tests, the smoke check and the
+benchmark's cpu_baseline leg import this; nothing in the product package does.
+
+Every wrapper takes and returns numpy arrays; in/out arguments are copied first, so callers' arrays never change.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import build as _build
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.isfile(_build.ORC_SO):
+            _build.build_oracle()
+        L = C.CDLL(_build.ORC_SO)
+        for n, r in (('orc_bf2f', C.c_float), ('orc_h2f', C.c_float), ('orc_row_ss', C.c_float), ('orc_bfly32_sum', C.c_float)):
+            getattr(L, n).restype = r
+        for n in ('orc_f2bf', 'orc_to_bf16', 'orc_f2h'):
+            getattr(L, n).restype = C.c_uint16
+            getattr(L, n).argtypes = [C.c_float]
+        L.orc_bf2f.argtypes = [C.c_uint16]; L.orc_h2f.argtypes = [C.c_uint16]
+        L.orc_row_ss.argtypes = [C.c_void_p, C.c_int]
+        L.orc_bfly32_sum.argtypes = [C.c_void_p]
+        _lib = L
+    return _lib
+
+
+def ref_codec():
+    """the reference's own_kv_codec.h compiled for the host (oracle/_ref), or None when it was never built here"""
+    global _ref
+    if _ref is None and os.path.isfile(_build.REF_SO):
+        _ref = C.CDLL(_build.REF_SO)
+    return _ref
+
+
+def _p(a):
+    return C.c_void_p(a.ctypes.data) if a is not None else C.c_void_p(None)
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+I, F, L64 = C.c_int, C.c_float, C.c_int64
+
+# ---- conversions -------------------------------------------------------------------------------------------------------
+
+
+def f2h(x):
+    x = _c(x, np.float32); y = np.empty(x.shape, np.uint16)
+    lib().orc_f2h_n(_p(x), _p(y), L64(x.size)); return y
+
+
+def h2f(h):
+    h = _c(h, np.uint16); y = np.empty(h.shape, np.float32)
+    lib().orc_h2f_n(_p(h), _p(y), L64(h.size)); return y
+
+
+def f2bf(x):
+    x = _c(x, np.float32); y = np.empty(x.shape, np.uint16)
+    lib().orc_cast_bf16(_p(x), _p(y), L64(x.size)); return y
+
+
+def bf2f(h):
+    return (_c(h, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def row_ss(x):
+    x = _c(x, np.float32); return np.float32(lib().orc_row_ss(_p(x), I(x.size)))
+
+
+# ---- q8_1 ----------------------------------------------------------------------------------------------------------------
+
+
+def q8_1(x, mode=0, rs=0.0, g=None):
+    """uint8 [ceil(n / 32), 36]"""
+    x = _c(x, np.float32).reshape(-1); n = x.size
+    g = _c(g, np.float32).reshape(-1) if g is not None else None
+    y = np.zeros(((n + 31) // 32, 36), np.uint8)
+    lib().orc_q8_1(_p(x), _p(y), L64(n), I(mode), F(rs), _p(g)); return y
+
+
+def k_pad(K):
+    return (int(K) + 511) // 512 * 512
+
+
+def mmq_q8_1(x, K, ncols, layout, s01=None, ids=None):
+    """uint8 [K_pad / 128, ncols, 144]"""
+    x = _c(x, np.float32); s01 = K if s01 is None else s01
+    ids = _c(ids, np.int32) if ids is not None else None
+    y = np.zeros((k_pad(K) // 128, ncols, 144), np.uint8)
+    lib().orc_mmq_q8_1(_p(x), _p(ids), _p(y), L64(K), L64(s01), I(ncols), I(layout)); return y
+
+
+def mmq_q8_1_scatter(x, K, ntok, ids_inv, k, layout, s_tok=None, fill=0):
+    x = _c(x, np.float32); s_tok = K if s_tok is None else s_tok
+    ids_inv = _c(ids_inv, np.int32)
+    y = np.full((k_pad(K) // 128, ntok * k, 144), fill, np.uint8)
+    lib().orc_mmq_q8_1_scatter(_p(x), _p(ids_inv), _p(y), L64(K), L64(s_tok), I(ntok), I(k), I(layout)); return y
+
+
+# ---- norms ---------------------------------------------------------------------------------------------------------------
+
+
+def add_rms16(x, nw, eps, d=None, w=None, S=0, want_q8=False):
+    """-> dict(x, h, h16[, q8]); x [n, N]"""
+    x = _c(x, np.float32).copy(); n, N = x.shape
+    d = _c(d, np.float32) if d is not None else None
+    w = _c(w, np.float32) if w is not None else None
+    nw = _c(nw, np.float32)
+    h = np.empty_like(x); h16 = np.empty(x.shape, np.uint16)
+    q8 = np.zeros((n, N // 32, 36), np.uint8) if want_q8 else None
+    lib().orc_add_rms16(_p(x), _p(d), _p(w), I(S), _p(nw), F(eps), _p(h), _p(h16), _p(q8), I(N), I(n))
+    out = dict(x=x, h=h, h16=h16)
+    if want_q8: out['q8'] = q8
+    return out
+
+
+def add_rms16_q35(x, nw, eps, d=None):
+    x = _c(x, np.float32).copy(); n, N = x.shape
+    d = _c(d, np.float32) if d is not None else None
+    h = np.empty_like(x); h16 = np.empty(x.shape, np.uint16)
+    lib().orc_add_rms16_q35(_p(x), _p(d), _p(_c(nw, np.float32)), F(eps), _p(h), _p(h16), I(N), I(n))
+    return dict(x=x, h=h, h16=h16)
+
+
+def add_rms_bf16(x, d, nw, eps):
+    x = _c(x, np.float32).copy(); n, N = x.shape
+    d = _c(d, np.uint16) if d is not None else None
+    h = np.empty_like(x); hbf = np.empty(x.shape, np.uint16)
+    lib().orc_add_rms_bf16(_p(x), _p(d), _p(_c(nw, np.float32)), F(eps), _p(h), _p(hbf), I(N), I(n))
+    return dict(x=x, h=h, hbf=hbf)
+
+
+def rms_mul(x, w, eps, want_q8=False):
+    x = _c(x, np.float32); R, K = x.shape
+    w = _c(w, np.float32).reshape(-1, K); wr = w.shape[0]
+    y = np.empty_like(x); ybf = np.empty(x.shape, np.uint16); scl = np.empty(R, np.float32)
+    q8 = np.zeros((R, K // 32, 36), np.uint8) if want_q8 else None
+    lib().orc_rms_mul(_p(x), _p(w), _p(y), _p(ybf), _p(scl), _p(q8), I(R), I(wr), I(K), F(eps))
+    out = dict(y=y, ybf=ybf, scale=scl)
+    if want_q8: out['q8'] = q8
+    return out
+
+
+def rmsnorm_f32(x, w, eps):
+    x = _c(x, np.float32); rows, D = x.shape; out = np.empty_like(x)
+    lib().orc_rmsnorm_f32(_p(x), _p(_c(w, np.float32)), _p(out), I(D), F(eps), I(rows)); return out
+
+
+# ---- core / fuse -----------------------------------------------------------------------------------------------------------
+
+
+def embedding_f32(tok, emb):
+    tok = _c(tok, np.int32); emb = _c(emb, np.float32); out = np.empty((tok.size, emb.shape[1]), np.float32)
+    lib().orc_embedding_f32(_p(tok), _p(emb), _p(out), I(emb.shape[1]), I(tok.size)); return out
+
+
+def silu_mul_bf16(gu):
+    gu = _c(gu, np.uint16); R, H2 = gu.shape; H = H2 // 2; act = np.empty((R, H), np.uint16)
+    lib().orc_silu_mul_bf16(_p(gu), _p(act), I(H), L64(R * H)); return act
+
+
+def residual3(x, m, y):
+    x = _c(x, np.float32); out = np.empty_like(x)
+    lib().orc_residual3(_p(x), _p(_c(m, np.uint16)), _p(_c(y, np.uint16)), _p(out), L64(x.size)); return out
+
+
+def copy_cols_bf16(inp, c_in, out, c_out, n):
+    inp = _c(inp, np.uint16); out = _c(out, np.uint16).copy()
+    lib().orc_copy_cols_bf16(_p(inp), I(inp.shape[1]), I(c_in), _p(out), I(out.shape[1]), I(c_out), I(n), L64(inp.shape[0])); return out
+
+
+def residual_slices_fwd(x, m, mlp, ys, pos):
+    x = _c(x, np.float32); d = x.shape[-1]; out = np.empty_like(x)
+    ys = _c(ys, np.uint16) if ys is not None else None
+    pos = _c(pos, np.int32) if pos is not None else None
+    lib().orc_residual_slices_fwd(_p(x), _p(_c(m, np.uint16)), _p(_c(mlp, np.uint16)), _p(ys), _p(pos), _p(out), I(d), L64(x.size // 4))
+    return out
+
+
+# ---- SwiGLU / gates / GDN ----------------------------------------------------------------------------------------------------
+
+
+def swiglu16(g, u):
+    g = _c(g, np.float32); y = np.empty(g.shape, np.uint16)
+    lib().orc_swiglu16(_p(g), _p(_c(u, np.float32)), _p(y), L64(g.size)); return y
+
+
+def silu_mul_f32(g, u):
+    g = _c(g, np.float32); y = np.empty_like(g)
+    lib().orc_silu_mul_f32(_p(g), _p(_c(u, np.float32)), _p(y), L64(g.size)); return y
+
+
+def gate_mul(a, gate, D, stride, off, f16=False):
+    a = _c(a, np.float32); gate = _c(gate, np.float32)
+    y = np.empty(a.shape, np.float32); y16 = np.empty(a.shape, np.uint16) if f16 else None
+    lib().orc_gate_mul(_p(a), _p(gate), _p(y), _p(y16), L64(a.size), I(D), I(stride), I(off))
+    return y16 if f16 else y
+
+
+def gdn_conv(x, w, st, ldx=None, ldy=None):
+    """-> (y [T, C], new state [C, 3]); x [T, ldx]"""
+    x = _c(x, np.float32); w = _c(w, np.float32); st = _c(st, np.float32).copy()
+    T = x.shape[0]; C_ = w.shape[0]; ldx = x.shape[1] if ldx is None else ldx; ldy = C_ if ldy is None else ldy
+    y = np.zeros((T, ldy), np.float32)
+    lib().orc_gdn_conv(_p(x), _p(w), _p(st), _p(y), I(C_), I(T), I(ldx), I(ldy))
+    lib().orc_conv_state(_p(x), _p(st), I(C_), I(T), I(ldx))
+    return y, st
+
+
+def gdn_l2(x, T, heads, K, eps, ldx=None):
+    x = _c(x, np.float32); ldx = heads * K if ldx is None else ldx
+    y = np.empty((T * heads, K), np.float32)
+    lib().orc_gdn_l2(_p(x), _p(y), I(T), I(heads), I(K), I(ldx), F(np.float32(eps / K))); return y
+
+
+# ---- rotary ---------------------------------------------------------------------------------------------------------------
+
+
+def qk_nr(x, head_stride, heads, w, D, n_rot, theta_scale, eps, pos0, T):
+    x = _c(x, np.float32); out = np.empty((T * heads, D), np.float32)
+    lib().orc_qk_nr(_p(x), I(head_stride), I(heads), _p(_c(w, np.float32)), I(D), I(n_rot), F(theta_scale), F(eps), I(pos0), _p(out), I(T))
+    return out
+
+
+def qk_rope(qkv, nh, nkv, par, n, pos0=0, pos=None, yarn=False, q8=False, cache=None, rows=None,
+            page_table=None, page=256, n_pages=0):
+    """-> (q16 uint16 [n, nh, 128], cache, err). cache: given (copied) or zeros of `rows` rows; fp16 rows as uint16
+    [rows, 2 M], Q8 rows as uint8 [rows, row_bytes]."""
+    qkv = _c(qkv, np.float32); ldq = qkv.shape[1]; M = nkv * 128
+    par = _c(par, np.float32)
+    q16 = np.zeros((n, nh, 128), np.uint16)
+    if cache is None:
+        cache = np.zeros((rows, 2 * (M // 32) * 34), np.uint8) if q8 else np.zeros((rows, 2 * M), np.uint16)
+    else:
+        cache = cache.copy()
+    err = np.zeros(1, np.int32)
+    pos = _c(pos, np.int32) if pos is not None else None
+    pt = _c(page_table, np.int32) if page_table is not None else None
+    lib().orc_qk_rope(_p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(pos0), _p(pos), _p(q16), _p(cache), I(n), I(int(yarn)), I(int(q8)),
+                      _p(err), _p(pt), I(pt.shape[1] if pt is not None else 0), I(page), I(n_pages))
+    return q16, cache, int(err[0])
+
+
+# ---- Hadamard / KV codec ------------------------------------------------------------------------------------------------------
+
+
+def hadamard128(x):
+    x = _c(x, np.float32); y = np.empty_like(x)
+    lib().orc_hadamard128(_p(x), _p(y), L64(x.size // 128)); return y
+
+
+def hadamard_n(x, n):
+    x = _c(x, np.float32).copy()
+    lib().orc_hadamard_n(_p(x), L64(x.size // n), I(n)); return x
+
+
+def kv_q8_encode(blocks, fill=0xa5):
+    """blocks float32 [nb, 32] -> (bytes uint8 [nb, 34] (refused blocks keep `fill`), ok uint8 [nb])"""
+    b = _c(blocks, np.float32).reshape(-1, 32); raw = np.full((b.shape[0], 34), fill, np.uint8); ok = np.zeros(b.shape[0], np.uint8)
+    lib().orc_kv_q8_encode(_p(b), _p(raw), _p(ok), L64(b.shape[0])); return raw, ok
+
+
+def ref_kv_q8_encode(blocks, fill=0xa5):
+    """the same through the compiled reference header (None when oracle/_ref was not built)"""
+    r = ref_codec()
+    if r is None: return None
+    b = _c(blocks, np.float32).reshape(-1, 32); raw = np.full((b.shape[0], 34), fill, np.uint8); ok = np.zeros(b.shape[0], np.uint8)
+    r.ref_kv_q8_encode(_p(b), _p(raw), _p(ok), C.c_long(b.shape[0])); return raw, ok
+
+
+def kv_q8_append(k, ldk, v, ldv, M, cache, pos0, T, rows=None):
+    """-> (cache bytes (copy), err)"""
+    k = _c(k, np.float32); v = _c(v, np.float32); cache = _c(cache, np.uint8).copy()
+    rb = 2 * (M // 32) * 34 if M >= 32 else 1
+    rows = cache.size // rb if rows is None else rows
+    err = np.zeros(1, np.int32)
+    lib().orc_kv_q8_append(_p(k), I(ldk), _p(v), I(ldv), I(M), _p(cache), I(pos0), I(rows), I(T), _p(err))
+    return cache, int(err[0])
+
+
+def pf_kv_append(k, ldk, v, ldv, M, cache, pos0, T, rows=None):
+    k = _c(k, np.float32); v = _c(v, np.float32); cache = _c(cache, np.uint8).copy()
+    rb = 2 * (M // 32) * 34
+    rows = cache.size // rb if rows is None else rows
+    err = np.zeros(1, np.int32)
+    lib().orc_pf_kv_append(_p(k), I(ldk), _p(v), I(ldv), I(M), _p(cache), I(pos0), I(rows), I(T), _p(err))
+    return cache, int(err[0])
+
+
+# ---- quantized embedding rows ---------------------------------------------------------------------------------------------------
+
+
+def emb_q4k(W, vocab, toks, N):
+    W = _c(W, np.uint8); toks = _c(toks, np.int32); rb = N // 256 * 144
+    x = np.empty((toks.size, N), np.float32); xbf = np.empty((toks.size, N), np.uint16)
+    lib().orc_emb_q4k(_p(W), I(rb), I(vocab), _p(toks), _p(x), _p(xbf), I(N), I(toks.size)); return x, xbf
+
+
+def emb_q8_0(W, vocab, toks, N):
+    W = _c(W, np.uint8); toks = _c(toks, np.int32); rb = N // 32 * 34
+    x = np.empty((toks.size, N), np.float32); xbf = np.empty((toks.size, N), np.uint16)
+    lib().orc_emb_q8_0(_p(W), I(rb), I(vocab), _p(toks), _p(x), _p(xbf), I(N), I(toks.size)); return x, xbf
+
+
+# ---- actq -----------------------------------------------------------------------------------------------------------------------
+
+
+def actq_fwd(x, clip=1.0, qmax=7, bf16=False):
+    """-> (y bf16 bits [M, K], s [M], codes uint8 [M, K / 2])"""
+    x = _c(x, np.uint16 if bf16 else np.float32); M, K = x.shape
+    y = np.empty((M, K), np.uint16); s = np.empty(M, np.float32); c = np.zeros((M, K // 2), np.uint8)
+    lib().orc_actq_fwd(_p(x), I(int(bf16)), _p(y), _p(s), _p(c), I(M), I(K), F(clip), I(qmax)); return y, s, c
+
+
+def silu_mul_actq_fwd(gu, clip=1.0, qmax=7):
+    gu = _c(gu, np.uint16); M, F2 = gu.shape; Fh = F2 // 2
+    y = np.empty((M, Fh), np.uint16); s = np.empty(M, np.float32); c = np.zeros((M, Fh // 2), np.uint8)
+    lib().orc_silu_mul_actq_fwd(_p(gu), I(F2), I(Fh), _p(y), _p(s), _p(c), I(M), F(clip), I(qmax)); return y, s, c
+
+
+def block_entry_fwd(x, nw, wab, eps, clip=1.0, qmax=7):
+    x = _c(x, np.float32); M, d = x.shape
+    nab = 0 if wab is None else wab.shape[0]
+    wab = _c(wab, np.uint16) if nab else None
+    y = np.empty((M, d), np.uint16); s = np.empty(M, np.float32); c = np.zeros((M, d // 2), np.uint8)
+    ab = np.zeros((M, max(nab, 1)), np.uint16); rstd = np.empty(M, np.float32)
+    lib().orc_block_entry_fwd(_p(x), _p(_c(nw, np.float32)), _p(wab), I(nab), F(eps), _p(y), _p(s), _p(c), _p(ab), _p(rstd),
+                              I(M), I(d), F(clip), I(qmax))
+    return y, s, c, ab[:, :nab], rstd

@@ -1,0 +1,77 @@
+"""GPU parity of the residual add + RMSNorm family against the CPU oracle (bit-exact under the contract tree)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from gpu_util import F, I, NULL, bits_equal, call, dev, host, outliers, ptr
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('n,N,S,weighted', [(1, 2048, 1, False), (5, 2048, 8, True), (3, 256, 0, False), (7, 1024, 3, True), (256, 2048, 1, False)])
+def test_q3p_add_rms16(n, N, S, weighted):
+    rng = np.random.default_rng(1001 + n + N + S)
+    x = outliers(rng, (n, N)); d = outliers(rng, (n, max(S, 1), N)); w = rng.random((n, max(S, 1))).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    ref = O.add_rms16(x, nw, 1e-6, d=d if S else None, w=w if weighted else None, S=S)
+    xd, dd, wd, nwd = dev(x), dev(d), dev(w), dev(nw)
+    h = dev(np.zeros((n, N), np.float32)); h16 = dev(np.zeros((n, N), np.uint16))
+    call('camx_q3p_add_rms16', ptr(xd), ptr(dd) if S else NULL, ptr(wd) if weighted else NULL, I(S), ptr(nwd), F(1e-6), ptr(h), ptr(h16), I(N), I(n))
+    assert bits_equal(host(xd), ref['x'])
+    assert bits_equal(host(h), ref['h'])
+    assert bits_equal(host(h16, np.uint16), ref['h16'])
+
+
+@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096)])
+def test_q35p_add_rms16(n, N):
+    rng = np.random.default_rng(7 + N)
+    x = outliers(rng, (n, N)); d = outliers(rng, (n, N)); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    for dd_ in (d, None):
+        ref = O.add_rms16_q35(x, nw, 1e-6, d=dd_)
+        xd = dev(x); h = dev(np.zeros((n, N), np.float32)); h16 = dev(np.zeros((n, N), np.uint16)); nwd = dev(nw)
+        ddv = dev(dd_) if dd_ is not None else None
+        call('camx_q35p_add_rms16', ptr(xd), ptr(ddv), ptr(nwd), F(1e-6), ptr(h), ptr(h16), I(N), I(n))
+        assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
+
+
+@pytest.mark.parametrize('n,N', [(4, 2048), (256, 2048), (2, 5120)])
+def test_add_rms_q8_1(n, N):
+    rng = np.random.default_rng(1002 + N)
+    x = outliers(rng, (n, N)); d = outliers(rng, (n, 1, N)); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    ref = O.add_rms16(x, nw, 1e-6, d=d, S=1, want_q8=True)
+    xd, dd, nwd = dev(x), dev(d), dev(nw)
+    h = dev(np.zeros((n, N), np.float32)); q8 = dev(np.zeros((n, N // 32, 36), np.uint8))
+    call('camx_add_rms_q8_1', ptr(xd), ptr(dd), NULL, I(1), ptr(nwd), F(1e-6), ptr(h), NULL, ptr(q8), I(N), I(n))
+    assert bits_equal(host(h), ref['h'])
+    assert bits_equal(host(q8), ref['q8'])
+
+
+@pytest.mark.parametrize('n,N', [(3, 5120), (64, 5120), (2, 2048)])
+def test_add_rms_bf16(n, N):
+    rng = np.random.default_rng(1003 + N)
+    x = outliers(rng, (n, N)); d = O.f2bf(outliers(rng, (n, N))); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    ref = O.add_rms_bf16(x, d, nw, 1e-6)
+    xd, dd, nwd = dev(x), dev(d), dev(nw)
+    h = dev(np.zeros((n, N), np.float32)); hbf = dev(np.zeros((n, N), np.uint16))
+    call('camx_add_rms_bf16', ptr(xd), ptr(dd), ptr(nwd), F(1e-6), ptr(h), ptr(hbf), I(N), I(n))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(hbf, np.uint16), ref['hbf'])
+
+
+@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2)])
+def test_rms_mul_and_rmsnorm(R, K, wr):
+    rng = np.random.default_rng(R * K)
+    x = outliers(rng, (R, K)); w = (1 + 0.1 * rng.standard_normal((wr, K))).astype(np.float32)
+    if R % wr: R = R // wr * wr; x = x[:R]
+    ref = O.rms_mul(x, w, 1e-6, want_q8=K % 32 == 0)
+    xd, wd = dev(x), dev(w)
+    y = dev(np.zeros((R, K), np.float32)); ybf = dev(np.zeros((R, K), np.uint16)); scl = dev(np.zeros(R, np.float32))
+    call('camx_pf_rms_mul', ptr(xd), ptr(wd), ptr(y), ptr(ybf), ptr(scl), I(R), I(wr), F(1e-6), I(K))
+    assert bits_equal(host(y), ref['y']) and bits_equal(host(ybf, np.uint16), ref['ybf']) and bits_equal(host(scl), ref['scale'])
+    if K % 32 == 0:
+        q8 = dev(np.zeros((R, K // 32, 36), np.uint8)); y2 = dev(np.zeros((R, K), np.float32))
+        call('camx_op_rms_mul', ptr(xd), ptr(wd), ptr(y2), ptr(q8), I(R), I(wr), I(K), F(1e-6))
+        assert bits_equal(host(y2), ref['y']) and bits_equal(host(q8), ref['q8'])
+    if wr == 1:
+        out = dev(np.zeros((R, K), np.float32))
+        call('camx_rmsnorm_f32', ptr(xd), ptr(wd), ptr(out), I(K), F(1e-6), I(R))
+        assert bits_equal(host(out), O.rmsnorm_f32(x, w[0], 1e-6))
