@@ -1,0 +1,281 @@
+// Elementwise and small row kernels for gfx950: SwiGLU and sigmoid gates, the GDN short convolution and L2 norm, and the
+// S1 core's gather / cast / residual kernels. Replaces q3p_swiglu / OP_OWN_SWIGLU16 (kernels/q3m_prefill.hip:516-518,
+// kernels/k3_own_ops.h:258-262), gg_silu_mul (kernels/k3_gguf.hip:74-77), pf_gate_mul / q35p_gate_mul16
+// (kernels/prefill_attn.hip:379-386, kernels/q35_prefill.hip:960-969), pf_gdn_conv / pf_conv_state
+// (kernels/prefill_glue.hip:314-341), pf_gdn_l2 (kernels/prefill_gdn.hip:66-78), kernels/core.hip and
+// residual_slices_fwd (kernels/fuse.hip:19-33). Four elements per lane, 128-bit accesses where alignment allows.
+#include "common.cuh"
+
+CAMX_DEV float silu_f(float x) { return x / (1.0f + expf(-x)); }
+CAMX_DEV float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+#define GRID_1D(n4) dim3((unsigned)((((n4) + 255) / 256) < 1048576 ? (((n4) + 255) / 256) : 1048576))
+
+// y16[i] = fp16(silu(g[i]) * u[i]); out_f32: y32[i] = silu(g[i]) * u[i]
+template <bool F16OUT>
+__global__ void __launch_bounds__(256) swiglu_f32(const float * __restrict__ g, const float * __restrict__ u, void * __restrict__ y, long n, int vec) {
+    const long stride = (long)gridDim.x * 256;
+    for (long q = (long)blockIdx.x * 256 + threadIdx.x; q * 4 < n; q += stride) {
+        const long i = q * 4;
+        float gv[4], uv[4], r[4];
+        if (vec && i + 3 < n) {
+            const f32x4 a = *(const f32x4 *)(g + i), b = *(const f32x4 *)(u + i);
+            gv[0] = a.x; gv[1] = a.y; gv[2] = a.z; gv[3] = a.w; uv[0] = b.x; uv[1] = b.y; uv[2] = b.z; uv[3] = b.w;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; k++) { gv[k] = i + k < n ? g[i + k] : 0.0f; uv[k] = i + k < n ? u[i + k] : 0.0f; }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) r[k] = gv[k] / (1.0f + expf(-gv[k])) * uv[k];
+        if (vec && i + 3 < n) {
+            if (F16OUT) *(u32x2 *)((uint16_t *)y + i) = pack_f16x4((f32x4){r[0], r[1], r[2], r[3]});
+            else *(f32x4 *)((float *)y + i) = (f32x4){r[0], r[1], r[2], r[3]};
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                if (i + k < n) { if (F16OUT) ((uint16_t *)y)[i + k] = f2h_bits(r[k]); else ((float *)y)[i + k] = r[k]; }
+        }
+    }
+}
+
+// silu_mul_bf16: act[r][c] = bf16(bf16(silu(g)) * u), gu rows = [g (H) | u (H)]
+__global__ void __launch_bounds__(256) silu_mul_bf16_k(const uint16_t * __restrict__ gu, uint16_t * __restrict__ act, int H, long n, int vec) {
+    const long stride = (long)gridDim.x * 256;
+    for (long q = (long)blockIdx.x * 256 + threadIdx.x; q * 4 < n; q += stride) {
+        const long i = q * 4;
+        if (vec) {     // H % 4 == 0: the four elements share a row
+            const long r = i / H, c = i - r * H;
+            const f32x4 g = unpack_bf16x4(*(const u32x2 *)(gu + r * 2 * H + c)), u = unpack_bf16x4(*(const u32x2 *)(gu + r * 2 * H + H + c));
+            f32x4 a;
+            a.x = rbf(silu_f(g.x)) * u.x; a.y = rbf(silu_f(g.y)) * u.y; a.z = rbf(silu_f(g.z)) * u.z; a.w = rbf(silu_f(g.w)) * u.w;
+            *(u32x2 *)(act + i) = pack_f2bf_x4(a);
+        } else {
+            for (int k = 0; k < 4 && i + k < n; k++) {
+                const long r = (i + k) / H, c = (i + k) - r * H;
+                const float g = bf2f(gu[r * 2 * H + c]), u = bf2f(gu[r * 2 * H + H + c]);
+                act[i + k] = f2bf(rbf(silu_f(g)) * u);
+            }
+        }
+    }
+}
+
+// y[i] = a[i] * sigmoid(gate[(i / D) * stride + off + i % D]); IO 0: fp32 a, gate -> fp32 y; 1: fp32 -> fp16 y;
+// 2: bf16 a, gate -> bf16 y (to_bf16)
+template <int IO>
+__global__ void __launch_bounds__(256) gate_mul_k(const void * __restrict__ a, const void * __restrict__ gt, void * __restrict__ y, long N, int D,
+                                                  int stride, int off) {
+    const long step = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < N; i += step) {
+        const long h = i / D; const int d = (int)(i - h * D);
+        const size_t gi = (size_t)h * stride + off + d;
+        const float gv = IO == 2 ? bf2f(((const uint16_t *)gt)[gi]) : ((const float *)gt)[gi];
+        const float av = IO == 2 ? bf2f(((const uint16_t *)a)[i]) : ((const float *)a)[i];
+        const float sgm = 1.0f / (1.0f + expf(-gv));
+        const float v = av * sgm;
+        if (IO == 0) ((float *)y)[i] = v; else if (IO == 1) ((uint16_t *)y)[i] = f2h_bits(v); else ((uint16_t *)y)[i] = to_bf16(v);
+    }
+}
+
+// y[t, c] = silu(fma chain over [x(t-3), x(t-2), x(t-1), x(t)] . w[c]), negative times from st[c] = [x(-3), x(-2), x(-1)]
+template <bool BF16>
+__global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
+                                                  void * __restrict__ y, int C, int T, int ldx, int ldy) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)T * C) return;
+    const int t = (int)(i / C), c = (int)(i - (long)t * C);
+    const f32x4 w4 = *(const f32x4 *)(w + (size_t)c * 4);
+    float in[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int tj = t - 3 + j;
+        if (tj >= 0) in[j] = BF16 ? bf2f(((const uint16_t *)x)[(size_t)tj * ldx + c]) : ((const float *)x)[(size_t)tj * ldx + c];
+        else in[j] = st[(size_t)c * 3 + 3 + tj];
+    }
+    float sumf = 0.0f;
+    sumf = __builtin_fmaf(in[0], w4.x, sumf); sumf = __builtin_fmaf(in[1], w4.y, sumf);
+    sumf = __builtin_fmaf(in[2], w4.z, sumf); sumf = __builtin_fmaf(in[3], w4.w, sumf);
+    const float r = silu_f(sumf);
+    if (BF16) ((uint16_t *)y)[(size_t)t * ldy + c] = to_bf16(r); else ((float *)y)[(size_t)t * ldy + c] = r;
+}
+template <bool BF16>
+__global__ void __launch_bounds__(256) conv_state_k(const void * __restrict__ x, float * __restrict__ st, int C, int T, int ldx) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float s[3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int tj = T - 3 + j;
+        if (tj >= 0) s[j] = BF16 ? bf2f(((const uint16_t *)x)[(size_t)tj * ldx + c]) : ((const float *)x)[(size_t)tj * ldx + c];
+        else s[j] = st[(size_t)c * 3 + 3 + tj];
+    }
+#pragma unroll
+    for (int j = 0; j < 3; j++) st[(size_t)c * 3 + j] = s[j];
+}
+
+// per head of K <= 512 values: y = (scale * x) * (1 / sqrt(K)), scale = 1 / sqrt(sum x^2 / K + rs); one wave per head
+template <bool BF16>
+__global__ void __launch_bounds__(256) gdn_l2_k(const void * __restrict__ x, void * __restrict__ y, int heads, int K, int ldx, float rs, int total) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (t >= total) return;
+    const int tt = t / heads, hh = t - tt * heads;
+    const size_t xo = (size_t)tt * ldx + (size_t)hh * K, yo = (size_t)t * K;
+    float xv[2][4];
+    f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = 256 * j + 4 * lane + k;
+            xv[j][k] = 0.0f;
+            if (i < K) xv[j][k] = BF16 ? bf2f(((const uint16_t *)x)[xo + i]) : ((const float *)x)[xo + i];
+        }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {   // (an absent element adds fma(0, 0, s) = s: the tree's threads past K hold 0)
+        ss.x = __builtin_fmaf(xv[j][0], xv[j][0], ss.x); ss.y = __builtin_fmaf(xv[j][1], xv[j][1], ss.y);
+        ss.z = __builtin_fmaf(xv[j][2], xv[j][2], ss.z); ss.w = __builtin_fmaf(xv[j][3], xv[j][3], ss.w);
+    }
+    const float tot = wave_groups_in_order(group32_sum(ss));
+    const float scale = rsqrt_exact(tot / (float)K + rs), s2 = 1.0f / sqrtf((float)K);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = 256 * j + 4 * lane + k;
+            if (i < K) {
+                const float v = (scale * xv[j][k]) * s2;
+                if (BF16) ((uint16_t *)y)[yo + i] = to_bf16(v); else ((float *)y)[yo + i] = v;
+            }
+        }
+}
+
+// ---- S1 core / fuse ----------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) embedding_f32_k(const int * __restrict__ tok, const float * __restrict__ emb, float * __restrict__ out, int D) {
+    const int t = blockIdx.x;
+    const float * src = emb + (size_t)tok[t] * D;
+    for (int j = threadIdx.x; j < D; j += 256) out[(size_t)t * D + j] = src[j];
+}
+__global__ void __launch_bounds__(256) residual3_k(const float * __restrict__ x, const uint16_t * __restrict__ m, const uint16_t * __restrict__ y,
+                                                   float * __restrict__ out, long n) {
+    const long step = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += step) out[i] = (x[i] + bf2f(m[i])) + bf2f(y[i]);
+}
+__global__ void __launch_bounds__(256) cast_bf16_k(const float * __restrict__ x, uint16_t * __restrict__ out, long n) {
+    const long step = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += step) out[i] = f2bf(x[i]);
+}
+__global__ void __launch_bounds__(256) copy_cols_bf16_k(const uint16_t * __restrict__ in, int ld_in, int c_in, uint16_t * __restrict__ out, int ld_out,
+                                                        int c_out, int n, long rows) {
+    const long step = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < rows * n; i += step) {
+        const long r = i / n, c = i - r * n;
+        out[r * ld_out + c_out + c] = in[r * ld_in + c_in + c];
+    }
+}
+// out = ((x + m) + mlp) + (pos[r] >= 0 ? ys[pos[r]] : 0), four columns per thread (d % 4 == 0)
+__global__ void __launch_bounds__(256) residual_slices_fwd_k(const float * __restrict__ x, const uint16_t * __restrict__ m, const uint16_t * __restrict__ mlp,
+                                                             const uint16_t * __restrict__ ys, const int * __restrict__ pos, float * __restrict__ out, int d, long n4) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const long e = i * 4; const int r = (int)(e / d), c = (int)(e % d);
+    const f32x4 xv = *(const f32x4 *)(x + e);
+    const f32x4 mv = unpack_bf16x4(*(const u32x2 *)(m + e)), lv = unpack_bf16x4(*(const u32x2 *)(mlp + e));
+    const int p = pos ? pos[r] : -1;
+    f32x4 sv = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (p >= 0) sv = unpack_bf16x4(*(const u32x2 *)(ys + (size_t)p * d + c));
+    f32x4 o;
+    o.x = ((xv.x + mv.x) + lv.x) + sv.x; o.y = ((xv.y + mv.y) + lv.y) + sv.y;
+    o.z = ((xv.z + mv.z) + lv.z) + sv.z; o.w = ((xv.w + mv.w) + lv.w) + sv.w;
+    *(f32x4 *)(out + e) = o;
+}
+
+extern "C" {
+
+int camx_q3p_swiglu(const float * g, const float * u, uint16_t * y, int n, hipStream_t st) {
+    if (!g || !u || !y || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const int vec = !(((uintptr_t)g | (uintptr_t)u) & 15) && !((uintptr_t)y & 7);
+    swiglu_f32<true><<<GRID_1D(((long)n + 3) / 4), dim3(256), 0, st>>>(g, u, y, n, vec);
+    CAMX_LAUNCH_RET();
+}
+int camx_gg_silu_mul(const float * g, const float * u, float * h, int n, hipStream_t st) {
+    if (!g || !u || !h || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const int vec = !(((uintptr_t)g | (uintptr_t)u | (uintptr_t)h) & 15);
+    swiglu_f32<false><<<GRID_1D(((long)n + 3) / 4), dim3(256), 0, st>>>(g, u, h, n, vec);
+    CAMX_LAUNCH_RET();
+}
+int camx_silu_mul_bf16(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st) {
+    if (!gu || !act || H < 1 || n < 0 || n % H) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const int vec = H % 4 == 0 && !(((uintptr_t)gu | (uintptr_t)act) & 7);
+    silu_mul_bf16_k<<<GRID_1D((n + 3) / 4), dim3(256), 0, st>>>(gu, act, H, n, vec);
+    CAMX_LAUNCH_RET();
+}
+// io: 0 fp32 -> fp32 (pf_gate_mul), 1 fp32 -> fp16 (q35p_gate_mul16), 2 bf16 -> bf16
+int camx_gate_mul(const void * a, const void * gt, void * y, long N, int D, int stride, int off, int io, hipStream_t st) {
+    if (!a || !gt || !y || N < 0 || D < 1 || N % D || off < 0 || off + D > stride || io < 0 || io > 2) return CAMX_EINVAL;
+    if (N == 0) return CAMX_OK;
+    const dim3 grid = GRID_1D(N), block(256);
+    if (io == 0) gate_mul_k<0><<<grid, block, 0, st>>>(a, gt, y, N, D, stride, off);
+    else if (io == 1) gate_mul_k<1><<<grid, block, 0, st>>>(a, gt, y, N, D, stride, off);
+    else gate_mul_k<2><<<grid, block, 0, st>>>(a, gt, y, N, D, stride, off);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void * y, int C, int T, int ldx, int ldy, int bf16, hipStream_t st) {
+    if (!x || !w || !state || !y || C < 1 || T < 1 || ldx < C || ldy < C || ((uintptr_t)w & 15)) return CAMX_EINVAL;
+    const dim3 grid((unsigned)(((long)T * C + 255) / 256)), block(256);
+    if (bf16) gdn_conv_k<true><<<grid, block, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
+    else gdn_conv_k<false><<<grid, block, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_conv_state(const void * x, float * state, int C, int T, int ldx, int bf16, hipStream_t st) {
+    if (!x || !state || C < 1 || T < 1 || ldx < C) return CAMX_EINVAL;
+    const dim3 grid((C + 255) / 256), block(256);
+    if (bf16) conv_state_k<true><<<grid, block, 0, st>>>(x, state, C, T, ldx);
+    else conv_state_k<false><<<grid, block, 0, st>>>(x, state, C, T, ldx);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs, int T, int bf16, hipStream_t st) {
+    if (!x || !y || heads < 1 || K < 1 || K > 512 || T < 0 || ldx < heads * K) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    const int total = T * heads;
+    const dim3 grid((total + 3) / 4), block(256);
+    if (bf16) gdn_l2_k<true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total);
+    else gdn_l2_k<false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total);
+    CAMX_LAUNCH_RET();
+}
+int camx_embedding_f32(const int * tok, const float * emb, float * out, int D, int T, hipStream_t st) {
+    if (!tok || !emb || !out || D < 1 || T < 0) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    embedding_f32_k<<<dim3(T), dim3(256), 0, st>>>(tok, emb, out, D);
+    CAMX_LAUNCH_RET();
+}
+int camx_residual3(const float * x, const uint16_t * m, const uint16_t * y, float * out, long n, hipStream_t st) {
+    if (!x || !m || !y || !out || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    residual3_k<<<GRID_1D(n), dim3(256), 0, st>>>(x, m, y, out, n);
+    CAMX_LAUNCH_RET();
+}
+int camx_cast_bf16(const float * x, uint16_t * out, long n, hipStream_t st) {
+    if (!x || !out || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    cast_bf16_k<<<GRID_1D(n), dim3(256), 0, st>>>(x, out, n);
+    CAMX_LAUNCH_RET();
+}
+int camx_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out, int ld_out, int c_out, int n, long rows, hipStream_t st) {
+    if (!in || !out || n < 0 || rows < 0 || c_in < 0 || c_out < 0 || c_in + n > ld_in || c_out + n > ld_out) return CAMX_EINVAL;
+    if (n == 0 || rows == 0) return CAMX_OK;
+    copy_cols_bf16_k<<<GRID_1D(rows * n), dim3(256), 0, st>>>(in, ld_in, c_in, out, ld_out, c_out, n, rows);
+    CAMX_LAUNCH_RET();
+}
+int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t * mlp, const uint16_t * ys, const int * pos, float * out,
+                             int d, long n4, hipStream_t st) {
+    if (!x || !m || !mlp || !out || d < 4 || d % 4 || n4 < 0 || ((uintptr_t)x & 15) || ((uintptr_t)out & 15) || ((uintptr_t)m & 7) ||
+        ((uintptr_t)mlp & 7) || ((uintptr_t)ys & 7)) return CAMX_EINVAL;
+    if (n4 == 0) return CAMX_OK;
+    residual_slices_fwd_k<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st>>>(x, m, mlp, ys, pos, out, d, n4);
+    CAMX_LAUNCH_RET();
+}
+
+}   // extern "C"

@@ -1,0 +1,139 @@
+// Q8 KV wire codec and Walsh-Hadamard transforms for gfx950. Replaces own_kv_q8_append (kernels/kv_codec.hip:10-30 with
+// kernels/own_kv_codec.h:33-52), pf_kv_append's q8_0 rows (kernels/prefill_attn.hip:157-181) and pf_hadamard /
+// OP_HADAMARD (kernels/prefill_attn.hip:132-153, kernels/k3_gguf_ops.h:1699-1721).
+//
+// A row is [K blocks | V blocks], 34 bytes per 32 values (fp16 scale + 32 int8). 8 lanes x 4 values encode one block; a
+// wave encodes 8 blocks per step. Blocks are only 2-byte aligned, so codes go out as 16-bit stores and a refused block
+// keeps every one of its bytes.
+#include "common.cuh"
+
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+// Error bits: 1 position span, 2 numerical domain, 4 layout.
+__global__ void __launch_bounds__(256) kv_q8_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
+                                                         uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
+    if (M < 32 || M % 32 || ldk < M || ldv < M || rows < 1) {
+        if (threadIdx.x == 0) atomicOr(err, 4);
+        return;
+    }
+    const long pos = (long)pos0 + (long)blockIdx.x;      // widened before the sum: a bad position cannot wrap into a valid row
+    if (pos < 0 || pos >= rows) {
+        if (threadIdx.x == 0) atomicOr(err, 1);
+        return;
+    }
+    const size_t tt = blockIdx.x;
+    const int nb = M / 32, lane = threadIdx.x & 63, sub = lane & 7;
+    uint8_t * dst = cache + (size_t)pos * ((size_t)2 * nb * 34);
+    for (int b0 = (threadIdx.x >> 6) * 8; b0 < 2 * nb; b0 += 32) {
+        const int b = b0 + (lane >> 3);
+        const bool active = b < 2 * nb;
+        const int bb = active ? b : 0;
+        const float * x = (bb < nb ? k + tt * ldk : v + tt * ldv) + (size_t)(bb % nb) * 32 + 4 * sub;
+        const f32x4 xv = *(const f32x4_a4 *)x;
+        kv_q8_emit(xv, dst + (size_t)bb * 34, sub, err, active);
+    }
+}
+
+// pf_kv_append (q8_0 rows): no refusal rules; d stored as half, codes roundf(x * (1 / d)); err bit 1 for a row outside
+__global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
+                                                         uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
+    const int tt = blockIdx.x, pos = pos0 + tt;
+    if (pos < 0 || pos >= rows) { if (threadIdx.x == 0) atomicOr(err, 1); return; }
+    const int nb = M / 32, lane = threadIdx.x & 63, sub = lane & 7;
+    uint8_t * base = cache + (size_t)pos * ((size_t)2 * nb * 34);
+    for (int b0 = (threadIdx.x >> 6) * 8; b0 < 2 * nb; b0 += 32) {
+        const int b = b0 + (lane >> 3);
+        const bool active = b < 2 * nb;
+        const int bb = active ? b : 0;
+        const float * x = (bb < nb ? k + (size_t)tt * ldk : v + (size_t)tt * ldv) + (size_t)(bb % nb) * 32 + 4 * sub;
+        const f32x4 xv = *(const f32x4_a4 *)x;
+        const float amax = group8_max(absmax4(xv));
+        const float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
+        if (!active) continue;
+        f32x4 t; t.x = xv.x * id; t.y = xv.y * id; t.z = xv.z * id; t.w = xv.w * id;
+        const uint32_t q = pack_round_i8x4(t);
+        uint8_t * blk = base + (size_t)bb * 34;
+        uint16_t * o = (uint16_t *)(blk + 2 + 4 * sub);
+        o[0] = (uint16_t)q; o[1] = (uint16_t)(q >> 16);
+        if (sub == 0) *(uint16_t *)blk = f2h_bits(d);
+    }
+}
+
+// in-place orthonormal WHT of C chunks of n values, n in {64, 128, 256}: n / 4 lanes per chunk
+template <int N>
+__global__ void __launch_bounds__(256) hadamard_chunks(float * __restrict__ x, long C) {
+    constexpr int LPC = N / 4;                       // lanes per chunk
+    const int lane = threadIdx.x & 63;
+    const long wave = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long c = wave * (64 / LPC) + lane / LPC;
+    const int l = lane % LPC;
+    const bool active = c < C;
+    f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) v = *(const f32x4 *)(x + c * N + 4 * l);
+    float a, b;
+    a = v.x; b = v.y; v.x = a + b; v.y = a - b;
+    a = v.z; b = v.w; v.z = a + b; v.w = a - b;
+    a = v.x; b = v.z; v.x = a + b; v.z = a - b;
+    a = v.y; b = v.w; v.y = a + b; v.w = a - b;
+#pragma unroll
+    for (int m = 1; m < LPC; m <<= 1) {
+        const bool hi = (l & m) != 0;
+        const float p0 = __shfl_xor(v.x, m, 64), p1 = __shfl_xor(v.y, m, 64), p2 = __shfl_xor(v.z, m, 64), p3 = __shfl_xor(v.w, m, 64);
+        v.x = hi ? p0 - v.x : v.x + p0; v.y = hi ? p1 - v.y : v.y + p1;
+        v.z = hi ? p2 - v.z : v.z + p2; v.w = hi ? p3 - v.w : v.w + p3;
+    }
+    const float scale = 1.0f / sqrtf((float)N);
+    v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+    if (active) *(f32x4 *)(x + c * N + 4 * l) = v;
+}
+
+// out-of-place 128-point transform with the literal scale 0x1.6a09e6p-4f (the Q8 KV cache's rotation)
+__global__ void __launch_bounds__(256) hadamard128_heads(const float * __restrict__ x, float * __restrict__ y, long heads) {
+    const int lane = threadIdx.x & 63;
+    const long h = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+    const int l = lane & 31;
+    const bool active = h < heads;
+    f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) v = *(const f32x4 *)(x + h * 128 + 4 * l);
+    v = hadamard128_l4(v, l, true);
+    if (active) *(f32x4 *)(y + h * 128 + 4 * l) = v;
+}
+
+extern "C" {
+
+int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
+                          int T, hipStream_t st) {
+    if (!k || !v || !cache || !err || T < 0 || ((uintptr_t)k & 3) || ((uintptr_t)v & 3) || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    kv_q8_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
+    CAMX_LAUNCH_RET();
+}
+
+int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
+                      int T, hipStream_t st) {
+    if (!k || !v || !cache || !err || T < 0 || M < 32 || M % 32 || ldk < M || ldv < M || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    pf_kv_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
+    CAMX_LAUNCH_RET();
+}
+
+int camx_pf_hadamard(float * x, int C, int n, int rpb, hipStream_t st) {
+    (void)rpb;
+    if (!x || C < 0 || (n != 64 && n != 128 && n != 256) || ((uintptr_t)x & 15)) return CAMX_EINVAL;
+    if (C == 0) return CAMX_OK;
+    const int cpw = 256 / n;                                           // chunks per wave
+    const unsigned blocks = (unsigned)(((long)C + 4 * cpw - 1) / (4 * cpw));
+    if (n == 64) hadamard_chunks<64><<<dim3(blocks), dim3(256), 0, st>>>(x, C);
+    else if (n == 128) hadamard_chunks<128><<<dim3(blocks), dim3(256), 0, st>>>(x, C);
+    else hadamard_chunks<256><<<dim3(blocks), dim3(256), 0, st>>>(x, C);
+    CAMX_LAUNCH_RET();
+}
+
+int camx_hadamard128(const float * x, float * y, long heads, hipStream_t st) {
+    if (!x || !y || heads < 0 || ((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return CAMX_EINVAL;
+    if (heads == 0) return CAMX_OK;
+    hadamard128_heads<<<dim3((unsigned)((heads + 7) / 8)), dim3(256), 0, st>>>(x, y, heads);
+    CAMX_LAUNCH_RET();
+}
+
+}   // extern "C"

@@ -1,0 +1,228 @@
+// Per-head QK RMSNorm + rotary for gfx950, with the fp16 / Q8 KV row writers fused in. Replaces q3p_qk_rope and
+// q3p_qk_rope_q8 (kernels/q3m_prefill.hip:534-591, the OP_OWN_ATTS prologue kernels/k3_own_atts.h:183-274) and pf_qk_nr /
+// OP_QK_NR (kernels/prefill_attn.hip:106-129, kernels/k3_gguf_ops.h:1495-1518).
+//
+// One workgroup per token: the first wave computes the token's cos / sin row once into LDS (the reference recomputes it
+// per head), then each half-wave takes one 128-wide head: lane l holds dims 4l .. 4l + 3, the NeoX partner dim i ^ 64
+// sits in lane l ^ 16. Norm sum: x * x per dim, the 32-lane butterfly per 32 dims, the four group sums in order.
+//
+// The frequency of pair j is powf(theta_scale, j) in the reference; here it is (float)pow((double)theta_scale, j), the
+// correctly rounded single-precision power, so a CPU libm that rounds powf correctly gives the same angle bits.
+#include "common.cuh"
+
+CAMX_DEV float rope_freq(float theta_scale, int j) { return (float)pow((double)theta_scale, (double)j); }
+
+struct RopeArgs {
+    const float * qkv; int ldq, nh, nkv;
+    const float * par;               // q_norm[128] | k_norm[128] | theta_scale | eps | (yarn: freq[64] | mscale)
+    int pos0; const int32_t * pos;   // token t is at pos ? pos[t] : pos0 + t
+    uint16_t * q16;                  // fp16 [n][nh][128]
+    void * cache;                    // fp16 rows [K (nkv*128) | V] or Q8 rows
+    int * err;
+    const int32_t * page_table; int pt_stride, page, n_pages;   // paged addressing (null: row = position)
+    int n;
+};
+
+template <bool YARN, bool Q8>
+__global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
+    __shared__ __attribute__((aligned(16))) float rc[64];
+    __shared__ __attribute__((aligned(16))) float rs[64];
+    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, l = lane & 31;
+    const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+    if (tid < 64) {
+        float c, s;
+        if (YARN) { const float theta = (float)pos * a.par[258 + tid], ms = a.par[322]; c = cosf(theta) * ms; s = sinf(theta) * ms; }
+        else { const float theta = (float)pos * rope_freq(a.par[256], tid); c = cosf(theta); s = sinf(theta); }
+        rc[tid] = c; rs[tid] = s;
+    }
+    __syncthreads();
+    const float * row = a.qkv + (size_t)t * a.ldq;
+    const size_t M = (size_t)a.nkv * 128;
+    const size_t rb = Q8 ? 2 * (M / 32) * 34 : 4 * M;
+    uint8_t * cw = nullptr;
+    if (a.page_table) {
+        const int pg = a.page_table[(size_t)t * a.pt_stride + pos / a.page];
+        if (pg < 0 || pg >= a.n_pages) { if (tid == 0) atomicOr(a.err, 8); }
+        else cw = (uint8_t *)a.cache + ((size_t)pg * a.page + (size_t)(pos % a.page)) * rb;
+    } else cw = (uint8_t *)a.cache + (size_t)pos * rb;
+    const float eps = a.par[257];
+    const f32x4 c4 = *(const f32x4 *)(rc + 4 * (l & 15)), s4 = *(const f32x4 *)(rs + 4 * (l & 15));
+    const bool lo = l < 16;
+    // items: heads 0 .. nh + nkv - 1 take norm + rotary, items nh + nkv .. nh + 2 nkv - 1 are the V heads
+    const int items = a.nh + 2 * a.nkv;
+    for (int it0 = (tid >> 6) * 2; it0 < items; it0 += 8) {
+        const int it = it0 + (lane >> 5);
+        const bool active = it < items;
+        const int hy = active ? it : 0;
+        const f32x4 x = *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
+        if (hy >= a.nh + a.nkv) {                       // a V head: fp16 copy, or fp16-rounded then Q8 blocks
+            const int g = hy - a.nh - a.nkv;
+            if (Q8) {
+                f32x4 v; v.x = f16r(x.x); v.y = f16r(x.y); v.z = f16r(x.z); v.w = f16r(x.w);
+                kv_q8_emit(v, cw + (M / 32 + (size_t)g * 4 + (l >> 3)) * 34, l & 7, a.err, active && cw != nullptr);
+            } else if (active && cw) *(u32x2 *)((uint16_t *)cw + M + (size_t)g * 128 + 4 * l) = pack_f16x4(x);
+            continue;
+        }
+        const bool isq = hy < a.nh;
+        const f32x4 wn = *(const f32x4 *)(a.par + (isq ? 0 : 128) + 4 * l);
+        f32x4 sq; sq.x = x.x * x.x; sq.y = x.y * x.y; sq.z = x.z * x.z; sq.w = x.w * x.w;
+        const float tot = half_groups_in_order<4>(group32_sum(sq), lane & 32);
+        const float scale = rsqrt_exact(tot / 128 + eps);
+        f32x4 y1; y1.x = (scale * x.x) * wn.x; y1.y = (scale * x.y) * wn.y; y1.z = (scale * x.z) * wn.z; y1.w = (scale * x.w) * wn.w;
+        f32x4 p; p.x = lane_xor16(y1.x); p.y = lane_xor16(y1.y); p.z = lane_xor16(y1.z); p.w = lane_xor16(y1.w);
+        // dims below 64: fma(x0, c, -(x1 s)); dims from 64: fma(x1, c, x0 s), with x0 the low and x1 the high dim of the pair
+        f32x4 y;
+        y.x = __builtin_fmaf(y1.x, c4.x, lo ? -(p.x * s4.x) : p.x * s4.x); y.y = __builtin_fmaf(y1.y, c4.y, lo ? -(p.y * s4.y) : p.y * s4.y);
+        y.z = __builtin_fmaf(y1.z, c4.z, lo ? -(p.z * s4.z) : p.z * s4.z); y.w = __builtin_fmaf(y1.w, c4.w, lo ? -(p.w * s4.w) : p.w * s4.w);
+        if (Q8) {
+            y.x = f16r(y.x); y.y = f16r(y.y); y.z = f16r(y.z); y.w = f16r(y.w);
+            y = hadamard128_l4(y, l, true);
+        }
+        if (isq) {
+            if (Q8) { asm volatile("" : "+v"(y.x), "+v"(y.y), "+v"(y.z), "+v"(y.w)); }   // fp32 product first, then fp16
+            if (active) *(u32x2 *)(a.q16 + ((size_t)t * a.nh + hy) * 128 + 4 * l) = pack_f16x4(y);
+        } else {
+            const int g = hy - a.nh;
+            if (Q8) kv_q8_emit(y, cw + ((size_t)g * 4 + (l >> 3)) * 34, l & 7, a.err, active && cw != nullptr);
+            else if (active && cw) *(u32x2 *)((uint16_t *)cw + (size_t)g * 128 + 4 * l) = pack_f16x4(y);
+        }
+    }
+}
+
+// ---- pf_qk_nr: any head dim D <= 512, rotary on the first n_rot dims, input heads at head_stride ------------------------------
+struct NrArgs {
+    const void * x; int head_stride, heads; const float * w; int D, nrot; float theta_scale, eps; int pos0; const int32_t * pos; void * out; int T;
+};
+template <bool BF16>
+__global__ void __launch_bounds__(256) qk_nr_tokens(NrArgs a) {
+    __shared__ float rc[256], rs[256];
+    __shared__ float nrm[4][512];
+    const int tok = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = a.nrot / 2;
+    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    for (int j = tid; j < half; j += 256) {
+        const float theta = pos * rope_freq(a.theta_scale, j);
+        rc[j] = cosf(theta); rs[j] = sinf(theta);
+    }
+    __syncthreads();
+    for (int h = wave; h < a.heads; h += 4) {
+        const size_t t = (size_t)tok * a.heads + h;
+        const size_t xo = t * a.head_stride, yo = t * a.D;
+        float xv[2][4];
+        f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int i = 256 * j + 4 * lane + k;
+                xv[j][k] = 0.0f;
+                if (i < a.D) xv[j][k] = BF16 ? bf2f(((const uint16_t *)a.x)[xo + i]) : ((const float *)a.x)[xo + i];
+            }
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            ss.x = __builtin_fmaf(xv[j][0], xv[j][0], ss.x); ss.y = __builtin_fmaf(xv[j][1], xv[j][1], ss.y);
+            ss.z = __builtin_fmaf(xv[j][2], xv[j][2], ss.z); ss.w = __builtin_fmaf(xv[j][3], xv[j][3], ss.w);
+        }
+        const float tot = wave_groups_in_order(group32_sum(ss));
+        const float scale = rsqrt_exact(tot / (float)a.D + a.eps);
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int i = 256 * j + 4 * lane + k;
+                if (i < a.D) { xv[j][k] = (scale * xv[j][k]) * a.w[i]; nrm[wave][i] = xv[j][k]; }
+            }
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): this wave's LDS stores have landed before its reads
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int i = 256 * j + 4 * lane + k;
+                if (i < a.D) {
+                    float y = xv[j][k];
+                    if (i < a.nrot) {
+                        const int jj = i < half ? i : i - half;
+                        const float c = rc[jj], sn = rs[jj];
+                        const float x0 = nrm[wave][jj], x1 = nrm[wave][jj + half];
+                        y = i < half ? x0 * c - x1 * sn : x0 * sn + x1 * c;
+                    }
+                    if (BF16) ((uint16_t *)a.out)[yo + i] = to_bf16(y); else ((float *)a.out)[yo + i] = y;
+                }
+            }
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+    }
+}
+
+__global__ void rope_freqs_k(float theta_scale, int n, float * out) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < n) out[j] = rope_freq(theta_scale, j);
+}
+
+static int rope_check(const RopeArgs & a, bool q8) {
+    if (!a.qkv || !a.par || !a.q16 || !a.cache || a.n < 0 || a.nh < 1 || a.nkv < 1 || a.ldq < (a.nh + 2 * a.nkv) * 128 || (a.ldq & 3)) return CAMX_EINVAL;
+    if (((uintptr_t)a.qkv & 15) || ((uintptr_t)a.par & 15) || ((uintptr_t)a.q16 & 7) || ((uintptr_t)a.cache & (q8 ? 1 : 7))) return CAMX_EINVAL;
+    if (q8 && !a.err) return CAMX_EINVAL;
+    if (a.page_table && (a.page < 1 || a.n_pages < 1 || a.pt_stride < 1 || !a.err)) return CAMX_EINVAL;
+    return CAMX_OK;
+}
+static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st) {
+    if (rope_check(a, q8)) return CAMX_EINVAL;
+    if (a.n == 0) return CAMX_OK;
+    const dim3 grid(a.n), block(256);
+    if (q8) { if (yarn) qk_rope_tokens<true, true><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true><<<grid, block, 0, st>>>(a); }
+    else { if (yarn) qk_rope_tokens<true, false><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false><<<grid, block, 0, st>>>(a); }
+    CAMX_LAUNCH_RET();
+}
+
+extern "C" {
+
+// q3p_qk_rope: n tokens at positions pos0 .. pos0 + n - 1; cache = fp16 rows [K | V] indexed by position
+int camx_q3p_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
+                     int n, int yarn, hipStream_t st) {
+    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, nullptr, nullptr, 0, 0, 0, n};
+    return rope_launch(a, yarn, false, st);
+}
+// q3p_qk_rope_q8: the Q8 cache rows (K rotated by the 128-point Hadamard transform, V unrotated); err bit 2 on a refused block
+int camx_q3p_qk_rope_q8(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint8_t * cache,
+                        int * err, int n, int yarn, hipStream_t st) {
+    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, err, nullptr, 0, 0, 0, n};
+    return rope_launch(a, yarn, true, st);
+}
+// batched decode form: sequence t at its own position pos[t]; row address through a page table
+// (page_table[t * pt_stride + pos / page] * page + pos % page) when page_table is given, else row = pos[t].
+// err bit 8: a page id outside [0, n_pages) (that row is not written). q8 = 0 writes fp16 rows.
+int camx_qk_rope_paged(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16, void * cache,
+                       int * err, const int32_t * page_table, int pt_stride, int page, int n_pages, int n, int yarn, int q8, hipStream_t st) {
+    if (!pos) return CAMX_EINVAL;
+    RopeArgs a = {qkv, ldq, nh, nkv, par, 0, pos, q16, cache, err, page_table, pt_stride, page, n_pages, n};
+    return rope_launch(a, yarn, q8 != 0, st);
+}
+
+// pf_qk_nr: out [T][heads][D] = rotary(rms_norm(x head) * w) at position pos0 + row; io 0 fp32, 1 bf16 in / out
+int camx_pf_qk_nr(const void * xin, int head_stride, int heads, const float * w, int D, int nrot, float theta_scale, float eps, int pos0,
+                  void * out, int T, int io, hipStream_t st) {
+    if (!xin || !w || !out || T < 0 || heads < 1 || D < 1 || D > 512 || head_stride < D || nrot < 0 || nrot > D || (nrot & 1) || io < 0 || io > 1) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    NrArgs a = {xin, head_stride, heads, w, D, nrot, theta_scale, eps, pos0, nullptr, out, T};
+    if (io) qk_nr_tokens<true><<<dim3(T), dim3(256), 0, st>>>(a); else qk_nr_tokens<false><<<dim3(T), dim3(256), 0, st>>>(a);
+    CAMX_LAUNCH_RET();
+}
+// the same with one position per row (a speculative-verify batch)
+int camx_qk_nr_pos(const void * xin, int head_stride, int heads, const float * w, int D, int nrot, float theta_scale, float eps,
+                   const int32_t * pos, void * out, int T, int io, hipStream_t st) {
+    if (!xin || !w || !out || !pos || T < 0 || heads < 1 || D < 1 || D > 512 || head_stride < D || nrot < 0 || nrot > D || (nrot & 1) || io < 0 || io > 1) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    NrArgs a = {xin, head_stride, heads, w, D, nrot, theta_scale, eps, 0, pos, out, T};
+    if (io) qk_nr_tokens<true><<<dim3(T), dim3(256), 0, st>>>(a); else qk_nr_tokens<false><<<dim3(T), dim3(256), 0, st>>>(a);
+    CAMX_LAUNCH_RET();
+}
+// the per-pair frequencies the rotary kernels use: out[j] = (float)pow((double)theta_scale, j), j < n
+int camx_rope_freqs(float theta_scale, int n, float * out, hipStream_t st) {
+    if (!out || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    rope_freqs_k<<<dim3((n + 63) / 64), dim3(64), 0, st>>>(theta_scale, n, out);
+    CAMX_LAUNCH_RET();
+}
+
+}   // extern "C"

@@ -29,7 +29,8 @@ def host(t, dtype=None):
 
 
 def ptr(t):
-    return C.c_void_p(t.data_ptr()) if t is not None else NULL
+    """marks a device-buffer argument; the tensor itself travels to call(), which keeps it alive until the kernel is done"""
+    return t if t is not None else NULL
 
 
 def stream():
@@ -37,7 +38,8 @@ def stream():
 
 
 def call(name, *args):
-    err = getattr(camx(), name)(*args, stream())
+    argv = [C.c_void_p(a.data_ptr()) if isinstance(a, torch.Tensor) else a for a in args]
+    err = getattr(camx(), name)(*argv, stream())
     _lib.check(err)
     torch.cuda.synchronize()
 
@@ -53,3 +55,21 @@ def outliers(rng, shape, frac=1e-3, scale=50.0):
     m = rng.random(shape) < frac
     x[m] *= np.float32(scale)
     return x
+
+
+def close_fp32(a, ref, rel=1e-5):
+    """|a - ref| <= rel * max |ref| elementwise (the fp32 tolerance class)"""
+    a = np.asarray(a, np.float64); ref = np.asarray(ref, np.float64)
+    return bool((np.abs(a - ref) <= rel * max(float(np.abs(ref).max()), 1e-30)).all())
+
+
+def close_16(bits, ref_bits, kind, rel=1e-5):
+    """16-bit outputs within one unit in the last place of the reference value (+ rel * max |ref|); kind 'f16' | 'bf16'"""
+    bits = np.asarray(bits, np.uint16); ref_bits = np.asarray(ref_bits, np.uint16)
+    if kind == 'f16':
+        a = bits.view(np.float16).astype(np.float64); r = ref_bits.view(np.float16).astype(np.float64)
+        ulp = np.abs(np.spacing(np.abs(ref_bits.view(np.float16)))).astype(np.float64)
+    else:
+        a = (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64); r = (ref_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        ulp = np.abs(r) * 2.0 ** -7 + 2.0 ** -133
+    return bool((np.abs(a - r) <= ulp + rel * max(float(np.abs(r).max()), 1e-30)).all())

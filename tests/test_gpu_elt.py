@@ -1,0 +1,96 @@
+"""GPU parity of the elementwise / small row kernels against the CPU oracle: exact where no transcendental is involved,
+1e-5 relative (fp32) / one 16-bit ulp otherwise."""
+import numpy as np
+import pytest
+
+import oracle as O
+from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, close_fp32, dev, host, outliers, ptr
+
+pytestmark = pytest.mark.gpu
+EXTREMES = np.array([30, -30, 0, -0.0, 1e-3, -88, 88, 5], np.float32)
+
+
+@pytest.mark.parametrize('n', [8 * 768, 1001, 7])
+def test_swiglu(n):
+    rng = np.random.default_rng(n)
+    g = outliers(rng, n); u = outliers(rng, n); g[:min(8, n)] = EXTREMES[:min(8, n)]
+    y16 = dev(np.zeros(n, np.uint16)); y32 = dev(np.zeros(n, np.float32)); gd, ud = dev(g), dev(u)
+    call('camx_q3p_swiglu', ptr(gd), ptr(ud), ptr(y16), I(n))
+    call('camx_gg_silu_mul', ptr(gd), ptr(ud), ptr(y32), I(n))
+    assert close_16(host(y16, np.uint16), O.swiglu16(g, u), 'f16')
+    assert close_fp32(host(y32), O.silu_mul_f32(g, u))
+
+
+@pytest.mark.parametrize('R,H', [(4, 17408), (3, 7)])
+def test_silu_mul_bf16(R, H):
+    rng = np.random.default_rng(H)
+    gu = O.f2bf(outliers(rng, (R, 2 * H)))
+    act = dev(np.zeros((R, H), np.uint16))
+    call('camx_silu_mul_bf16', ptr(dev(gu)), ptr(act), I(H), L64(R * H))
+    assert close_16(host(act, np.uint16), O.silu_mul_bf16(gu), 'bf16')
+
+
+def test_gate_mul():
+    rng = np.random.default_rng(1004)
+    T, H, D = 16, 24, 256
+    a = outliers(rng, (T * H, D)); qg = outliers(rng, (T * H, 2 * D)); qg[0, D:D + 8] = EXTREMES
+    ad, gd = dev(a), dev(qg)
+    y = dev(np.zeros_like(a)); y16 = dev(np.zeros(a.shape, np.uint16))
+    call('camx_gate_mul', ptr(ad), ptr(gd), ptr(y), L64(a.size), I(D), I(2 * D), I(D), I(0))
+    call('camx_gate_mul', ptr(ad), ptr(gd), ptr(y16), L64(a.size), I(D), I(2 * D), I(D), I(1))
+    assert close_fp32(host(y), O.gate_mul(a, qg, D, 2 * D, D))
+    assert close_16(host(y16, np.uint16), O.gate_mul(a, qg, D, 2 * D, D, f16=True), 'f16')
+    abf, gbf = O.f2bf(a), O.f2bf(qg)
+    ybf = dev(np.zeros(a.shape, np.uint16))
+    call('camx_gate_mul', ptr(dev(abf)), ptr(dev(gbf)), ptr(ybf), L64(a.size), I(D), I(2 * D), I(D), I(2))
+    assert close_16(host(ybf, np.uint16), O.f2bf(O.gate_mul(O.bf2f(abf), O.bf2f(gbf), D, 2 * D, D)), 'bf16')
+
+
+@pytest.mark.parametrize('T,C', [(16, 10240), (1, 64), (2, 100), (5, 256)])
+def test_gdn_conv(T, C):
+    rng = np.random.default_rng(C)
+    ldx = C + 4
+    x = outliers(rng, (T, ldx)); w = rng.standard_normal((C, 4)).astype(np.float32); st = rng.standard_normal((C, 3)).astype(np.float32)
+    ref_y, ref_st = O.gdn_conv(x, w, st, ldx=ldx)
+    xd, wd, sd = dev(x), dev(w), dev(st); y = dev(np.zeros((T, C), np.float32))
+    call('camx_pf_gdn_conv', ptr(xd), ptr(wd), ptr(sd), ptr(y), I(C), I(T), I(ldx), I(C), I(0))
+    call('camx_pf_conv_state', ptr(xd), ptr(sd), I(C), I(T), I(ldx), I(0))
+    assert close_fp32(host(y), ref_y) and bits_equal(host(sd), ref_st)
+
+
+@pytest.mark.parametrize('T,heads,K', [(16, 32, 128), (16, 48, 128), (3, 5, 256), (2, 3, 96)])
+def test_gdn_l2(T, heads, K):
+    rng = np.random.default_rng(K + heads)
+    ldx = heads * K + 64
+    x = outliers(rng, (T, ldx))
+    y = dev(np.zeros((T * heads, K), np.float32))
+    call('camx_pf_gdn_l2', ptr(dev(x)), ptr(y), I(heads), I(K), I(ldx), F(np.float32(1e-6 / K)), I(T), I(0))
+    assert bits_equal(host(y), O.gdn_l2(x, T, heads, K, 1e-6, ldx=ldx))
+
+
+def test_core_and_fuse():
+    rng = np.random.default_rng(5)
+    T, D, V = 9, 896, 50
+    emb = rng.standard_normal((V, D)).astype(np.float32); tok = rng.integers(0, V, T).astype(np.int32)
+    out = dev(np.zeros((T, D), np.float32))
+    call('camx_embedding_f32', ptr(dev(tok)), ptr(dev(emb)), ptr(out), I(D), I(T))
+    assert bits_equal(host(out), O.embedding_f32(tok, emb))
+    x = outliers(rng, (T, D))
+    m = O.f2bf(outliers(rng, (T, D))); y = O.f2bf(outliers(rng, (T, D)))
+    o = dev(np.zeros((T, D), np.float32))
+    call('camx_residual3', ptr(dev(x)), ptr(dev(m)), ptr(dev(y)), ptr(o), L64(T * D))
+    assert bits_equal(host(o), O.residual3(x, m, y))
+    x[0, :6] = [np.nan, np.inf, -np.inf, 1e-40, -np.nan, 3.3895314e38]
+    c = dev(np.zeros((T, D), np.uint16))
+    call('camx_cast_bf16', ptr(dev(x)), ptr(c), L64(T * D))
+    assert bits_equal(host(c, np.uint16), O.f2bf(x))
+    dst = rng.integers(0, 65536, (T, 64)).astype(np.uint16); dd = dev(dst)
+    call('camx_copy_cols_bf16', ptr(dev(m)), I(D), I(5), ptr(dd), I(64), I(3), I(40), L64(T))
+    assert bits_equal(host(dd, np.uint16), O.copy_cols_bf16(m, 5, dst, 3, 40))
+    ys = O.f2bf(outliers(rng, (4, D))); pos = np.array([-1, 0, 3, -1, 2, 1, -1, -1, 0], np.int32)
+    x2 = outliers(rng, (T, D))
+    for has in (True, False):
+        o2 = dev(np.zeros((T, D), np.float32))
+        call('camx_residual_slices_fwd', ptr(dev(x2)), ptr(dev(m)), ptr(dev(y)), ptr(dev(ys)) if has else NULL, ptr(dev(pos)) if has else NULL,
+             ptr(o2), I(D), L64(T * D // 4))
+        assert bits_equal(host(o2), O.residual_slices_fwd(x2, m, y, ys if has else None, pos if has else None))

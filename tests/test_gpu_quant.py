@@ -1,0 +1,78 @@
+"""GPU parity of the activation quantizers (q8_1 blocks and the MMQ layout) against the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle as O
+from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, dev, host, outliers, ptr
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('n', [32, 2048, 1000, 31, 256 * 2048, 4097])
+def test_q8_1_plain(n):
+    rng = np.random.default_rng(n)
+    x = outliers(rng, n)
+    x[:32] = 0.0                                         # an all-zero block
+    if n >= 96: x[64:96] = np.float32(127.0) * np.sign(rng.standard_normal(32)).astype(np.float32)
+    y = dev(np.full(((n + 31) // 32, 36), 0xa5, np.uint8))
+    call('camx_gg_quantize_q8_1', ptr(dev(x)), ptr(y), L64(n), I(0), F(0), NULL)
+    assert bits_equal(host(y), O.q8_1(x))
+
+
+@pytest.mark.parametrize('mode', [1, 2])
+def test_q8_1_silu_modes(mode):
+    rng = np.random.default_rng(mode)
+    n = 8 * 768
+    x = outliers(rng, n); g = outliers(rng, n)
+    x[:8] = [30, -30, 0, -0.0, 1e-3, -88, 88, 5]
+    y = dev(np.zeros((n // 32, 36), np.uint8))
+    xd, gd = dev(x), dev(g)
+    call('camx_gg_quantize_q8_1', ptr(xd), ptr(y), L64(n), I(mode), F(0.37), ptr(gd) if mode == 2 else NULL)
+    got = host(y); ref = O.q8_1(x, mode=mode, rs=0.37, g=g)
+    # transcendental inside: scales within one fp16 step, codes within one step of the oracle's
+    d_g, d_r = got[:, 0:2].copy().view(np.float16).astype(np.float64), ref[:, 0:2].copy().view(np.float16).astype(np.float64)
+    assert np.all(np.abs(d_g - d_r) <= np.abs(d_r) * 2.0 ** -9 + 1e-12)
+    assert np.abs(got[:, 4:].view(np.int8).astype(int) - ref[:, 4:].view(np.int8).astype(int)).max() <= 1
+
+
+@pytest.mark.parametrize('K,ncols,layout', [(512, 3, 0), (2048, 17, 1), (17408, 5, 1), (896, 4, 0), (100 * 4, 2, 1)])
+def test_mmq_quantize(K, ncols, layout):
+    rng = np.random.default_rng(K + ncols)
+    s01 = K + 8
+    x = outliers(rng, (ncols + 2, s01)); x[0, :128] = 0
+    ids = rng.permutation(ncols + 2)[:ncols].astype(np.int32)
+    for use_ids in (False, True):
+        ref = O.mmq_q8_1(x, K, ncols, layout, s01=s01, ids=ids if use_ids else None)
+        y = dev(np.zeros(ref.shape, np.uint8))
+        call('camx_quantize_mmq_q8_1', ptr(dev(x)), ptr(dev(ids)) if use_ids else NULL, ptr(y), L64(K), L64(s01), L64(0), L64(0),
+             L64(O.k_pad(K)), I(ncols), I(1), I(0), I(layout))
+        assert bits_equal(host(y), ref)
+
+
+@pytest.mark.parametrize('K,ntok,k', [(768, 9, 8), (2048, 4, 2)])
+def test_mmq_quantize_scatter(K, ntok, k):
+    rng = np.random.default_rng(K)
+    x = outliers(rng, (ntok, K))
+    ids_inv = rng.permutation(ntok * k).astype(np.int32)
+    for layout in (0, 1):
+        ref = O.mmq_q8_1_scatter(x, K, ntok, ids_inv, k, layout)
+        y = dev(np.zeros(ref.shape, np.uint8))
+        call('camx_quantize_mmq_q8_1_scatter', ptr(dev(x)), ptr(dev(ids_inv)), ptr(y), L64(K), L64(0), L64(K), L64(0), L64(O.k_pad(K)),
+             I(ntok * k), I(1), I(k), I(layout), I(ntok))
+        assert bits_equal(host(y), ref)
+
+
+@pytest.mark.parametrize('T,Fh', [(3, 17408), (8, 768), (5, 1024)])
+def test_swiglu_mmq(T, Fh):
+    """fused SwiGLU -> MMQ: the bf16 activation within one bf16 ulp of the oracle's; the blocks bit-exact given the
+    kernel's own activation bits"""
+    rng = np.random.default_rng(1003 + Fh)
+    gu = O.f2bf(outliers(rng, (T, 2 * Fh)))
+    y = dev(np.zeros((O.k_pad(Fh) // 128, T, 144), np.uint8)); act = dev(np.zeros((T, Fh), np.uint16))
+    call('camx_swiglu_mmq_q8_1', ptr(dev(gu)), L64(2 * Fh), L64(Fh), ptr(y), ptr(act), I(T), I(1))
+    a = host(act, np.uint16)
+    assert close_16(a, O.silu_mul_bf16(gu), 'bf16')
+    assert bits_equal(host(y), O.mmq_q8_1(O.bf2f(a), Fh, T, 1))
+    y2 = dev(np.zeros((O.k_pad(Fh) // 128, T, 144), np.uint8))
+    call('camx_swiglu_mmq_q8_1', ptr(dev(gu)), L64(2 * Fh), L64(Fh), ptr(y2), NULL, I(T), I(1))
+    assert bits_equal(host(y2), host(y))

@@ -1,0 +1,128 @@
+"""GPU parity of QK-norm + rotary (+ fp16 / Q8 KV rows, paged) against the CPU oracle.
+
+Float outputs: within one fp16 ulp + 1e-5 x max (the reference's own bound, tests/engine/test_q3m_yarn_rope.py:9-11).
+Q8 rows: bit-exact bytes of the oracle's codec applied to the fp16 row the F16 form of the same kernel wrote, which is
+where the reference places the stage boundary (tests/engine/test_q3m_kvq8_atts.py:2-7)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from caminus_amd import rope
+from gpu_util import F, I, NULL, bits_equal, call, close_16, close_fp32, dev, host, outliers, ptr
+from vectors import qk_par
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('base', [1e6, 1e7, 1e4, 5e5])
+def test_rope_freqs_match_libm_powf(base):
+    ts = np.float32(np.float32(base) ** np.float32(-2.0 / 128))
+    out = dev(np.zeros(128, np.float32))
+    call('camx_rope_freqs', F(ts), I(128), ptr(out))
+    want = np.array([np.float32(float(ts) ** j) for j in range(128)], np.float32)      # correctly rounded from float64
+    assert bits_equal(host(out), want)
+
+
+def _run_pair(nh, nkv, n, pos0, yarn, rng, rows):
+    tab = rope.yarn_table(128, 1e6, 4.0, 32768) if yarn else None
+    par = qk_par(rng, yarn_table=tab)
+    ldq = (nh + 2 * nkv) * 128 + 16
+    qkv = (rng.standard_normal((n, ldq)) * 1.3).astype(np.float32)
+    M = nkv * 128
+    pd, qd = dev(par), dev(qkv)
+    # F16 form
+    q16 = dev(np.zeros((n, nh, 128), np.uint16)); c16 = dev(np.zeros((rows, 2 * M), np.uint16))
+    call('camx_q3p_qk_rope', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), I(pos0), ptr(q16), ptr(c16), I(n), I(int(yarn)))
+    rq, rc, _ = O.qk_rope(qkv, nh, nkv, par, n, pos0=pos0, yarn=yarn, rows=rows)
+    gq, gc = host(q16, np.uint16), host(c16, np.uint16)
+    assert close_16(gq, rq, 'f16') and close_16(gc[pos0:pos0 + n, :M], rc[pos0:pos0 + n, :M], 'f16')
+    assert bits_equal(gc[:, M:], rc[:, M:])                              # V is an exact fp16 rounding
+    assert not gc[:pos0].any() and not gc[pos0 + n:].any()
+    # Q8 form
+    rb = 2 * (M // 32) * 34
+    q16b = dev(np.zeros((n, nh, 128), np.uint16)); c8 = dev(np.full((rows, rb), 0xa5, np.uint8)); err = dev(np.zeros(1, np.int32))
+    call('camx_q3p_qk_rope_q8', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), I(pos0), ptr(q16b), ptr(c8), ptr(err), I(n), I(int(yarn)))
+    assert int(host(err)[0]) == 0
+    k16 = O.h2f(gc[pos0:pos0 + n, :M]).reshape(n * nkv, 128); v16 = O.h2f(gc[pos0:pos0 + n, M:]).reshape(n * nkv * 4, 32)
+    kb, ok1 = O.kv_q8_encode(O.hadamard128(k16).reshape(-1, 32)); vb, ok2 = O.kv_q8_encode(v16)
+    assert ok1.all() and ok2.all()
+    want = np.concatenate([kb.reshape(n, -1), vb.reshape(n, -1)], axis=1)
+    g8 = host(c8)
+    assert bits_equal(g8[pos0:pos0 + n], want)
+    assert (g8[:pos0] == 0xa5).all() and (g8[pos0 + n:] == 0xa5).all()
+    assert bits_equal(host(q16b, np.uint16), O.f2h(O.hadamard128(O.h2f(gq).reshape(-1, 128))).reshape(n, nh, 128))
+    return qkv, par
+
+
+@pytest.mark.parametrize('nh,nkv,n,pos0,yarn', [(32, 4, 1, 1234, False), (32, 4, 5, 0, False), (64, 8, 9, 4090, True), (16, 2, 3, 131000, True),
+                                                (5, 3, 4, 77, False)])
+def test_qk_rope_f16_and_q8(nh, nkv, n, pos0, yarn):
+    _run_pair(nh, nkv, n, pos0, yarn, np.random.default_rng(1001 + nh + n), rows=pos0 + n + 2)
+
+
+def test_qk_rope_position_zero_is_norm_only():
+    rng = np.random.default_rng(3)
+    par = qk_par(rng); nh, nkv = 4, 1
+    qkv = rng.standard_normal((1, 6 * 128)).astype(np.float32)
+    q16 = dev(np.zeros((1, nh, 128), np.uint16)); c16 = dev(np.zeros((1, 256), np.uint16))
+    call('camx_q3p_qk_rope', ptr(dev(qkv)), I(768), I(nh), I(nkv), ptr(dev(par)), I(0), ptr(q16), ptr(c16), I(1), I(0))
+    x = qkv[0, :nh * 128].reshape(nh, 128).astype(np.float64)
+    want = x / np.sqrt((x * x).mean(1, keepdims=True) + 1e-6) * par[:128]
+    assert close_16(host(q16, np.uint16).reshape(nh, 128), O.f2h(want.astype(np.float32)), 'f16')
+
+
+def test_qk_rope_paged_decode_batch():
+    """config-5 shape: every sequence at its own position, rows addressed through a page table; each row's bytes equal the
+    unpaged row's, untouched pages stay untouched, a bad page id sets bit 8 and writes nothing for that row"""
+    rng = np.random.default_rng(1005)
+    nh, nkv, n, page, n_pages, maxp = 32, 4, 64, 256, 1024, 512
+    par = qk_par(rng); M = nkv * 128; rb = 2 * (M // 32) * 34
+    qkv = outliers(rng, (n, (nh + 2 * nkv) * 128))
+    pos = rng.integers(0, 131072, n).astype(np.int32)
+    pt = rng.permutation(n_pages)[:n * 8].reshape(n, 8).astype(np.int32)
+    table = np.full((n, maxp), -7, np.int32)
+    for t in range(n): table[t, pos[t] // page] = pt[t, 0]
+    table[5, pos[5] // page] = n_pages + 3                                   # out of range: refused row
+    pd, qd, posd, td = dev(par), dev(qkv), dev(pos), dev(table)
+    c8 = dev(np.full((n_pages * page, rb), 0xa5, np.uint8)); err = dev(np.zeros(1, np.int32)); q16 = dev(np.zeros((n, nh, 128), np.uint16))
+    call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16), ptr(c8), ptr(err), ptr(td), I(maxp),
+         I(page), I(n_pages), I(n), I(0), I(1))
+    assert int(host(err)[0]) == 8
+    # the unpaged form at the same positions, one sequence per launch row, as the reference for the row bytes
+    c_flat = dev(np.full((131072, rb), 0xa5, np.uint8)); q16f = dev(np.zeros((n, nh, 128), np.uint16)); err2 = dev(np.zeros(1, np.int32))
+    call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16f), ptr(c_flat), ptr(err2), NULL, I(0),
+         I(0), I(0), I(n), I(0), I(1))
+    assert int(host(err2)[0]) == 0
+    g, flat = host(c8).reshape(n_pages, page, rb), host(c_flat)
+    touched = np.zeros((n_pages, page), bool)
+    for t in range(n):
+        if t == 5: continue
+        pg = table[t, pos[t] // page]
+        assert bits_equal(g[pg, pos[t] % page], flat[pos[t]])
+        touched[pg, pos[t] % page] = True
+    assert (g[~touched] == 0xa5).all()
+    assert bits_equal(host(q16, np.uint16), host(q16f, np.uint16))
+    # the oracle on the same inputs: q16 within tolerance, and the same error word
+    rq, _, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos, q8=True, rows=n_pages * page, page_table=table, page=page, n_pages=n_pages)
+    assert oerr == 8 and close_16(host(q16, np.uint16), rq, 'f16')
+
+
+@pytest.mark.parametrize('T,heads,D,n_rot,stride,base', [(16, 24, 256, 64, 512, 1e7), (16, 4, 256, 64, 256, 1e7), (3, 5, 128, 128, 128, 1e6),
+                                                         (2, 3, 96, 32, 100, 1e4), (2, 2, 512, 128, 512, 1e6)])
+def test_pf_qk_nr(T, heads, D, n_rot, stride, base):
+    rng = np.random.default_rng(1004 + D + heads)
+    x = outliers(rng, (T * heads, stride)); w = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    ts = float(np.float32(np.float32(base) ** np.float32(-2.0 / n_rot)))
+    pos0 = 60000
+    ref = O.qk_nr(x, stride, heads, w, D, n_rot, ts, 1e-6, pos0, T)
+    out = dev(np.zeros((T * heads, D), np.float32))
+    call('camx_pf_qk_nr', ptr(dev(x)), I(stride), I(heads), ptr(dev(w)), I(D), I(n_rot), F(ts), F(1e-6), I(pos0), ptr(out), I(T), I(0))
+    got = host(out)
+    assert close_fp32(got, ref)
+    assert bits_equal(got[:, n_rot:], ref[:, n_rot:])                     # the pass-through dims carry no transcendental
+    # bf16 in / out, one position per row
+    xb = O.f2bf(x); pos = rng.integers(0, 65536, T).astype(np.int32)
+    outb = dev(np.zeros((T * heads, D), np.uint16))
+    call('camx_qk_nr_pos', ptr(dev(xb)), I(stride), I(heads), ptr(dev(w)), I(D), I(n_rot), F(ts), F(1e-6), ptr(dev(pos)), ptr(outb), I(T), I(1))
+    refb = np.concatenate([O.qk_nr(O.bf2f(xb)[t * heads:(t + 1) * heads], stride, heads, w, D, n_rot, ts, 1e-6, int(pos[t]), 1) for t in range(T)])
+    assert close_16(host(outb, np.uint16), O.f2bf(refb), 'bf16')
