@@ -1,0 +1,303 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused per-layer row kernels on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A step is one pass of the dense 27B-class prefill chunk's three fused op-sets over one synthetic batch that is already
+resident in HBM (4096 tokens x hidden 5120, bf16 activations, fp32 residual):
+  (i)   residual add (bf16 addend) + RMSNorm -> fp32 residual + bf16 normed rows          camx_add_rms_bf16
+  (ii)  QK-norm + YaRN rotary on 64 Q + 8 KV heads (+ 8 V heads) of dim 128 -> fp16          camx_qk_rope_bf16
+  (iii) SwiGLU on a 4096 x 17408 gate / up pair -> q8_1 blocks in the MMQ layout              camx_swiglu_mmq_q8_1
+The value is algorithmic bytes (every input read once, every output written once) per second over the whole step.
+One JSON line goes to stdout; `roofline` describes the dominant kernel, `cpu_baseline` the CPU oracle timed on a bounded
+sample of the same workload on this host, `opsets` the other shapes (decode token, embedding gather, hybrid verify
+batch, batched decode with the Q8 KV codec) in microseconds and GB/s per launch.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+I, F, L64 = C.c_int, C.c_float, C.c_int64
+NULL = C.c_void_p(None)
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else NULL
+
+
+class Bench:
+    def __init__(self):
+        import torch
+        from caminus_amd.device import lib
+        self.torch = torch
+        self.L = lib.load()
+        self.check = lib.check
+        self.dev = torch.device('cuda:0')
+        torch.cuda.set_device(self.dev)
+        self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.flush_buf = None
+
+    def call(self, name, *args):
+        self.check(getattr(self.L, name)(*args, self.stream))
+
+    def acts(self, shape, dtype, seed, frac=1e-3, scale=50.0):
+        """N(0, 1) with `frac` of the entries scaled by `scale`, generated on the device"""
+        torch = self.torch
+        g = torch.Generator(device=self.dev); g.manual_seed(seed)
+        x = torch.randn(shape, generator=g, device=self.dev, dtype=torch.float32)
+        m = torch.rand(shape, generator=g, device=self.dev) < frac
+        x = torch.where(m, x * scale, x)
+        return x.to(dtype).contiguous()
+
+    def gamma(self, n, seed):
+        torch = self.torch
+        g = torch.Generator(device=self.dev); g.manual_seed(seed)
+        return (1.0 + 0.1 * torch.randn(n, generator=g, device=self.dev)).contiguous()
+
+    def flush(self):
+        """push the previous launch's lines out of L2 / MALL: a 512 MiB fill (untimed)"""
+        torch = self.torch
+        if self.flush_buf is None: self.flush_buf = torch.empty(512 << 20, dtype=torch.uint8, device=self.dev)
+        self.flush_buf.fill_(1)
+
+    def time_launch(self, fn, reps=50, warm=10, flush=False):
+        """median and mean duration (us) of one launch of fn, HIP events on the launch stream"""
+        torch = self.torch
+        for _ in range(warm): fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            if flush: self.flush()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); fn(); b.record(); b.synchronize()
+            ts.append(a.elapsed_time(b) * 1e3)
+        ts.sort()
+        return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def yarn_par(torch, dev, seed, base=1e6, eps=1e-6, yarn=True):
+    import numpy as np
+    from caminus_amd import rope
+    rng = np.random.default_rng(seed)
+    qn = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32); kn = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32)
+    ts = np.float32(np.float32(base) ** np.float32(-2.0 / 128))
+    par = np.concatenate([qn, kn, np.array([ts, eps], np.float32)])
+    if yarn: par = np.concatenate([par, rope.yarn_table(128, base, 4.0, 32768)])
+    return torch.from_numpy(par.astype(np.float32)).to(dev), par.astype(np.float32)
+
+
+def config3(B, T=4096, H=5120, nh=64, nkv=8, Fh=17408):
+    """the dense prefill chunk: buffers and the three launches"""
+    torch = B.torch
+    w = dict(T=T, H=H, nh=nh, nkv=nkv, Fh=Fh)
+    w['x'] = B.acts((T, H), torch.float32, 1003)
+    w['d'] = B.acts((T, H), torch.bfloat16, 1004)
+    w['nw'] = B.gamma(H, 1005)
+    w['hbf'] = torch.empty((T, H), dtype=torch.bfloat16, device=B.dev)
+    ldq = (nh + 2 * nkv) * 128
+    w['qkv'] = B.acts((T, ldq), torch.bfloat16, 1006)
+    w['par'], w['par_np'] = yarn_par(torch, B.dev, 1007)
+    w['q16'] = torch.empty((T, nh, 128), dtype=torch.float16, device=B.dev)
+    w['cache'] = torch.empty((T, 2 * nkv * 128), dtype=torch.float16, device=B.dev)
+    w['gu'] = B.acts((T, 2 * Fh), torch.bfloat16, 1008)
+    kp = (Fh + 511) // 512 * 512
+    w['y'] = torch.empty((kp // 128, T, 144), dtype=torch.uint8, device=B.dev)
+    w['ldq'] = ldq
+    w['bytes'] = {
+        'add_rms_bf16': T * H * (4 + 2 + 4 + 2) + H * 4,
+        'qk_rope_bf16': T * ldq * 2 + 323 * 4 + T * ldq * 2,
+        'swiglu_mmq_q8_1': T * 2 * Fh * 2 + (kp // 128) * T * 144,
+    }
+    w['launch'] = {
+        'add_rms_bf16': lambda: B.call('camx_add_rms_bf16', _p(w['x']), _p(w['d']), _p(w['nw']), F(1e-6), NULL, _p(w['hbf']), I(H), I(T)),
+        'qk_rope_bf16': lambda: B.call('camx_qk_rope_bf16', _p(w['qkv']), I(ldq), I(nh), I(nkv), _p(w['par']), I(0), _p(w['q16']), _p(w['cache']), I(T), I(1)),
+        'swiglu_mmq_q8_1': lambda: B.call('camx_swiglu_mmq_q8_1', _p(w['gu']), L64(2 * Fh), L64(Fh), _p(w['y']), NULL, I(T), I(1)),
+    }
+    return w
+
+
+def extra_opsets(B):
+    """the other shapes, one launch each: (name, algorithmic bytes, launch)"""
+    import numpy as np
+    torch = B.torch
+    out = []
+    # decode token, hidden 2048 (batch 1)
+    N = 2048
+    x = B.acts((1, N), torch.float32, 11); d = B.acts((1, 1, N), torch.float32, 12); nw = B.gamma(N, 13)
+    h = torch.empty((1, N), device=B.dev); h16 = torch.empty((1, N), dtype=torch.float16, device=B.dev)
+    q8 = torch.empty((N // 32) * 36, dtype=torch.uint8, device=B.dev)
+    out.append(('c1_add_rms_h_h16', N * 4 * 3 + N * 4 * 2 + N * 2,
+                lambda: B.call('camx_q3p_add_rms16', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), _p(h), _p(h16), I(N), I(1))))
+    out.append(('c1_q8_1', N * 4 + N // 32 * 36, lambda: B.call('camx_gg_quantize_q8_1', _p(h), _p(q8), L64(N), I(0), F(0), NULL)))
+    nh, nkv = 32, 4
+    ldq = (nh + 2 * nkv) * 128
+    qkv = B.acts((1, ldq), torch.float32, 14); par, _ = yarn_par(torch, B.dev, 15, yarn=False)
+    q16 = torch.empty((1, nh, 128), dtype=torch.float16, device=B.dev); cache = torch.zeros((4096, 2 * nkv * 128), dtype=torch.float16, device=B.dev)
+    out.append(('c1_qk_rope', ldq * 4 + 258 * 4 + nh * 128 * 2 + 2 * nkv * 128 * 2,
+                lambda: B.call('camx_q3p_qk_rope', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(1234), _p(q16), _p(cache), I(1), I(0))))
+    n = 8 * 768
+    g = B.acts((n,), torch.float32, 16); u = B.acts((n,), torch.float32, 17); y16 = torch.empty(n, dtype=torch.float16, device=B.dev)
+    out.append(('c1_swiglu', n * 10, lambda: B.call('camx_q3p_swiglu', _p(g), _p(u), _p(y16), I(n))))
+    # embedding gather, 151936 x 2048, 256 ids
+    V, n_tok = 151936, 256
+    rng = np.random.default_rng(1002)
+    toks = torch.from_numpy(rng.integers(0, V, n_tok).astype(np.int32)).to(B.dev)
+    gq = torch.Generator(device=B.dev); gq.manual_seed(1002)
+    for fmt, name, rb, blk in ((0, 'q4_k', N // 256 * 144, 144), (1, 'q8_0', N // 32 * 34, 34)):
+        tab = torch.randint(0, 256, (V, rb), generator=gq, device=B.dev, dtype=torch.uint8)
+        sc = (torch.rand((V, rb // blk, 2 if fmt == 0 else 1), generator=gq, device=B.dev) * 9e-3 + 1e-3).to(torch.float16)
+        tab.view(V, rb // blk, blk)[:, :, :(4 if fmt == 0 else 2)] = sc.view(torch.uint8).view(V, rb // blk, -1)
+        xo = torch.empty((n_tok, N), device=B.dev); xbf = torch.empty((n_tok, N), dtype=torch.bfloat16, device=B.dev)
+        hh = torch.empty((n_tok, N), device=B.dev); qq = torch.empty(n_tok * (N // 32) * 36, dtype=torch.uint8, device=B.dev)
+        out.append((f'c2_gather_{name}_f32_bf16', n_tok * (rb + 4 + N * 6),
+                    (lambda tab=tab, rb=rb, fmt=fmt, xo=xo, xbf=xbf: B.call('camx_emb_gather', _p(tab), L64(rb), I(V), _p(toks), _p(xo), _p(xbf), I(N), I(n_tok), I(fmt)))))
+        out.append((f'c2_gather_{name}_add_rms_q8_1', n_tok * (rb + 4 + N * 4 + N * 2 + N // 32 * 36) + N * 4,
+                    (lambda tab=tab, rb=rb, fmt=fmt, xo=xo, xbf=xbf, qq=qq: B.call('camx_emb_gather_add_rms', _p(tab), L64(rb), I(V), _p(toks), _p(xo), _p(xbf), NULL, _p(nw),
+                                                                                   F(1e-6), NULL, NULL, _p(qq), I(N), I(n_tok), I(fmt)))))
+    # hybrid verify batch: 16 tokens, hidden 5120
+    T4, D4 = 16, 256
+    qg = B.acts((T4 * 24, 2 * D4), torch.bfloat16, 41); w4 = B.gamma(D4, 42)
+    pos = torch.from_numpy(rng.integers(0, 65536, T4).astype(np.int32)).to(B.dev)
+    o4 = torch.empty((T4 * 24, D4), dtype=torch.bfloat16, device=B.dev)
+    ts7 = float(np.float32(np.float32(1e7) ** np.float32(-2.0 / 64)))
+    out.append(('c4_qk_nr_partial_rotary_q', T4 * 24 * D4 * 4 + D4 * 4,
+                lambda: B.call('camx_qk_nr_pos', _p(qg), I(2 * D4), I(24), _p(w4), I(D4), I(64), F(ts7), F(1e-6), _p(pos), _p(o4), I(T4), I(1))))
+    a4 = B.acts((T4 * 24, D4), torch.bfloat16, 43)
+    out.append(('c4_sigmoid_gate', T4 * 24 * D4 * 6,
+                lambda: B.call('camx_gate_mul', _p(a4), _p(qg), _p(o4), L64(T4 * 24 * D4), I(D4), I(2 * D4), I(D4), I(2))))
+    Cc = 10240
+    xc = B.acts((T4, Cc), torch.bfloat16, 44); wc = B.acts((Cc, 4), torch.float32, 45, frac=0); st = B.acts((Cc, 3), torch.float32, 46, frac=0)
+    yc = torch.empty((T4, Cc), dtype=torch.bfloat16, device=B.dev)
+    out.append(('c4_conv4_silu', T4 * Cc * 4 + Cc * 16 + Cc * 12,
+                lambda: B.call('camx_pf_gdn_conv', _p(xc), _p(wc), _p(st), _p(yc), I(Cc), I(T4), I(Cc), I(Cc), I(1))))
+    l2o = torch.empty((T4 * 32, 128), dtype=torch.bfloat16, device=B.dev)
+    out.append(('c4_l2norm_qk', T4 * 32 * 128 * 4,
+                lambda: B.call('camx_pf_gdn_l2', _p(yc), _p(l2o), I(32), I(128), I(Cc), F(1e-6 / 128), I(T4), I(1))))
+    # batched decode: 256 sequences, Q8 KV codec into a paged cache
+    S5 = 256
+    x5 = B.acts((S5, N), torch.float32, 51); d5 = B.acts((S5, 1, N), torch.float32, 52)
+    h5 = torch.empty((S5, N), device=B.dev); h516 = torch.empty((S5, N), dtype=torch.float16, device=B.dev)
+    out.append(('c5_add_rms_256x2048', S5 * N * (12 + 6) + N * 4,
+                lambda: B.call('camx_q3p_add_rms16', _p(x5), _p(d5), NULL, I(1), _p(nw), F(1e-6), _p(h5), _p(h516), I(N), I(S5))))
+    qkv5 = B.acts((S5, ldq), torch.float32, 53)
+    page, n_pages = 256, 65536
+    rbq = 2 * (nkv * 128 // 32) * 34
+    pos5 = rng.integers(0, 131072, S5).astype(np.int32)
+    pt = rng.integers(0, n_pages, (S5, 512)).astype(np.int32)
+    pt[np.arange(S5), pos5 // page] = rng.permutation(n_pages)[:S5]          # the pages this launch writes are distinct
+    cache5 = torch.zeros(n_pages * page * rbq, dtype=torch.uint8, device=B.dev)
+    err5 = torch.zeros(1, dtype=torch.int32, device=B.dev)
+    pos5d, ptd = torch.from_numpy(pos5).to(B.dev), torch.from_numpy(pt).to(B.dev)
+    q165 = torch.empty((S5, nh, 128), dtype=torch.float16, device=B.dev)
+    out.append(('c5_qk_rope_hadamard_q8_paged', S5 * (ldq * 4 + 8 + nh * 128 * 2 + rbq) + 258 * 4,
+                lambda: B.call('camx_qk_rope_paged', _p(qkv5), I(ldq), I(nh), I(nkv), _p(par), _p(pos5d), _p(q165), _p(cache5), _p(err5), _p(ptd), I(512),
+                               I(page), I(n_pages), I(S5), I(0), I(1))))
+    out.append(('_keep', 0, [x, d, nw, h, h16, q8, qkv, par, q16, cache, g, u, y16, toks, qg, w4, pos, o4, a4, xc, wc, st, yc, l2o, x5, d5, h5, h516, qkv5,
+                             cache5, err5, pos5d, ptd, q165]))
+    return out
+
+
+def cpu_baseline(w, sample_tokens=128):
+    """the CPU oracle on the first sample_tokens tokens of the same three op-sets; GB/s by the same byte accounting"""
+    import numpy as np
+    import oracle as O
+    T, H, nh, nkv, Fh, ldq = sample_tokens, w['H'], w['nh'], w['nkv'], w['Fh'], w['ldq']
+    import torch
+
+    def bf_bits(t):
+        return t[:T].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+    x = w['x'][:T].cpu().numpy(); d = bf_bits(w['d']); nw = w['nw'].cpu().numpy()
+    qkv = O.bf2f(bf_bits(w['qkv'])); gu = bf_bits(w['gu'])
+    threads = int(os.environ.get('OMP_NUM_THREADS', '0')) or min(os.cpu_count() or 1, 16)
+    frac = T / w['T']
+    by = sum(w['bytes'].values()) * frac
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.add_rms_bf16(x, d, nw, 1e-6)
+        O.qk_rope(qkv, nh, nkv, w['par_np'], T, pos0=0, yarn=True, rows=T)
+        act = O.silu_mul_bf16(gu)
+        O.mmq_q8_1(O.bf2f(act), Fh, T, 1)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {'value': round(by / best / 1e9, 3), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
+            'sample': f'first {T} of {w["T"]} tokens of the same three op-sets, best of 3, {best * 1e3:.1f} ms'}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--no-cpu', action='store_true')
+    ap.add_argument('--no-extra', action='store_true')
+    ap.add_argument('--only', default=None, help='run a single kernel of the step (for profiling)')
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f'bench.py: this build measures one GPU only (--gpus {a.gpus} is not supported): the row kernels shard by token with no '
+              f'communication, so a multi-GPU figure would be N independent copies of this run', file=sys.stderr)
+        sys.exit(2)
+    B = Bench()
+    torch = B.torch
+    w = config3(B)
+    names = list(w['launch']) if not a.only else [a.only]
+
+    def step():
+        for n in names: w['launch'][n]()
+
+    for _ in range(a.warmup): step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(a.steps): step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = e0.elapsed_time(e1) / a.steps
+    total_bytes = sum(w['bytes'][n] for n in names)
+    # per-kernel average durations, measured live with events on the launch stream (steady state, same order as the step)
+    per = {}
+    for n in names:
+        med, mean = B.time_launch(w['launch'][n], reps=max(20, a.steps), warm=3)
+        per[n] = {'us': round(mean, 2), 'us_median': round(med, 2), 'bytes': w['bytes'][n], 'GBps': round(w['bytes'][n] / (mean * 1e-6) / 1e9, 1),
+                  'frac_of_8TBps': round(w['bytes'][n] / (mean * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+    dom = max(per, key=lambda n: per[n]['us'])
+    achieved = per[dom]['bytes'] / (per[dom]['us'] * 1e-6) / 1e9
+    out = {
+        'metric': 'fused-op HBM GB/s (% of MI355X peak) + us per layer op-set, 1 GPU', 'value': round(total_bytes / (ms_step * 1e-3) / 1e9, 1), 'unit': 'GB/s',
+        'n_gpus': 1, 'steps': a.steps, 'warmup': a.warmup, 'ms_per_step': round(ms_step, 4), 'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'dense 27B-class prefill chunk: 4096 tokens x hidden 5120, bf16 activations, fp32 residual and norms; op-sets add+RMSNorm, '
+                               'QK-norm+YaRN rotary (64 Q + 8 KV heads x 128), SwiGLU 4096x17408 -> q8_1 MMQ (DS4)', 'tokens': 4096, 'hidden': 5120,
+                   'kernels': names},
+        'frac_of_hbm_peak': round(total_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        'wall_ms_per_step': round(wall * 1e3 / a.steps, 4),
+        'roofline': {'bound': 'hbm', 'kernel': dom, 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': None},
+        'kernels': per,
+    }
+    if not a.no_extra and not a.only:
+        ops = {}
+        for name, by, fn in extra_opsets(B):
+            if name == '_keep': continue
+            med, mean = B.time_launch(fn, reps=50, warm=10, flush=True)
+            med_hot, _ = B.time_launch(fn, reps=50, warm=10, flush=False)
+            ops[name] = {'us': round(med, 2), 'us_cache_hot': round(med_hot, 2), 'bytes': by, 'GBps': round(by / (med * 1e-6) / 1e9, 1),
+                         'frac_of_8TBps': round(by / (med * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+        out['opsets'] = ops
+    if not a.no_cpu and not a.only:
+        out['cpu_baseline'] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

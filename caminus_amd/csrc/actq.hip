@@ -35,7 +35,7 @@ struct RmsSrc {
 template <typename Src>
 CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * __restrict__ s_out, int K, float clip, int qmax,
                            uint16_t * __restrict__ codes, float * lds) {
-    const int tid = threadIdx.x, l = tid & 31, hw = tid >> 5, nch = K / 128;
+    const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
     f32x4 u[MAXR];
     float amax = 0.0f;
 #pragma unroll
@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(256) actq_fwd_k(Src src, uint16_t * y, float *
 template <typename F>
 CAMX_DEV float row_tree_sum(F term, int d, float * slot) {
     if (threadIdx.x < 64) {
-        const int lane = threadIdx.x;
+        const int lane = slot_of(threadIdx.x);
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
         for (int base = 0; base < d; base += 256) {
             const int k = base + 4 * lane;

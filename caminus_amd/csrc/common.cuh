@@ -6,9 +6,15 @@
 //
 // The reference's reductions are stated for 256 logical threads in 32-lane groups (thread t owns elements t, t + 256, ..;
 // xor butterfly 16, 8, 4, 2, 1 inside each group of 32; the 8 group sums added in order). In L4, logical thread
-// t = 4 p + k, so a group of 32 logical threads is 8 consecutive lanes x 4 registers, and the butterfly becomes
-// lane xor 4, lane xor 2, lane xor 1, then register pairs (k, k ^ 2) and (k, k ^ 1): the same pairs in the same order,
+// t = 4 p + k, so a group of 32 logical threads is 8 consecutive slots x 4 registers, and the butterfly becomes
+// slot xor 4, slot xor 2, slot xor 1, then register pairs (k, k ^ 2) and (k, k ^ 1): the same pairs in the same order,
 // hence the same bits. The group sums are then read with v_readlane from lanes 0, 8, .., 56 and added in order.
+//
+// Slots and lanes: the position p above is a logical slot; slot u lives in lane slot_to_lane(u), which differs from u
+// only inside each group of 8: slots 4..7 sit in lanes 7..4. With that placement every slot exchange the kernels need is
+// one DPP modifier on the consuming VALU op (no LDS crossbar): slot ^ 1 and slot ^ 2 are quad permutes, slot ^ 4 is
+// row_half_mirror (lane 7 - l), slot ^ 8 is row_ror:8. Only slot ^ 16 takes a ds_swizzle. Kernels compute addresses from
+// slot_of(lane); a wave still touches the same contiguous bytes per instruction.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -24,10 +30,13 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 #define CAMX_DEV __device__ __forceinline__
 
-// ---- lane permutes (all 64 lanes must be active) ----------------------------------------------------------------------
+// lane -> the logical slot it holds (and back: the map is an involution)
+CAMX_DEV int slot_of(int lane) { const int s = lane & 7; return (lane & ~7) | (s < 4 ? s : 11 - s); }
+
+// ---- slot exchanges (every lane of the exchanging group must be active) ---------------------------------------------------
 CAMX_DEV float lane_xor1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)); }   // quad_perm [1,0,3,2]
 CAMX_DEV float lane_xor2(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)); }   // quad_perm [2,3,0,1]
-CAMX_DEV float lane_xor4(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x101f)); }               // swizzle SWAP,4
+CAMX_DEV float lane_xor4(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false)); }  // row_half_mirror
 CAMX_DEV float lane_xor8(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false)); }  // row_ror:8
 CAMX_DEV float lane_xor16(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401f)); }              // swizzle SWAP,16
 CAMX_DEV float lane_read(float v, int lane) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane)); }
@@ -113,7 +122,8 @@ CAMX_DEV f32x4 unpack_bf16x4(u32x2 w) {
 }
 
 // roundf (half away from zero) of a value known to fit int8 after rounding, as a signed byte in the low 8 bits
-CAMX_DEV uint32_t round_i8(float v) { return (uint32_t)(int)roundf(v) & 0xffu; }
+// trunc(v + copysign(0.49999997f, v)) equals roundf(v) for every float with |v| <= 256 (checked exhaustively on a CPU)
+CAMX_DEV uint32_t round_i8(float v) { return (uint32_t)(int)(v + __builtin_copysignf(0.49999997f, v)) & 0xffu; }
 CAMX_DEV uint32_t pack_round_i8x4(f32x4 v) {
     return round_i8(v.x) | (round_i8(v.y) << 8) | (round_i8(v.z) << 16) | (round_i8(v.w) << 24);
 }

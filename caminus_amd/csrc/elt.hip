@@ -115,7 +115,7 @@ __global__ void __launch_bounds__(256) conv_state_k(const void * __restrict__ x,
 // per head of K <= 512 values: y = (scale * x) * (1 / sqrt(K)), scale = 1 / sqrt(sum x^2 / K + rs); one wave per head
 template <bool BF16>
 __global__ void __launch_bounds__(256) gdn_l2_k(const void * __restrict__ x, void * __restrict__ y, int heads, int K, int ldx, float rs, int total) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (t >= total) return;
     const int tt = t / heads, hh = t - tt * heads;

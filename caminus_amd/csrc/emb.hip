@@ -57,7 +57,7 @@ struct EmbArgs {
 
 template <int FMT, int NI_MAX, bool TAIL>
 __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (t >= a.n) return;
     int tok = a.toks[t]; tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;

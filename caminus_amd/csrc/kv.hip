@@ -22,7 +22,7 @@ __global__ void __launch_bounds__(256) kv_q8_append_rows(const float * __restric
         return;
     }
     const size_t tt = blockIdx.x;
-    const int nb = M / 32, lane = threadIdx.x & 63, sub = lane & 7;
+    const int nb = M / 32, lane = slot_of(threadIdx.x & 63), sub = lane & 7;
     uint8_t * dst = cache + (size_t)pos * ((size_t)2 * nb * 34);
     for (int b0 = (threadIdx.x >> 6) * 8; b0 < 2 * nb; b0 += 32) {
         const int b = b0 + (lane >> 3);
@@ -39,7 +39,7 @@ __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restric
                                                          uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
     const int tt = blockIdx.x, pos = pos0 + tt;
     if (pos < 0 || pos >= rows) { if (threadIdx.x == 0) atomicOr(err, 1); return; }
-    const int nb = M / 32, lane = threadIdx.x & 63, sub = lane & 7;
+    const int nb = M / 32, lane = slot_of(threadIdx.x & 63), sub = lane & 7;
     uint8_t * base = cache + (size_t)pos * ((size_t)2 * nb * 34);
     for (int b0 = (threadIdx.x >> 6) * 8; b0 < 2 * nb; b0 += 32) {
         const int b = b0 + (lane >> 3);
@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(256) hadamard_chunks(float * __restrict__ x, l
 
 // out-of-place 128-point transform with the literal scale 0x1.6a09e6p-4f (the Q8 KV cache's rotation)
 __global__ void __launch_bounds__(256) hadamard128_heads(const float * __restrict__ x, float * __restrict__ y, long heads) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const long h = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
     const int l = lane & 31;
     const bool active = h < heads;

