@@ -1,0 +1,195 @@
+/* camx.h - C ABI of libcamx.so: the fused per-layer row kernels of the Caminus inference engine for AMD Instinct MI355X
+ * (gfx950). Plain pointers and sizes, no C++ or PyTorch types. Every pointer is a device pointer unless said otherwise.
+ *
+ * Conventions
+ *   - Every entry point queues work on `stream` (a hipStream_t; NULL = the default stream) and returns at once:
+ *     0, or a hipError_t value (1 = invalid value: a shape, alignment or pointer argument was refused and nothing was
+ *     launched). camx_error_string() names the value.
+ *   - The library allocates nothing per call and keeps no state between calls, except a 128 KiB lookup table that
+ *     camx_swiglu_mmq_q8_1 fills once per device on its first call.
+ *   - bf16 / fp16 values travel as uint16_t bit patterns. "rows" / "n" / "T" arguments that the reference kernels took
+ *     from their launch grid are explicit trailing arguments here.
+ *   - Device-side errors are sticky int32 words OR-ed by the kernels and never cleared by them; bit meanings are given at
+ *     each function.
+ *   - Each declaration cites the reference kernel or op it replaces (paths relative to the reference checkout).
+ *
+ * Numeric contract (see oracle/camx_oracle.c for the executable statement): sums of squares are formed as the reference
+ * forms them (256 logical threads, fmaf chains in element order, 32-lane xor butterfly, 8 group sums in order); rsqrt is
+ * 1 / sqrt with IEEE square root and division; quantizer outputs (q8_1, MMQ q8_1, Q8 KV blocks, actq codes), Hadamard
+ * transforms and GGUF dequantization are bit-exact; values that pass through expf / cosf / sinf are within 1e-5 relative
+ * (fp32 outputs) or one unit in the last place (fp16 / bf16 outputs).
+ */
+#ifndef CAMX_H
+#define CAMX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t * camx_stream_t;      /* = hipStream_t */
+
+/* ---- library ---------------------------------------------------------------------------------------------------------- */
+int camx_version(void);
+const char * camx_arch(void);                     /* "gfx950" */
+const char * camx_error_string(int err);          /* hipGetErrorString; replaces device/hip.py:35-37's lookup */
+
+/* ---- residual add + RMSNorm -------------------------------------------------------------------------------------------- */
+/* q3p_add_rms16 (kernels/q3m_prefill.hip:385-415) = OP_OWN_ADD_RMS16 (kernels/k3_own_ops.h:326-383).
+ * Per token t < n: x[t] += sum over slots s < S of w[t][s] * d[t][s] (fma in slot order from 0; w NULL: acc + d; S = 0 or
+ * d NULL: no add), x written back; h = (x * scale) * nw, h16 = fp16(h). N = 256 NI <= 2048, S <= 8. h may be NULL. */
+int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
+                       uint16_t * h16, int N, int n, camx_stream_t stream);
+/* q35p_add_rms16 (kernels/q35_prefill.hip:636-660) = the dense line's OP_OWN_ADD_RMS16 (kernels/k3_q35_ops.h:79-145).
+ * x = x + d (d NULL: no add), any N = 256 NI <= 65536; h and h16 are both written. */
+int camx_q35p_add_rms16(float * x, const float * d, const float * nw, float eps, float * h, uint16_t * h16, int N, int n,
+                        camx_stream_t stream);
+/* The same row pass with a q8_1 copy of h (36-byte blocks, [n][N / 32]): OP_RMS_MUL's optional q8_1 output
+ * (kernels/k3_gguf_ops.h:1233-1268, q8_emit :158-162) on q3p_add_rms16's add. h, h16, q8 optional; N % 32 == 0. */
+int camx_add_rms_q8_1(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
+                      uint16_t * h16, void * q8, int N, int n, camx_stream_t stream);
+/* Dense bf16 prefill form: x (fp32 residual) = x + bf16 addend d (kernels/core.hip:57-61's promotion; d NULL: no add), then
+ * q35p_add_rms16's norm; hbf = bf16 copy of h by round-to-nearest-even (kernels/prefill_glue.hip:77-80). h, hbf optional. */
+int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps, float * h, uint16_t * hbf, int N, int n,
+                      camx_stream_t stream);
+/* pf_rms_mul (kernels/prefill_glue.hip:94-124): y[r] = (x[r] * scale_r) * w[r % wr] for R rows of K values; y (may be x),
+ * ybf (bf16 copy), scl (row scale [R]) each optional. The reference kernel is built for K = 2560; K is an argument here. */
+int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf, float * scl, int R, int wr, float eps, int K,
+                    camx_stream_t stream);
+/* OP_RMS_MUL (kernels/k3_gguf_ops.h:1233-1268; Seg fields: a = x, W = w, y, asum = q8, N = R, K, pad1 = wr, rs = eps). */
+int camx_op_rms_mul(const float * x, const float * w, float * y, void * q8, int R, int wr, int K, float eps, camx_stream_t stream);
+/* rmsnorm_f32 (kernels/core.hip:30-46): out = x * inv * w over `rows` rows of D values (any D). */
+int camx_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows, camx_stream_t stream);
+
+/* ---- q8_1 activation quantizers ------------------------------------------------------------------------------------------ */
+/* gg_quantize_q8_1 (kernels/k3_gguf.hip:29-36) and OP_GG_Q8_1 (kernels/k3_gguf_ops.h:55-77): y = ceil(n / 32) blocks of
+ * {half d, half sum, int8 qs[32]}; mode 0 plain, 1 silu(x * rs), 2 silu(x) * g[i]; values past n quantize as 0. */
+int camx_gg_quantize_q8_1(const float * x, void * y, long n, int mode, float rs, const float * g, camx_stream_t stream);
+/* quantize_mmq_q8_1<layout, false> (kernels/ggml_mmq/quantize_mmq.cuh:41-140; launched by prefill/mmq.py:245-261):
+ * column c of vy = row (ids ? ids[c] : c) of x (row stride s01 floats), blocks of 144 bytes per 128 values in
+ * [ne0 / 128][ne1] order, ne00 = K, ne0 = K padded to 512 (padding quantizes as zeros). layout 0 = D4, 1 = DS4.
+ * s02, s03 must be 0 and ne2 1 (the reference's callers pass exactly that). */
+int camx_quantize_mmq_q8_1(const float * x, const int32_t * ids, void * vy, long ne00, long s01, long s02, long s03, long ne0,
+                           int ne1, int ne2, int n_expert_used, int layout, camx_stream_t stream);
+/* quantize_mmq_q8_1<layout, true> (same source; prefill/mmq.py:263-276): token t's row (stride s02 floats) quantized once and
+ * written to the columns ids[t * n_expert_used + slot] of the ne1 = ntok * n_expert_used compact columns. */
+int camx_quantize_mmq_q8_1_scatter(const float * x, const int32_t * ids, void * vy, long ne00, long s01, long s02, long s03,
+                                   long ne0, int ne1, int ne2, int n_expert_used, int layout, int ntok, camx_stream_t stream);
+/* Fused SwiGLU -> MMQ q8_1: gu bf16 [T][ld] = [g (F) | u (F)]; act = bf16(bf16(silu g) * u) (silu_mul_bf16,
+ * kernels/core.hip:48-55) quantized as quantize_mmq_q8_1 of the fp32-widened act. act (optional, bf16 [T][F]) receives
+ * the activation. Fills a per-device lookup table on its first call (synchronizes `stream` once). */
+int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16_t * act, int T, int layout, camx_stream_t stream);
+
+/* ---- SwiGLU, gates ------------------------------------------------------------------------------------------------------------ */
+/* q3p_swiglu (kernels/q3m_prefill.hip:516-518) = OP_OWN_SWIGLU16 (kernels/k3_own_ops.h:258-262): y16 = fp16(silu(g) * u). */
+int camx_q3p_swiglu(const float * g, const float * u, uint16_t * y16, int n, camx_stream_t stream);
+/* gg_silu_mul (kernels/k3_gguf.hip:74-77): h = silu(g) * u in fp32. */
+int camx_gg_silu_mul(const float * g, const float * u, float * h, int n, camx_stream_t stream);
+/* silu_mul_bf16 (kernels/core.hip:48-55): act[r][c] = bf16(bf16(silu(g)) * u), gu rows = [g (H) | u (H)], n = rows * H. */
+int camx_silu_mul_bf16(const uint16_t * gu, uint16_t * act, int H, long n, camx_stream_t stream);
+/* pf_gate_mul (kernels/prefill_attn.hip:379-386; io 0: fp32 -> fp32), q35p_gate_mul16 / OP_GATE_MUL16
+ * (kernels/q35_prefill.hip:960-969, kernels/k3_q35_ops.h:381-391; io 1: fp32 -> fp16), io 2: bf16 a and gate -> bf16:
+ * y[i] = a[i] * sigmoid(gate[(i / D) * stride + off + i % D]) over N elements. */
+int camx_gate_mul(const void * a, const void * gate, void * y, long N, int D, int stride, int off, int io, camx_stream_t stream);
+
+/* ---- QK-norm + rotary, KV rows ------------------------------------------------------------------------------------------------ */
+/* q3p_qk_rope (kernels/q3m_prefill.hip:534-591, F16 form; yarn = the Q3P_YARN build): n tokens at positions pos0 + t;
+ * qkv fp32 [n][ldq] = q (nh heads of 128) | k (nkv) | v (nkv); par = q_norm[128] | k_norm[128] | theta_scale | eps
+ * (| freq[64] | mscale when yarn); q16 fp16 [n][nh][128]; cache = fp16 rows [K | V] indexed by position. The caller has
+ * checked the positions against the cache's rows (prefill/q3m_ops.py:103-117). */
+int camx_q3p_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
+                     int n, int yarn, camx_stream_t stream);
+/* q3p_qk_rope_q8 (same source under Q3P_KV_Q8; rotation kernels/own_kv_rot128.h:21-33, block encode
+ * kernels/own_kv_codec.h:57-72): K = Hadamard-128 of the fp16-rounded rotary output, V = fp16-rounded v, both as Q8 blocks;
+ * q16 = fp16 of the same transform of q. err: bit 2 ORed when a block is refused (its bytes stay untouched). */
+int camx_q3p_qk_rope_q8(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint8_t * cache,
+                        int * err, int n, int yarn, camx_stream_t stream);
+/* The same statements on bf16 activations (qkv bf16, widened exactly), F16 rows: a dense bf16 prefill chunk. */
+int camx_qk_rope_bf16(const uint16_t * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
+                      int n, int yarn, camx_stream_t stream);
+/* Batched decode form of the two kernels above: sequence t at its own position pos[t]; with page_table the row address is
+ * (page_table[t * pt_stride + pos / page] * page + pos % page) * row_bytes, else pos * row_bytes. q8 selects the row format.
+ * err bit 8: a page id outside [0, n_pages) (that sequence's row is not written). Paging has no reference counterpart:
+ * each row's bytes equal the unpaged kernel's. */
+int camx_qk_rope_paged(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16,
+                       void * cache, int * err, const int32_t * page_table, int pt_stride, int page, int n_pages, int n, int yarn,
+                       int q8, camx_stream_t stream);
+/* pf_qk_nr (kernels/prefill_attn.hip:106-129) = OP_QK_NR (kernels/k3_gguf_ops.h:1495-1518, kernels/k3_q35_ops.h:341-364):
+ * out [T][heads][D] = rotary on the first nrot dims of rms_norm(x head) * w, row r at position pos0 + r; input heads sit
+ * head_stride elements apart; D <= 512. io 0: fp32 in / out, 1: bf16 in / out. */
+int camx_pf_qk_nr(const void * xin, int head_stride, int heads, const float * w, int D, int nrot, float theta_scale, float eps,
+                  int pos0, void * out, int T, int io, camx_stream_t stream);
+/* The same with one position per row (a speculative-verify batch). */
+int camx_qk_nr_pos(const void * xin, int head_stride, int heads, const float * w, int D, int nrot, float theta_scale, float eps,
+                   const int32_t * pos, void * out, int T, int io, camx_stream_t stream);
+/* out[j] = the frequency of rotary pair j as the kernels above compute it: the correctly rounded theta_scale ** j. */
+int camx_rope_freqs(float theta_scale, int n, float * out, camx_stream_t stream);
+
+/* own_kv_q8_append (kernels/kv_codec.hip:10-30 with kernels/own_kv_codec.h:33-52; launcher device/kv_codec.py:48-83):
+ * T rows of M values from k / v (row strides ldk / ldv) to cache rows pos0 + t of 2 * (M / 32) blocks of 34 bytes.
+ * err bits: 1 position outside [0, rows), 2 refused block (bytes untouched), 4 layout (M < 32, M % 32, ld < M, rows < 1). */
+int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows,
+                          int * err, int T, camx_stream_t stream);
+/* pf_kv_append, q8_0 rows (kernels/prefill_attn.hip:157-181) = OP_KV_APPEND work 1 (kernels/k3_gguf_ops.h:1532-1553):
+ * no refusal rules; err bit 1 for a row outside [0, rows). */
+int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
+                      int T, camx_stream_t stream);
+/* pf_hadamard (kernels/prefill_attn.hip:132-153) = OP_HADAMARD (kernels/k3_gguf_ops.h:1699-1721): in place, C chunks of
+ * n in {64, 128, 256} values, scale 1 / sqrtf(n). rpb (the reference's chunks per workgroup) is accepted and ignored. */
+int camx_pf_hadamard(float * x, int C, int n, int rpb, camx_stream_t stream);
+/* own_kv_rot128 as a kernel of its own (kernels/own_kv_rot128.h:21-33; CPU reference python/caminus/ref_kv.py:72-89):
+ * y = H128 x per head of 128 values, scale 0x1.6a09e6p-4f. */
+int camx_hadamard128(const float * x, float * y, long heads, camx_stream_t stream);
+
+/* ---- quantized embedding rows ------------------------------------------------------------------------------------------------ */
+/* q3p_emb (kernels/q3m_prefill.hip:364-380) = OP_OWN_EMB (kernels/k3_own_ops.h:279-304): x [n][N] fp32 = the Q4_K rows
+ * toks[i] of W (rb bytes per row), ids clamped to [0, vocab). */
+int camx_q3p_emb(const uint8_t * W, int rb, int vocab, const int32_t * toks, float * x, int N, int n, camx_stream_t stream);
+/* Gather + dequant to fp32 (x) and / or bf16 (xbf); fmt 0 = Q4_K (as q3p_emb), 1 = Q8_0 (the host decoder's arithmetic,
+ * python/caminus/own_dequant.py:202-206). N = 256 NI <= 8192. */
+int camx_emb_gather(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int N, int n, int fmt,
+                    camx_stream_t stream);
+/* Gather + dequant + (x += d) + RMSNorm * nw with fp32 / fp16 / q8_1 copies of the normed row in one pass per row
+ * (q3p_emb followed by q3p_add_rms16 and OP_RMS_MUL's q8_1 copy). xbf = bf16 of the gathered row; x = the residual row. */
+int camx_emb_gather_add_rms(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, const float * d,
+                            const float * nw, float eps, float * h, uint16_t * h16, void * q8, int N, int n, int fmt,
+                            camx_stream_t stream);
+
+/* ---- GDN short convolution and L2 norm ------------------------------------------------------------------------------------------ */
+/* pf_gdn_conv (kernels/prefill_glue.hip:314-332) = OP_GDN_CONV (kernels/k3_q35_ops.h:152-177): y[t][c] = silu(fma chain
+ * of [x(t-3) .. x(t)] . w[c]), times before 0 from state[c] = [x(-3), x(-2), x(-1)]. bf16 != 0: x and y are bf16. */
+int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void * y, int C, int T, int ldx, int ldy, int bf16,
+                     camx_stream_t stream);
+/* pf_conv_state (kernels/prefill_glue.hip:334-341): state[c] = the last 3 inputs of [state[c], x[0 .. T-1][c]]. */
+int camx_pf_conv_state(const void * x, float * state, int C, int T, int ldx, int bf16, camx_stream_t stream);
+/* pf_gdn_l2 (kernels/prefill_gdn.hip:66-78) = OP_GDN_L2 (kernels/k3_q35_ops.h:181-194): per head of K <= 512 values
+ * y = (scale * x) * (1 / sqrt(K)), scale = 1 / sqrt(sum x^2 / K + rs); head h of token t at x + t * ldx + h * K. */
+int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs, int T, int bf16, camx_stream_t stream);
+
+/* ---- S1 core and fused residual (kernels/core.hip, kernels/fuse.hip) ------------------------------------------------------------- */
+int camx_embedding_f32(const int * tok, const float * emb, float * out, int D, int T, camx_stream_t stream);          /* core.hip:23-28 */
+int camx_residual3(const float * x, const uint16_t * m, const uint16_t * y, float * out, long n, camx_stream_t stream); /* core.hip:57-61 */
+int camx_cast_bf16(const float * x, uint16_t * out, long n, camx_stream_t stream);                                     /* core.hip:63-66 */
+int camx_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out, int ld_out, int c_out, int n, long rows,
+                        camx_stream_t stream);                                                                          /* core.hip:69-75 */
+/* residual_slices_fwd (kernels/fuse.hip:19-33): out = ((x + m) + mlp) + (pos[r] >= 0 ? ys[pos[r]] : 0); ys / pos may be NULL. */
+int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t * mlp, const uint16_t * ys, const int * pos,
+                             float * out, int d, long n4, camx_stream_t stream);
+
+/* ---- activation fake-quant, forward (kernels/actq.hip) ------------------------------------------------------------------------------ */
+/* actq_fwd_{f32,bf16} and actq_fwd_codes_{f32,bf16} (kernels/actq.hip:96-132, 315-326): M rows of K values (K % 128 == 0,
+ * K <= 8192); y bf16 [M][K] (optional when codes are written), s [M] (optional), codes [M][K / 2] bytes (optional). */
+int camx_actq_fwd(const void * x, int is_bf16, uint16_t * y, float * s, uint16_t * codes, int K, float clip, int qmax, int M,
+                  camx_stream_t stream);
+/* silu_mul_actq_fwd (kernels/actq.hip:307-310): the source is bf16(bf16(silu g) * u) of gu rows (stride ld) = [g (F) | u (F)]. */
+int camx_silu_mul_actq_fwd(const uint16_t * gu, int ld, int F, uint16_t * y, float * s, uint16_t * codes, float clip, int qmax, int M,
+                           camx_stream_t stream);
+/* block_entry_fwd (kernels/actq.hip:247-274): RMSNorm(x) never materialized -> actq -> nab gate projections. */
+int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y, float * s,
+                         uint16_t * codes, uint16_t * ab, float * rstd_out, int d, float clip, int qmax, int M, camx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CAMX_H */
