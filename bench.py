@@ -24,6 +24,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of each kernel of the step, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file
+# (KiB per dispatch, scaled by what the same counters read for the 256 MiB copy of --only copy_ref: FETCH_SIZE reads half
+# the bytes moved, WRITE_SIZE reads them all); the summaries are kept under profiles/
+HBM_TRAFFIC = {'add_rms_bf16': 126495 * 1024 + 122880 * 1024, 'qk_rope_bf16': 82001 * 1024 + 81920 * 1024,
+               'swiglu_mmq_q8_1': 279708 * 1024 + 78336 * 1024}
 I, F, L64 = C.c_int, C.c_float, C.c_int64
 NULL = C.c_void_p(None)
 
@@ -247,29 +252,39 @@ def main():
         sys.exit(2)
     B = Bench()
     torch = B.torch
+    if a.only == 'copy_ref':
+        # a plain device copy of known size (256 MiB read + 256 MiB written per launch): the yardstick that FETCH_SIZE / WRITE_SIZE
+        # counter readings of the kernels above are scaled by
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=B.dev); dst = torch.empty_like(src)
+        med, mean = B.time_launch(lambda: dst.copy_(src), reps=a.steps, warm=a.warmup)
+        print(json.dumps({'kernel': 'copy_ref', 'bytes_read': src.numel(), 'bytes_written': src.numel(), 'us': round(mean, 2),
+                          'GBps': round(2 * src.numel() / (mean * 1e-6) / 1e9, 1)}))
+        return
     w = config3(B)
     names = list(w['launch']) if not a.only else [a.only]
 
-    def step():
+    for _ in range(a.warmup):
         for n in names: w['launch'][n]()
-
-    for _ in range(a.warmup): step()
     torch.cuda.synchronize()
+    # the timed region: K steps, a HIP event on the launch stream before and after every kernel, so the same K steps give the
+    # step time (first event to last) and each kernel's average duration in the order and cache state of the real step
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(a.steps)]
     t0 = time.perf_counter()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(a.steps): step()
-    e1.record()
+    for k in range(a.steps):
+        ev[k][0].record()
+        for i, n in enumerate(names):
+            w['launch'][n]()
+            ev[k][i + 1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_step = e0.elapsed_time(e1) / a.steps
+    ms_step = ev[0][0].elapsed_time(ev[-1][-1]) / a.steps
     total_bytes = sum(w['bytes'][n] for n in names)
-    # per-kernel average durations, measured live with events on the launch stream (steady state, same order as the step)
     per = {}
-    for n in names:
-        med, mean = B.time_launch(w['launch'][n], reps=max(20, a.steps), warm=3)
+    for i, n in enumerate(names):
+        ts = sorted(ev[k][i].elapsed_time(ev[k][i + 1]) * 1e3 for k in range(a.steps))
+        mean, med = sum(ts) / len(ts), ts[len(ts) // 2]
         per[n] = {'us': round(mean, 2), 'us_median': round(med, 2), 'bytes': w['bytes'][n], 'GBps': round(w['bytes'][n] / (mean * 1e-6) / 1e9, 1),
-                  'frac_of_8TBps': round(w['bytes'][n] / (mean * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+                  'frac_of_8TBps': round(w['bytes'][n] / (mean * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), 'hbm_traffic_bytes': HBM_TRAFFIC.get(n)}
     dom = max(per, key=lambda n: per[n]['us'])
     achieved = per[dom]['bytes'] / (per[dom]['us'] * 1e-6) / 1e9
     out = {
@@ -282,7 +297,7 @@ def main():
         'frac_of_hbm_peak': round(total_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         'wall_ms_per_step': round(wall * 1e3 / a.steps, 4),
         'roofline': {'bound': 'hbm', 'kernel': dom, 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': None},
+                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': HBM_TRAFFIC.get(dom)},
         'kernels': per,
     }
     if not a.no_extra and not a.only:
