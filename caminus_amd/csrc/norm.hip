@@ -74,9 +74,9 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) {
-                const f32x4 dv = unpack_bf16x4(*(const u32x2 *)(dr + 256 * j + 4 * lane));
+                const f32x4 dv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane)));
                 xv[j] = xv[j] + dv;
-                *(f32x4 *)(xr + 256 * j + 4 * lane) = xv[j];
+                __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
             }
     }
     // sum of squares: logical thread 4 lane + k chains its elements in j order
@@ -100,7 +100,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
             const size_t o = (size_t)row * N + 256 * j + 4 * lane;
             if (a.h) *(f32x4 *)(a.h + o) = v;
             if (a.h16) *(u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane) = pack_f16x4(v);
-            if (a.hbf) *(u32x2 *)(a.hbf + o) = pack_bf16x4_rne(v);
+            if (a.hbf) __builtin_nontemporal_store(pack_bf16x4_rne(v), (u32x2 *)(a.hbf + o));
             if (a.q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
         }
 }

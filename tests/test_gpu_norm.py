@@ -22,7 +22,7 @@ def test_q3p_add_rms16(n, N, S, weighted):
     assert bits_equal(host(h16, np.uint16), ref['h16'])
 
 
-@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096)])
+@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096), (520, 4096), (513, 8192), (600, 3072)])
 def test_q35p_add_rms16(n, N):
     rng = np.random.default_rng(7 + N)
     x = outliers(rng, (n, N)); d = outliers(rng, (n, N)); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
@@ -46,7 +46,7 @@ def test_add_rms_q8_1(n, N):
     assert bits_equal(host(q8), ref['q8'])
 
 
-@pytest.mark.parametrize('n,N', [(3, 5120), (64, 5120), (2, 2048)])
+@pytest.mark.parametrize('n,N', [(3, 5120), (64, 5120), (2, 2048), (600, 5120), (515, 6144), (512, 7168)])
 def test_add_rms_bf16(n, N):
     rng = np.random.default_rng(1003 + N)
     x = outliers(rng, (n, N)); d = O.f2bf(outliers(rng, (n, N))); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
@@ -57,7 +57,7 @@ def test_add_rms_bf16(n, N):
     assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(hbf, np.uint16), ref['hbf'])
 
 
-@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2)])
+@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2), (516, 3072, 4), (512, 5120, 1)])
 def test_rms_mul_and_rmsnorm(R, K, wr):
     rng = np.random.default_rng(R * K)
     x = outliers(rng, (R, K)); w = (1 + 0.1 * rng.standard_normal((wr, K))).astype(np.float32)

@@ -126,3 +126,23 @@ def test_pf_qk_nr(T, heads, D, n_rot, stride, base):
     call('camx_qk_nr_pos', ptr(dev(xb)), I(stride), I(heads), ptr(dev(w)), I(D), I(n_rot), F(ts), F(1e-6), ptr(dev(pos)), ptr(outb), I(T), I(1))
     refb = np.concatenate([O.qk_nr(O.bf2f(xb)[t * heads:(t + 1) * heads], stride, heads, w, D, n_rot, ts, 1e-6, int(pos[t]), 1) for t in range(T)])
     assert close_16(host(outb, np.uint16), O.f2bf(refb), 'bf16')
+
+
+@pytest.mark.parametrize('nh,nkv,n,pos0,yarn,pad', [(64, 8, 7, 4089, True, 0), (32, 4, 3, 0, False, 8), (5, 3, 4, 77, False, 24), (96, 8, 2, 100, True, 0),
+                                                    (1, 1, 2, 5, False, 4)])
+def test_qk_rope_bf16(nh, nkv, n, pos0, yarn, pad):
+    """bf16 activations (a dense prefill chunk): the same statements on the exactly widened values; head counts that are not
+    multiples of four, rows longer than 80 heads and a row stride that defeats the 128-bit path are all covered"""
+    rng = np.random.default_rng(2003 + nh + n)
+    tab = rope.yarn_table(128, 1e6, 4.0, 32768) if yarn else None
+    par = qk_par(rng, yarn_table=tab)
+    ldq = (nh + 2 * nkv) * 128 + pad
+    qkv = O.f2bf(outliers(rng, (n, ldq)) * np.float32(1.3))
+    M = nkv * 128; rows = pos0 + n + 1
+    q16 = dev(np.zeros((n, nh, 128), np.uint16)); c16 = dev(np.zeros((rows, 2 * M), np.uint16))
+    call('camx_qk_rope_bf16', ptr(dev(qkv)), I(ldq), I(nh), I(nkv), ptr(dev(par)), I(pos0), ptr(q16), ptr(c16), I(n), I(int(yarn)))
+    rq, rc, _ = O.qk_rope(O.bf2f(qkv), nh, nkv, par, n, pos0=pos0, yarn=yarn, rows=rows)
+    gq, gc = host(q16, np.uint16), host(c16, np.uint16)
+    assert close_16(gq, rq, 'f16') and close_16(gc[pos0:pos0 + n, :M], rc[pos0:pos0 + n, :M], 'f16')
+    assert bits_equal(gc[:, M:], rc[:, M:])                              # V: an exact conversion
+    assert not gc[:pos0].any() and not gc[pos0 + n:].any()
