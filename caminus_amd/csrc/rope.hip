@@ -115,87 +115,138 @@ CAMX_DEV uint32_t pack_f16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, f16x2));
 }
 
-template <bool YARN>
+// v + (v of lane ^ 1), v + (v of lane ^ 2), (v of lane ^ 8 inside its row of 16) * m: the cross-lane move rides on the
+// arithmetic instruction as a DPP source modifier (every lane is active wherever these are used)
+template <int CTRL> CAMX_DEV float dpp_full(float v) {   // full row / bank masks and bound_ctrl: the backend folds the move into its user
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+CAMX_DEV float add_xor1(float v) { return dpp_full<0xB1>(v) + v; }
+CAMX_DEV float add_xor2(float v) { return dpp_full<0x4E>(v) + v; }
+CAMX_DEV float mul_ror8(float v, float m) { return dpp_full<0x128>(v) * m; }
+template <int S> CAMX_DEV float row_lane_bcast(float v) {   // every lane of a 16-lane row reads the row's lane S
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x10 | (S << 5)));
+}
+
+// TPW tokens per workgroup. With four, wave w computes the cos / sin row of token w while every wave's first loads are in
+// flight, one barrier publishes the four rows, and then each wave walks the four tokens on its own, loading token i + 1's
+// heads before it does token i's arithmetic. With one (small batches), wave 0 computes the row.
+template <bool YARN, int TPW>
 __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
-    __shared__ __attribute__((aligned(16))) float rc[64];
-    __shared__ __attribute__((aligned(16))) float rs[64];
+    __shared__ __attribute__((aligned(16))) float rc[TPW][64];
+    __shared__ __attribute__((aligned(16))) float rs[TPW][64];
     __shared__ __attribute__((aligned(16))) float nrm[256];                  // q_norm | k_norm
-    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, hq = lane >> 4;
-    const int pos = a.pos ? a.pos[t] : a.pos0 + t;
-    const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)t * a.ldq;
+    const int t0 = blockIdx.x * TPW, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, hq = lane >> 4;
     const int items = a.nh + 2 * a.nkv, nqk = a.nh + a.nkv;
     const size_t M = (size_t)a.nkv * 128;
-    uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
-    f32x4 c4[2], s4[2];
-    for (int base = 0; base < items; base += 16 * RB_STEPS) {
-        u32x4 xin[RB_STEPS];
+    const int lo = 128 * hq + 8 * l16;                                      // this lane's element offset inside a wave step
+    const int nchunk = (items + 16 * RB_STEPS - 1) / (16 * RB_STEPS);       // a row longer than 80 heads takes several passes
+    u32x4 xin[RB_STEPS], xnext[RB_STEPS];
+    auto load = [&](u32x4 (&buf)[RB_STEPS], int tok, int base) {
+        const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)tok * a.ldq;
 #pragma unroll
         for (int s = 0; s < RB_STEPS; s++) {                                // wave step s: heads base + 16 s + 4 wave + (0 .. 3)
-            const int h = base + 16 * s + 4 * wave + hq;
-            xin[s] = (u32x4){0u, 0u, 0u, 0u};
-            if (h < items) xin[s] = __builtin_nontemporal_load((const u32x4 *)(rowb + (size_t)h * 128 + 8 * l16));
+            const int h0 = base + 16 * s + 4 * wave;
+            buf[s] = (u32x4){0u, 0u, 0u, 0u};
+            if (tok < a.n && h0 + hq < items) buf[s] = __builtin_nontemporal_load((const u32x4 *)(rowb + (size_t)h0 * 128 + lo));
         }
-        if (base == 0) {
-            nrm[tid] = a.par[tid];
-            if (tid < 64) {
-                float c, sn;
-                if (YARN) { const float theta = (float)pos * a.par[258 + tid], ms = a.par[322]; c = cosf(theta) * ms; sn = sinf(theta) * ms; }
-                else { const float theta = (float)pos * rope_freq(a.par[256], tid); c = cosf(theta); sn = sinf(theta); }
-                rc[tid] = c; rs[tid] = sn;
-            }
-            __syncthreads();
-            const int j0 = 8 * (l16 & 7);
-            c4[0] = *(const f32x4 *)(rc + j0); c4[1] = *(const f32x4 *)(rc + j0 + 4);
-            s4[0] = *(const f32x4 *)(rs + j0); s4[1] = *(const f32x4 *)(rs + j0 + 4);
-            if (l16 < 8) { s4[0] = -s4[0]; s4[1] = -s4[1]; }                // dims below 64 take -(x1 s): the sign moves into s
+    };
+    load(xin, t0, 0);
+    nrm[tid] = a.par[tid];
+    {
+        const int tr = TPW == 1 ? 0 : wave;                                 // the token whose row this wave computes
+        if ((TPW > 1 || tid < 64) && t0 + tr < a.n) {
+            const int pos = a.pos ? a.pos[t0 + tr] : a.pos0 + t0 + tr;
+            float c, sn;
+            if (YARN) { const float theta = (float)pos * a.par[258 + lane], ms = a.par[322]; c = cosf(theta) * ms; sn = sinf(theta) * ms; }
+            else { const float theta = (float)pos * rope_freq(a.par[256], lane); c = cosf(theta); sn = sinf(theta); }
+            rc[tr][lane] = c; rs[tr][lane] = sn;
         }
-        const float eps = a.par[257];
+    }
+    __syncthreads();
+    const float eps = a.par[257];
+    for (int it = 0; it < TPW * nchunk; it++) {
+        const int ti = it / nchunk, base = (it - ti * nchunk) * 16 * RB_STEPS, t = t0 + ti;
+        if (t >= a.n) break;
+        if (it + 1 < TPW * nchunk) { const int tn = (it + 1) / nchunk; load(xnext, t0 + tn, ((it + 1) - tn * nchunk) * 16 * RB_STEPS); }
+        const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+        uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
+        uint16_t * qw = a.q16 + (size_t)t * a.nh * 128;
+        const int j0 = 8 * (l16 & 7);
+        f32x4 c4[2], s4[2];
+        c4[0] = *(const f32x4 *)(rc[ti] + j0); c4[1] = *(const f32x4 *)(rc[ti] + j0 + 4);
+        s4[0] = *(const f32x4 *)(rs[ti] + j0); s4[1] = *(const f32x4 *)(rs[ti] + j0 + 4);
+        if (l16 < 8) { s4[0] = -s4[0]; s4[1] = -s4[1]; }                    // dims below 64 take -(x1 s): the sign moves into s
+        // phase 1: the sum of squares of every step's heads (V heads included: their sums are never used)
+        float x[RB_STEPS][8], tot[RB_STEPS];
 #pragma unroll
         for (int s = 0; s < RB_STEPS; s++) {
-            const int h = base + 16 * s + 4 * wave + hq;
-            if (base + 16 * s + 4 * wave >= items) break;                   // wave-uniform: no head of this step exists
-            const bool active = h < items;
-            float x[8];
 #pragma unroll
-            for (int p = 0; p < 4; p++) { x[2 * p] = __builtin_bit_cast(float, xin[s][p] << 16); x[2 * p + 1] = __builtin_bit_cast(float, xin[s][p] & 0xffff0000u); }
-            u32x4 out;
-            if (__builtin_amdgcn_readfirstlane(base + 16 * s + 4 * wave) >= nqk) {          // the whole step is V heads: fp16 copy
-#pragma unroll
-                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[2 * p], x[2 * p + 1]);
-                if (active) *(u32x4 *)(cw + M + (size_t)(h - nqk) * 128 + 8 * l16) = out;
-                continue;
-            }
+            for (int p = 0; p < 4; p++) { x[s][2 * p] = __builtin_bit_cast(float, xin[s][p] << 16); x[s][2 * p + 1] = __builtin_bit_cast(float, xin[s][p] & 0xffff0000u); }
             float sq[8];
 #pragma unroll
-            for (int k = 0; k < 8; k++) sq[k] = x[k] * x[k];
+            for (int k = 0; k < 8; k++) sq[k] = x[s][k] * x[s][k];
 #pragma unroll
-            for (int k = 0; k < 8; k++) sq[k] += dpp_xor2(sq[k]);           // thread ^ 16
+            for (int k = 0; k < 8; k++) sq[k] = add_xor2(sq[k]);            // thread ^ 16
 #pragma unroll
-            for (int k = 0; k < 8; k++) sq[k] += dpp_xor1(sq[k]);           // thread ^ 8
+            for (int k = 0; k < 8; k++) sq[k] = add_xor1(sq[k]);            // thread ^ 8
             const float b0 = sq[0] + sq[4], b1 = sq[1] + sq[5], b2 = sq[2] + sq[6], b3 = sq[3] + sq[7];   // thread ^ 4
             const float e0 = b0 + b2, e1 = b1 + b3;                         // thread ^ 2
             const float g = e0 + e1;                                        // thread ^ 1
-            const float tot = ((swz_group(g, 0) + swz_group(g, 1)) + swz_group(g, 2)) + swz_group(g, 3);
-            const float scale = rsqrt_exact(tot / 128 + eps);
-            const bool isq = h < a.nh, isv = h >= nqk;
-            const float * wp = nrm + (isq ? 0 : 128) + 8 * l16;
-            const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
-            float y1[8], y[8];
+            tot[s] = ((swz_group(g, 0) + swz_group(g, 1)) + swz_group(g, 2)) + swz_group(g, 3);
+        }
+        // phase 2: one IEEE sqrt + divide per row for all steps: lane s of a row takes step s, the row reads it back
+        float tv = tot[0];
 #pragma unroll
-            for (int k = 0; k < 8; k++) y1[k] = (scale * x[k]) * (k < 4 ? w0[k] : w1[k - 4]);
+        for (int s = 1; s < RB_STEPS; s++) tv = l16 == s ? tot[s] : tv;
+        const float sc = rsqrt_exact(tv / 128 + eps);
+        float scale[RB_STEPS];
+        scale[0] = row_lane_bcast<0>(sc); scale[1] = row_lane_bcast<1>(sc); scale[2] = row_lane_bcast<2>(sc);
+        scale[3] = row_lane_bcast<3>(sc); scale[4] = row_lane_bcast<4>(sc);
+        static_assert(RB_STEPS == 5, "the broadcasts above are written out for five steps");
+        // phase 3: scale, rotate, convert, store
+#pragma unroll
+        for (int s = 0; s < RB_STEPS; s++) {
+            const int h0 = base + 16 * s + 4 * wave;                        // wave-uniform
+            if (h0 >= items) break;
+            u32x4 out;
+            if (h0 >= nqk) {                                                // V heads only: fp16 copy
+#pragma unroll
+                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[s][2 * p], x[s][2 * p + 1]);
+                if (h0 + hq < items) *(u32x4 *)(cw + M + (size_t)(h0 - nqk) * 128 + lo) = out;
+                continue;
+            }
+            const bool allq = h0 + 3 < a.nh, allk = h0 >= a.nh && h0 + 3 < nqk;
+            const int h = h0 + hq;
+            const bool isq = h < a.nh, isv = h >= nqk;
+            const float * wp = nrm + ((allq || (!allk && isq)) ? 0 : 128) + 8 * l16;
+            const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
+            float y[8];
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                const float pk = dpp_ror8(y1[k]);
-                y[k] = __builtin_fmaf(y1[k], k < 4 ? c4[0][k] : c4[1][k - 4], pk * (k < 4 ? s4[0][k] : s4[1][k - 4]));
-                if (isv) y[k] = x[k];                                       // a V head inside a mixed step (nh + nkv not a multiple of 4)
+                const float y1 = (scale[s] * x[s][k]) * (k < 4 ? w0[k] : w1[k - 4]);
+                y[k] = __builtin_fmaf(y1, k < 4 ? c4[0][k] : c4[1][k - 4], mul_ror8(y1, k < 4 ? s4[0][k] : s4[1][k - 4]));
             }
+            if (allq) {
 #pragma unroll
-            for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
-            if (active) {
-                uint16_t * dst = isq ? a.q16 + ((size_t)t * a.nh + h) * 128 : (isv ? cw + M + (size_t)(h - nqk) * 128 : cw + (size_t)(h - a.nh) * 128);
-                *(u32x4 *)(dst + 8 * l16) = out;
+                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
+                *(u32x4 *)(qw + (size_t)h0 * 128 + lo) = out;
+            } else if (allk) {
+#pragma unroll
+                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
+                *(u32x4 *)(cw + (size_t)(h0 - a.nh) * 128 + lo) = out;
+            } else {                                                        // a step that straddles q | k | v or the end of the row
+#pragma unroll
+                for (int k = 0; k < 8; k++) if (isv) y[k] = x[s][k];
+#pragma unroll
+                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
+                if (h < items) {
+                    uint16_t * dst = isq ? qw + (size_t)h * 128 : (isv ? cw + M + (size_t)(h - nqk) * 128 : cw + (size_t)(h - a.nh) * 128);
+                    *(u32x4 *)(dst + 8 * l16) = out;
+                }
             }
         }
+#pragma unroll
+        for (int s = 0; s < RB_STEPS; s++) xin[s] = xnext[s];
     }
 }
 
@@ -287,7 +338,11 @@ static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bo
     if (a.n == 0) return CAMX_OK;
     const bool wide = bf16in && !q8 && !a.page_table && (a.ldq & 7) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
                       ((uintptr_t)a.cache & 15) == 0;
-    if (wide) { if (yarn) qk_rope_bf16_tokens<true><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false><<<dim3(a.n), dim3(256), 0, st>>>(a); }
+    if (wide && a.n >= 2048) {          // enough tokens to fill the chip four to a workgroup
+        const dim3 g4((a.n + 3) / 4);
+        if (yarn) qk_rope_bf16_tokens<true, 4><<<g4, dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false, 4><<<g4, dim3(256), 0, st>>>(a);
+    }
+    else if (wide) { if (yarn) qk_rope_bf16_tokens<true, 1><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false, 1><<<dim3(a.n), dim3(256), 0, st>>>(a); }
     else if (bf16in) rope_dispatch<true>(a, yarn, q8, st); else rope_dispatch<false>(a, yarn, q8, st);
     CAMX_LAUNCH_RET();
 }

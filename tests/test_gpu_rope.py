@@ -129,7 +129,7 @@ def test_pf_qk_nr(T, heads, D, n_rot, stride, base):
 
 
 @pytest.mark.parametrize('nh,nkv,n,pos0,yarn,pad', [(64, 8, 7, 4089, True, 0), (32, 4, 3, 0, False, 8), (5, 3, 4, 77, False, 24), (96, 8, 2, 100, True, 0),
-                                                    (1, 1, 2, 5, False, 4)])
+                                                    (1, 1, 2, 5, False, 4), (8, 2, 2051, 3, True, 0), (96, 8, 2048, 0, False, 0), (5, 3, 2049, 9, False, 8)])
 def test_qk_rope_bf16(nh, nkv, n, pos0, yarn, pad):
     """bf16 activations (a dense prefill chunk): the same statements on the exactly widened values; head counts that are not
     multiples of four, rows longer than 80 heads and a row stride that defeats the 128-bit path are all covered"""
