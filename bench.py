@@ -317,7 +317,11 @@ def main():
             if name == '_keep': continue
             med, mean = B.time_launch(fn, reps=50, warm=10, flush=True)
             med_hot, _ = B.time_launch(fn, reps=50, warm=10, flush=False)
-            ops[name] = {'us': round(med, 2), 'us_cache_hot': round(med_hot, 2), 'bytes': by, 'GBps': round(by / (med * 1e-6) / 1e9, 1),
+            q0, q1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            q0.record()
+            for _ in range(50): fn()
+            q1.record(); q1.synchronize()
+            ops[name] = {'us': round(med, 2), 'us_cache_hot': round(med_hot, 2), 'us_queued': round(q0.elapsed_time(q1) * 1e3 / 50, 2), 'bytes': by, 'GBps': round(by / (med * 1e-6) / 1e9, 1),
                          'frac_of_8TBps': round(by / (med * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
         out['opsets'] = ops
     if not a.no_cpu and not a.only:

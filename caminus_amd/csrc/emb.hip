@@ -63,6 +63,18 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     int tok = a.toks[t]; tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;
     const uint8_t * row = a.W + (size_t)tok * a.rb;
     const int N = a.N, ni = N >> 8;
+    // short rows: the addend and gamma do not depend on the token id, so they are requested before the table row is decoded
+    // (one memory round trip after the id instead of three)
+    constexpr bool PRE = TAIL && NI_MAX <= 8;
+    f32x4 gpre[PRE ? NI_MAX : 1], dpre[PRE ? NI_MAX : 1];
+    if (PRE) {
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) {
+                gpre[j] = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
+                if (a.d) dpre[j] = *(const f32x4 *)(a.d + (size_t)t * N + 256 * j + 4 * lane);
+            }
+    }
     f32x4 xv[NI_MAX];
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
@@ -78,7 +90,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) {
                 const size_t o = (size_t)t * N + 256 * j + 4 * lane;
-                xv[j] = xv[j] + *(const f32x4 *)(a.d + o);
+                xv[j] = xv[j] + (PRE ? dpre[j] : *(const f32x4 *)(a.d + o));
                 if (a.x) *(f32x4 *)(a.x + o) = xv[j];
             }
     }
@@ -94,7 +106,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) {
-            const f32x4 g = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
+            const f32x4 g = PRE ? gpre[j] : *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
             f32x4 v;
             v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
             const size_t o = (size_t)t * N + 256 * j + 4 * lane;

@@ -38,6 +38,16 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) xv[j] = *(const f32x4 *)(xr + 256 * j + 4 * lane);
+    // short rows (few of them in a decode step: latency, not bandwidth, sets the time): gamma is fetched with the row, so
+    // the scaling pass does not start a second memory round trip after the reduction
+    constexpr bool PRE_G = NI_MAX <= 8;
+    const float * gw = a.nw + (size_t)(row % a.wr) * N;
+    f32x4 gpre[PRE_G ? NI_MAX : 1];
+    if (PRE_G) {
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) gpre[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+    }
     if (ADD == ADD_F32_SLOTS && a.S > 0) {
         const float * dr = (const float *)a.d + (size_t)row * a.S * N;
         const float * wr = a.w ? a.w + (size_t)row * a.S : nullptr;
@@ -90,11 +100,10 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     const float tot = wave_groups_in_order(group32_sum(ss));
     const float scale = rsqrt_exact(tot / (float)N + a.eps);
     if (a.scl && lane == 0) a.scl[row] = scale;
-    const float * gw = a.nw + (size_t)(row % a.wr) * N;
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) {
-            const f32x4 g = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+            const f32x4 g = PRE_G ? gpre[j] : *(const f32x4 *)(gw + 256 * j + 4 * lane);
             f32x4 v;
             v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
             const size_t o = (size_t)row * N + 256 * j + 4 * lane;

@@ -29,6 +29,26 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rs[64];
     const int t = blockIdx.x, tid = threadIdx.x, lane = slot_of(tid & 63), l = lane & 31;
     const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+    const float * row = (const float *)a.qkv + (size_t)t * a.ldq;
+    const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)t * a.ldq;
+    // items: heads 0 .. nh + nkv - 1 take norm + rotary, items nh + nkv .. nh + 2 nkv - 1 are the V heads. A wave step is two
+    // heads (one per half-wave); the loads of up to QR_STEPS steps are issued before the cos / sin row is computed, so a
+    // decode token pays one memory round trip, not one per head.
+    const int items = a.nh + 2 * a.nkv;
+    constexpr int QR_STEPS = 5;
+    const int it_w = (tid >> 6) * 2 + (lane >> 5);                      // this half-wave's head inside a step of 8 heads
+    f32x4 xin[QR_STEPS];
+    auto load = [&](int base) {
+#pragma unroll
+        for (int s = 0; s < QR_STEPS; s++) {
+            const int it = base + 8 * s + it_w;
+            const int hy = it < items ? it : 0;
+            xin[s] = BF16IN ? unpack_bf16x4(*(const u32x2 *)(rowb + (size_t)hy * 128 + 4 * l)) : *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
+        }
+    };
+    load(0);
+    const f32x4 wq = *(const f32x4 *)(a.par + 4 * l), wk = *(const f32x4 *)(a.par + 128 + 4 * l);
+    const float eps = a.par[257];
     if (tid < 64) {
         float c, s;
         if (YARN) { const float theta = (float)pos * a.par[258 + tid], ms = a.par[322]; c = cosf(theta) * ms; s = sinf(theta) * ms; }
@@ -36,8 +56,6 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         rc[tid] = c; rs[tid] = s;
     }
     __syncthreads();
-    const float * row = (const float *)a.qkv + (size_t)t * a.ldq;
-    const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)t * a.ldq;
     const size_t M = (size_t)a.nkv * 128;
     const size_t rb = Q8 ? 2 * (M / 32) * 34 : 4 * M;
     uint8_t * cw = nullptr;
@@ -46,46 +64,48 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         if (pg < 0 || pg >= a.n_pages) { if (tid == 0) atomicOr(a.err, 8); }
         else cw = (uint8_t *)a.cache + ((size_t)pg * a.page + (size_t)(pos % a.page)) * rb;
     } else cw = (uint8_t *)a.cache + (size_t)pos * rb;
-    const float eps = a.par[257];
     const f32x4 c4 = *(const f32x4 *)(rc + 4 * (l & 15)), s4 = *(const f32x4 *)(rs + 4 * (l & 15));
     const bool lo = l < 16;
-    // items: heads 0 .. nh + nkv - 1 take norm + rotary, items nh + nkv .. nh + 2 nkv - 1 are the V heads
-    const int items = a.nh + 2 * a.nkv;
-    for (int it0 = (tid >> 6) * 2; it0 < items; it0 += 8) {
-        const int it = it0 + (lane >> 5);
-        const bool active = it < items;
-        const int hy = active ? it : 0;
-        const f32x4 x = BF16IN ? unpack_bf16x4(*(const u32x2 *)(rowb + (size_t)hy * 128 + 4 * l)) : *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
-        if (hy >= a.nh + a.nkv) {                       // a V head: fp16 copy, or fp16-rounded then Q8 blocks
-            const int g = hy - a.nh - a.nkv;
+    for (int base = 0; base < items; base += 8 * QR_STEPS) {
+        if (base) load(base);
+#pragma unroll
+        for (int st = 0; st < QR_STEPS; st++) {
+            if (base + 8 * st + (tid >> 6) * 2 >= items) break;        // wave-uniform: neither half-wave has a head
+            const int it = base + 8 * st + it_w;
+            const bool active = it < items;
+            const int hy = active ? it : 0;
+            const f32x4 x = xin[st];
+            if (hy >= a.nh + a.nkv) {                       // a V head: fp16 copy, or fp16-rounded then Q8 blocks
+                const int g = hy - a.nh - a.nkv;
+                if (Q8) {
+                    f32x4 v; v.x = f16r(x.x); v.y = f16r(x.y); v.z = f16r(x.z); v.w = f16r(x.w);
+                    kv_q8_emit(v, cw + (M / 32 + (size_t)g * 4 + (l >> 3)) * 34, l & 7, a.err, active && cw != nullptr);
+                } else if (active && cw) *(u32x2 *)((uint16_t *)cw + M + (size_t)g * 128 + 4 * l) = pack_f16x4(x);
+                continue;
+            }
+            const bool isq = hy < a.nh;
+            const f32x4 wn = isq ? wq : wk;
+            f32x4 sq; sq.x = x.x * x.x; sq.y = x.y * x.y; sq.z = x.z * x.z; sq.w = x.w * x.w;
+            const float tot = half_groups_in_order<4>(group32_sum(sq), lane & 32);
+            const float scale = rsqrt_exact(tot / 128 + eps);
+            f32x4 y1; y1.x = (scale * x.x) * wn.x; y1.y = (scale * x.y) * wn.y; y1.z = (scale * x.z) * wn.z; y1.w = (scale * x.w) * wn.w;
+            f32x4 p; p.x = lane_xor16(y1.x); p.y = lane_xor16(y1.y); p.z = lane_xor16(y1.z); p.w = lane_xor16(y1.w);
+            // dims below 64: fma(x0, c, -(x1 s)); dims from 64: fma(x1, c, x0 s), with x0 the low and x1 the high dim of the pair
+            f32x4 y;
+            y.x = __builtin_fmaf(y1.x, c4.x, lo ? -(p.x * s4.x) : p.x * s4.x); y.y = __builtin_fmaf(y1.y, c4.y, lo ? -(p.y * s4.y) : p.y * s4.y);
+            y.z = __builtin_fmaf(y1.z, c4.z, lo ? -(p.z * s4.z) : p.z * s4.z); y.w = __builtin_fmaf(y1.w, c4.w, lo ? -(p.w * s4.w) : p.w * s4.w);
             if (Q8) {
-                f32x4 v; v.x = f16r(x.x); v.y = f16r(x.y); v.z = f16r(x.z); v.w = f16r(x.w);
-                kv_q8_emit(v, cw + (M / 32 + (size_t)g * 4 + (l >> 3)) * 34, l & 7, a.err, active && cw != nullptr);
-            } else if (active && cw) *(u32x2 *)((uint16_t *)cw + M + (size_t)g * 128 + 4 * l) = pack_f16x4(x);
-            continue;
-        }
-        const bool isq = hy < a.nh;
-        const f32x4 wn = *(const f32x4 *)(a.par + (isq ? 0 : 128) + 4 * l);
-        f32x4 sq; sq.x = x.x * x.x; sq.y = x.y * x.y; sq.z = x.z * x.z; sq.w = x.w * x.w;
-        const float tot = half_groups_in_order<4>(group32_sum(sq), lane & 32);
-        const float scale = rsqrt_exact(tot / 128 + eps);
-        f32x4 y1; y1.x = (scale * x.x) * wn.x; y1.y = (scale * x.y) * wn.y; y1.z = (scale * x.z) * wn.z; y1.w = (scale * x.w) * wn.w;
-        f32x4 p; p.x = lane_xor16(y1.x); p.y = lane_xor16(y1.y); p.z = lane_xor16(y1.z); p.w = lane_xor16(y1.w);
-        // dims below 64: fma(x0, c, -(x1 s)); dims from 64: fma(x1, c, x0 s), with x0 the low and x1 the high dim of the pair
-        f32x4 y;
-        y.x = __builtin_fmaf(y1.x, c4.x, lo ? -(p.x * s4.x) : p.x * s4.x); y.y = __builtin_fmaf(y1.y, c4.y, lo ? -(p.y * s4.y) : p.y * s4.y);
-        y.z = __builtin_fmaf(y1.z, c4.z, lo ? -(p.z * s4.z) : p.z * s4.z); y.w = __builtin_fmaf(y1.w, c4.w, lo ? -(p.w * s4.w) : p.w * s4.w);
-        if (Q8) {
-            y.x = f16r(y.x); y.y = f16r(y.y); y.z = f16r(y.z); y.w = f16r(y.w);
-            y = hadamard128_l4(y, l, true);
-        }
-        if (isq) {
-            if (Q8) { asm volatile("" : "+v"(y.x), "+v"(y.y), "+v"(y.z), "+v"(y.w)); }   // fp32 product first, then fp16
-            if (active) *(u32x2 *)(a.q16 + ((size_t)t * a.nh + hy) * 128 + 4 * l) = pack_f16x4(y);
-        } else {
-            const int g = hy - a.nh;
-            if (Q8) kv_q8_emit(y, cw + ((size_t)g * 4 + (l >> 3)) * 34, l & 7, a.err, active && cw != nullptr);
-            else if (active && cw) *(u32x2 *)((uint16_t *)cw + (size_t)g * 128 + 4 * l) = pack_f16x4(y);
+                y.x = f16r(y.x); y.y = f16r(y.y); y.z = f16r(y.z); y.w = f16r(y.w);
+                y = hadamard128_l4(y, l, true);
+            }
+            if (isq) {
+                if (Q8) { asm volatile("" : "+v"(y.x), "+v"(y.y), "+v"(y.z), "+v"(y.w)); }   // fp32 product first, then fp16
+                if (active) *(u32x2 *)(a.q16 + ((size_t)t * a.nh + hy) * 128 + 4 * l) = pack_f16x4(y);
+            } else {
+                const int g = hy - a.nh;
+                if (Q8) kv_q8_emit(y, cw + ((size_t)g * 4 + (l >> 3)) * 34, l & 7, a.err, active && cw != nullptr);
+                else if (active && cw) *(u32x2 *)((uint16_t *)cw + (size_t)g * 128 + 4 * l) = pack_f16x4(y);
+            }
         }
     }
 }
@@ -254,65 +274,97 @@ __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
 struct NrArgs {
     const void * x; int head_stride, heads; const float * w; int D, nrot; float theta_scale, eps; int pos0; const int32_t * pos; void * out; int T;
 };
-template <bool BF16>
-__global__ void __launch_bounds__(256) qk_nr_tokens(NrArgs a) {
-    __shared__ float rc[256], rs[256];
-    __shared__ float nrm[4][512];
-    const int tok = blockIdx.x, tid = threadIdx.x, lane = slot_of(tid & 63), wave = tid >> 6, half = a.nrot / 2;
-    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
-    for (int j = tid; j < half; j += 256) {
-        const float theta = pos * rope_freq(a.theta_scale, j);
-        rc[j] = cosf(theta); rs[j] = sinf(theta);
-    }
-    __syncthreads();
-    for (int h = wave; h < a.heads; h += 4) {
-        const size_t t = (size_t)tok * a.heads + h;
-        const size_t xo = t * a.head_stride, yo = t * a.D;
-        float xv[2][4];
-        f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+// One wave per (token, head), four per workgroup, nothing shared between them: each wave issues its head's loads, computes
+// the token's cos / sin for the rotated pairs into its own LDS rows while they are in flight, normalizes, parks the normed
+// head in LDS for the partner reads of the rotation, and stores. No barrier; a verify batch of 16 tokens x 28 heads is 448
+// independent waves instead of 16 workgroups that loop over their heads.
+template <bool BF16, bool VEC>
+__global__ void __launch_bounds__(256) qk_nr_heads(NrArgs a) {
+    __shared__ float rc[4][256], rs[4][256];
+    __shared__ __attribute__((aligned(16))) float nrm[4][512];
+    const int tid = threadIdx.x, lraw = tid & 63, lane = slot_of(lraw), wave = tid >> 6, half = a.nrot / 2;
+    const long gw = (long)blockIdx.x * 4 + wave;
+    if (gw >= (long)a.T * a.heads) return;
+    const int tok = (int)(gw / a.heads);
+    const size_t xo = (size_t)gw * a.head_stride, yo = (size_t)gw * a.D;
+    float xv[2][4];
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+    for (int j = 0; j < 2; j++) {
+        const int i0 = 256 * j + 4 * lane;
+        if (VEC) {                                               // D, head_stride multiples of 4, aligned bases: i0 .. i0 + 3 are in or out together
+            f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (i0 < a.D) v = BF16 ? unpack_bf16x4(*(const u32x2 *)((const uint16_t *)a.x + xo + i0)) : *(const f32x4 *)((const float *)a.x + xo + i0);
+            xv[j][0] = v.x; xv[j][1] = v.y; xv[j][2] = v.z; xv[j][3] = v.w;
+        } else {
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const int i = 256 * j + 4 * lane + k;
+                const int i = i0 + k;
                 xv[j][k] = 0.0f;
                 if (i < a.D) xv[j][k] = BF16 ? bf2f(((const uint16_t *)a.x)[xo + i]) : ((const float *)a.x)[xo + i];
             }
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            ss.x = __builtin_fmaf(xv[j][0], xv[j][0], ss.x); ss.y = __builtin_fmaf(xv[j][1], xv[j][1], ss.y);
-            ss.z = __builtin_fmaf(xv[j][2], xv[j][2], ss.z); ss.w = __builtin_fmaf(xv[j][3], xv[j][3], ss.w);
         }
-        const float tot = wave_groups_in_order(group32_sum(ss));
-        const float scale = rsqrt_exact(tot / (float)a.D + a.eps);
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const int i = 256 * j + 4 * lane + k;
-                if (i < a.D) { xv[j][k] = (scale * xv[j][k]) * a.w[i]; nrm[wave][i] = xv[j][k]; }
-            }
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): this wave's LDS stores have landed before its reads
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const int i = 256 * j + 4 * lane + k;
-                if (i < a.D) {
-                    float y = xv[j][k];
-                    if (i < a.nrot) {
-                        const int jj = i < half ? i : i - half;
-                        const float c = rc[jj], sn = rs[jj];
-                        const float x0 = nrm[wave][jj], x1 = nrm[wave][jj + half];
-                        y = i < half ? x0 * c - x1 * sn : x0 * sn + x1 * c;
-                    }
-                    if (BF16) ((uint16_t *)a.out)[yo + i] = to_bf16(y); else ((float *)a.out)[yo + i] = y;
-                }
-            }
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_s_waitcnt(0xc07f);
     }
+    float wv[2][4];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const int i = 256 * j + 4 * lane + k; wv[j][k] = i < a.D ? a.w[i] : 0.0f; }
+    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    for (int j = lraw; j < half; j += 64) {
+        const float theta = pos * rope_freq(a.theta_scale, j);
+        rc[wave][j] = cosf(theta); rs[wave][j] = sinf(theta);
+    }
+    f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        ss.x = __builtin_fmaf(xv[j][0], xv[j][0], ss.x); ss.y = __builtin_fmaf(xv[j][1], xv[j][1], ss.y);
+        ss.z = __builtin_fmaf(xv[j][2], xv[j][2], ss.z); ss.w = __builtin_fmaf(xv[j][3], xv[j][3], ss.w);
+    }
+    const float tot = wave_groups_in_order(group32_sum(ss));
+    const float scale = rsqrt_exact(tot / (float)a.D + a.eps);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = 256 * j + 4 * lane + k;
+            if (i < a.D) { xv[j][k] = (scale * xv[j][k]) * wv[j][k]; nrm[wave][i] = xv[j][k]; }
+        }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): this wave's LDS stores have landed before its reads
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        float y[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = 256 * j + 4 * lane + k;
+            y[k] = xv[j][k];
+            if (i < a.D && i < a.nrot) {
+                const int jj = i < half ? i : i - half;
+                const float c = rc[wave][jj], sn = rs[wave][jj];
+                const float x0 = nrm[wave][jj], x1 = nrm[wave][jj + half];
+                y[k] = i < half ? x0 * c - x1 * sn : x0 * sn + x1 * c;
+            }
+        }
+        const int i0 = 256 * j + 4 * lane;
+        if (VEC) {
+            if (i0 < a.D) {
+                const f32x4 v = {y[0], y[1], y[2], y[3]};
+                if (BF16) *(u32x2 *)((uint16_t *)a.out + yo + i0) = pack_bf16x4_rne(v); else *(f32x4 *)((float *)a.out + yo + i0) = v;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                if (i0 + k < a.D) { if (BF16) ((uint16_t *)a.out)[yo + i0 + k] = to_bf16(y[k]); else ((float *)a.out)[yo + i0 + k] = y[k]; }
+        }
+    }
+}
+
+static void launch_nr(const NrArgs & a, int io, hipStream_t st) {
+    const int es = io ? 2 : 4;
+    const bool vec = (a.D & 3) == 0 && (a.head_stride & 3) == 0 && ((uintptr_t)a.x & (4 * es - 1)) == 0 && ((uintptr_t)a.out & (4 * es - 1)) == 0;
+    const dim3 grid((unsigned)(((long)a.T * a.heads + 3) / 4)), block(256);
+    if (io) { if (vec) qk_nr_heads<true, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<true, false><<<grid, block, 0, st>>>(a); }
+    else { if (vec) qk_nr_heads<false, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<false, false><<<grid, block, 0, st>>>(a); }
 }
 
 __global__ void rope_freqs_k(float theta_scale, int n, float * out) {
@@ -384,7 +436,7 @@ int camx_pf_qk_nr(const void * xin, int head_stride, int heads, const float * w,
     if (!xin || !w || !out || T < 0 || heads < 1 || D < 1 || D > 512 || head_stride < D || nrot < 0 || nrot > D || (nrot & 1) || io < 0 || io > 1) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     NrArgs a = {xin, head_stride, heads, w, D, nrot, theta_scale, eps, pos0, nullptr, out, T};
-    if (io) qk_nr_tokens<true><<<dim3(T), dim3(256), 0, st>>>(a); else qk_nr_tokens<false><<<dim3(T), dim3(256), 0, st>>>(a);
+    launch_nr(a, io, st);
     CAMX_LAUNCH_RET();
 }
 // the same with one position per row (a speculative-verify batch)
@@ -393,7 +445,7 @@ int camx_qk_nr_pos(const void * xin, int head_stride, int heads, const float * w
     if (!xin || !w || !out || !pos || T < 0 || heads < 1 || D < 1 || D > 512 || head_stride < D || nrot < 0 || nrot > D || (nrot & 1) || io < 0 || io > 1) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     NrArgs a = {xin, head_stride, heads, w, D, nrot, theta_scale, eps, 0, pos, out, T};
-    if (io) qk_nr_tokens<true><<<dim3(T), dim3(256), 0, st>>>(a); else qk_nr_tokens<false><<<dim3(T), dim3(256), 0, st>>>(a);
+    launch_nr(a, io, st);
     CAMX_LAUNCH_RET();
 }
 // the per-pair frequencies the rotary kernels use: out[j] = (float)pow((double)theta_scale, j), j < n
