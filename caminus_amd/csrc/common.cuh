@@ -90,7 +90,9 @@ CAMX_DEV uint16_t to_bf16(float f) {       // the same rounding without the NaN 
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
 }
 CAMX_DEV float rbf(float f) { return bf2f(f2bf(f)); }
-CAMX_DEV uint16_t f2h_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+// fp32 -> fp16 of a value that is already rounded to fp32: the empty asm keeps the backend from folding the producing
+// multiply / fma and the convert into one mixed-precision instruction (v_fma_mix*: one rounding where the contract has two)
+CAMX_DEV uint16_t f2h_bits(float f) { asm volatile("" : "+v"(f)); return __builtin_bit_cast(uint16_t, (_Float16)f); }
 CAMX_DEV float h2f_bits(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 // fp32 -> fp16 -> fp32 of a value that is already rounded to fp32: the opaque copy keeps the backend from folding the
 // producing fma and the convert into one mixed-precision instruction (one rounding instead of two)

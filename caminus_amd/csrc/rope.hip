@@ -131,6 +131,7 @@ CAMX_DEV float dpp_xor1(float v) { return __builtin_bit_cast(float, __builtin_am
 CAMX_DEV float dpp_xor2(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)); }
 CAMX_DEV float dpp_ror8(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false)); }
 CAMX_DEV uint32_t pack_f16x2(float lo, float hi) {
+    asm volatile("" : "+v"(lo), "+v"(hi));                       // already rounded to fp32: never fused with the producer
     const f32x2 in = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, f16x2));
 }

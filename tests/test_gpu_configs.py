@@ -1,0 +1,232 @@
+"""The five workload configurations at their full sizes, seeded as the measurement plan states (seeds 1001 .. 1005), each
+op-set through the C ABI against the CPU oracle on the same inputs, plus the size-independent properties the domain
+offers (chunk-split invariance, paged rows equal unpaged rows, a checksum over the untouched part of the paged cache).
+
+Tolerances: bit-exact for everything that does not pass a transcendental (norms, q8_1 / MMQ / Q8 KV bytes given their
+fp16 / bf16 inputs, dequantized rows); one fp16 / bf16 unit in the last place + 1e-5 x max for rotary, SwiGLU, gates, conv.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from caminus_amd import rope
+from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, dev, host, outliers, ptr
+from vectors import q4k_table, q80_table, qk_par
+
+pytestmark = pytest.mark.gpu
+
+
+def _gamma(rng, n):
+    return (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+
+
+def test_config1_decode_token():
+    """Qwen3-30B-A3B-shaped single decode token: add + RMSNorm over 2048, q8_1 of the normed row, QK-norm + NeoX rotary on
+    32 Q + 4 KV heads of 128 at a random position below 4096 (theta 1e6), SwiGLU for 8 experts x 768"""
+    rng = np.random.default_rng(1001)
+    N, nh, nkv = 2048, 32, 4
+    x = outliers(rng, (1, N)); d = outliers(rng, (1, 1, N)); nw = _gamma(rng, N)
+    ref = O.add_rms16(x, nw, 1e-6, d=d, S=1, want_q8=True)
+    xd = dev(x); h = dev(np.zeros((1, N), np.float32)); h16 = dev(np.zeros((1, N), np.uint16)); q8 = dev(np.zeros((N // 32, 36), np.uint8))
+    call('camx_q3p_add_rms16', ptr(xd), ptr(dev(d)), NULL, I(1), ptr(dev(nw)), F(1e-6), ptr(h), ptr(h16), I(N), I(1))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
+    call('camx_gg_quantize_q8_1', ptr(h), ptr(q8), L64(N), I(0), F(0), NULL)
+    assert bits_equal(host(q8), ref['q8'][0]) and bits_equal(host(q8), O.q8_1(ref['h'][0]))
+    # the fused form gives the same blocks in one launch
+    x2 = dev(x); q8b = dev(np.zeros((N // 32, 36), np.uint8))
+    call('camx_add_rms_q8_1', ptr(x2), ptr(dev(d)), NULL, I(1), ptr(dev(nw)), F(1e-6), NULL, NULL, ptr(q8b), I(N), I(1))
+    assert bits_equal(host(q8b), host(q8))
+
+    par = qk_par(rng, theta_base=1e6)
+    pos = int(rng.integers(0, 4096))
+    ldq = (nh + 2 * nkv) * 128
+    qkv = outliers(rng, (1, ldq)); M = nkv * 128
+    q16 = dev(np.zeros((1, nh, 128), np.uint16)); c16 = dev(np.zeros((4096, 2 * M), np.uint16))
+    call('camx_q3p_qk_rope', ptr(dev(qkv)), I(ldq), I(nh), I(nkv), ptr(dev(par)), I(pos), ptr(q16), ptr(c16), I(1), I(0))
+    rq, rc, _ = O.qk_rope(qkv, nh, nkv, par, 1, pos0=pos, rows=4096)
+    gc = host(c16, np.uint16)
+    assert close_16(host(q16, np.uint16), rq, 'f16') and close_16(gc[pos, :M], rc[pos, :M], 'f16') and bits_equal(gc[pos, M:], rc[pos, M:])
+    gc[pos] = 0
+    assert not gc.any()
+
+    n = 8 * 768
+    g = outliers(rng, n); u = outliers(rng, n)
+    y16 = dev(np.zeros(n, np.uint16))
+    call('camx_q3p_swiglu', ptr(dev(g)), ptr(dev(u)), ptr(y16), I(n))
+    assert close_16(host(y16, np.uint16), O.swiglu16(g, u), 'f16')
+
+
+@pytest.mark.parametrize('fmt', [0, 1])
+def test_config2_embedding_gather_full_table(fmt):
+    """151936 x 2048 table, Q4_K (175 MB) or Q8_0 (331 MB): 256 uniformly drawn ids to fp32 and bf16, then add + RMSNorm +
+    q8_1 of the gathered rows, every output bit-exact"""
+    rng = np.random.default_rng(1002)
+    V, N, n = 151936, 2048, 256
+    table = (q4k_table if fmt == 0 else q80_table)(rng, V, N)
+    toks = rng.integers(0, V, n).astype(np.int32)
+    nw = _gamma(rng, N); d = outliers(rng, (n, 1, N))
+    orc = O.emb_q4k if fmt == 0 else O.emb_q8_0
+    ref_x, ref_bf = orc(table, V, toks, N)
+    Wd, td = dev(table), dev(toks)
+    x = dev(np.zeros((n, N), np.float32)); xbf = dev(np.zeros((n, N), np.uint16))
+    call('camx_emb_gather', ptr(Wd), L64(table.shape[1]), I(V), ptr(td), ptr(x), ptr(xbf), I(N), I(n), I(fmt))
+    assert bits_equal(host(x), ref_x) and bits_equal(host(xbf, np.uint16), ref_bf)
+    # the independent numpy decoder on the same rows
+    from oracle import np_dequant
+    want = np.stack([np_dequant.dequant(table[t], 'Q4_K' if fmt == 0 else 'Q8_0', N) for t in toks[:16]])
+    assert bits_equal(host(x)[:16], want)
+    for addend in (None, d):
+        ref = O.add_rms16(ref_x, nw, 1e-6, d=addend, S=0 if addend is None else 1, want_q8=True)
+        xr = dev(np.zeros((n, N), np.float32)); q8 = dev(np.zeros((n, N // 32, 36), np.uint8)); h = dev(np.zeros((n, N), np.float32))
+        call('camx_emb_gather_add_rms', ptr(Wd), L64(table.shape[1]), I(V), ptr(td), ptr(xr), NULL, ptr(dev(addend)) if addend is not None else NULL,
+             ptr(dev(nw)), F(1e-6), ptr(h), NULL, ptr(q8), I(N), I(n), I(fmt))
+        assert bits_equal(host(xr), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(q8), ref['q8'])
+
+
+def test_config3_add_rms_full_chunk():
+    """4096 x 5120, fp32 residual + bf16 addend -> fp32 residual + bf16 normed rows, bit-exact; the same rows in two launches
+    of 1000 and 3096 tokens give the same bits (chunk geometry does not matter)"""
+    rng = np.random.default_rng(1003)
+    T, H = 4096, 5120
+    x = outliers(rng, (T, H)); d = O.f2bf(outliers(rng, (T, H))); nw = _gamma(rng, H)
+    ref = O.add_rms_bf16(x, d, nw, 1e-6)
+    xd, dd, nwd = dev(x), dev(d), dev(nw); hbf = dev(np.zeros((T, H), np.uint16))
+    call('camx_add_rms_bf16', ptr(xd), ptr(dd), ptr(nwd), F(1e-6), NULL, ptr(hbf), I(H), I(T))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(hbf, np.uint16), ref['hbf'])
+    x2 = dev(x); h2 = dev(np.zeros((T, H), np.uint16))
+    call('camx_add_rms_bf16', ptr(x2), ptr(dd), ptr(nwd), F(1e-6), NULL, ptr(h2), I(H), I(1000))
+    call('camx_add_rms_bf16', ptr(x2[1000:]), ptr(dd[1000:]), ptr(nwd), F(1e-6), NULL, ptr(h2[1000:]), I(H), I(T - 1000))
+    assert torch.equal(x2, xd) and torch.equal(h2, hbf)
+
+
+def test_config3_qk_rope_yarn_full_chunk():
+    """64 Q + 8 KV (+ 8 V) heads of 128 in bf16, YaRN factor 4 from 32768, theta 1e6, positions 0 .. 4095"""
+    rng = np.random.default_rng(1003)
+    T, nh, nkv = 4096, 64, 8
+    par = qk_par(rng, theta_base=1e6, yarn_table=rope.yarn_table(128, 1e6, 4.0, 32768))
+    ldq = (nh + 2 * nkv) * 128; M = nkv * 128
+    qkv = O.f2bf(outliers(rng, (T, ldq)))
+    q16 = dev(np.zeros((T, nh, 128), np.uint16)); c16 = dev(np.zeros((T, 2 * M), np.uint16))
+    call('camx_qk_rope_bf16', ptr(dev(qkv)), I(ldq), I(nh), I(nkv), ptr(dev(par)), I(0), ptr(q16), ptr(c16), I(T), I(1))
+    rq, rc, _ = O.qk_rope(O.bf2f(qkv), nh, nkv, par, T, pos0=0, yarn=True, rows=T)
+    gq, gc = host(q16, np.uint16), host(c16, np.uint16)
+    assert close_16(gq, rq, 'f16') and close_16(gc[:, :M], rc[:, :M], 'f16') and bits_equal(gc[:, M:], rc[:, M:])
+    # position 0 is the identity rotation times mscale: norm preserved per pair up to mscale^2
+    ms = float(par[322])
+    k0 = O.h2f(gc[0, :M]).reshape(nkv, 128).astype(np.float64)
+    xk = O.bf2f(qkv[0, nh * 128:(nh + nkv) * 128]).reshape(nkv, 128).astype(np.float64)
+    want = xk / np.sqrt((xk * xk).mean(1, keepdims=True) + 1e-6) * par[128:256] * ms
+    assert np.abs(k0 - want).max() <= 2.0 ** -10 * np.abs(want).max() + 1e-5
+
+
+def test_config3_swiglu_mmq_full_chunk():
+    """4096 x 17408 gate / up pair in bf16 -> q8_1 blocks in the MMQ layout (DS4): activation within one bf16 ulp of the
+    oracle's, blocks bit-exact given the kernel's own activation bits; without the activation output the blocks are the same"""
+    rng = np.random.default_rng(1003)
+    T, Fh = 4096, 17408
+    gu = O.f2bf(outliers(rng, (T, 2 * Fh)))
+    gud = dev(gu)
+    y = dev(np.zeros((O.k_pad(Fh) // 128, T, 144), np.uint8)); act = dev(np.zeros((T, Fh), np.uint16))
+    call('camx_swiglu_mmq_q8_1', ptr(gud), L64(2 * Fh), L64(Fh), ptr(y), ptr(act), I(T), I(1))
+    a = host(act, np.uint16)
+    assert close_16(a, O.silu_mul_bf16(gu), 'bf16')
+    assert bits_equal(host(y), O.mmq_q8_1(O.bf2f(a), Fh, T, 1))
+    y2 = dev(np.zeros((O.k_pad(Fh) // 128, T, 144), np.uint8))
+    call('camx_swiglu_mmq_q8_1', ptr(gud), L64(2 * Fh), L64(Fh), ptr(y2), NULL, I(T), I(1))
+    assert torch.equal(y2, y)
+    # q * d reconstructs the activation within half a quantization step, block by block (layout-independent invariant)
+    blocks = host(y).reshape(-1, T, 144)
+    dsc = blocks[:, :, :16].copy().view(np.float16).reshape(-1, T, 4, 2)[..., 0].astype(np.float32)       # [kb][t][group]
+    q = blocks[:, :, 16:].view(np.int8).reshape(-1, T, 4, 32).astype(np.float32)
+    recon = (q * dsc[..., None]).transpose(1, 0, 2, 3).reshape(T, -1)[:, :Fh]
+    af = O.bf2f(a)
+    step = np.repeat(dsc.transpose(1, 0, 2).reshape(T, -1), 32, axis=1)[:, :Fh]
+    assert (np.abs(recon - af) <= 0.57 * step + 1e-30).all()            # d / 2, plus 127 codes x the half rounding of the stored d
+
+
+def test_config4_hybrid_verify_batch():
+    """16-token verify batch: 24 Q heads (stride 512: q | gate) and 4 KV heads of 256 with rotary over the first 64 dims
+    (theta 1e7), sigmoid output gate, SiLU short conv of width 4 over 10240 channels, L2 norm of 32 (and 48) heads of 128;
+    bf16 activations, positions uniform below 65536"""
+    rng = np.random.default_rng(1004)
+    T, D, nrot = 16, 256, 64
+    ts = float(np.float32(np.float32(1e7) ** np.float32(-2.0 / nrot)))
+    pos = rng.integers(0, 65536, T).astype(np.int32)
+    w = _gamma(rng, D)
+    for heads, stride in ((24, 512), (4, 256)):
+        xb = O.f2bf(outliers(rng, (T * heads, stride)))
+        out = dev(np.zeros((T * heads, D), np.uint16))
+        call('camx_qk_nr_pos', ptr(dev(xb)), I(stride), I(heads), ptr(dev(w)), I(D), I(nrot), F(ts), F(1e-6), ptr(dev(pos)), ptr(out), I(T), I(1))
+        ref = np.concatenate([O.qk_nr(O.bf2f(xb)[t * heads:(t + 1) * heads], stride, heads, w, D, nrot, ts, 1e-6, int(pos[t]), 1) for t in range(T)])
+        got = host(out, np.uint16)
+        assert close_16(got, O.f2bf(ref), 'bf16')
+        assert bits_equal(got[:, nrot:], O.f2bf(ref)[:, nrot:])                 # the pass-through dims carry no transcendental
+    a = O.f2bf(outliers(rng, (T * 24, D))); qg = O.f2bf(outliers(rng, (T * 24, 2 * D)))
+    y = dev(np.zeros((T * 24, D), np.uint16))
+    call('camx_gate_mul', ptr(dev(a)), ptr(dev(qg)), ptr(y), L64(a.size), I(D), I(2 * D), I(D), I(2))
+    assert close_16(host(y, np.uint16), O.f2bf(O.gate_mul(O.bf2f(a), O.bf2f(qg), D, 2 * D, D)), 'bf16')
+    C = 10240
+    xc = O.f2bf(outliers(rng, (T, C))); wc = rng.standard_normal((C, 4)).astype(np.float32); st = rng.standard_normal((C, 3)).astype(np.float32)
+    ry, rst = O.gdn_conv(O.bf2f(xc), wc, st)
+    xcd, std = dev(xc), dev(st); yc = dev(np.zeros((T, C), np.uint16))
+    call('camx_pf_gdn_conv', ptr(xcd), ptr(dev(wc)), ptr(std), ptr(yc), I(C), I(T), I(C), I(C), I(1))
+    call('camx_pf_conv_state', ptr(xcd), ptr(std), I(C), I(T), I(C), I(1))
+    assert close_16(host(yc, np.uint16), O.f2bf(ry), 'bf16') and bits_equal(host(std), rst)
+    # the same 16 tokens as two passes of 5 and 11 (state carried between them) give the same outputs
+    st2 = dev(st); y2 = dev(np.zeros((T, C), np.uint16))
+    for lo, hi in ((0, 5), (5, 16)):
+        call('camx_pf_gdn_conv', ptr(xcd[lo:]), ptr(dev(wc)), ptr(st2), ptr(y2[lo:]), I(C), I(hi - lo), I(C), I(C), I(1))
+        call('camx_pf_conv_state', ptr(xcd[lo:]), ptr(st2), I(C), I(hi - lo), I(C), I(1))
+    assert torch.equal(y2, yc) and torch.equal(st2, std)
+    for heads in (32, 48):
+        xl = O.f2bf(outliers(rng, (T, heads * 128)))
+        yl = dev(np.zeros((T * heads, 128), np.uint16))
+        call('camx_pf_gdn_l2', ptr(dev(xl)), ptr(yl), I(heads), I(128), I(heads * 128), F(np.float32(1e-6 / 128)), I(T), I(1))
+        assert bits_equal(host(yl, np.uint16), O.f2bf(O.gdn_l2(O.bf2f(xl), T, heads, 128, 1e-6)))
+
+
+def test_config5_batched_decode_paged_q8():
+    """256 sequences at the Qwen3-30B-A3B shape: add + RMSNorm, then QK-norm -> rotary at each sequence's own position below
+    131072 -> fp16 -> Hadamard-128 -> Q8 blocks into a paged cache (page 256 tokens, random table over 65536 pages, 18 GB).
+    Row bytes equal the unpaged kernel's rows, which equal the oracle codec applied to the fp16 rows the F16 form wrote; restoring
+    the fill in the written rows leaves the whole cache uniform: nothing else was touched."""
+    rng = np.random.default_rng(1005)
+    S, N, nh, nkv, page, n_pages = 256, 2048, 32, 4, 256, 65536
+    x = outliers(rng, (S, N)); d = outliers(rng, (S, 1, N)); nw = _gamma(rng, N)
+    ref = O.add_rms16(x, nw, 1e-6, d=d, S=1)
+    xd = dev(x); h = dev(np.zeros((S, N), np.float32)); h16 = dev(np.zeros((S, N), np.uint16))
+    call('camx_q3p_add_rms16', ptr(xd), ptr(dev(d)), NULL, I(1), ptr(dev(nw)), F(1e-6), ptr(h), ptr(h16), I(N), I(S))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
+
+    par = qk_par(rng, theta_base=1e6)
+    M = nkv * 128; rb = 2 * (M // 32) * 34; ldq = (nh + 2 * nkv) * 128
+    qkv = outliers(rng, (S, ldq))
+    pos = rng.choice(131072, S, replace=False).astype(np.int32)          # distinct: the unpaged comparison run below shares one flat cache
+    table = rng.integers(0, n_pages, (S, 512)).astype(np.int32)
+    table[np.arange(S), pos // page] = rng.permutation(n_pages)[:S]                # the pages this batch writes are distinct
+    qd, pd, posd, td = dev(qkv), dev(par), dev(pos), dev(table)
+    cache = torch.full((n_pages * page * rb,), 0xa5, dtype=torch.uint8, device='cuda:0')
+    err = dev(np.zeros(1, np.int32)); q16 = dev(np.zeros((S, nh, 128), np.uint16))
+    call('camx_qk_rope_paged', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16), ptr(cache), ptr(err), ptr(td), I(512), I(page),
+         I(n_pages), I(S), I(0), I(1))
+    assert int(host(err)[0]) == 0
+    rowid = table[np.arange(S), pos // page].astype(np.int64) * page + pos % page
+    rows = host(cache.view(-1, rb)[torch.from_numpy(rowid).to('cuda:0')])
+    # everything else still holds the fill: put the fill back into the written rows and the whole 18 GB must be uniform
+    assert not (rows == 0xa5).all(axis=1).any()
+    cache.view(-1, rb)[torch.from_numpy(rowid).to('cuda:0')] = 0xa5
+    fill_word = int(np.frombuffer(bytes([0xa5] * 8), np.int64)[0])
+    assert bool((cache.view(torch.int64) == fill_word).all())
+    del cache
+    # the unpaged F16 form at the same positions: the stage boundary the Q8 bytes are defined from
+    c16 = dev(np.zeros((131072, 2 * M), np.uint16)); q16f = dev(np.zeros((S, nh, 128), np.uint16)); e2 = dev(np.zeros(1, np.int32))
+    call('camx_qk_rope_paged', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16f), ptr(c16), ptr(e2), NULL, I(0), I(0), I(0), I(S), I(0), I(0))
+    rows16 = host(c16, np.uint16)[pos]
+    rq, rc, _ = O.qk_rope(qkv, nh, nkv, par, S, pos=pos, rows=131072)
+    assert close_16(host(q16f, np.uint16), rq, 'f16') and close_16(rows16[:, :M], rc[pos][:, :M], 'f16') and bits_equal(rows16[:, M:], rc[pos][:, M:])
+    k16 = O.h2f(rows16[:, :M]).reshape(S * nkv, 128); v16 = O.h2f(rows16[:, M:]).reshape(-1, 32)
+    kb, ok1 = O.kv_q8_encode(O.hadamard128(k16).reshape(-1, 32)); vb, ok2 = O.kv_q8_encode(v16)
+    assert ok1.all() and ok2.all()
+    assert bits_equal(rows, np.concatenate([kb.reshape(S, -1), vb.reshape(S, -1)], axis=1))
+    assert bits_equal(host(q16, np.uint16), O.f2h(O.hadamard128(O.h2f(host(q16f, np.uint16)).reshape(-1, 128))).reshape(S, nh, 128))
