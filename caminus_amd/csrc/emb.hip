@@ -55,17 +55,18 @@ struct EmbArgs {
     float * h; uint16_t * h16; uint8_t * q8;
 };
 
-template <int FMT, int NI_MAX, bool TAIL>
+// EXACT: the row has exactly NI_MAX slabs (straight-line loops: the loads are issued as one batch)
+template <int FMT, int NI_MAX, bool TAIL, bool EXACT>
 __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     const int lane = slot_of(threadIdx.x & 63);
     const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (t >= a.n) return;
     int tok = a.toks[t]; tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;
     const uint8_t * row = a.W + (size_t)tok * a.rb;
-    const int N = a.N, ni = N >> 8;
+    const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
     // short rows: the addend and gamma do not depend on the token id, so they are requested before the table row is decoded
     // (one memory round trip after the id instead of three)
-    constexpr bool PRE = TAIL && NI_MAX <= 8;
+    constexpr bool PRE = TAIL;
     f32x4 gpre[PRE ? NI_MAX : 1], dpre[PRE ? NI_MAX : 1];
     if (PRE) {
 #pragma unroll
@@ -75,11 +76,15 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
                 if (a.d) dpre[j] = *(const f32x4 *)(a.d + (size_t)t * N + 256 * j + 4 * lane);
             }
     }
+    // every table load first, then the stores: a load written after a store that might alias it cannot be hoisted above it,
+    // and the row would cost one memory round trip per slab
     f32x4 xv[NI_MAX];
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
+        if (j < ni) xv[j] = FMT == FMT_Q4_K ? q4k_decode4(row + (size_t)j * 144, lane) : q80_decode4(row + (size_t)j * 272, lane);
+#pragma unroll
+    for (int j = 0; j < NI_MAX; j++)
         if (j < ni) {
-            xv[j] = FMT == FMT_Q4_K ? q4k_decode4(row + (size_t)j * 144, lane) : q80_decode4(row + (size_t)j * 272, lane);
             const size_t o = (size_t)t * N + 256 * j + 4 * lane;
             if (!TAIL || !a.d) { if (a.x) *(f32x4 *)(a.x + o) = xv[j]; }
             if (a.xbf) *(u32x2 *)(a.xbf + o) = pack_f2bf_x4(xv[j]);
@@ -122,8 +127,9 @@ static int launch_emb(const EmbArgs & a, hipStream_t st) {
     const dim3 grid((a.n + 3) / 4), block(256);
     const int ni = a.N >> 8;
     const bool tail = a.nw != nullptr;
-#define CAMX_EMB(NI) (tail ? emb_rows<FMT, NI, true><<<grid, block, 0, st>>>(a) : emb_rows<FMT, NI, false><<<grid, block, 0, st>>>(a))
-    if (ni <= 8) CAMX_EMB(8); else if (ni <= 16) CAMX_EMB(16); else if (ni <= 24) CAMX_EMB(24); else CAMX_EMB(32);
+#define CAMX_EMB(NI, EX) (tail ? emb_rows<FMT, NI, true, EX><<<grid, block, 0, st>>>(a) : emb_rows<FMT, NI, false, EX><<<grid, block, 0, st>>>(a))
+    if (ni == 8) CAMX_EMB(8, true); else if (ni == 16) CAMX_EMB(16, true); else if (ni == 20) CAMX_EMB(20, true); else if (ni == 4) CAMX_EMB(4, true);
+    else if (ni <= 8) CAMX_EMB(8, false); else if (ni <= 16) CAMX_EMB(16, false); else if (ni <= 24) CAMX_EMB(24, false); else CAMX_EMB(32, false);
 #undef CAMX_EMB
     CAMX_LAUNCH_RET();
 }

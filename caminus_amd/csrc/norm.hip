@@ -27,27 +27,25 @@ struct NormArgs {
     int N, rows;
 };
 
-template <int NI_MAX, int ADD>
+// EXACT: the row has exactly NI_MAX slabs, so every loop below is straight-line code: no scalar branch stands between the
+// loads, which the backend then issues as one batch (with a run-time slab count each `j < ni` is a branch that loads do
+// not cross, and a 4096 x 5120 launch loses 17 % to it).
+template <int NI_MAX, int ADD, bool EXACT>
 __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     const int lane = slot_of(threadIdx.x & 63);
     const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (row >= a.rows) return;
-    const int N = a.N, ni = N >> 8;
+    const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
     float * xr = a.x + (size_t)row * N;
     f32x4 xv[NI_MAX];
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) xv[j] = *(const f32x4 *)(xr + 256 * j + 4 * lane);
-    // short rows (few of them in a decode step: latency, not bandwidth, sets the time): gamma is fetched with the row, so
-    // the scaling pass does not start a second memory round trip after the reduction
-    constexpr bool PRE_G = NI_MAX <= 8;
+    // Loads never sit behind a store they might alias: the compiler cannot prove that x, d, gamma and the outputs are
+    // distinct, so a load written after a store waits for everything before it (one memory round trip per slab instead of
+    // one per row). Hence: every addend load, then the x stores; gamma is requested before the reduction and arrives
+    // while it runs.
     const float * gw = a.nw + (size_t)(row % a.wr) * N;
-    f32x4 gpre[PRE_G ? NI_MAX : 1];
-    if (PRE_G) {
-#pragma unroll
-        for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) gpre[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
-    }
     if (ADD == ADD_F32_SLOTS && a.S > 0) {
         const float * dr = (const float *)a.d + (size_t)row * a.S * N;
         const float * wr = a.w ? a.w + (size_t)row * a.S : nullptr;
@@ -56,38 +54,53 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         for (int j = 0; j < NI_MAX; j++) acc[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
         for (int s = 0; s < a.S; s++) {
             const float ws = wr ? wr[s] : 1.0f;
+            f32x4 dv[NI_MAX];
+#pragma unroll
+            for (int j = 0; j < NI_MAX; j++)
+                if (j < ni) dv[j] = *(const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane);
 #pragma unroll
             for (int j = 0; j < NI_MAX; j++)
                 if (j < ni) {
-                    const f32x4 dv = *(const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane);
                     if (wr) {
-                        acc[j].x = __builtin_fmaf(ws, dv.x, acc[j].x); acc[j].y = __builtin_fmaf(ws, dv.y, acc[j].y);
-                        acc[j].z = __builtin_fmaf(ws, dv.z, acc[j].z); acc[j].w = __builtin_fmaf(ws, dv.w, acc[j].w);
-                    } else acc[j] = acc[j] + dv;
+                        acc[j].x = __builtin_fmaf(ws, dv[j].x, acc[j].x); acc[j].y = __builtin_fmaf(ws, dv[j].y, acc[j].y);
+                        acc[j].z = __builtin_fmaf(ws, dv[j].z, acc[j].z); acc[j].w = __builtin_fmaf(ws, dv[j].w, acc[j].w);
+                    } else acc[j] = acc[j] + dv[j];
                 }
         }
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) { xv[j] = xv[j] + acc[j]; *(f32x4 *)(xr + 256 * j + 4 * lane) = xv[j]; }
+            if (j < ni) xv[j] = xv[j] + acc[j];
     }
     if (ADD == ADD_F32_DIRECT && a.d) {
         const float * dr = (const float *)a.d + (size_t)row * N;
+        f32x4 dv[NI_MAX];
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) {
-                xv[j] = xv[j] + *(const f32x4 *)(dr + 256 * j + 4 * lane);
-                *(f32x4 *)(xr + 256 * j + 4 * lane) = xv[j];
-            }
+            if (j < ni) dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + 256 * j + 4 * lane));
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) xv[j] = xv[j] + dv[j];
     }
     if (ADD == ADD_BF16 && a.d) {
         const uint16_t * dr = (const uint16_t *)a.d + (size_t)row * N;
+        u32x2 dv[NI_MAX];
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) {
-                const f32x4 dv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane)));
-                xv[j] = xv[j] + dv;
-                __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
-            }
+            if (j < ni) dv[j] = __builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane));
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) xv[j] = xv[j] + unpack_bf16x4(dv[j]);
+    }
+    f32x4 g[NI_MAX];
+#pragma unroll
+    for (int j = 0; j < NI_MAX; j++)
+        if (j < ni) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+    if ((ADD == ADD_F32_SLOTS && a.S > 0) || ((ADD == ADD_F32_DIRECT || ADD == ADD_BF16) && a.d)) {
+        // the updated residual goes back to the lines it was read from (plain loads above, nontemporal stores here: a
+        // nontemporal load followed by a store to the same line is slow on gfx950)
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
     }
     // sum of squares: logical thread 4 lane + k chains its elements in j order
     f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -103,9 +116,8 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) {
-            const f32x4 g = PRE_G ? gpre[j] : *(const f32x4 *)(gw + 256 * j + 4 * lane);
             f32x4 v;
-            v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
+            v.x = (xv[j].x * scale) * g[j].x; v.y = (xv[j].y * scale) * g[j].y; v.z = (xv[j].z * scale) * g[j].z; v.w = (xv[j].w * scale) * g[j].w;
             const size_t o = (size_t)row * N + 256 * j + 4 * lane;
             if (a.h) *(f32x4 *)(a.h + o) = v;
             if (a.h16) *(u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane) = pack_f16x4(v);
@@ -179,10 +191,17 @@ static int launch_norm(const NormArgs & a, hipStream_t st) {
                      ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.nw & 15) == 0 && ((uintptr_t)a.d & 15) == 0 && ((uintptr_t)a.h & 15) == 0 &&
                      ((uintptr_t)a.h16 & 7) == 0 && ((uintptr_t)a.hbf & 7) == 0 && ((uintptr_t)a.q8 & 3) == 0;
     if (!vec) add_rms_rows_any<ADD><<<grid, block, 0, st>>>(a);
-    else if (ni <= 8) add_rms_rows<8, ADD><<<grid, block, 0, st>>>(a);
-    else if (ni <= 16) add_rms_rows<16, ADD><<<grid, block, 0, st>>>(a);
-    else if (ni <= 24) add_rms_rows<24, ADD><<<grid, block, 0, st>>>(a);
-    else add_rms_rows<32, ADD><<<grid, block, 0, st>>>(a);
+    else switch (ni) {
+#define CAMX_NORM_EXACT(NI) case NI: add_rms_rows<NI, ADD, true><<<grid, block, 0, st>>>(a); break;
+        CAMX_NORM_EXACT(1) CAMX_NORM_EXACT(2) CAMX_NORM_EXACT(3) CAMX_NORM_EXACT(4) CAMX_NORM_EXACT(5) CAMX_NORM_EXACT(6) CAMX_NORM_EXACT(7)
+        CAMX_NORM_EXACT(8) CAMX_NORM_EXACT(10) CAMX_NORM_EXACT(12) CAMX_NORM_EXACT(14) CAMX_NORM_EXACT(16) CAMX_NORM_EXACT(20)
+        CAMX_NORM_EXACT(24) CAMX_NORM_EXACT(28) CAMX_NORM_EXACT(32)
+#undef CAMX_NORM_EXACT
+        default:
+            if (ni <= 16) add_rms_rows<16, ADD, false><<<grid, block, 0, st>>>(a);
+            else if (ni <= 24) add_rms_rows<24, ADD, false><<<grid, block, 0, st>>>(a);
+            else add_rms_rows<32, ADD, false><<<grid, block, 0, st>>>(a);
+    }
     CAMX_LAUNCH_RET();
 }
 
