@@ -8,6 +8,11 @@
 
 CAMX_DEV float silu_f(float x) { return x / (1.0f + expf(-x)); }
 CAMX_DEV float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+// for results that are rounded to 16 bits right away (tolerance: one unit of the 16-bit format): v_exp_f32 and v_rcp_f32, each
+// good to about 1e-6 relative, in place of the library exponential and the IEEE division (6 instructions instead of 30: the
+// 16-bit elementwise kernels are otherwise bound by the vector ALU, not by HBM). exp overflow gives 1 / inf = 0, as the division does.
+CAMX_DEV float sigmoid_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+CAMX_DEV float silu_fast(float x) { return x * sigmoid_fast(x); }
 
 #define GRID_1D(n4) dim3((unsigned)((((n4) + 255) / 256) < 1048576 ? (((n4) + 255) / 256) : 1048576))
 
@@ -76,6 +81,42 @@ __global__ void __launch_bounds__(256) gate_mul_k(const void * __restrict__ a, c
     }
 }
 
+// the same, VW consecutive values per thread with 128-bit accesses (VW = 4 for fp32 inputs, 8 for bf16): D, stride, off
+// multiples of VW and 16-byte aligned bases, so a vector never straddles a head
+template <int IO>
+__global__ void __launch_bounds__(256) gate_mul_vec(const void * __restrict__ a, const void * __restrict__ gt, void * __restrict__ y, long nvec, int dv,
+                                                    int stride, int off) {
+    constexpr int VW = IO == 2 ? 8 : 4;
+    const long step = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < nvec; i += step) {
+        const long h = i / dv; const int d = (int)(i - h * dv) * VW;
+        const size_t gi = (size_t)h * stride + off + d, ai = (size_t)i * VW;
+        float av[VW], gv[VW], v[VW];
+        if (IO == 2) {
+            const u32x4 aw = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)a + ai)), gw = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)gt + gi));
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                av[2 * p] = __builtin_bit_cast(float, aw[p] << 16); av[2 * p + 1] = __builtin_bit_cast(float, aw[p] & 0xffff0000u);
+                gv[2 * p] = __builtin_bit_cast(float, gw[p] << 16); gv[2 * p + 1] = __builtin_bit_cast(float, gw[p] & 0xffff0000u);
+            }
+        } else {
+            const f32x4 aw = __builtin_nontemporal_load((const f32x4 *)((const float *)a + ai)), gw = __builtin_nontemporal_load((const f32x4 *)((const float *)gt + gi));
+#pragma unroll
+            for (int k = 0; k < 4; k++) { av[k] = aw[k]; gv[k] = gw[k]; }
+        }
+#pragma unroll
+        for (int k = 0; k < VW; k++) { const float sgm = IO == 0 ? 1.0f / (1.0f + expf(-gv[k])) : sigmoid_fast(gv[k]); v[k] = av[k] * sgm; }
+        if (IO == 0) *(f32x4 *)((float *)y + ai) = (f32x4){v[0], v[1], v[2], v[3]};
+        else if (IO == 1) *(u32x2 *)((uint16_t *)y + ai) = pack_f16x4((f32x4){v[0], v[1], v[2], v[3]});
+        else {
+            u32x4 o;
+#pragma unroll
+            for (int p = 0; p < 4; p++) o[p] = (uint32_t)to_bf16(v[2 * p]) | ((uint32_t)to_bf16(v[2 * p + 1]) << 16);
+            *(u32x4 *)((uint16_t *)y + ai) = o;
+        }
+    }
+}
+
 // y[t, c] = silu(fma chain over [x(t-3), x(t-2), x(t-1), x(t)] . w[c]), negative times from st[c] = [x(-3), x(-2), x(-1)]
 template <bool BF16>
 __global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
@@ -97,6 +138,67 @@ __global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, c
     const float r = silu_f(sumf);
     if (BF16) ((uint16_t *)y)[(size_t)t * ldy + c] = to_bf16(r); else ((float *)y)[(size_t)t * ldy + c] = r;
 }
+// the same with VW consecutive channels per thread (VW = 8 for bf16, 4 for fp32) and a sliding window over CONV_TT tokens:
+// every input is read once (plus a three-token halo per chunk) with 128-bit loads that are all issued before the first
+// output is computed; the loaded vectors stay packed (4 registers per token) and are widened as the window reaches them
+#define CONV_TT 16
+template <bool BF16>
+__global__ void __launch_bounds__(256) gdn_conv_vec(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
+                                                    void * __restrict__ y, int C, int T, int ldx, int ldy) {
+    constexpr int VW = BF16 ? 8 : 4;
+    const int cv = blockIdx.x * 256 + threadIdx.x;
+    if (cv * VW >= C) return;
+    const int c0 = cv * VW, t0 = blockIdx.y * CONV_TT;
+    const int nt = T - t0 < CONV_TT ? T - t0 : CONV_TT;
+    u32x4 raw[CONV_TT + 3];                                  // tokens t0 - 3 .. t0 + nt - 1 (those at or after time 0)
+#pragma unroll
+    for (int j = 0; j < CONV_TT + 3; j++) {
+        const int tj = t0 - 3 + j;
+        raw[j] = (u32x4){0u, 0u, 0u, 0u};
+        if (j < nt + 3 && tj >= 0)
+            raw[j] = BF16 ? *(const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0) : *(const u32x4 *)((const float *)x + (size_t)tj * ldx + c0);
+    }
+    f32x4 w4[VW];
+#pragma unroll
+    for (int k = 0; k < VW; k++) w4[k] = *(const f32x4 *)(w + (size_t)(c0 + k) * 4);
+    auto widen = [&](float (&o)[VW], int j) {                 // the inputs of window slot j: from the state before time 0
+        const int tj = t0 - 3 + j;
+        if (tj < 0) {
+#pragma unroll
+            for (int k = 0; k < VW; k++) o[k] = st[(size_t)(c0 + k) * 3 + 3 + tj];
+        } else if (BF16) {
+#pragma unroll
+            for (int p = 0; p < 4; p++) { o[2 * p] = __builtin_bit_cast(float, raw[j][p] << 16); o[2 * p + 1] = __builtin_bit_cast(float, raw[j][p] & 0xffff0000u); }
+        } else {
+            const f32x4 v = __builtin_bit_cast(f32x4, raw[j]);
+            o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+        }
+    };
+    float win[4][VW];
+    widen(win[0], 0); widen(win[1], 1); widen(win[2], 2);
+#pragma unroll
+    for (int j = 0; j < CONV_TT; j++) {
+        if (j < nt) {
+            widen(win[(j + 3) & 3], j + 3);
+            float r[VW];
+#pragma unroll
+            for (int k = 0; k < VW; k++) {
+                float sumf = 0.0f;
+                sumf = __builtin_fmaf(win[j & 3][k], w4[k].x, sumf); sumf = __builtin_fmaf(win[(j + 1) & 3][k], w4[k].y, sumf);
+                sumf = __builtin_fmaf(win[(j + 2) & 3][k], w4[k].z, sumf); sumf = __builtin_fmaf(win[(j + 3) & 3][k], w4[k].w, sumf);
+                r[k] = BF16 ? silu_fast(sumf) : silu_f(sumf);
+            }
+            const size_t o = (size_t)(t0 + j) * ldy + c0;
+            if (BF16) {
+                u32x4 ov;
+#pragma unroll
+                for (int p = 0; p < 4; p++) ov[p] = (uint32_t)to_bf16(r[2 * p]) | ((uint32_t)to_bf16(r[2 * p + 1]) << 16);
+                *(u32x4 *)((uint16_t *)y + o) = ov;
+            } else *(f32x4 *)((float *)y + o) = (f32x4){r[0], r[1], r[2], r[3]};
+        }
+    }
+}
+
 template <bool BF16>
 __global__ void __launch_bounds__(256) conv_state_k(const void * __restrict__ x, float * __restrict__ st, int C, int T, int ldx) {
     const int c = blockIdx.x * 256 + threadIdx.x;
@@ -113,7 +215,7 @@ __global__ void __launch_bounds__(256) conv_state_k(const void * __restrict__ x,
 }
 
 // per head of K <= 512 values: y = (scale * x) * (1 / sqrt(K)), scale = 1 / sqrt(sum x^2 / K + rs); one wave per head
-template <bool BF16>
+template <bool BF16, bool VEC>
 __global__ void __launch_bounds__(256) gdn_l2_k(const void * __restrict__ x, void * __restrict__ y, int heads, int K, int ldx, float rs, int total) {
     const int lane = slot_of(threadIdx.x & 63);
     const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -123,13 +225,21 @@ __global__ void __launch_bounds__(256) gdn_l2_k(const void * __restrict__ x, voi
     float xv[2][4];
     f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < 2; j++) {
+        const int i0 = 256 * j + 4 * lane;
+        if (VEC) {                                          // K, ldx multiples of 4 and aligned bases: four values in or out together
+            f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (i0 < K) v = BF16 ? unpack_bf16x4(*(const u32x2 *)((const uint16_t *)x + xo + i0)) : *(const f32x4 *)((const float *)x + xo + i0);
+            xv[j][0] = v.x; xv[j][1] = v.y; xv[j][2] = v.z; xv[j][3] = v.w;
+        } else {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int i = 256 * j + 4 * lane + k;
-            xv[j][k] = 0.0f;
-            if (i < K) xv[j][k] = BF16 ? bf2f(((const uint16_t *)x)[xo + i]) : ((const float *)x)[xo + i];
+            for (int k = 0; k < 4; k++) {
+                const int i = i0 + k;
+                xv[j][k] = 0.0f;
+                if (i < K) xv[j][k] = BF16 ? bf2f(((const uint16_t *)x)[xo + i]) : ((const float *)x)[xo + i];
+            }
         }
+    }
 #pragma unroll
     for (int j = 0; j < 2; j++) {   // (an absent element adds fma(0, 0, s) = s: the tree's threads past K hold 0)
         ss.x = __builtin_fmaf(xv[j][0], xv[j][0], ss.x); ss.y = __builtin_fmaf(xv[j][1], xv[j][1], ss.y);
@@ -138,15 +248,39 @@ __global__ void __launch_bounds__(256) gdn_l2_k(const void * __restrict__ x, voi
     const float tot = wave_groups_in_order(group32_sum(ss));
     const float scale = rsqrt_exact(tot / (float)K + rs), s2 = 1.0f / sqrtf((float)K);
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < 2; j++) {
+        const int i0 = 256 * j + 4 * lane;
+        f32x4 v;
+        v.x = (scale * xv[j][0]) * s2; v.y = (scale * xv[j][1]) * s2; v.z = (scale * xv[j][2]) * s2; v.w = (scale * xv[j][3]) * s2;
+        if (VEC) {
+            if (i0 < K) { if (BF16) *(u32x2 *)((uint16_t *)y + yo + i0) = pack_bf16x4_rne(v); else *(f32x4 *)((float *)y + yo + i0) = v; }
+        } else {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int i = 256 * j + 4 * lane + k;
-            if (i < K) {
-                const float v = (scale * xv[j][k]) * s2;
-                if (BF16) ((uint16_t *)y)[yo + i] = to_bf16(v); else ((float *)y)[yo + i] = v;
-            }
+            for (int k = 0; k < 4; k++)
+                if (i0 + k < K) { if (BF16) ((uint16_t *)y)[yo + i0 + k] = to_bf16(v[k]); else ((float *)y)[yo + i0 + k] = v[k]; }
         }
+    }
+}
+
+// K = 128 (the GDN key heads): a half-wave per head, two heads per wave, 128-bit accesses. The logical threads past 128
+// hold zeros in the reference's tree, so the four group sums of the head added in order are the whole sum.
+template <bool BF16>
+__global__ void __launch_bounds__(256) gdn_l2_128(const void * __restrict__ x, void * __restrict__ y, int heads, int ldx, float rs, int total) {
+    const int lane = slot_of(threadIdx.x & 63), l = lane & 31;
+    const int t = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+    const bool active = t < total;
+    const int tc = active ? t : 0;
+    const int tt = tc / heads, hh = tc - tt * heads;
+    const size_t xo = (size_t)tt * ldx + (size_t)hh * 128 + 4 * l, yo = (size_t)tc * 128 + 4 * l;
+    const f32x4 v = BF16 ? unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)((const uint16_t *)x + xo)))
+                         : __builtin_nontemporal_load((const f32x4 *)((const float *)x + xo));
+    f32x4 ss;
+    ss.x = __builtin_fmaf(v.x, v.x, 0.0f); ss.y = __builtin_fmaf(v.y, v.y, 0.0f); ss.z = __builtin_fmaf(v.z, v.z, 0.0f); ss.w = __builtin_fmaf(v.w, v.w, 0.0f);
+    const float tot = half_groups_in_order<4>(group32_sum(ss), lane & 32);
+    const float scale = rsqrt_exact(tot / 128.0f + rs), s2 = 1.0f / sqrtf(128.0f);
+    f32x4 o;
+    o.x = (scale * v.x) * s2; o.y = (scale * v.y) * s2; o.z = (scale * v.z) * s2; o.w = (scale * v.w) * s2;
+    if (active) { if (BF16) *(u32x2 *)((uint16_t *)y + yo) = pack_bf16x4_rne(o); else *(f32x4 *)((float *)y + yo) = o; }
 }
 
 // ---- S1 core / fuse ----------------------------------------------------------------------------------------------------------
@@ -216,6 +350,16 @@ int camx_silu_mul_bf16(const uint16_t * gu, uint16_t * act, int H, long n, hipSt
 int camx_gate_mul(const void * a, const void * gt, void * y, long N, int D, int stride, int off, int io, hipStream_t st) {
     if (!a || !gt || !y || N < 0 || D < 1 || N % D || off < 0 || off + D > stride || io < 0 || io > 2) return CAMX_EINVAL;
     if (N == 0) return CAMX_OK;
+    const int vw = io == 2 ? 8 : 4, es = io == 2 ? 2 : 4;
+    if (D % vw == 0 && stride % vw == 0 && off % vw == 0 && !(((uintptr_t)a | (uintptr_t)gt) & 15) && !((uintptr_t)y & (io == 1 ? 7 : 15))) {
+        (void)es;
+        const long nvec = N / vw;
+        const dim3 gv = GRID_1D(nvec), bv(256);
+        if (io == 0) gate_mul_vec<0><<<gv, bv, 0, st>>>(a, gt, y, nvec, D / vw, stride, off);
+        else if (io == 1) gate_mul_vec<1><<<gv, bv, 0, st>>>(a, gt, y, nvec, D / vw, stride, off);
+        else gate_mul_vec<2><<<gv, bv, 0, st>>>(a, gt, y, nvec, D / vw, stride, off);
+        CAMX_LAUNCH_RET();
+    }
     const dim3 grid = GRID_1D(N), block(256);
     if (io == 0) gate_mul_k<0><<<grid, block, 0, st>>>(a, gt, y, N, D, stride, off);
     else if (io == 1) gate_mul_k<1><<<grid, block, 0, st>>>(a, gt, y, N, D, stride, off);
@@ -224,6 +368,13 @@ int camx_gate_mul(const void * a, const void * gt, void * y, long N, int D, int 
 }
 int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void * y, int C, int T, int ldx, int ldy, int bf16, hipStream_t st) {
     if (!x || !w || !state || !y || C < 1 || T < 1 || ldx < C || ldy < C || ((uintptr_t)w & 15)) return CAMX_EINVAL;
+    const int vw = bf16 ? 8 : 4;
+    if (C % vw == 0 && ldx % vw == 0 && ldy % vw == 0 && !(((uintptr_t)x | (uintptr_t)y) & 15)) {
+        const dim3 gv((unsigned)((C / vw + 255) / 256), (unsigned)((T + CONV_TT - 1) / CONV_TT)), bv(256);
+        if (bf16) gdn_conv_vec<true><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
+        else gdn_conv_vec<false><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
+        CAMX_LAUNCH_RET();
+    }
     const dim3 grid((unsigned)(((long)T * C + 255) / 256)), block(256);
     if (bf16) gdn_conv_k<true><<<grid, block, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
     else gdn_conv_k<false><<<grid, block, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
@@ -241,8 +392,14 @@ int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs
     if (T == 0) return CAMX_OK;
     const int total = T * heads;
     const dim3 grid((total + 3) / 4), block(256);
-    if (bf16) gdn_l2_k<true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total);
-    else gdn_l2_k<false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total);
+    const bool vec = K % 4 == 0 && ldx % 4 == 0 && !((uintptr_t)x & (bf16 ? 7 : 15)) && !((uintptr_t)y & (bf16 ? 7 : 15));
+    if (vec && K == 128) {
+        const dim3 g2((total + 7) / 8);
+        if (bf16) gdn_l2_128<true><<<g2, block, 0, st>>>(x, y, heads, ldx, rs, total); else gdn_l2_128<false><<<g2, block, 0, st>>>(x, y, heads, ldx, rs, total);
+        CAMX_LAUNCH_RET();
+    }
+    if (bf16) { if (vec) gdn_l2_k<true, true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); else gdn_l2_k<true, false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); }
+    else { if (vec) gdn_l2_k<false, true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); else gdn_l2_k<false, false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); }
     CAMX_LAUNCH_RET();
 }
 int camx_embedding_f32(const int * tok, const float * emb, float * out, int D, int T, hipStream_t st) {
