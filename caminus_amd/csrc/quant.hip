@@ -9,38 +9,80 @@
 CAMX_DEV float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
 // ---- q8_1, flat -------------------------------------------------------------------------------------------------------------
-// mode 0 plain, 1 silu(x * rs), 2 silu(x) * g[i]; values past n quantize as 0; blocks = ceil(n / 32)
+// mode 0 plain, 1 silu(x * rs), 2 silu(x) * g[i]; values past n quantize as 0; blocks = ceil(n / 32).
+// A wave takes 1024 consecutive values per step: four 128-bit loads per lane issued together, then the 32 blocks (1152
+// contiguous bytes) are assembled in the wave's own LDS and leave as 72 aligned 16-byte pieces, instead of 4-byte stores
+// that cover each 64-byte line in several partial writes. The last, partial step (and an unaligned y) stores directly.
+CAMX_DEV f32x4 q8_1_pre(f32x4 v, f32x4 gv, int mode, float rs, long i0, long n) {
+    if (mode == 1) {
+        if (i0 + 0 < n) { const float t = v.x * rs; v.x = silu_f(t); }
+        if (i0 + 1 < n) { const float t = v.y * rs; v.y = silu_f(t); }
+        if (i0 + 2 < n) { const float t = v.z * rs; v.z = silu_f(t); }
+        if (i0 + 3 < n) { const float t = v.w * rs; v.w = silu_f(t); }
+    } else if (mode == 2) {
+        if (i0 + 0 < n) v.x = silu_f(v.x) * gv.x;
+        if (i0 + 1 < n) v.y = silu_f(v.y) * gv.y;
+        if (i0 + 2 < n) v.z = silu_f(v.z) * gv.z;
+        if (i0 + 3 < n) v.w = silu_f(v.w) * gv.w;
+    }
+    return v;
+}
 __global__ void __launch_bounds__(256) q8_1_flat(const float * __restrict__ x, uint8_t * __restrict__ y, long n, int mode, float rs,
-                                                 const float * __restrict__ g, int vec) {
-    const int lane = slot_of(threadIdx.x & 63);
-    const long wave = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+                                                 const float * __restrict__ g, int vec, int vecst) {
+    __shared__ __attribute__((aligned(16))) uint32_t stage[4][288];
+    const int lane = slot_of(threadIdx.x & 63), lraw = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const long wave = (long)blockIdx.x * 4 + wv;
     const long nwaves = (long)gridDim.x * 4;
-    const long nslab = (n + 255) >> 8, nb = (n + 31) >> 5;
-    for (long s = wave; s < nslab; s += nwaves) {
-        const long i0 = s * 256 + 4 * lane;
-        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f}, gv = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (vec && i0 + 3 < n) {
-            v = *(const f32x4 *)(x + i0);
-            if (mode == 2) gv = *(const f32x4 *)(g + i0);
-        } else {
-            float t[4] = {0.0f, 0.0f, 0.0f, 0.0f}, tg[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const long nstep = (n + 1023) >> 10, nb = (n + 31) >> 5;
+    f32x4 v[4], gv[4];
+    auto load = [&](f32x4 (&v)[4], f32x4 (&gv)[4], long s) {
+        const long base = s * 1024;
+        if (vec && base + 1024 <= n) {
 #pragma unroll
-            for (int k = 0; k < 4; k++) if (i0 + k < n) { t[k] = x[i0 + k]; if (mode == 2) tg[k] = g[i0 + k]; }
-            v = (f32x4){t[0], t[1], t[2], t[3]}; gv = (f32x4){tg[0], tg[1], tg[2], tg[3]};
+            for (int j = 0; j < 4; j++) v[j] = __builtin_nontemporal_load((const f32x4 *)(x + base + 256 * j + 4 * lane));
+            if (mode == 2) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) gv[j] = __builtin_nontemporal_load((const f32x4 *)(g + base + 256 * j + 4 * lane));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const long i0 = base + 256 * j + 4 * lane;
+                float t[4] = {0.0f, 0.0f, 0.0f, 0.0f}, tg[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int k = 0; k < 4; k++) if (i0 + k < n) { t[k] = x[i0 + k]; if (mode == 2) tg[k] = g[i0 + k]; }
+                v[j] = (f32x4){t[0], t[1], t[2], t[3]}; gv[j] = (f32x4){tg[0], tg[1], tg[2], tg[3]};
+            }
         }
-        if (mode == 1) {
-            if (i0 + 0 < n) { const float t = v.x * rs; v.x = silu_f(t); }
-            if (i0 + 1 < n) { const float t = v.y * rs; v.y = silu_f(t); }
-            if (i0 + 2 < n) { const float t = v.z * rs; v.z = silu_f(t); }
-            if (i0 + 3 < n) { const float t = v.w * rs; v.w = silu_f(t); }
-        } else if (mode == 2) {
-            if (i0 + 0 < n) v.x = silu_f(v.x) * gv.x;
-            if (i0 + 1 < n) v.y = silu_f(v.y) * gv.y;
-            if (i0 + 2 < n) v.z = silu_f(v.z) * gv.z;
-            if (i0 + 3 < n) v.w = silu_f(v.w) * gv.w;
+    };
+    for (long s = wave; s < nstep; s += nwaves) {
+        const long base = s * 1024;
+        load(v, gv, s);
+        const bool whole = vecst && s * 32 + 32 <= nb;             // all 32 blocks of the step exist
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const f32x4 q = q8_1_pre(v[j], gv[j], mode, rs, base + 256 * j + 4 * lane, n);
+            const long b = s * 32 + 8 * j + (lane >> 3);
+            if (whole) {
+                const float amax = group8_max(absmax4(q));
+                const float sum = group32_sum(q);
+                const float d = amax / 127.0f;
+                uint32_t codes = 0;
+                if (amax != 0.0f) { f32x4 t; t.x = q.x / d; t.y = q.y / d; t.z = q.z / d; t.w = q.w / d; codes = pack_round_i8x4(t); }
+                uint32_t * blk = stage[wv] + (8 * j + (lane >> 3)) * 9;
+                blk[1 + (lane & 7)] = codes;
+                if ((lane & 7) == 0) blk[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
+            } else if (b < nb) q8_1_emit(q, y + b * 36, lane & 7);     // (a group of 8 lanes is wholly inside or outside)
         }
-        const long b = s * 8 + (lane >> 3);
-        if (b < nb) q8_1_emit(v, y + b * 36, lane & 7);     // (a group of 8 lanes is wholly inside or outside)
+        if (whole) {
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_s_waitcnt(0xc07f);                        // lgkmcnt(0): the wave's LDS stores have landed
+            u32x4 * dst = (u32x4 *)(y + s * 1152);
+            dst[lraw] = *(const u32x4 *)(stage[wv] + 4 * lraw);
+            if (lraw < 8) dst[64 + lraw] = *(const u32x4 *)(stage[wv] + 4 * (64 + lraw));
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_s_waitcnt(0xc07f);                        // read out before the next step overwrites it
+        }
     }
 }
 
@@ -310,10 +352,11 @@ extern "C" {
 int camx_gg_quantize_q8_1(const float * x, void * y, long n, int mode, float rs, const float * g, hipStream_t st) {
     if (n < 0 || !x || !y || mode < 0 || mode > 2 || (mode == 2 && !g) || ((uintptr_t)y & 3)) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
-    const long nslab = (n + 255) >> 8;
+    const long nstep = (n + 1023) >> 10;
     const int vec = ((uintptr_t)x & 15) == 0 && (mode != 2 || ((uintptr_t)g & 15) == 0);
-    const long blocks = (nslab + 3) / 4;
-    q8_1_flat<<<dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st>>>(x, (uint8_t *)y, n, mode, rs, g, vec);
+    const int vecst = ((uintptr_t)y & 15) == 0;
+    const long blocks = (nstep + 3) / 4;
+    q8_1_flat<<<dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st>>>(x, (uint8_t *)y, n, mode, rs, g, vec, vecst);
     CAMX_LAUNCH_RET();
 }
 
