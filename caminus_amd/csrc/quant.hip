@@ -214,42 +214,63 @@ struct SwmItem { u32x4 gw[2], uw[2]; };
 // issue the four 128-bit loads of work item (token t, slab). Every lane always issues all four (a lane past the row's
 // end, or a whole wave without work, reads 16 zero bytes instead): with a fixed number of loads in flight the compiler
 // can wait for exactly the older item's data and leave this item's loads outstanding across the other item's arithmetic.
-CAMX_DEV void swm_load(SwmItem & it, const uint16_t * __restrict__ gu, long ld, long F, int t, int slab, int lane, bool valid) {
+template <int SRC>
+CAMX_DEV void swm_load(SwmItem & it, const void * __restrict__ src, const int32_t * __restrict__ ids, long ld, long F, int t, int slab, int lane, bool valid) {
     const long e0 = (long)slab * SWM_SLAB + 8 * lane;           // load i covers elements e0 + 512 i .. + 7
-    const uint16_t * r = gu + (size_t)(valid ? t : 0) * ld + e0;
+    if (SRC == SRC_SWIGLU_BF16) {
+        const uint16_t * r = (const uint16_t *)src + (size_t)(valid ? t : 0) * ld + e0;
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const bool ok = valid && e0 + 512 * i < F;
-        const u32x4 * pg = ok ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
-        const u32x4 * pu = ok ? (const u32x4 *)(r + F + 512 * i) : (const u32x4 *)g_zero16;
-        it.gw[i] = __builtin_nontemporal_load(pg); it.uw[i] = __builtin_nontemporal_load(pu);     // read once, never written: +15 % over plain loads
+        for (int i = 0; i < 2; i++) {
+            const bool ok = valid && e0 + 512 * i < F;
+            const u32x4 * pg = ok ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
+            const u32x4 * pu = ok ? (const u32x4 *)(r + F + 512 * i) : (const u32x4 *)g_zero16;
+            it.gw[i] = __builtin_nontemporal_load(pg); it.uw[i] = __builtin_nontemporal_load(pu);     // read once, never written: +15 % over plain loads
+        }
+    } else {                                                    // fp32 rows: gw[i] = values 0 .. 3, uw[i] = values 4 .. 7 of the lane's eight
+        const long row = valid ? (ids ? ids[t] : t) : 0;
+        const float * r = (const float *)src + (size_t)row * ld + e0;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const u32x4 * p0 = valid && e0 + 512 * i < F ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
+            const u32x4 * p1 = valid && e0 + 512 * i + 4 < F ? (const u32x4 *)(r + 512 * i + 4) : (const u32x4 *)g_zero16;
+            it.gw[i] = __builtin_nontemporal_load(p0); it.uw[i] = __builtin_nontemporal_load(p1);
+        }
     }
 }
 
 // the item's arithmetic; the wave's 8 blocks go to stage[kb][token slot][144]
-template <int LAYOUT>
+template <int LAYOUT, int SRC>
 CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int t, int slab,
                           int lane, int wave) {
     const int lq = lane & 3;
     const long e0 = (long)slab * SWM_SLAB + 8 * lane;
-    uint32_t pk[2][4];
+    float val[2][8];                                                   // the lane's eight values of each half, as quantized
     float amax[2], sum[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         float m = 0.0f, s0 = 0.0f, s1 = 0.0f;
+        uint32_t pk[4];
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            const uint32_t sl = lut[it.gw[i][p] & 0xffffu], sh = lut[it.gw[i][p] >> 16];
-            const float u0 = __builtin_bit_cast(float, it.uw[i][p] << 16), u1 = __builtin_bit_cast(float, it.uw[i][p] & 0xffff0000u);
-            const float a0 = __builtin_bit_cast(float, sl << 16) * u0, a1 = __builtin_bit_cast(float, sh << 16) * u1;
-            pk[i][p] = cvt_pk_bf16(a0, a1);
-            const float v0 = __builtin_bit_cast(float, pk[i][p] << 16), v1 = __builtin_bit_cast(float, pk[i][p] & 0xffff0000u);
+            float v0, v1;
+            if (SRC == SRC_SWIGLU_BF16) {
+                const uint32_t sl = lut[it.gw[i][p] & 0xffffu], sh = lut[it.gw[i][p] >> 16];
+                const float u0 = __builtin_bit_cast(float, it.uw[i][p] << 16), u1 = __builtin_bit_cast(float, it.uw[i][p] & 0xffff0000u);
+                const float a0 = __builtin_bit_cast(float, sl << 16) * u0, a1 = __builtin_bit_cast(float, sh << 16) * u1;
+                pk[p] = cvt_pk_bf16(a0, a1);
+                v0 = __builtin_bit_cast(float, pk[p] << 16); v1 = __builtin_bit_cast(float, pk[p] & 0xffff0000u);
+            } else {
+                const u32x4 w = p < 2 ? it.gw[i] : it.uw[i];
+                const uint32_t b0 = w[2 * (p & 1)], b1 = w[2 * (p & 1) + 1];     // (a bit cast applied straight to a vector element reads element 0)
+                v0 = __builtin_bit_cast(float, b0); v1 = __builtin_bit_cast(float, b1);
+            }
+            val[i][2 * p] = v0; val[i][2 * p + 1] = v1;
             m = max3_abs(v0, v1, m);
             if (LAYOUT == MMQ_DS4) {      // per thread ((x0 + x1) + x2) + x3: pairs p = 0, 1 are thread h = 0, pairs 2, 3 thread h = 1
                 if (p == 0) s0 = v0 + v1; else if (p == 1) s0 = (s0 + v0) + v1; else if (p == 2) s1 = v0 + v1; else s1 = (s1 + v0) + v1;
             }
         }
-        if (act && e0 + 512 * i < F) *(u32x4 *)(act + (size_t)t * F + e0 + 512 * i) = (u32x4){pk[i][0], pk[i][1], pk[i][2], pk[i][3]};
+        if (SRC == SRC_SWIGLU_BF16 && act && e0 + 512 * i < F) *(u32x4 *)(act + (size_t)t * F + e0 + 512 * i) = (u32x4){pk[0], pk[1], pk[2], pk[3]};
         m = fmaxf(m, lane_xor2(m)); amax[i] = fmaxf(m, lane_xor1(m));
         sum[i] = 0.0f;
         if (LAYOUT == MMQ_DS4) {
@@ -269,10 +290,7 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
     for (int i = 0; i < 2; i++) {
         int q[8];
 #pragma unroll
-        for (int p = 0; p < 4; p++) {
-            q[2 * p] = round_i32(__builtin_bit_cast(float, pk[i][p] << 16) * di[i]);
-            q[2 * p + 1] = round_i32(__builtin_bit_cast(float, pk[i][p] & 0xffff0000u) * di[i]);
-        }
+        for (int p = 0; p < 8; p++) q[p] = round_i32(val[i][p] * di[i]);
         *(u32x2 *)(blk0 + i * (4 * SWM_TOK * 144) + 16 + 8 * (lane & 15)) = (u32x2){pack_i8x4(q[0], q[1], q[2], q[3]), pack_i8x4(q[4], q[5], q[6], q[7])};
     }
     if (lq < 2)
@@ -280,11 +298,12 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
             LAYOUT == MMQ_DS4 ? ((uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sm) << 16)) : __builtin_bit_cast(uint32_t, d);
 }
 
-template <int LAYOUT>
-__global__ void __launch_bounds__(1024) swiglu_mmq_lut(const uint16_t * __restrict__ gu, long ld, long F, long Kp, uint8_t * __restrict__ y,
-                                                       uint16_t * __restrict__ act, int T, int ngroups, int nslab) {
+// SRC_F32 (quantize_mmq_q8_1 without scatter): the same work split and copy-out on fp32 rows (column c = row ids[c] or c), no table
+template <int LAYOUT, int SRC>
+__global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__ gu, const int32_t * __restrict__ ids, long ld, long F, long Kp,
+                                                       uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T, int ngroups, int nslab) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
-    uint8_t * stage = (uint8_t *)lut + 131072;
+    uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 131072 : 0);
     const int xcd = blockIdx.x & 7, wgx = blockIdx.x >> 3, nwgx = gridDim.x >> 3;
     const int per = (ngroups + 7) >> 3, lim = per * nslab;       // token groups per XCD, work items per XCD
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -294,10 +313,12 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const uint16_t * __restri
 #define SWM_OK(j) ((j) < lim && SWM_G(j) < ngroups && SWM_T(j) < T)
     SwmItem A, B, C;                                                          // three items in rotation: two steps of loads in flight
     int j = wgx;
-    swm_load(A, gu, ld, F, SWM_T(j), j % nslab, lane, SWM_OK(j));             // in flight while the table is copied
-    swm_load(B, gu, ld, F, SWM_T(j + nwgx), (j + nwgx) % nslab, lane, SWM_OK(j + nwgx));
-    for (int i = threadIdx.x; i < 8192; i += 1024) ((u32x4 *)lut)[i] = ((const u32x4 *)g_silu_lut)[i];
-    __syncthreads();
+    swm_load<SRC>(A, gu, ids, ld, F, SWM_T(j), j % nslab, lane, SWM_OK(j));             // in flight while the table is copied
+    swm_load<SRC>(B, gu, ids, ld, F, SWM_T(j + nwgx), (j + nwgx) % nslab, lane, SWM_OK(j + nwgx));
+    if (SRC == SRC_SWIGLU_BF16) {
+        for (int i = threadIdx.x; i < 8192; i += 1024) ((u32x4 *)lut)[i] = ((const u32x4 *)g_silu_lut)[i];
+        __syncthreads();
+    }
     // copy-out of a finished step: block row kb of the step = 2304 contiguous bytes = 144 lanes x 16 B
     auto flush = [&](int jj) {
         const int grp = SWM_G(jj), slab = jj % nslab;
@@ -312,8 +333,8 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const uint16_t * __restri
 #define SWM_STEP(CUR, NXT2, jc)                                                                                              \
     {                                                                                                                        \
         const int jn = (jc) + 2 * nwgx;                                                                                      \
-        swm_load(NXT2, gu, ld, F, SWM_T(jn), jn % nslab, lane, SWM_OK(jn));                                                  \
-        if (SWM_OK(jc)) swm_compute<LAYOUT>(CUR, lut, stage, F, act, SWM_T(jc), (jc) % nslab, lane, wave);                   \
+        swm_load<SRC>(NXT2, gu, ids, ld, F, SWM_T(jn), jn % nslab, lane, SWM_OK(jn));                                        \
+        if (SWM_OK(jc)) swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, SWM_T(jc), (jc) % nslab, lane, wave);              \
         __syncthreads();                                                                                                     \
         if ((jc) < lim && SWM_G(jc) < ngroups) flush(jc);                                                                    \
         __syncthreads();                                                                                                     \
@@ -338,8 +359,8 @@ static int silu_lut_ready(hipStream_t st) {
         silu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
-        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
-        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
+        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
+        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
         if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
         done[dev] = true;
     }
@@ -367,6 +388,15 @@ int camx_quantize_mmq_q8_1(const float * x, const int32_t * ids, void * vy, long
     (void)s02; (void)s03; (void)n_expert_used;
     if (!x || !vy || ne00 < 4 || ne00 % 4 || s01 < ne00 || s01 % 4 || ne0 % 512 || ne0 < ne00 || ne0 >= ne00 + 512 || ne1 < 0 || ne2 != 1 ||
         (layout != MMQ_D4 && layout != MMQ_DS4) || ((uintptr_t)x & 15) || ((uintptr_t)vy & 15)) return CAMX_EINVAL;
+    if (ne1 >= 256 && ne00 % 4 == 0) {       // enough columns to fill the chip: persistent workgroups, block rows stored as whole aligned runs
+        int dev = 0, ncu = 256;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return CAMX_EINVAL;
+        const int ngroups = (ne1 + SWM_TOK - 1) / SWM_TOK, nslab = (int)((ne0 + SWM_SLAB - 1) / SWM_SLAB);
+        const dim3 grid((unsigned)((ncu + 7) / 8 * 8)), block(1024);
+        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, ne0, (uint8_t *)vy, nullptr, ne1, ngroups, nslab);
+        else swiglu_mmq_lut<MMQ_D4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, ne0, (uint8_t *)vy, nullptr, ne1, ngroups, nslab);
+        CAMX_LAUNCH_RET();
+    }
     MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s01, ne1, ne1, 0};
     return launch_mmq<SRC_F32>(a, layout, st);
 }
@@ -398,8 +428,8 @@ int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16
         const long Kp = (F + 511) / 512 * 512;
         const int ngroups = (T + SWM_TOK - 1) / SWM_TOK, nslab = (int)((Kp + SWM_SLAB - 1) / SWM_SLAB);
         const dim3 grid((unsigned)((ncu + 7) / 8 * 8)), block(1024);
-        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4><<<grid, block, SWM_LDS, st>>>(gu, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
-        else swiglu_mmq_lut<MMQ_D4><<<grid, block, SWM_LDS, st>>>(gu, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
+        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
+        else swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
         CAMX_LAUNCH_RET();
     }
     MmqArgs a = {gu, nullptr, (uint8_t *)vy, act, F, (F + 511) / 512 * 512, ld, T, T, 0};

@@ -35,7 +35,8 @@ def test_q8_1_silu_modes(mode):
     assert np.abs(got[:, 4:].view(np.int8).astype(int) - ref[:, 4:].view(np.int8).astype(int)).max() <= 1
 
 
-@pytest.mark.parametrize('K,ncols,layout', [(512, 3, 0), (2048, 17, 1), (17408, 5, 1), (896, 4, 0), (100 * 4, 2, 1)])
+@pytest.mark.parametrize('K,ncols,layout', [(512, 3, 0), (2048, 17, 1), (17408, 5, 1), (896, 4, 0), (100 * 4, 2, 1), (2048, 300, 1), (900, 257, 0),
+                                            (6144, 1030, 1)])
 def test_mmq_quantize(K, ncols, layout):
     rng = np.random.default_rng(K + ncols)
     s01 = K + 8
