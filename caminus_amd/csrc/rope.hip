@@ -23,54 +23,85 @@ struct RopeArgs {
     int n;
 };
 
-template <bool YARN, bool Q8, bool BF16IN>
+// TPW tokens per workgroup: 1 for decode-sized batches (wave 0 computes the token's cos / sin row); 4 for prefill chunks, where
+// wave w computes token w's row, one barrier publishes all four, and each wave then walks the tokens with the next token's
+// (or next pass's) loads in flight during the current one's arithmetic.
+template <int S> CAMX_DEV float half_lane_bcast(float v) {   // every lane of a 32-lane half reads the half's lane S
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x00 | (S << 5)));
+}
+
+template <bool YARN, bool Q8, bool BF16IN, int TPW>
 __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
-    __shared__ __attribute__((aligned(16))) float rc[64];
-    __shared__ __attribute__((aligned(16))) float rs[64];
-    const int t = blockIdx.x, tid = threadIdx.x, lane = slot_of(tid & 63), l = lane & 31;
-    const int pos = a.pos ? a.pos[t] : a.pos0 + t;
-    const float * row = (const float *)a.qkv + (size_t)t * a.ldq;
-    const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)t * a.ldq;
+    __shared__ __attribute__((aligned(16))) float rc[TPW][64];
+    __shared__ __attribute__((aligned(16))) float rs[TPW][64];
+    const int t0 = blockIdx.x * TPW, tid = threadIdx.x, lraw = tid & 63, lane = slot_of(lraw), l = lane & 31, wave = tid >> 6;
     // items: heads 0 .. nh + nkv - 1 take norm + rotary, items nh + nkv .. nh + 2 nkv - 1 are the V heads. A wave step is two
-    // heads (one per half-wave); the loads of up to QR_STEPS steps are issued before the cos / sin row is computed, so a
-    // decode token pays one memory round trip, not one per head.
+    // heads (one per half-wave); the loads of up to QR_STEPS steps (one pass) are issued together, and before the cos / sin
+    // rows are computed, so a decode token pays one memory round trip, not one per head.
     const int items = a.nh + 2 * a.nkv;
     constexpr int QR_STEPS = 5;
-    const int it_w = (tid >> 6) * 2 + (lane >> 5);                      // this half-wave's head inside a step of 8 heads
-    f32x4 xin[QR_STEPS];
-    auto load = [&](int base) {
+    const int npass = (items + 8 * QR_STEPS - 1) / (8 * QR_STEPS);
+    const int it_w = wave * 2 + (lane >> 5);                            // this half-wave's head inside a step of 8 heads
+    f32x4 xin[QR_STEPS], xnext[QR_STEPS];
+    auto load = [&](f32x4 (&buf)[QR_STEPS], int tok, int base) {
+        const int tk = tok < a.n ? tok : 0;
+        const float * row = (const float *)a.qkv + (size_t)tk * a.ldq;
+        const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)tk * a.ldq;
 #pragma unroll
         for (int s = 0; s < QR_STEPS; s++) {
             const int it = base + 8 * s + it_w;
             const int hy = it < items ? it : 0;
-            xin[s] = BF16IN ? unpack_bf16x4(*(const u32x2 *)(rowb + (size_t)hy * 128 + 4 * l)) : *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
+            buf[s] = BF16IN ? unpack_bf16x4(*(const u32x2 *)(rowb + (size_t)hy * 128 + 4 * l)) : *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
         }
     };
-    load(0);
+    load(xin, t0, 0);
     const f32x4 wq = *(const f32x4 *)(a.par + 4 * l), wk = *(const f32x4 *)(a.par + 128 + 4 * l);
     const float eps = a.par[257];
-    if (tid < 64) {
-        float c, s;
-        if (YARN) { const float theta = (float)pos * a.par[258 + tid], ms = a.par[322]; c = cosf(theta) * ms; s = sinf(theta) * ms; }
-        else { const float theta = (float)pos * rope_freq(a.par[256], tid); c = cosf(theta); s = sinf(theta); }
-        rc[tid] = c; rs[tid] = s;
+    for (int tr = wave; tr < TPW; tr += 4) {                               // the tokens whose cos / sin rows this wave computes
+        if (t0 + tr < a.n) {
+            const int pos = a.pos ? a.pos[t0 + tr] : a.pos0 + t0 + tr;
+            float c, s;
+            if (YARN) { const float theta = (float)pos * a.par[258 + lraw], ms = a.par[322]; c = cosf(theta) * ms; s = sinf(theta) * ms; }
+            else { const float theta = (float)pos * rope_freq(a.par[256], lraw); c = cosf(theta); s = sinf(theta); }
+            rc[tr][lraw] = c; rs[tr][lraw] = s;
+        }
     }
     __syncthreads();
     const size_t M = (size_t)a.nkv * 128;
     const size_t rb = Q8 ? 2 * (M / 32) * 34 : 4 * M;
-    uint8_t * cw = nullptr;
-    if (a.page_table) {
-        const int pg = a.page_table[(size_t)t * a.pt_stride + pos / a.page];
-        if (pg < 0 || pg >= a.n_pages) { if (tid == 0) atomicOr(a.err, 8); }
-        else cw = (uint8_t *)a.cache + ((size_t)pg * a.page + (size_t)(pos % a.page)) * rb;
-    } else cw = (uint8_t *)a.cache + (size_t)pos * rb;
-    const f32x4 c4 = *(const f32x4 *)(rc + 4 * (l & 15)), s4 = *(const f32x4 *)(rs + 4 * (l & 15));
     const bool lo = l < 16;
-    for (int base = 0; base < items; base += 8 * QR_STEPS) {
-        if (base) load(base);
+    for (int it_tp = 0; it_tp < TPW * npass; it_tp++) {
+        const int ti = it_tp / npass, base = (it_tp - ti * npass) * 8 * QR_STEPS, t = t0 + ti;
+        if (t >= a.n) break;
+        if (it_tp + 1 < TPW * npass) { const int tn = (it_tp + 1) / npass; load(xnext, t0 + tn, ((it_tp + 1) - tn * npass) * 8 * QR_STEPS); }
+        const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+        uint8_t * cw = nullptr;
+        if (a.page_table) {
+            const int pg = a.page_table[(size_t)t * a.pt_stride + pos / a.page];
+            if (pg < 0 || pg >= a.n_pages) { if (tid == 0 && base == 0) atomicOr(a.err, 8); }
+            else cw = (uint8_t *)a.cache + ((size_t)pg * a.page + (size_t)(pos % a.page)) * rb;
+        } else cw = (uint8_t *)a.cache + (size_t)pos * rb;
+        const f32x4 c4 = *(const f32x4 *)(rc[ti] + 4 * (l & 15)), s4 = *(const f32x4 *)(rs[ti] + 4 * (l & 15));
+        // the sums of squares of all steps first (every lane active), then ONE IEEE sqrt + divide per half-wave for all of
+        // them: lane s of a half-wave takes step s, and the half-wave reads it back
+        float tot[QR_STEPS];
 #pragma unroll
         for (int st = 0; st < QR_STEPS; st++) {
-            if (base + 8 * st + (tid >> 6) * 2 >= items) break;        // wave-uniform: neither half-wave has a head
+            const f32x4 x = xin[st];
+            f32x4 sq; sq.x = x.x * x.x; sq.y = x.y * x.y; sq.z = x.z * x.z; sq.w = x.w * x.w;
+            tot[st] = half_groups_in_order<4>(group32_sum(sq), lane & 32);
+        }
+        float tv = tot[0];
+#pragma unroll
+        for (int st = 1; st < QR_STEPS; st++) tv = (lraw & 31) == st ? tot[st] : tv;
+        const float sc = rsqrt_exact(tv / 128 + eps);
+        float scl[QR_STEPS];
+        scl[0] = half_lane_bcast<0>(sc); scl[1] = half_lane_bcast<1>(sc); scl[2] = half_lane_bcast<2>(sc); scl[3] = half_lane_bcast<3>(sc);
+        scl[4] = half_lane_bcast<4>(sc);
+        static_assert(QR_STEPS == 5, "the broadcasts above are written out for five steps");
+#pragma unroll
+        for (int st = 0; st < QR_STEPS; st++) {
+            if (base + 8 * st + wave * 2 >= items) break;               // wave-uniform: neither half-wave has a head
             const int it = base + 8 * st + it_w;
             const bool active = it < items;
             const int hy = active ? it : 0;
@@ -85,9 +116,7 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
             }
             const bool isq = hy < a.nh;
             const f32x4 wn = isq ? wq : wk;
-            f32x4 sq; sq.x = x.x * x.x; sq.y = x.y * x.y; sq.z = x.z * x.z; sq.w = x.w * x.w;
-            const float tot = half_groups_in_order<4>(group32_sum(sq), lane & 32);
-            const float scale = rsqrt_exact(tot / 128 + eps);
+            const float scale = scl[st];
             f32x4 y1; y1.x = (scale * x.x) * wn.x; y1.y = (scale * x.y) * wn.y; y1.z = (scale * x.z) * wn.z; y1.w = (scale * x.w) * wn.w;
             f32x4 p; p.x = lane_xor16(y1.x); p.y = lane_xor16(y1.y); p.z = lane_xor16(y1.z); p.w = lane_xor16(y1.w);
             // dims below 64: fma(x0, c, -(x1 s)); dims from 64: fma(x1, c, x0 s), with x0 the low and x1 the high dim of the pair
@@ -107,6 +136,8 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
                 else if (active && cw) *(u32x2 *)((uint16_t *)cw + (size_t)g * 128 + 4 * l) = pack_f16x4(y);
             }
         }
+#pragma unroll
+        for (int st = 0; st < QR_STEPS; st++) xin[st] = xnext[st];
     }
 }
 
@@ -463,11 +494,11 @@ static int rope_check(const RopeArgs & a, bool q8, bool bf16in) {
     if (a.page_table && (a.page < 1 || a.n_pages < 1 || a.pt_stride < 1 || !a.err)) return CAMX_EINVAL;
     return CAMX_OK;
 }
-template <bool BF16IN>
+template <bool BF16IN, int TPW>
 static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st) {
-    const dim3 grid(a.n), block(256);
-    if (q8) { if (yarn) qk_rope_tokens<true, true, BF16IN><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true, BF16IN><<<grid, block, 0, st>>>(a); }
-    else { if (yarn) qk_rope_tokens<true, false, BF16IN><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false, BF16IN><<<grid, block, 0, st>>>(a); }
+    const dim3 grid((a.n + TPW - 1) / TPW), block(256);
+    if (q8) { if (yarn) qk_rope_tokens<true, true, BF16IN, TPW><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true, BF16IN, TPW><<<grid, block, 0, st>>>(a); }
+    else { if (yarn) qk_rope_tokens<true, false, BF16IN, TPW><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false, BF16IN, TPW><<<grid, block, 0, st>>>(a); }
 }
 static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bool bf16in = false) {
     if (rope_check(a, q8, bf16in)) return CAMX_EINVAL;
@@ -479,7 +510,8 @@ static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bo
         if (yarn) qk_rope_bf16_tokens<true, 4><<<g4, dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false, 4><<<g4, dim3(256), 0, st>>>(a);
     }
     else if (wide) { if (yarn) qk_rope_bf16_tokens<true, 1><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false, 1><<<dim3(a.n), dim3(256), 0, st>>>(a); }
-    else if (bf16in) rope_dispatch<true>(a, yarn, q8, st); else rope_dispatch<false>(a, yarn, q8, st);
+    else if (bf16in) rope_dispatch<true, 1>(a, yarn, q8, st);
+    else rope_dispatch<false, 1>(a, yarn, q8, st);
     CAMX_LAUNCH_RET();
 }
 
