@@ -141,8 +141,7 @@ __global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, c
 // the same with VW consecutive channels per thread (VW = 8 for bf16, 4 for fp32) and a sliding window over CONV_TT tokens:
 // every input is read once (plus a three-token halo per chunk) with 128-bit loads that are all issued before the first
 // output is computed; the loaded vectors stay packed (4 registers per token) and are widened as the window reaches them
-#define CONV_TT 16
-template <bool BF16>
+template <bool BF16, int CONV_TT>
 __global__ void __launch_bounds__(256) gdn_conv_vec(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
                                                     void * __restrict__ y, int C, int T, int ldx, int ldy) {
     constexpr int VW = BF16 ? 8 : 4;
@@ -369,10 +368,10 @@ int camx_gate_mul(const void * a, const void * gt, void * y, long N, int D, int 
 int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void * y, int C, int T, int ldx, int ldy, int bf16, hipStream_t st) {
     if (!x || !w || !state || !y || C < 1 || T < 1 || ldx < C || ldy < C || ((uintptr_t)w & 15)) return CAMX_EINVAL;
     const int vw = bf16 ? 8 : 4;
-    if (C % vw == 0 && ldx % vw == 0 && ldy % vw == 0 && !(((uintptr_t)x | (uintptr_t)y) & 15)) {
-        const dim3 gv((unsigned)((C / vw + 255) / 256), (unsigned)((T + CONV_TT - 1) / CONV_TT)), bv(256);
-        if (bf16) gdn_conv_vec<true><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
-        else gdn_conv_vec<false><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
+    if ((long)T * C >= (1L << 20) && C % vw == 0 && ldx % vw == 0 && ldy % vw == 0 && !(((uintptr_t)x | (uintptr_t)y) & 15)) {
+        const int tt = 16;      // (a decode / verify batch takes the one-value-per-thread kernel below: it fills the chip, a 16-token window would not)
+        const dim3 gv((unsigned)((C / vw + 255) / 256), (unsigned)((T + tt - 1) / tt)), bv(256);
+        { if (bf16) gdn_conv_vec<true, 16><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy); else gdn_conv_vec<false, 16><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy); }
         CAMX_LAUNCH_RET();
     }
     const dim3 grid((unsigned)(((long)T * C + 255) / 256)), block(256);

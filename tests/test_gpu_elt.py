@@ -46,7 +46,7 @@ def test_gate_mul():
     assert close_16(host(ybf, np.uint16), O.f2bf(O.gate_mul(O.bf2f(abf), O.bf2f(gbf), D, 2 * D, D)), 'bf16')
 
 
-@pytest.mark.parametrize('T,C', [(16, 10240), (1, 64), (2, 100), (5, 256), (37, 512), (3, 6)])
+@pytest.mark.parametrize('T,C', [(16, 10240), (1, 64), (2, 100), (5, 256), (37, 512), (3, 6), (520, 8192), (130, 8200)])
 def test_gdn_conv(T, C):
     rng = np.random.default_rng(C)
     ldx = C + 4
