@@ -203,8 +203,18 @@ def extra_opsets(B):
     out.append(('c5_qk_rope_hadamard_q8_paged', S5 * (ldq * 4 + 8 + nh * 128 * 2 + rbq) + 258 * 4,
                 lambda: B.call('camx_qk_rope_paged', _p(qkv5), I(ldq), I(nh), I(nkv), _p(par), _p(pos5d), _p(q165), _p(cache5), _p(err5), _p(ptd), I(512),
                                I(page), I(n_pages), I(S5), I(0), I(1))))
+    # hyper-connection glue at the one shape the reference publishes per-op times for (T = 2048, 4 streams of 2560; RX 7900 XTX:
+    # hc_post_rms with bf16 copy and scale 0.466 ms, hc_mean 0.267 ms; docs/specs/spec-prefill-cache.md:276)
+    Th, HC, Nh = 2048, 4, 2560
+    bh = B.acts((Th, Nh), torch.float32, 61); injh = B.acts((Th, HC), torch.float32, 62, frac=0); resh = B.acts((Th, HC, Nh), torch.float32, 63)
+    wh = B.gamma(HC * Nh, 64); xnbf = torch.empty((Th, HC, Nh), dtype=torch.bfloat16, device=B.dev); sclh = torch.empty(Th * HC, device=B.dev)
+    gh = B.acts((Th, HC, Nh), torch.float32, 65); outh = torch.empty((Th, Nh), device=B.dev)
+    out.append(('hc_post_rms_2048x4x2560_bf16_scale', Th * Nh * 4 + Th * HC * Nh * (4 + 4 + 2) + HC * Nh * 4 + Th * HC * 8,
+                lambda: B.call('camx_pf_hc_post_rms', _p(bh), _p(injh), _p(resh), _p(wh), NULL, _p(xnbf), _p(sclh), I(Th), I(HC), F(0.25), F(1e-6), I(Nh))))
+    out.append(('hc_mean_2048x4x2560_from_residual', Th * HC * Nh * 8 + Th * Nh * 4 + HC * Nh * 4 + Th * HC * 4,
+                lambda: B.call('camx_pf_hc_mean', _p(resh), _p(sclh), _p(wh), _p(gh), _p(outh), I(Th), I(HC), I(Nh), F(0.25))))
     out.append(('_keep', 0, [x, d, nw, h, h16, q8, qkv, par, q16, cache, g, u, y16, toks, qg, w4, pos, o4, a4, xc, wc, st, yc, l2o, x5, d5, h5, h516, qkv5,
-                             cache5, err5, pos5d, ptd, q165]))
+                             cache5, err5, pos5d, ptd, q165, bh, injh, resh, wh, xnbf, sclh, gh, outh]))
     return out
 
 
@@ -323,6 +333,9 @@ def main():
             q1.record(); q1.synchronize()
             ops[name] = {'us': round(med, 2), 'us_cache_hot': round(med_hot, 2), 'us_queued': round(q0.elapsed_time(q1) * 1e3 / 50, 2), 'bytes': by, 'GBps': round(by / (med * 1e-6) / 1e9, 1),
                          'frac_of_8TBps': round(by / (med * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+        # the only per-op times the reference publishes for this path (another GPU: RX 7900 XTX, docs/specs/spec-prefill-cache.md:276)
+        for k, ref_us in (('hc_post_rms_2048x4x2560_bf16_scale', 466.0), ('hc_mean_2048x4x2560_from_residual', 267.0)):
+            if k in ops: ops[k]['reference_rx7900xtx_us'] = ref_us
         out['opsets'] = ops
     if not a.no_cpu and not a.only:
         out['cpu_baseline'] = cpu_baseline(w)

@@ -282,6 +282,76 @@ __global__ void __launch_bounds__(256) gdn_l2_128(const void * __restrict__ x, v
     if (active) { if (BF16) *(u32x2 *)((uint16_t *)y + yo) = pack_bf16x4_rne(o); else *(f32x4 *)((float *)y + yo) = o; }
 }
 
+// ---- hyper-connection glue (kernels/prefill_glue.hip:172-206) -----------------------------------------------------------------
+// pf_hc_post: res[t][h][i] = fma(b[t][i], 2 sigmoid(inj[t][h] * rs), res[t][h][i]); four consecutive i per thread when D % 4 == 0
+template <bool VEC>
+__global__ void __launch_bounds__(256) hc_post_k(const float * __restrict__ b, const float * __restrict__ inj, float * __restrict__ res, int T, int HC,
+                                                 int D, float rs) {
+    constexpr int VW = VEC ? 4 : 1;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * VW;
+    if (i >= (long)T * D) return;
+    const int tt = (int)(i / D), ii = (int)(i - (long)tt * D);
+    float bv[VW];
+    if (VEC) { const f32x4 v = *(const f32x4 *)(b + i); bv[0] = v.x; if (VW > 1) { bv[1] = v.y; bv[2] = v.z; bv[3] = v.w; } }
+    else bv[0] = b[i];
+    for (int h = 0; h < HC; h++) {
+        const float v = inj[tt * HC + h] * rs;
+        const float sgm = 1.0f / (1.0f + expf(-v));
+        const float ph = sgm * 2.0f;
+        const size_t o = (size_t)(tt * HC + h) * D + ii;
+        if (VEC) {
+            f32x4 r = *(const f32x4 *)(res + o);
+            r.x = __builtin_fmaf(bv[0], ph, r.x); r.y = __builtin_fmaf(bv[1 % VW], ph, r.y); r.z = __builtin_fmaf(bv[2 % VW], ph, r.z); r.w = __builtin_fmaf(bv[3 % VW], ph, r.w);
+            __builtin_nontemporal_store(r, (f32x4 *)(res + o));
+        } else res[o] = __builtin_fmaf(bv[0], ph, res[o]);
+    }
+}
+// pf_hc_mean: out[t][i] = rs * sum over h (fma chain from 0) of xn[t][h][i] * sigmoid(g[t][h][i]); xn given, or recomputed from
+// the residual as (x * scl[t * HC + h]) * w[h][i]. The loads of all HC streams (up to 8) are issued before the arithmetic.
+template <bool VEC>
+__global__ void __launch_bounds__(256) hc_mean_k(const float * __restrict__ x, const float * __restrict__ scl, const float * __restrict__ w,
+                                                 const float * __restrict__ g, float * __restrict__ out, int T, int HC, int D, float rs) {
+    constexpr int VW = VEC ? 4 : 1;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * VW;
+    if (i >= (long)T * D) return;
+    const int tt = (int)(i / D), ii = (int)(i - (long)tt * D);
+    float sum[VW];
+#pragma unroll
+    for (int k = 0; k < VW; k++) sum[k] = 0.0f;
+    for (int h0 = 0; h0 < HC; h0 += 8) {
+        float xv[8][VW], gv[8][VW], sc[8], wv[8][VW];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int h = h0 + u;
+            if (h < HC) {
+                const size_t o = (size_t)(tt * HC + h) * D + ii;
+                if (VEC) {
+                    const f32x4 a = __builtin_nontemporal_load((const f32x4 *)(x + o)), c = __builtin_nontemporal_load((const f32x4 *)(g + o));
+                    xv[u][0] = a.x; gv[u][0] = c.x;
+                    if (VW > 1) { xv[u][1] = a.y; xv[u][2] = a.z; xv[u][3] = a.w; gv[u][1] = c.y; gv[u][2] = c.z; gv[u][3] = c.w; }
+                } else { xv[u][0] = x[o]; gv[u][0] = g[o]; }
+                if (scl) {
+                    sc[u] = scl[tt * HC + h];
+                    if (VEC) { const f32x4 q = *(const f32x4 *)(w + (size_t)h * D + ii); wv[u][0] = q.x; if (VW > 1) { wv[u][1] = q.y; wv[u][2] = q.z; wv[u][3] = q.w; } }
+                    else wv[u][0] = w[(size_t)h * D + ii];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            if (h0 + u < HC) {
+#pragma unroll
+                for (int k = 0; k < VW; k++) {
+                    const float xn = scl ? (xv[u][k] * sc[u]) * wv[u][k] : xv[u][k];
+                    sum[k] = __builtin_fmaf(xn, 1.0f / (1.0f + expf(-gv[u][k])), sum[k]);
+                }
+            }
+        }
+    }
+    if (VEC) *(f32x4 *)(out + i) = (f32x4){rs * sum[0], rs * sum[1 % VW], rs * sum[2 % VW], rs * sum[3 % VW]};
+    else out[i] = rs * sum[0];
+}
+
 // ---- S1 core / fuse ----------------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) embedding_f32_k(const int * __restrict__ tok, const float * __restrict__ emb, float * __restrict__ out, int D) {
     const int t = blockIdx.x;
@@ -399,6 +469,22 @@ int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs
     }
     if (bf16) { if (vec) gdn_l2_k<true, true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); else gdn_l2_k<true, false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); }
     else { if (vec) gdn_l2_k<false, true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); else gdn_l2_k<false, false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); }
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_hc_post(const float * b, const float * inj, float * res, int T, int HC, int D, float rs, hipStream_t st) {
+    if (!b || !inj || !res || T < 0 || HC < 1 || D < 1) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    const bool vec = D % 4 == 0 && !(((uintptr_t)b | (uintptr_t)res) & 15);
+    const long n = (long)T * D / (vec ? 4 : 1);
+    if (vec) hc_post_k<true><<<GRID_1D(n), dim3(256), 0, st>>>(b, inj, res, T, HC, D, rs); else hc_post_k<false><<<GRID_1D(n), dim3(256), 0, st>>>(b, inj, res, T, HC, D, rs);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_hc_mean(const float * x, const float * scl, const float * w, const float * g, float * out, int T, int HC, int D, float rs, hipStream_t st) {
+    if (!x || !g || !out || T < 0 || HC < 1 || D < 1 || ((scl == nullptr) != (w == nullptr))) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    const bool vec = D % 4 == 0 && !(((uintptr_t)x | (uintptr_t)g | (uintptr_t)out | (uintptr_t)w) & 15);
+    const long n = (long)T * D / (vec ? 4 : 1);
+    if (vec) hc_mean_k<true><<<GRID_1D(n), dim3(256), 0, st>>>(x, scl, w, g, out, T, HC, D, rs); else hc_mean_k<false><<<GRID_1D(n), dim3(256), 0, st>>>(x, scl, w, g, out, T, HC, D, rs);
     CAMX_LAUNCH_RET();
 }
 int camx_embedding_f32(const int * tok, const float * emb, float * out, int D, int T, hipStream_t st) {

@@ -8,7 +8,8 @@
 // 8 group sums in order; scale = 1 / sqrt(tot / N + eps) with IEEE sqrt and divide; h = (x * scale) * w.
 #include "common.cuh"
 
-enum { ADD_NONE = 0, ADD_F32_SLOTS = 1, ADD_BF16 = 2, ADD_F32_DIRECT = 3 };   // DIRECT: x = x + d (no 0 + d first)
+enum { ADD_NONE = 0, ADD_F32_SLOTS = 1, ADD_BF16 = 2, ADD_F32_DIRECT = 3, ADD_HC = 4 };   // DIRECT: x = x + d (no 0 + d first)
+// ADD_HC (pf_hc_post_rms): row q = token q / HC, stream q % HC; x = fma(d[token], 2 sigmoid(inj[q] * rs), x); gamma row q % HC
 
 struct NormArgs {
     float * x;               // [rows][N] residual, updated in place when an addend is given
@@ -25,6 +26,7 @@ struct NormArgs {
     uint8_t * q8;            // optional q8_1 blocks [rows][N / 32][36]
     float * scl;             // optional row scale [rows]
     int N, rows;
+    const float * inj; int HC; float rs;   // ADD_HC only
 };
 
 // EXACT: the row has exactly NI_MAX slabs, so every loop below is straight-line code: no scalar branch stands between the
@@ -91,11 +93,27 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) xv[j] = xv[j] + unpack_bf16x4(dv[j]);
     }
+    if (ADD == ADD_HC) {
+        const float * dr = (const float *)a.d + (size_t)(row / a.HC) * N;
+        f32x4 dv[NI_MAX];
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) dv[j] = *(const f32x4 *)(dr + 256 * j + 4 * lane);       // (plain: the HC rows of a token share it)
+        const float v = a.inj[row] * a.rs;
+        const float sgm = 1.0f / (1.0f + expf(-v));
+        const float p = sgm * 2.0f;
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) {
+                xv[j].x = __builtin_fmaf(dv[j].x, p, xv[j].x); xv[j].y = __builtin_fmaf(dv[j].y, p, xv[j].y);
+                xv[j].z = __builtin_fmaf(dv[j].z, p, xv[j].z); xv[j].w = __builtin_fmaf(dv[j].w, p, xv[j].w);
+            }
+    }
     f32x4 g[NI_MAX];
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
-    if ((ADD == ADD_F32_SLOTS && a.S > 0) || ((ADD == ADD_F32_DIRECT || ADD == ADD_BF16) && a.d)) {
+    if (ADD == ADD_HC || (ADD == ADD_F32_SLOTS && a.S > 0) || ((ADD == ADD_F32_DIRECT || ADD == ADD_BF16) && a.d)) {
         // the updated residual goes back to the lines it was read from (plain loads above, nontemporal stores here: a
         // nontemporal load followed by a store to the same line is slow on gfx950)
 #pragma unroll
@@ -151,6 +169,10 @@ __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
                 }
                 if (ADD == ADD_F32_DIRECT && a.d) { xv = xv + ((const float *)a.d)[(size_t)row * N + i]; xr[i] = xv; }
                 if (ADD == ADD_BF16 && a.d) { xv = xv + bf2f(((const uint16_t *)a.d)[(size_t)row * N + i]); xr[i] = xv; }
+                if (ADD == ADD_HC) {
+                    const float v = a.inj[row] * a.rs; const float sgm = 1.0f / (1.0f + expf(-v)); const float p = sgm * 2.0f;
+                    xv = __builtin_fmaf(((const float *)a.d)[(size_t)(row / a.HC) * N + i], p, xv); xr[i] = xv;
+                }
                 ssk[k] = __builtin_fmaf(xv, xv, ssk[k]);
             }
         }
@@ -210,44 +232,52 @@ extern "C" {
 int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
                        uint16_t * h16, int N, int n, hipStream_t st) {
     if (N < 256 || N % 256 || N > 2048 || S < 0 || S > 8 || n < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
-    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n};
+    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
     return launch_norm<ADD_F32_SLOTS>(a, st);
 }
 
 int camx_q35p_add_rms16(float * x, const float * d, const float * nw, float eps, float * h, uint16_t * h16, int N, int n, hipStream_t st) {
     if (N < 256 || N % 256 || N > 65536 || n < 0 || !x || !nw || !h || !h16) return CAMX_EINVAL;
-    NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n};
+    NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
     return launch_norm<ADD_F32_DIRECT>(a, st);
 }
 
 int camx_add_rms_q8_1(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
                       uint16_t * h16, uint8_t * q8, int N, int n, hipStream_t st) {
     if (N < 32 || N % 32 || S < 0 || S > 8 || n < 0 || !x || !nw || (S > 0 && !d)) return CAMX_EINVAL;
-    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, q8, nullptr, N, n};
+    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, q8, nullptr, N, n, nullptr, 1, 0.0f};
     return launch_norm<ADD_F32_SLOTS>(a, st);
 }
 
 int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps, float * h, uint16_t * hbf, int N, int n, hipStream_t st) {
     if (N < 1 || n < 0 || !x || !nw) return CAMX_EINVAL;
-    NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, nullptr, N, hbf, nullptr, nullptr, N, n};
+    NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, nullptr, N, hbf, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
     return launch_norm<ADD_BF16>(a, st);
 }
 
 int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf, float * scl, int R, int wr, float eps, int K, hipStream_t st) {
     if (K < 1 || R < 0 || wr < 1 || !x || !w) return CAMX_EINVAL;
-    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, ybf, nullptr, scl, K, R};
+    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, ybf, nullptr, scl, K, R, nullptr, 1, 0.0f};
     return launch_norm<ADD_NONE>(a, st);
 }
 
 int camx_op_rms_mul(const float * x, const float * w, float * y, uint8_t * q8, int R, int wr, int K, float eps, hipStream_t st) {
     if (K < 1 || R < 0 || wr < 1 || !x || !w || (q8 && K % 32)) return CAMX_EINVAL;
-    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, nullptr, q8, nullptr, K, R};
+    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, nullptr, q8, nullptr, K, R, nullptr, 1, 0.0f};
     return launch_norm<ADD_NONE>(a, st);
+}
+
+// pf_hc_post_rms: res [T * HC][N] updated in place, then its norm with w [HC][N]; xn, xnbf, scl optional
+int camx_pf_hc_post_rms(const float * b, const float * inj, float * res, const float * w, float * xn, uint16_t * xnbf, float * scl, int T, int HC,
+                        float rs, float eps, int N, hipStream_t st) {
+    if (!b || !inj || !res || !w || T < 0 || HC < 1 || N < 1 || (long)T * HC > 0x7fffffffL) return CAMX_EINVAL;
+    NormArgs a = {res, b, nullptr, 0, w, HC, eps, xn, nullptr, N, xnbf, nullptr, scl, N, T * HC, inj, HC, rs};
+    return launch_norm<ADD_HC>(a, st);
 }
 
 int camx_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows, hipStream_t st) {
     if (D < 1 || rows < 0 || !x || !w || !out) return CAMX_EINVAL;
-    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, 1, eps, out, nullptr, D, nullptr, nullptr, nullptr, D, rows};
+    NormArgs a = {(float *)x, nullptr, nullptr, 0, w, 1, eps, out, nullptr, D, nullptr, nullptr, nullptr, D, rows, nullptr, 1, 0.0f};
     return launch_norm<ADD_NONE>(a, st);
 }
 

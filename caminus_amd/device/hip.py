@@ -130,6 +130,8 @@ def _q3m(yarn, q8):
 
 def _glue(K):
     return {'pf_rms_mul': _pf_rms_mul(K),
+            'pf_hc_post_rms': ('camx_pf_hc_post_rms', lambda g, b, v: list(v) + [I(K)]),
+            'pf_hc_post': _plain('camx_pf_hc_post'), 'pf_hc_mean': _plain('camx_pf_hc_mean'),
             'pf_gdn_conv': ('camx_pf_gdn_conv', lambda g, b, v: list(v) + [I(0)]),
             'pf_conv_state': ('camx_pf_conv_state', lambda g, b, v: list(v) + [I(0)])}
 

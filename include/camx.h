@@ -59,6 +59,17 @@ int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf,
                     camx_stream_t stream);
 /* OP_RMS_MUL (kernels/k3_gguf_ops.h:1233-1268; Seg fields: a = x, W = w, y, asum = q8, N = R, K, pad1 = wr, rs = eps). */
 int camx_op_rms_mul(const float * x, const float * w, float * y, void * q8, int R, int wr, int K, float eps, camx_stream_t stream);
+/* pf_hc_post_rms (kernels/prefill_glue.hip:130-170): row q = t * HC + h of N values: res[q] = fma(b[t], 2 sigmoid(inj[q] * rs),
+ * res[q]) in place, then the norm of the updated row with w[h]: xn fp32, xnbf bf16, scl the row scale [T * HC], each optional.
+ * The reference kernel is built for N = 2560; N is an argument here. */
+int camx_pf_hc_post_rms(const float * b, const float * inj, float * res, const float * w, float * xn, uint16_t * xnbf, float * scl,
+                        int T, int HC, float rs, float eps, int N, camx_stream_t stream);
+/* pf_hc_post (kernels/prefill_glue.hip:172-188): the residual update alone. */
+int camx_pf_hc_post(const float * b, const float * inj, float * res, int T, int HC, int D, float rs, camx_stream_t stream);
+/* pf_hc_mean (kernels/prefill_glue.hip:190-206): out[t][i] = rs * sum over h of xn[t][h][i] * sigmoid(g[t][h][i]) (fma chain from
+ * 0); xn = x, or (scl and w given) recomputed from the residual x as (x * scl[t * HC + h]) * w[h][i]. */
+int camx_pf_hc_mean(const float * x, const float * scl, const float * w, const float * g, float * out, int T, int HC, int D, float rs,
+                    camx_stream_t stream);
 /* rmsnorm_f32 (kernels/core.hip:30-46): out = x * inv * w over `rows` rows of D values (any D). */
 int camx_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows, camx_stream_t stream);
 

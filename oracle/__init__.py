@@ -150,6 +150,31 @@ def rms_mul(x, w, eps, want_q8=False):
     return out
 
 
+def hc_post_rms(b, inj, res, w, eps, rs=0.25):
+    """-> dict(res, xn, xnbf, scale); b [T, N], inj [T, HC], res [T, HC, N], w [HC, N]"""
+    b = _c(b, np.float32); inj = _c(inj, np.float32); res = _c(res, np.float32).copy(); w = _c(w, np.float32)
+    T, HC, N = res.shape
+    xn = np.empty_like(res); xnbf = np.empty(res.shape, np.uint16); scl = np.empty(T * HC, np.float32)
+    lib().orc_hc_post_rms(_p(b), _p(inj), _p(res), _p(w), _p(xn), _p(xnbf), _p(scl), I(T), I(HC), I(N), F(rs), F(eps))
+    return dict(res=res, xn=xn, xnbf=xnbf, scale=scl)
+
+
+def hc_post(b, inj, res, rs=0.25):
+    b = _c(b, np.float32); inj = _c(inj, np.float32); res = _c(res, np.float32).copy()
+    T, HC, D = res.shape
+    lib().orc_hc_post(_p(b), _p(inj), _p(res), I(T), I(HC), I(D), F(rs))
+    return res
+
+
+def hc_mean(x, g, rs=0.25, scale=None, w=None):
+    x = _c(x, np.float32); g = _c(g, np.float32)
+    T, HC, D = x.shape
+    out = np.empty((T, D), np.float32)
+    lib().orc_hc_mean(_p(x), _p(_c(scale, np.float32)) if scale is not None else _p(None), _p(_c(w, np.float32)) if w is not None else _p(None),
+                      _p(g), _p(out), I(T), I(HC), I(D), F(rs))
+    return out
+
+
 def rmsnorm_f32(x, w, eps):
     x = _c(x, np.float32); rows, D = x.shape; out = np.empty_like(x)
     lib().orc_rmsnorm_f32(_p(x), _p(_c(w, np.float32)), _p(out), I(D), F(eps), I(rows)); return out

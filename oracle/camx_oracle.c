@@ -275,6 +275,55 @@ ORC_API void orc_rms_mul(const float * x, const float * w, float * y, uint16_t *
         }
     }
 }
+/* pf_hc_post_rms (kernels/prefill_glue.hip:130-170): per (token, stream) row q = t * HC + h of N values:
+ * p = (1 / (1 + expf(-(inj[q] * rs)))) * 2 (contract off), res[q][i] = fmaf(b[t][i], p, res[q][i]) in place, then the
+ * norm of the updated row with w[h]: xn fp32, xnbf bf16, scl the row scale, each optional. FP class through expf. */
+ORC_API void orc_hc_post_rms(const float * b, const float * inj, float * res, const float * w, float * xn, uint16_t * xnbf,
+                             float * scl, int T, int HC, int N, float rs, float eps) {
+#pragma omp parallel for schedule(static)
+    for (int q = 0; q < T * HC; q++) {
+        const int h = q % HC, t = q / HC;
+        float * rr = res + (size_t)q * N;
+        const float * br = b + (size_t)t * N, * wv = w + (size_t)h * N;
+        const float v = inj[q] * rs;
+        const float sgm = 1.0f / (1.0f + expf(-v));
+        const float p = sgm * 2.0f;
+        for (int i = 0; i < N; i++) rr[i] = fmaf(br[i], p, rr[i]);
+        const float scale = rsqrt_c(row_ss(rr, N) / (float)N + eps);
+        if (scl) scl[q] = scale;
+        for (int i = 0; i < N; i++) {
+            const float y = (rr[i] * scale) * wv[i];
+            if (xn) xn[(size_t)q * N + i] = y;
+            if (xnbf) xnbf[(size_t)q * N + i] = orc_to_bf16(y);
+        }
+    }
+}
+/* pf_hc_post (kernels/prefill_glue.hip:172-188): the residual update alone, any D */
+ORC_API void orc_hc_post(const float * b, const float * inj, float * res, int T, int HC, int D, float rs) {
+#pragma omp parallel for schedule(static)
+    for (int q = 0; q < T * HC; q++) {
+        const int t = q / HC;
+        const float v = inj[q] * rs;
+        const float sgm = 1.0f / (1.0f + expf(-v));
+        const float p = sgm * 2.0f;
+        for (int i = 0; i < D; i++) res[(size_t)q * D + i] = fmaf(b[(size_t)t * D + i], p, res[(size_t)q * D + i]);
+    }
+}
+/* pf_hc_mean (kernels/prefill_glue.hip:190-206): out[t][i] = rs * sum over h (fmaf chain from 0) of xn[t][h][i] *
+ * (1 / (1 + expf(-g[t][h][i]))); xn given, or recomputed (scl, w given) as (x * scl[t * HC + h]) * w[h][i] */
+ORC_API void orc_hc_mean(const float * x, const float * scl, const float * w, const float * g, float * out, int T, int HC, int D, float rs) {
+#pragma omp parallel for schedule(static)
+    for (int t = 0; t < T; t++)
+        for (int i = 0; i < D; i++) {
+            float sum = 0.0f;
+            for (int h = 0; h < HC; h++) {
+                const size_t o = ((size_t)t * HC + h) * D + i;
+                const float xv = scl ? (x[o] * scl[t * HC + h]) * w[(size_t)h * D + i] : x[o];
+                sum = fmaf(xv, 1.0f / (1.0f + expf(-g[o])), sum);
+            }
+            out[(size_t)t * D + i] = rs * sum;
+        }
+}
 /* rmsnorm_f32 (kernels/core.hip:30-46): out = x * inv * w = (x * inv) * w; the squares accumulate by fmaf (the
  * reference's `s += x * x` under hipcc's default contraction) */
 ORC_API void orc_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows) {

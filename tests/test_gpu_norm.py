@@ -75,3 +75,31 @@ def test_rms_mul_and_rmsnorm(R, K, wr):
         out = dev(np.zeros((R, K), np.float32))
         call('camx_rmsnorm_f32', ptr(xd), ptr(wd), ptr(out), I(K), F(1e-6), I(R))
         assert bits_equal(host(out), O.rmsnorm_f32(x, w[0], 1e-6))
+
+
+@pytest.mark.parametrize('T,HC,N', [(5, 4, 2560), (2048, 4, 2560), (3, 2, 2048), (7, 3, 100), (130, 4, 5120)])
+def test_hc_glue(T, HC, N):
+    """hyper-connection glue: the residual update passes expf (tolerance class: 1e-5 x max), everything behind it is exact given
+    the updated residual; inj = 0 makes the gate exactly 1, so those rows are compared bit for bit"""
+    from gpu_util import close_16, close_fp32
+    rng = np.random.default_rng(T + N)
+    b = outliers(rng, (T, N)); inj = rng.standard_normal((T, HC)).astype(np.float32); inj[0] = 0.0
+    res = outliers(rng, (T, HC, N)); w = (1 + 0.1 * rng.standard_normal((HC, N))).astype(np.float32)
+    ref = O.hc_post_rms(b, inj, res, w, 1e-6)
+    rd = dev(res); xn = dev(np.zeros((T, HC, N), np.float32)); xnbf = dev(np.zeros((T, HC, N), np.uint16)); scl = dev(np.zeros(T * HC, np.float32))
+    bd, injd, wd = dev(b), dev(inj), dev(w)
+    call('camx_pf_hc_post_rms', ptr(bd), ptr(injd), ptr(rd), ptr(wd), ptr(xn), ptr(xnbf), ptr(scl), I(T), I(HC), F(0.25), F(1e-6), I(N))
+    gres, gxn = host(rd), host(xn)
+    assert close_fp32(gres, ref['res']) and close_fp32(gxn, ref['xn']) and close_16(host(xnbf, np.uint16), ref['xnbf'], 'bf16')
+    assert bits_equal(gres[0], ref['res'][0]) and bits_equal(gxn[0], ref['xn'][0]) and bits_equal(host(scl)[:HC], ref['scale'][:HC])
+    # exact given the device's own residual: the norm of it by the oracle's rms_mul
+    again = O.rms_mul(gres.reshape(T * HC, N), w, 1e-6)
+    assert bits_equal(gxn.reshape(T * HC, N), again['y']) and bits_equal(host(scl), again['scale']) and bits_equal(host(xnbf, np.uint16).reshape(T * HC, N), again['ybf'])
+    r2 = dev(res)
+    call('camx_pf_hc_post', ptr(bd), ptr(injd), ptr(r2), I(T), I(HC), I(N), F(0.25))
+    assert bits_equal(host(r2), gres)                                      # the same statements: the same bits as the fused kernel
+    g = outliers(rng, (T, HC, N))
+    out = dev(np.zeros((T, N), np.float32)); out2 = dev(np.zeros((T, N), np.float32))
+    call('camx_pf_hc_mean', ptr(xn), NULL, NULL, ptr(dev(g)), ptr(out), I(T), I(HC), I(N), F(0.25))
+    call('camx_pf_hc_mean', ptr(rd), ptr(scl), ptr(wd), ptr(dev(g)), ptr(out2), I(T), I(HC), I(N), F(0.25))
+    assert close_fp32(host(out), O.hc_mean(gxn, g)) and bits_equal(host(out2), host(out))

@@ -489,3 +489,28 @@ def test_actq_invariants():
     assert (s > 0).all() and np.allclose(s, np.abs(u).reshape(M, K).max(1) * 0.9 / qmax, rtol=2e-2)
     z, sz, cz = O.actq_fwd(np.zeros((1, 128), f32))
     assert sz[0] == f32(1e-8) and not cz.any() and not z.any()
+
+
+def test_hc_glue_against_float64():
+    """hyper-connection glue (kernels/prefill_glue.hip:130-206): float64 closed forms; inj = 0 gives the gate exactly 1; the
+    mean from the residual + scale equals the mean from the stored norm bit for bit (the same expression on the same bits)"""
+    rng = np.random.default_rng(44)
+    T, HC, N = 6, 4, 2560
+    b = rng.standard_normal((T, N)).astype(f32); inj = rng.standard_normal((T, HC)).astype(f32); inj[2] = 0
+    res = rng.standard_normal((T, HC, N)).astype(f32); w = (1 + 0.1 * rng.standard_normal((HC, N))).astype(f32)
+    r = O.hc_post_rms(b, inj, res, w, 1e-6)
+    p = 2 / (1 + np.exp(-inj.astype(np.float64) * 0.25))
+    r64 = res + b[:, None, :] * p[:, :, None]
+    xn64 = r64 / np.sqrt((r64 * r64).mean(-1, keepdims=True) + 1e-6) * w
+    assert np.abs(r['res'] - r64).max() <= 1e-6 * np.abs(r64).max() and np.abs(r['xn'] - xn64).max() <= 2e-6 * np.abs(xn64).max()
+    assert np.array_equal(r['res'][2], res[2] + b[2][None, :])                 # p = 1 exactly: one exact fma per element
+    assert np.array_equal(r['xnbf'], O.f2bf(r['xn'])) and np.array_equal(O.hc_post(b, inj, res), r['res'])
+    again = O.rms_mul(r['res'].reshape(T * HC, N), w, 1e-6)
+    assert np.array_equal(again['y'], r['xn'].reshape(T * HC, N)) and np.array_equal(again['scale'], r['scale'])
+    g = rng.standard_normal((T, HC, N)).astype(f32)
+    m = O.hc_mean(r['xn'], g)
+    m64 = 0.25 * (r['xn'].astype(np.float64) / (1 + np.exp(-g.astype(np.float64)))).sum(1)
+    assert np.abs(m - m64).max() <= 1e-6 * np.abs(m64).max()
+    assert np.array_equal(O.hc_mean(r['res'], g, scale=r['scale'], w=w), m)
+    one = O.hc_mean(np.ones((1, 1, 8), f32), np.zeros((1, 1, 8), f32), rs=1.0)      # sigmoid(0) = 0.5 exactly
+    assert np.array_equal(one, np.full((1, 8), 0.5, f32))
