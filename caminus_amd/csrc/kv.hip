@@ -59,6 +59,41 @@ __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restric
     }
 }
 
+// The reader: cache rows back to K / V values, value = (float)code * (float)half scale (one fp32 multiply, exact in the
+// sense of the attention kernels' own decode: q3p_q8_stage, kernels/q3m_prefill.hip:617-632; host reference decode_q8_kv,
+// python/caminus/ref_kv.py:127-144); F16: rounded to fp16 (the prefill staging's operand format). One workgroup per row,
+// 8 lanes x 4 codes per block as in the writer; outputs leave as 16-byte (fp32) or 8-byte (fp16) stores per lane.
+template <bool F16>
+__global__ void __launch_bounds__(256) kv_q8_read_rows(const uint8_t * __restrict__ cache, const int32_t * __restrict__ row_ids, int pos0, int rows, int M,
+                                                       void * __restrict__ k, int ldk, void * __restrict__ v, int ldv, int * __restrict__ err) {
+    if (M < 32 || M % 32 || ldk < M || ldv < M || rows < 1) {
+        if (threadIdx.x == 0) atomicOr(err, 4);
+        return;
+    }
+    const size_t tt = blockIdx.x;
+    const long pos = row_ids ? (long)row_ids[tt] : (long)pos0 + (long)blockIdx.x;
+    if (pos < 0 || pos >= rows) {
+        if (threadIdx.x == 0) atomicOr(err, 1);
+        return;
+    }
+    const int nb = M / 32, lane = threadIdx.x & 63, sub = lane & 7;
+    const uint8_t * src = cache + (size_t)pos * ((size_t)2 * nb * 34);
+    for (int b0 = (threadIdx.x >> 6) * 8; b0 < 2 * nb; b0 += 32) {
+        const int b = b0 + (lane >> 3);
+        if (b >= 2 * nb) continue;
+        const uint8_t * blk = src + (size_t)b * 34;
+        const float d = h2f_bits(*(const uint16_t *)blk);
+        const uint16_t * c = (const uint16_t *)(blk + 2 + 4 * sub);
+        const uint32_t w = (uint32_t)c[0] | ((uint32_t)c[1] << 16);
+        f32x4 y;
+        y.x = (float)(int8_t)(w & 0xff) * d; y.y = (float)(int8_t)((w >> 8) & 0xff) * d;
+        y.z = (float)(int8_t)((w >> 16) & 0xff) * d; y.w = (float)(int8_t)(w >> 24) * d;
+        const size_t o = (b < nb ? tt * ldk : tt * ldv) + (size_t)(b % nb) * 32 + 4 * sub;
+        if (F16) *(u32x2 *)((uint16_t *)(b < nb ? k : v) + o) = pack_f16x4(y);
+        else *(f32x4_a4 *)((float *)(b < nb ? k : v) + o) = y;
+    }
+}
+
 // in-place orthonormal WHT of C chunks of n values, n in {64, 128, 256}: n / 4 lanes per chunk
 template <int N>
 __global__ void __launch_bounds__(256) hadamard_chunks(float * __restrict__ x, long C) {
@@ -109,6 +144,18 @@ int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, in
     CAMX_LAUNCH_RET();
 }
 
+// The Q8 KV reader (no kernel of its own in the reference: the decode is inlined in its attention kernels). Row t = row_ids ?
+// row_ids[t] : pos0 + t; k, v [T][ld] fp32 (f16 = 0) or fp16 bits (f16 = 1). err bits: 1 a row outside [0, rows) (its outputs
+// stay untouched), 4 layout.
+int camx_own_kv_q8_read(const uint8_t * cache, const int32_t * row_ids, int pos0, int rows, int M, void * k, int ldk, void * v, int ldv,
+                        int * err, int T, int f16, hipStream_t st) {
+    if (!cache || !k || !v || !err || T < 0 || ((uintptr_t)cache & 1) || ((uintptr_t)k & (f16 ? 7 : 3)) || ((uintptr_t)v & (f16 ? 7 : 3)) ||
+        (f16 && ((ldk | ldv) & 3))) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    if (f16) kv_q8_read_rows<true><<<dim3(T), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, err);
+    else kv_q8_read_rows<false><<<dim3(T), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, err);
+    CAMX_LAUNCH_RET();
+}
 int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
                       int T, hipStream_t st) {
     if (!k || !v || !cache || !err || T < 0 || M < 32 || M % 32 || ldk < M || ldv < M || ((uintptr_t)cache & 1)) return CAMX_EINVAL;

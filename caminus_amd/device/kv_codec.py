@@ -62,6 +62,7 @@ class Q8KVCodec:
     def __init__(self, device, module=None):
         self.dev = _explicit_cuda_device(device)
         self.module = module
+        self.reader = module             # read() binds the library's own entry point lazily (a recorder serves both)
 
     def append(self, k, ldk, v, ldv, M, cache, pos0, T, err, rows=None):
         """Queue the encode of rows pos0 .. pos0 + T - 1 from k[t * ldk : t * ldk + M] and v[t * ldv : t * ldv + M].
@@ -94,6 +95,39 @@ class Q8KVCodec:
             if self.module is None:
                 self.module = Module('kv_codec')
             self.module.own_kv_q8_append((T,), (256,), k, c_int(ldk), v, c_int(ldv), c_int(M), cache, c_int(pos0), c_int(rows), err)
+
+    def read(self, cache, M, k, ldk, v, ldv, pos0, T, err, rows=None, row_ids=None):
+        """Queue the decode of rows pos0 .. pos0 + T - 1 (or rows row_ids[0 .. T - 1], int32 on this device) into k / v: fp32, or
+        fp16 (rounded from the fp32 value) when k is float16. The reference launcher has no decoder (its attention kernels
+        decode blocks in place); the checks and the error word follow append()."""
+        M = _integer(M, 'M', _BLOCK_VALUES)
+        if M % _BLOCK_VALUES:
+            raise ValueError('kv_codec: M must be divisible by 32')
+        T = _integer(T, 'T', 1)
+        ldk, ldv = _integer(ldk, 'ldk', M), _integer(ldv, 'ldv', M)
+        pos0 = _integer(pos0, 'pos0')
+        row_bytes = 2 * (M // _BLOCK_VALUES) * _BLOCK_BYTES
+        rows = _cache_rows(cache, row_bytes, rows)
+        if row_ids is None:
+            from ..engine.k3 import check_span
+            check_span(pos0, T, rows, what='own Q8 KV read')
+        if not isinstance(k, torch.Tensor) or k.dtype not in (torch.float32, torch.float16):
+            raise ValueError('kv_codec: k must be float32 or float16')
+        operands = {
+            'cache': (cache, torch.uint8, rows * row_bytes, 2),
+            'k': (k, k.dtype, (T - 1) * ldk + M, 8 if k.dtype == torch.float16 else 4),
+            'v': (v, k.dtype, (T - 1) * ldv + M, 8 if k.dtype == torch.float16 else 4),
+            'err': (err, torch.int32, 1),
+        }
+        if row_ids is not None:
+            operands['row_ids'] = (row_ids, torch.int32, T)
+        _check(self.dev, 'own_kv_q8_read', operands, ('k', 'v', 'err'))
+        c_int = ctypes.c_int
+        with torch.cuda.device(self.dev):
+            if self.reader is None:
+                self.reader = Module('camx')
+            self.reader.camx_own_kv_q8_read((T,), (256,), cache, row_ids if row_ids is not None else ctypes.c_void_p(None), c_int(pos0), c_int(rows),
+                                            c_int(M), k, c_int(ldk), v, c_int(ldv), err, c_int(T), c_int(int(k.dtype == torch.float16)))
 
     def check(self, err):
         """Synchronize the device, read the word, raise RuntimeError if any bit is set. The word is left as it is."""

@@ -142,6 +142,13 @@ int camx_rope_freqs(float theta_scale, int n, float * out, camx_stream_t stream)
  * err bits: 1 position outside [0, rows), 2 refused block (bytes untouched), 4 layout (M < 32, M % 32, ld < M, rows < 1). */
 int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows,
                           int * err, int T, camx_stream_t stream);
+/* The reader of those rows. The reference has no kernel of its own for it: its attention kernels decode blocks in place
+ * (q3p_q8_stage, kernels/q3m_prefill.hip:617-632; host reference decode_q8_kv, python/caminus/ref_kv.py:127-144). Row t =
+ * row_ids ? row_ids[t] : pos0 + t; value = (float)code * (float)half scale; k, v [T][ld] fp32 (f16 = 0) or fp16 bits rounded
+ * from that value (f16 = 1, the prefill staging's operand format). err bits: 1 a row outside [0, rows) (outputs untouched), 4
+ * layout. */
+int camx_own_kv_q8_read(const uint8_t * cache, const int32_t * row_ids, int pos0, int rows, int M, void * k, int ldk, void * v, int ldv,
+                        int * err, int T, int f16, camx_stream_t stream);
 /* pf_kv_append, q8_0 rows (kernels/prefill_attn.hip:157-181) = OP_KV_APPEND work 1 (kernels/k3_gguf_ops.h:1532-1553):
  * no refusal rules; err bit 1 for a row outside [0, rows). */
 int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,

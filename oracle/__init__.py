@@ -312,6 +312,19 @@ def kv_q8_append(k, ldk, v, ldv, M, cache, pos0, T, rows=None):
     return cache, int(err[0])
 
 
+def kv_q8_read(cache, M, T, pos0=0, row_ids=None, rows=None, f16=False, fill=None):
+    """-> (k, v, err): [T, M] float32, or fp16 bits (uint16) when f16; rows outside [0, rows) keep `fill`"""
+    cache = _c(cache, np.uint8).reshape(-1); rb = 2 * (M // 32) * 34
+    rows = cache.size // rb if rows is None else rows
+    dt = np.uint16 if f16 else np.float32
+    k = np.zeros((T, M), dt); v = np.zeros((T, M), dt)
+    if fill is not None: k[:] = fill; v[:] = fill
+    err = np.zeros(1, np.int32)
+    ids = _c(row_ids, np.int32) if row_ids is not None else None
+    lib().orc_kv_q8_read(_p(cache), _p(ids), I(pos0), I(rows), I(M), _p(k), I(M), _p(v), I(M), I(T), I(int(f16)), _p(err))
+    return k, v, int(err[0])
+
+
 def pf_kv_append(k, ldk, v, ldv, M, cache, pos0, T, rows=None):
     k = _c(k, np.float32); v = _c(v, np.float32); cache = _c(cache, np.uint8).copy()
     rb = 2 * (M // 32) * 34

@@ -492,6 +492,31 @@ ORC_API void orc_kv_q8_append(const float * k, int ldk, const float * v, int ldv
         }
     }
 }
+/* The Q8 KV reader: the decode of a wire block as the attention kernels do it (q3p_q8_stage, kernels/q3m_prefill.hip:617-632;
+ * host reference decode_q8_kv, python/caminus/ref_kv.py:127-144): value = (float)code * (float)half scale, one fp32
+ * multiply; f16: that value rounded to fp16 (the prefill staging). Row t = row_ids ? row_ids[t] : pos0 + t; a row outside
+ * [0, rows) sets err bit 1 and leaves its outputs untouched. k, v: [T][ld] fp32 or fp16 bits. */
+ORC_API void orc_kv_q8_read(const uint8_t * cache, const int32_t * row_ids, int pos0, int rows, int M, void * k, int ldk, void * v,
+                            int ldv, int T, int f16, int32_t * err) {
+    if (M < 32 || M % 32 || ldk < M || ldv < M || rows < 1) { *err |= 4; return; }
+    const int nb = M / 32;
+    const size_t rb = (size_t)2 * nb * 34;
+    for (int t = 0; t < T; t++) {
+        const int64_t pos = row_ids ? (int64_t)row_ids[t] : (int64_t)pos0 + t;
+        if (pos < 0 || pos >= rows) { *err |= 1; continue; }
+        const uint8_t * src = cache + (size_t)pos * rb;
+        for (int b = 0; b < 2 * nb; b++) {
+            const uint8_t * blk = src + (size_t)b * 34;
+            uint16_t hd; memcpy(&hd, blk, 2);
+            const float d = orc_h2f(hd);
+            const size_t o = (b < nb ? (size_t)t * ldk : (size_t)t * ldv) + (size_t)(b % nb) * 32;
+            for (int j = 0; j < 32; j++) {
+                const float val = (float)(int8_t)blk[2 + j] * d;
+                if (f16) ((uint16_t *)(b < nb ? k : v))[o + j] = orc_f2h(val); else ((float *)(b < nb ? k : v))[o + j] = val;
+            }
+        }
+    }
+}
 /* pf_kv_append, q8_0 rows (kernels/prefill_attn.hip:157-181): no refusal rules; d stored as half, code by x * (1 / d) */
 ORC_API void orc_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0,
                               int rows, int T, int32_t * err) {

@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 import oracle as O
-from gpu_util import I, L64, bits_equal, call, dev, host, ptr
+from gpu_util import I, L64, NULL, bits_equal, call, dev, host, ptr
 from vectors import kv_invalid_blocks, kv_valid_blocks
 
 pytestmark = pytest.mark.gpu
@@ -89,3 +89,35 @@ def test_hadamard128():
     y = dev(np.zeros_like(xs))
     call('camx_hadamard128', ptr(dev(xs)), ptr(y), L64(len(xs)))
     assert bits_equal(host(y), O.hadamard128(xs))
+
+
+@pytest.mark.parametrize('M,T,f16', [(512, 300, False), (512, 300, True), (64, 5, False), (1024, 17, True)])
+def test_kv_q8_read_round_trip(M, T, f16):
+    """the reader: bit-exact against the oracle and the independent numpy decoder; encode -> decode stays within half a
+    quantization step of the input (any size); rows addressed by id; a row outside the cache raises bit 1 and is left alone"""
+    from oracle import np_kv
+    rng = np.random.default_rng(M + T)
+    k = (rng.standard_normal((T, M)) * np.exp2(rng.integers(-8, 8, (T, 1)))).astype(np.float32); v = rng.standard_normal((T, M)).astype(np.float32)
+    rb = 2 * (M // 32) * 34
+    cache, werr = O.kv_q8_append(k, M, v, M, M, np.zeros(T * rb, np.uint8), 0, T)
+    assert werr == 0
+    rk, rv, _ = O.kv_q8_read(cache, M, T, f16=f16)
+    nk, nv = np_kv.decode_q8_kv(cache.reshape(T, rb), np_kv.Q8KVLayout(M // 32, 32))
+    if not f16:
+        assert bits_equal(rk, nk.reshape(T, M)) and bits_equal(rv, nv.reshape(T, M))
+    else:
+        assert bits_equal(rk, nk.reshape(T, M).astype(np.float16).view(np.uint16)) and bits_equal(rv, nv.reshape(T, M).astype(np.float16).view(np.uint16))
+    dt = np.uint16 if f16 else np.float32
+    cd = dev(cache); kd = dev(np.zeros((T, M + 8), dt)); vd = dev(np.zeros((T, M + 4), dt)); err = dev(np.zeros(1, np.int32))
+    call('camx_own_kv_q8_read', ptr(cd), NULL, I(0), I(T), I(M), ptr(kd), I(M + 8), ptr(vd), I(M + 4), ptr(err), I(T), I(int(f16)))
+    gk, gv = host(kd, dt), host(vd, dt)
+    assert int(host(err)[0]) == 0 and bits_equal(gk[:, :M], rk) and bits_equal(gv[:, :M], rv) and not gk[:, M:].any() and not gv[:, M:].any()
+    if not f16:
+        step = np.repeat(np.abs(k.reshape(T, -1, 32)).max(-1) / 127, 32, axis=1)
+        assert (np.abs(gk[:, :M] - k) <= 0.5 * step * (1 + 2.0 ** -9) + np.abs(k) * 2.0 ** -10).all()
+    ids = rng.permutation(T)[:max(T // 2, 2)].astype(np.int32); ids[1] = T + 3
+    k2 = dev(np.full((len(ids), M), 7, dt)); v2 = dev(np.full((len(ids), M), 7, dt)); err2 = dev(np.zeros(1, np.int32))
+    call('camx_own_kv_q8_read', ptr(cd), ptr(dev(ids)), I(0), I(T), I(M), ptr(k2), I(M), ptr(v2), I(M), ptr(err2), I(len(ids)), I(int(f16)))
+    ok, ov, oerr = O.kv_q8_read(cache, M, len(ids), row_ids=ids, f16=f16, fill=7)
+    assert int(host(err2)[0]) == oerr == 1 and bits_equal(host(k2, dt), ok) and bits_equal(host(v2, dt), ov)
+    assert (host(k2, dt)[1] == 7).all()

@@ -514,3 +514,23 @@ def test_hc_glue_against_float64():
     assert np.array_equal(O.hc_mean(r['res'], g, scale=r['scale'], w=w), m)
     one = O.hc_mean(np.ones((1, 1, 8), f32), np.zeros((1, 1, 8), f32), rs=1.0)      # sigmoid(0) = 0.5 exactly
     assert np.array_equal(one, np.full((1, 8), 0.5, f32))
+
+
+def test_kv_q8_reader_against_numpy_decoder_and_literals():
+    """the reader's decode (code x half scale in fp32) against the independent numpy decoder on encoder output, on literal
+    blocks with negative scales and the -128 code (which the encoder never writes but a reader must decode), and the error bits"""
+    rng = np.random.default_rng(9)
+    M, T = 256, 11
+    k = (rng.standard_normal((T, M)) * 3).astype(f32); v = rng.standard_normal((T, M)).astype(f32)
+    rb = 2 * (M // 32) * 34
+    cache, err = O.kv_q8_append(k, M, v, M, M, np.zeros(T * rb, np.uint8), 0, T)
+    rk, rv, rerr = O.kv_q8_read(cache, M, T)
+    nk, nv = ref_kv.decode_q8_kv(cache.reshape(T, rb), ref_kv.Q8KVLayout(2, 128))
+    assert err == rerr == 0 and np.array_equal(rk, nk.reshape(T, M)) and np.array_equal(rv, nv.reshape(T, M))
+    blk = np.zeros((1, 2 * 34), np.uint8)
+    blk[0, :2] = np.array([-0.5], '<f2').view(np.uint8); blk[0, 2:6] = np.array([-128, 127, 1, 0], np.int8).view(np.uint8)
+    lk, lv, _ = O.kv_q8_read(blk, 32, 1)
+    assert lk[0, :4].tolist() == [64.0, -63.5, -0.5, -0.0] and not lv.any()
+    hk, _, _ = O.kv_q8_read(blk, 32, 1, f16=True)
+    assert np.array_equal(hk, lk.astype(np.float16).view(np.uint16))
+    assert O.kv_q8_read(cache, M, 2, pos0=T - 1)[2] == 1 and O.kv_q8_read(cache, 48, 1)[2] == 4
