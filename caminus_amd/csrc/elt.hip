@@ -511,6 +511,23 @@ int camx_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out
     copy_cols_bf16_k<<<GRID_1D(rows * n), dim3(256), 0, st>>>(in, ld_in, c_in, out, ld_out, c_out, n, rows);
     CAMX_LAUNCH_RET();
 }
+// residual_slices_bwd (kernels/fuse.hip:35-47): dm = dmlp = bf16(dout) (f2bf), dys[pos[r]] = bf16(dout[r]) for the routed rows
+__global__ void __launch_bounds__(256) residual_slices_bwd_k(const float * __restrict__ dout, const int * __restrict__ pos, uint16_t * __restrict__ dm,
+                                                             uint16_t * __restrict__ dmlp, uint16_t * __restrict__ dys, int d, long n4) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const long e = i * 4; const int r = (int)(e / d), c = (int)(e % d);
+    const u32x2 b = pack_f2bf_x4(__builtin_nontemporal_load((const f32x4 *)(dout + e)));
+    *(u32x2 *)(dm + e) = b; *(u32x2 *)(dmlp + e) = b;
+    const int p = pos ? pos[r] : -1;
+    if (p >= 0) *(u32x2 *)(dys + (size_t)p * d + c) = b;
+}
+int camx_residual_slices_bwd(const float * dout, const int * pos, uint16_t * dm, uint16_t * dmlp, uint16_t * dys, int d, long n4, hipStream_t st) {
+    if (!dout || !dm || !dmlp || d < 4 || d % 4 || n4 < 0 || (pos && !dys) || (((uintptr_t)dout) & 15) || (((uintptr_t)dm | (uintptr_t)dmlp | (uintptr_t)dys) & 7)) return CAMX_EINVAL;
+    if (n4 == 0) return CAMX_OK;
+    residual_slices_bwd_k<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st>>>(dout, pos, dm, dmlp, dys, d, n4);
+    CAMX_LAUNCH_RET();
+}
 int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t * mlp, const uint16_t * ys, const int * pos, float * out,
                              int d, long n4, hipStream_t st) {
     if (!x || !m || !mlp || !out || d < 4 || d % 4 || n4 < 0 || ((uintptr_t)x & 15) || ((uintptr_t)out & 15) || ((uintptr_t)m & 7) ||

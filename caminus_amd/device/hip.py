@@ -112,7 +112,8 @@ _CORE = {
     'cast_bf16': ('camx_cast_bf16', lambda g, b, v: [v[0], v[1], L64(_val(v[2]))]),
     'copy_cols_bf16': ('camx_copy_cols_bf16', lambda g, b, v: list(v[:7]) + [L64(_val(v[7]))]),
 }
-_FUSE = {'residual_slices_fwd': ('camx_residual_slices_fwd', lambda g, b, v: list(v[:7]) + [L64(_val(v[7]))])}
+_FUSE = {'residual_slices_fwd': ('camx_residual_slices_fwd', lambda g, b, v: list(v[:7]) + [L64(_val(v[7]))]),
+         'residual_slices_bwd': ('camx_residual_slices_bwd', lambda g, b, v: list(v[:6]) + [L64(_val(v[6]))])}
 _ACTQ = {
     'actq_fwd_f32': _actq(False, False), 'actq_fwd_bf16': _actq(True, False),
     'actq_fwd_codes_f32': _actq(False, True), 'actq_fwd_codes_bf16': _actq(True, True),

@@ -1,7 +1,7 @@
 """Residual sum fused with the scatter of routed rows: out = ((x + m) + mlp) + ys[pos] in one pass over the rows.
 
 Offers the reference's entry point residual_slices(x, m, mlp, ys, pos) (python/caminus/train/fuse.py:16-45) on top of this
-library's residual_slices_fwd. Only the forward kernel exists here; asking autograd for a gradient raises.
+library's residual_slices_fwd / residual_slices_bwd. Backward: dx = dout, dm = dmlp = bf16(dout), dys[pos[r]] = bf16(dout[r]).
 
   x    fp32  [..., d]      residual stream
   m    bf16  [..., d]      first addend (mixer output)
@@ -42,14 +42,34 @@ def _launch_forward(x, m, mlp, ys, pos):
     return out
 
 
+def _launch_backward(dout, pos, nys):
+    dout = dout.contiguous()
+    d = dout.shape[-1]
+    quads = dout.numel() // 4
+    dm = torch.empty(dout.shape, device=dout.device, dtype=torch.bfloat16)
+    dmlp = torch.empty_like(dm)
+    routed = pos is not None
+    dys = torch.empty(nys, d, device=dout.device, dtype=torch.bfloat16) if routed else None      # every row of ys is named by one pos
+    null = ctypes.c_void_p(None)
+    grid = (quads + _BLOCK - 1) // _BLOCK
+    _module().residual_slices_bwd((grid,), (_BLOCK,), dout, pos if routed else null, dm, dmlp, dys if routed else null,
+                                  ctypes.c_int(d), ctypes.c_long(quads))
+    return dout, dm, dmlp, dys
+
+
 class ResidualSlices(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, m, mlp, ys, pos):
+        routed = ys is not None and ys.numel() > 0
+        ctx.save_for_backward(pos if routed else None)
+        ctx.nys = ys.shape[0] if routed else 0
         return _launch_forward(x, m, mlp, ys, pos)
 
     @staticmethod
     def backward(ctx, dout):
-        raise NotImplementedError('residual_slices: the backward kernel is outside this library (forward only)')
+        (pos,) = ctx.saved_tensors
+        dx, dm, dmlp, dys = _launch_backward(dout, pos, ctx.nys)
+        return dx, dm, dmlp, dys, None
 
 
 def residual_slices(x, m, mlp, ys, pos):

@@ -195,6 +195,11 @@ int camx_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out
 int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t * mlp, const uint16_t * ys, const int * pos,
                              float * out, int d, long n4, camx_stream_t stream);
 
+/* residual_slices_bwd (kernels/fuse.hip:35-47): dm = dmlp = bf16(dout); dys[pos[r]] = bf16(dout[r]) where pos[r] >= 0 (dx = dout is
+ * the caller's). pos / dys may be NULL. */
+int camx_residual_slices_bwd(const float * dout, const int * pos, uint16_t * dm, uint16_t * dmlp, uint16_t * dys, int d, long n4,
+                             camx_stream_t stream);
+
 /* ---- activation fake-quant, forward (kernels/actq.hip) ------------------------------------------------------------------------------ */
 /* actq_fwd_{f32,bf16} and actq_fwd_codes_{f32,bf16} (kernels/actq.hip:96-132, 315-326): M rows of K values (K % 128 == 0,
  * K <= 8192); y bf16 [M][K] (optional when codes are written), s [M] (optional), codes [M][K / 2] bytes (optional). */

@@ -203,6 +203,14 @@ def copy_cols_bf16(inp, c_in, out, c_out, n):
     lib().orc_copy_cols_bf16(_p(inp), I(inp.shape[1]), I(c_in), _p(out), I(out.shape[1]), I(c_out), I(n), L64(inp.shape[0])); return out
 
 
+def residual_slices_bwd(dout, pos, nys):
+    """-> (dm, dmlp, dys) bf16 bits; dys [nys, d] rows that no pos names stay 0"""
+    dout = _c(dout, np.float32); d = dout.shape[-1]
+    dm = np.empty(dout.shape, np.uint16); dmlp = np.empty(dout.shape, np.uint16); dys = np.zeros((nys, d), np.uint16)
+    lib().orc_residual_slices_bwd(_p(dout), _p(_c(pos, np.int32)) if pos is not None else _p(None), _p(dm), _p(dmlp), _p(dys), I(d), L64(dout.size))
+    return dm, dmlp, dys
+
+
 def residual_slices_fwd(x, m, mlp, ys, pos):
     x = _c(x, np.float32); d = x.shape[-1]; out = np.empty_like(x)
     ys = _c(ys, np.uint16) if ys is not None else None

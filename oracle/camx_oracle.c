@@ -355,6 +355,15 @@ ORC_API void orc_cast_bf16(const float * x, uint16_t * out, int64_t n) { for (in
 ORC_API void orc_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out, int ld_out, int c_out, int n, int64_t rows) {
     for (int64_t r = 0; r < rows; r++) for (int c = 0; c < n; c++) out[r * ld_out + c_out + c] = in[r * ld_in + c_in + c];
 }
+/* residual_slices_bwd (kernels/fuse.hip:35-47) */
+ORC_API void orc_residual_slices_bwd(const float * dout, const int32_t * pos, uint16_t * dm, uint16_t * dmlp, uint16_t * dys, int d, int64_t n) {
+    for (int64_t e = 0; e < n; e++) {
+        const uint16_t b = orc_f2bf(dout[e]);
+        dm[e] = b; dmlp[e] = b;
+        const int p = pos ? pos[e / d] : -1;
+        if (p >= 0) dys[(size_t)p * d + e % d] = b;
+    }
+}
 /* residual_slices_fwd (kernels/fuse.hip:19-33) */
 ORC_API void orc_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t * mlp, const uint16_t * ys,
                                      const int32_t * pos, float * out, int d, int64_t n4) {

@@ -94,3 +94,29 @@ def test_core_and_fuse():
         call('camx_residual_slices_fwd', ptr(dev(x2)), ptr(dev(m)), ptr(dev(y)), ptr(dev(ys)) if has else NULL, ptr(dev(pos)) if has else NULL,
              ptr(o2), I(D), L64(T * D // 4))
         assert bits_equal(host(o2), O.residual_slices_fwd(x2, m, y, ys if has else None, pos if has else None))
+
+
+def test_residual_slices_bwd_and_autograd():
+    """the backward kernel against the oracle, and the autograd wrapper end to end against torch's own graph of the same sum"""
+    import torch
+    from caminus_amd.train.fuse import residual_slices
+    rng = np.random.default_rng(6)
+    T, D, nys = 11, 896, 5
+    dout = outliers(rng, (T, D)); dout[0, :3] = [np.nan, np.inf, 3.3895314e38]
+    pos = np.array([-1, 0, 3, -1, 2, 1, -1, -1, 4, -1, -1], np.int32)
+    rdm, rdmlp, rdys = O.residual_slices_bwd(dout, pos, nys)
+    dm = dev(np.zeros((T, D), np.uint16)); dmlp = dev(np.zeros((T, D), np.uint16)); dys = dev(np.zeros((nys, D), np.uint16))
+    call('camx_residual_slices_bwd', ptr(dev(dout)), ptr(dev(pos)), ptr(dm), ptr(dmlp), ptr(dys), I(D), L64(T * D // 4))
+    assert bits_equal(host(dm, np.uint16), rdm) and bits_equal(host(dmlp, np.uint16), rdmlp) and bits_equal(host(dys, np.uint16), rdys)
+    x = torch.randn(T, D, device='cuda:0', requires_grad=True)
+    m = torch.randn(T, D, device='cuda:0').bfloat16().requires_grad_(); mlp = torch.randn(T, D, device='cuda:0').bfloat16().requires_grad_()
+    ys = torch.randn(nys, D, device='cuda:0').bfloat16().requires_grad_(); pd = torch.from_numpy(pos).to('cuda:0')
+    out = residual_slices(x, m, mlp, ys, pd)
+    gsel = torch.zeros(T, D, device='cuda:0'); sel = pd >= 0
+    gsel[sel] = ys.detach().float()[pd[sel].long()]
+    want = ((x.detach() + m.detach().float()) + mlp.detach().float()) + gsel
+    assert torch.equal(out.detach(), want)
+    go = torch.randn(T, D, device='cuda:0')
+    out.backward(go)
+    assert torch.equal(x.grad, go) and torch.equal(m.grad, go.bfloat16()) and torch.equal(mlp.grad, go.bfloat16())
+    assert torch.equal(ys.grad[pd[sel].long()], go[sel].bfloat16())
