@@ -1,14 +1,18 @@
-// Fused activation fake-quant (forward) for gfx950: per row of K values (K % 128 == 0, K <= 8192) a 128-point Hadamard
-// rotation per chunk in bf16 steps, one int4-style scale per row, codes packed two per byte. Replaces actq_fwd_{f32,bf16},
-// actq_fwd_codes_{f32,bf16}, silu_mul_actq_fwd and block_entry_fwd (kernels/actq.hip:40-53, 96-132, 247-274, 305-326).
+// Fused activation fake-quant for gfx950, forward and backward: per row of K values (K % 128 == 0, K <= 8192) a 128-point
+// Hadamard rotation per chunk in bf16 steps, one int4-style scale per row, codes packed two per byte. Replaces actq_fwd_{f32,bf16},
+// actq_fwd_codes_{f32,bf16}, actq_bwd_{f32,bf16}, silu_mul_actq_{fwd,bwd} and block_entry_{fwd,bwd} (kernels/actq.hip:40-53,
+// 96-218, 247-333).
 //
 // One 256-thread workgroup per row. A half-wave (32 lanes) transforms one 128-chunk: lane l holds elements 4l .. 4l + 3,
-// butterfly stages 1-2 in registers, 4 .. 64 across lanes; a workgroup keeps 8 chunks in flight and up to 8 rounds of
-// them in registers across the row-wide amax.
+// butterfly stages 1-2 in registers, 4 .. 64 across lanes; half-wave h takes chunks h, h + 8, ... (the reference's wave h of
+// 32), NR = ceil(K / 1024) rounds of them stay in registers across the row-wide reductions. Kernels are instantiated per
+// NR, so a row of 2048 values runs two rounds and not the eight the limit allows.
+//
+// Sums of the backward pass (dL/ds, the tie count, the RMSNorm dot) follow one fixed tree: a lane adds its terms in chunk
+// order with fmaf, the 32 lanes of a half-wave combine by xor 16, 8, 4, 2, 1, the eight half-wave sums are added in order.
 #include "common.cuh"
 
 #define HSCALE 0.08837890625f      // bf16(1 / sqrt(128))
-#define MAXR 8                     // rounds of 8 chunks: K <= 8 * 8 * 128
 
 struct PlainF32 { const float * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); } };
 struct PlainBF16 { const uint16_t * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); } };
@@ -32,41 +36,59 @@ struct RmsSrc {
     }
 };
 
-template <typename Src>
-CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * __restrict__ s_out, int K, float clip, int qmax,
-                           uint16_t * __restrict__ codes, float * lds) {
-    const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
-    f32x4 u[MAXR];
+#define CAMX_EACH4(OP) OP(x) OP(y) OP(z) OP(w)
+
+CAMX_DEV f32x4 rbf4(f32x4 v) { v.x = rbf(v.x); v.y = rbf(v.y); v.z = rbf(v.z); v.w = rbf(v.w); return v; }
+CAMX_DEV f32x4 rbf4_scaled(f32x4 v) { v.x = rbf(v.x * HSCALE); v.y = rbf(v.y * HSCALE); v.z = rbf(v.z * HSCALE); v.w = rbf(v.w * HSCALE); return v; }
+
+// u = bf16(H128 . bf16(source)) for the NR rounds of this half-wave; returns the lane's max |u| over its active chunks
+template <int NR, typename Src>
+CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[NR]) {
+#pragma unroll
+    for (int c = 0; c < NR; c++) {
+        const int ch = hw + 8 * c;
+        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (ch < nch) v = src(row, ch * 128 + 4 * l);
+        u[c] = v;
+    }
     float amax = 0.0f;
 #pragma unroll
-    for (int c = 0; c < MAXR; c++) {
-        const int ch = hw + 8 * c;
-        const bool on = ch < nch;
-        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (on) v = src(row, ch * 128 + 4 * l);
-        v.x = rbf(v.x); v.y = rbf(v.y); v.z = rbf(v.z); v.w = rbf(v.w);        // autocast's bf16 input
-        v = hadamard128_l4(v, l, false);
-        v.x = rbf(v.x * HSCALE); v.y = rbf(v.y * HSCALE); v.z = rbf(v.z * HSCALE); v.w = rbf(v.w * HSCALE);
+    for (int c = 0; c < NR; c++) {
+        const f32x4 v = rbf4_scaled(hadamard128_l4(rbf4(u[c]), l, false));      // rbf4: autocast's bf16 input
         u[c] = v;
-        if (on) amax = fmaxf(amax, absmax4(v));
+        if (hw + 8 * c < nch) amax = fmaxf(amax, absmax4(v));
     }
-    // row-wide max (order-free)
+    return amax;
+}
+
+// row-wide max (order-free); lds: 4 floats
+CAMX_DEV float row_max(float amax, float * lds) {
+    const int tid = threadIdx.x;
 #pragma unroll
     for (int m = 32; m > 0; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
     __syncthreads();
     if ((tid & 63) == 0) lds[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
+    return fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
+}
+
+template <int NR, typename Src>
+CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * __restrict__ s_out, int K, float clip, int qmax,
+                           uint16_t * __restrict__ codes, float * lds) {
+    const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
+    f32x4 u[NR];
+    const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u), lds);
     const float s = fmaxf(amax * clip / (float)qmax, 1e-8f);
     if (tid == 0 && s_out) s_out[row] = s;
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
 #pragma unroll
-    for (int c = 0; c < MAXR; c++) {
+    for (int c = 0; c < NR; c++) {
         const int ch = hw + 8 * c;
         if (ch < nch) {
             f32x4 q;
-            q.x = fminf(fmaxf(rintf(u[c].x / s), lo), hi); q.y = fminf(fmaxf(rintf(u[c].y / s), lo), hi);
-            q.z = fminf(fmaxf(rintf(u[c].z / s), lo), hi); q.w = fminf(fmaxf(rintf(u[c].w / s), lo), hi);
+#define Q_(e) q.e = fminf(fmaxf(rintf(u[c].e / s), lo), hi);
+            CAMX_EACH4(Q_)
+#undef Q_
             if (y) { f32x4 d; d.x = q.x * s; d.y = q.y * s; d.z = q.z * s; d.w = q.w * s; *(u32x2 *)(y + (size_t)row * K + ch * 128 + 4 * l) = pack_f2bf_x4(d); }
             if (codes) {
                 const uint32_t pk = ((uint32_t)(int)q.x & 0xfu) | (((uint32_t)(int)q.y & 0xfu) << 4) | (((uint32_t)(int)q.z & 0xfu) << 8) | (((uint32_t)(int)q.w & 0xfu) << 12);
@@ -76,12 +98,102 @@ CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * 
     }
 }
 
-template <typename Src>
+template <int NR, typename Src>
 __global__ void __launch_bounds__(256) actq_fwd_k(Src src, uint16_t * y, float * s, uint16_t * codes, int K, float clip, int qmax) {
     __shared__ float lds[4];
-    actq_fwd_row(src, blockIdx.x, y, s, K, clip, qmax, codes, lds);
+    actq_fwd_row<NR>(src, blockIdx.x, y, s, K, clip, qmax, codes, lds);
 }
 
+// ---- backward ----------------------------------------------------------------------------------------------------------------
+// sum over the 32 lanes of a half-wave by xor 16, 8, 4, 2, 1 (slot space), then the eight half-wave sums in order
+CAMX_DEV float half32_sum(float v) {
+    v += lane_xor16(v); v += lane_xor8(v); v += lane_xor4(v); v += lane_xor2(v); v += lane_xor1(v);
+    return v;
+}
+CAMX_DEV void block8_sum2(float & a, float & b, float * lds16) {
+    const int tid = threadIdx.x;
+    a = half32_sum(a); b = half32_sum(b);
+    __syncthreads();
+    if ((tid & 31) == 0) { lds16[tid >> 5] = a; lds16[8 + (tid >> 5)] = b; }
+    __syncthreads();
+    a = lds16[0]; b = lds16[8];
+#pragma unroll
+    for (int w = 1; w < 8; w++) { a += lds16[w]; b += lds16[8 + w]; }
+}
+
+struct SinkF32 { float * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v) const { *(f32x4 *)(dx + (size_t)row * K + k) = v; } };
+struct SinkBF16 { uint16_t * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v) const { *(u32x2 *)(dx + (size_t)row * K + k) = pack_f2bf_x4(v); } };
+struct SinkLds { float * buf; CAMX_DEV void operator()(int, int k, f32x4 v) const { *(f32x4 *)(buf + k) = v; } };
+// dact back through act = bf16(bf16(silu g) * u): each product rounded to bf16, then silu's derivative
+// ds * sig * fma(g, 1 - sig, 1), into dgu = [dg | du] rows of 2F
+struct SinkSiluMul {
+    const uint16_t * gu; int ld, F; uint16_t * dgu;
+    CAMX_DEV void operator()(int row, int k, f32x4 dact) const {
+        const uint16_t * r = gu + (size_t)row * ld;
+        const f32x4 g = unpack_bf16x4(*(const u32x2 *)(r + k)), u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
+        f32x4 dg, du;
+#define S_(e) { const float ex = expf(-g.e), sl = rbf(g.e / (1.0f + ex)), sig = 1.0f / (1.0f + ex), ds = rbf(dact.e * u.e); \
+                du.e = dact.e * sl; dg.e = ds * sig * __builtin_fmaf(g.e, 1.0f - sig, 1.0f); }
+        CAMX_EACH4(S_)
+#undef S_
+        uint16_t * o = dgu + (size_t)row * (2 * F);
+        *(u32x2 *)(o + k) = pack_f2bf_x4(dg);
+        *(u32x2 *)(o + F + k) = pack_f2bf_x4(du);
+    }
+};
+
+// lds16: 16 floats. sink receives bf16-valued floats: the gradient of the bf16 source, before any widening store.
+template <int NR, typename Src, typename Sink>
+CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Sink sink, int K, float clip, int qmax, float * lds16) {
+    const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
+    f32x4 u[NR], gv[NR];
+#pragma unroll
+    for (int c = 0; c < NR; c++) {
+        const int ch = hw + 8 * c;
+        u32x2 raw = {0u, 0u};
+        if (ch < nch) raw = *(const u32x2 *)(g + (size_t)row * K + ch * 128 + 4 * l);
+        gv[c] = unpack_bf16x4(raw);
+    }
+    const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u), lds16);
+    const float s_raw = amax * clip / (float)qmax, s = fmaxf(s_raw, 1e-8f);
+    const float lo = (float)(-qmax - 1), hi = (float)qmax;
+    // dL/ds = sum g (q - m t) and the number of max-|u| elements; m: the rounded value lies strictly inside (lo, hi)
+    float dlds = 0.0f, ties = 0.0f;
+    uint32_t inside = 0;
+#pragma unroll
+    for (int c = 0; c < NR; c++) {
+        if (hw + 8 * c < nch) {
+            int bit = 4 * c;
+#define D_(e) { const float t = u[c].e / s, r = rintf(t), q = fminf(fmaxf(r, lo), hi); const bool m = r > lo && r < hi; \
+                dlds = __builtin_fmaf(gv[c].e, m ? q - t : q, dlds); ties += fabsf(u[c].e) == amax ? 1.0f : 0.0f; inside |= (uint32_t)m << bit; bit++; }
+            CAMX_EACH4(D_)
+#undef D_
+        }
+    }
+    block8_sum2(dlds, ties, lds16);
+    const float coef = s_raw >= 1e-8f ? dlds * clip / (float)qmax / ties : 0.0f;
+#pragma unroll
+    for (int c = 0; c < NR; c++) {
+        const int ch = hw + 8 * c;
+        if (ch < nch) {
+            f32x4 d;
+            int bit = 4 * c;
+#define V_(e) { float v = gv[c].e * ((inside >> bit) & 1u ? 1.0f : 0.0f); bit++; \
+                if (fabsf(u[c].e) == amax && u[c].e != 0.0f) v += u[c].e > 0.0f ? coef : -coef; d.e = rbf(v); }
+            CAMX_EACH4(V_)
+#undef V_
+            sink(row, ch * 128 + 4 * l, rbf4_scaled(hadamard128_l4(d, l, false)));
+        }
+    }
+}
+
+template <int NR, typename Src, typename Sink>
+__global__ void __launch_bounds__(256) actq_bwd_k(Src src, const uint16_t * g, Sink sink, int K, float clip, int qmax) {
+    __shared__ float lds[16];
+    actq_bwd_row<NR>(src, blockIdx.x, g, sink, K, clip, qmax, lds);
+}
+
+// ---- block entry: h = RMSNorm(x) never materialized ------------------------------------------------------------------------
 // row sum under the 256-thread tree, computed by the first wave (elements 256 j + 4 lane + k), result to all threads
 template <typename F>
 CAMX_DEV float row_tree_sum(F term, int d, float * slot) {
@@ -112,6 +224,7 @@ struct AbTerm {
     CAMX_DEV f32x4 other(int k) const { return unpack_bf16x4(*(const u32x2 *)(wab + k)); }
 };
 
+template <int NR>
 __global__ void __launch_bounds__(256) block_entry_fwd_k(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y,
                                                          float * s, uint16_t * codes, uint16_t * ab, float * rstd_out, int d, float clip, int qmax) {
     __shared__ float lds[4];
@@ -121,14 +234,64 @@ __global__ void __launch_bounds__(256) block_entry_fwd_k(const float * x, const 
     const float ss = row_tree_sum(SqTerm{xr}, d, &slot);
     const float rstd = rsqrt_exact(ss / (float)d + eps);
     if (threadIdx.x == 0 && rstd_out) rstd_out[row] = rstd;
-    actq_fwd_row(RmsSrc{x, nw, rstd, d}, row, y, s, d, clip, qmax, codes, lds);
+    actq_fwd_row<NR>(RmsSrc{x, nw, rstd, d}, row, y, s, d, clip, qmax, codes, lds);
     for (int j = 0; j < nab; j++) {
         const float v = row_tree_sum(AbTerm{xr, nw, rstd, wab + (size_t)j * d}, d, &slot);
         if (threadIdx.x == 0) ab[(size_t)row * nab + j] = f2bf(v);
     }
 }
 
+// dh = actq backward of dy, plus the two projection groups' input gradients (wab rows [0, nab / 2) and [nab / 2, nab), each
+// group's sum rounded to bf16); then the RMSNorm backward dx = rstd (dh w - xhat mean(dh w xhat)), xhat = x rstd. d <= 1024.
+// Thread t (slot space) owns elements t, t + 256, ...
+__global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const float * nw, const float * rstd_in, const uint16_t * wab, int nab,
+                                                         const uint16_t * dy, const uint16_t * dab, float * dx, int d, float clip, int qmax) {
+    __shared__ __attribute__((aligned(16))) float dh[1024];
+    __shared__ float lds[16];
+    __shared__ float dabs[16];
+    const int row = blockIdx.x, tid = threadIdx.x, t = slot_of(tid);
+    const float rstd = rstd_in[row];
+    const float * xr = x + (size_t)row * d;
+    actq_bwd_row<1>(RmsSrc{x, nw, rstd, d}, row, dy, SinkLds{dh}, d, clip, qmax, lds);
+    if (tid < nab) dabs[tid] = bf2f(dab[(size_t)row * nab + tid]);
+    __syncthreads();
+    const int half = nab / 2;
+    float dot = 0.0f, none = 0.0f, gk[4], xh[4], wk[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int k = t + 256 * i;
+        gk[i] = xh[i] = wk[i] = 0.0f;
+        if (k < d) {
+            float g = dh[k];
+            if (nab) {
+                float pa = 0.0f, pb = 0.0f;
+                for (int j = 0; j < half; j++) pa = __builtin_fmaf(dabs[j], bf2f(wab[(size_t)j * d + k]), pa);
+                for (int j = half; j < nab; j++) pb = __builtin_fmaf(dabs[j], bf2f(wab[(size_t)j * d + k]), pb);
+                g = (g + rbf(pa)) + rbf(pb);
+            }
+            gk[i] = g; wk[i] = nw[k]; xh[i] = xr[k] * rstd;
+            dot = __builtin_fmaf(g * wk[i], xh[i], dot);
+        }
+    }
+    block8_sum2(dot, none, lds);
+    dot = dot / (float)d;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int k = t + 256 * i;
+        if (k < d) dx[(size_t)row * d + k] = rstd * (gk[i] * wk[i] - xh[i] * dot);
+    }
+}
+
 static int actq_check(int K, int qmax, int M) { return (K < 128 || K % 128 || K > 8192 || qmax < 1 || M < 0) ? CAMX_EINVAL : CAMX_OK; }
+
+// one instance per number of rounds
+#define ACTQ_ROUNDS(K, CALL)                                                                                           \
+    switch (((K) + 1023) / 1024) {                                                                                     \
+        case 1: { constexpr int NR = 1; CALL; } break; case 2: { constexpr int NR = 2; CALL; } break;                   \
+        case 3: { constexpr int NR = 3; CALL; } break; case 4: { constexpr int NR = 4; CALL; } break;                   \
+        case 5: { constexpr int NR = 5; CALL; } break; case 6: { constexpr int NR = 6; CALL; } break;                   \
+        case 7: { constexpr int NR = 7; CALL; } break; default: { constexpr int NR = 8; CALL; } break;                  \
+    }
 
 extern "C" {
 
@@ -137,14 +300,14 @@ extern "C" {
 int camx_actq_fwd(const void * x, int is_bf16, uint16_t * y, float * s, uint16_t * codes, int K, float clip, int qmax, int M, hipStream_t st) {
     if (!x || (!y && !codes) || actq_check(K, qmax, M) || ((uintptr_t)x & (is_bf16 ? 7 : 15)) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    if (is_bf16) actq_fwd_k<<<dim3(M), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, y, s, codes, K, clip, qmax);
-    else actq_fwd_k<<<dim3(M), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, y, s, codes, K, clip, qmax);
+    if (is_bf16) { ACTQ_ROUNDS(K, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, y, s, codes, K, clip, qmax))) }
+    else { ACTQ_ROUNDS(K, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, y, s, codes, K, clip, qmax))) }
     CAMX_LAUNCH_RET();
 }
 int camx_silu_mul_actq_fwd(const uint16_t * gu, int ld, int F, uint16_t * y, float * s, uint16_t * codes, float clip, int qmax, int M, hipStream_t st) {
     if (!gu || (!y && !codes) || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    actq_fwd_k<<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F}, y, s, codes, F, clip, qmax);
+    ACTQ_ROUNDS(F, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F}, y, s, codes, F, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y, float * s, uint16_t * codes,
@@ -152,7 +315,32 @@ int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab
     if (!x || !nw || (!y && !codes) || actq_check(d, qmax, M) || nab < 0 || nab > 16 || (nab && (!wab || !ab)) || ((uintptr_t)x & 15) ||
         ((uintptr_t)nw & 15) || ((uintptr_t)wab & 7) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    block_entry_fwd_k<<<dim3(M), dim3(256), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax);
+    ACTQ_ROUNDS(d, (block_entry_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax)))
+    CAMX_LAUNCH_RET();
+}
+
+// actq_bwd_{f32,bf16}: g bf16 [M][K] the gradient of y; dx [M][K] in x's type
+int camx_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, int K, float clip, int qmax, int M, hipStream_t st) {
+    if (!x || !g || !dx || actq_check(K, qmax, M) || ((uintptr_t)x & (is_bf16 ? 7 : 15)) || ((uintptr_t)dx & (is_bf16 ? 7 : 15)) || ((uintptr_t)g & 7)) return CAMX_EINVAL;
+    if (M == 0) return CAMX_OK;
+    if (is_bf16) { ACTQ_ROUNDS(K, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, g, SinkBF16{(uint16_t *)dx, K}, K, clip, qmax))) }
+    else { ACTQ_ROUNDS(K, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, g, SinkF32{(float *)dx, K}, K, clip, qmax))) }
+    CAMX_LAUNCH_RET();
+}
+// silu_mul_actq_bwd: g bf16 [M][F] the gradient of y; dgu bf16 [M][2F] = [dg | du], contiguous
+int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, float clip, int qmax, int M, hipStream_t st) {
+    if (!gu || !g || !dgu || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)g & 7) || ((uintptr_t)dgu & 7)) return CAMX_EINVAL;
+    if (M == 0) return CAMX_OK;
+    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F}, g, SinkSiluMul{gu, ld, F, dgu}, F, clip, qmax)))
+    CAMX_LAUNCH_RET();
+}
+// block_entry_bwd: dy bf16 [M][d], dab bf16 [M][nab] (needed when nab > 0), rstd [M] from the forward; dx fp32 [M][d]; d <= 1024
+int camx_block_entry_bwd(const float * x, const float * nw, const float * rstd, const uint16_t * wab, int nab, const uint16_t * dy,
+                         const uint16_t * dab, float * dx, int d, float clip, int qmax, int M, hipStream_t st) {
+    if (!x || !nw || !rstd || !dy || !dx || actq_check(d, qmax, M) || d > 1024 || nab < 0 || nab > 16 || (nab & 1) || (nab && (!wab || !dab)) ||
+        ((uintptr_t)x & 15) || ((uintptr_t)nw & 15) || ((uintptr_t)dy & 7)) return CAMX_EINVAL;
+    if (M == 0) return CAMX_OK;
+    block_entry_bwd_k<<<dim3(M), dim3(256), 0, st>>>(x, nw, rstd, wab, nab, dy, dab, dx, d, clip, qmax);
     CAMX_LAUNCH_RET();
 }
 

@@ -105,6 +105,13 @@ def _actq(is_bf16, codes):
     return 'camx_actq_fwd', ad
 
 
+def _actq_bwd(is_bf16):
+    def ad(g, b, v):             # (x, g, dx, K, clip, qmax); grid M
+        x, gy, dx, K, clip, qmax = v
+        return [x, I(int(is_bf16)), gy, dx, K, clip, qmax, I(g[0])]
+    return 'camx_actq_bwd', ad
+
+
 _CORE = {
     'embedding_f32': _rows('camx_embedding_f32'), 'rmsnorm_f32': _rows('camx_rmsnorm_f32'),
     'silu_mul_bf16': ('camx_silu_mul_bf16', lambda g, b, v: [v[0], v[1], v[2], L64(_val(v[3]))]),
@@ -118,6 +125,8 @@ _ACTQ = {
     'actq_fwd_f32': _actq(False, False), 'actq_fwd_bf16': _actq(True, False),
     'actq_fwd_codes_f32': _actq(False, True), 'actq_fwd_codes_bf16': _actq(True, True),
     'silu_mul_actq_fwd': _rows('camx_silu_mul_actq_fwd'), 'block_entry_fwd': _rows('camx_block_entry_fwd'),
+    'actq_bwd_f32': _actq_bwd(False), 'actq_bwd_bf16': _actq_bwd(True),
+    'silu_mul_actq_bwd': _rows('camx_silu_mul_actq_bwd'), 'block_entry_bwd': _rows('camx_block_entry_bwd'),
 }
 _KV = {'own_kv_q8_append': _rows('camx_own_kv_q8_append')}
 _GG = {'gg_quantize_q8_1': ('camx_gg_quantize_q8_1', _gg_q8_1), 'gg_silu_mul': _plain('camx_gg_silu_mul')}

@@ -212,6 +212,18 @@ int camx_silu_mul_actq_fwd(const uint16_t * gu, int ld, int F, uint16_t * y, flo
 int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y, float * s,
                          uint16_t * codes, uint16_t * ab, float * rstd_out, int d, float clip, int qmax, int M, camx_stream_t stream);
 
+/* ---- activation fake-quant, backward (kernels/actq.hip) ----------------------------------------------------------------------------- */
+/* actq_bwd_{f32,bf16} (kernels/actq.hip:158-218, 327-333): x the forward's input, g bf16 [M][K] the gradient of y; dx [M][K] in
+ * x's type. Straight-through mask strictly inside the code range; the scale's gradient flows to the row's max-|u| elements. */
+int camx_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, int K, float clip, int qmax, int M, camx_stream_t stream);
+/* silu_mul_actq_bwd (kernels/actq.hip:137-153, 311-314): dgu bf16 [M][2F] = [dg | du], contiguous rows. */
+int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, float clip, int qmax, int M,
+                           camx_stream_t stream);
+/* block_entry_bwd (kernels/actq.hip:275-304): rstd [M] as the forward wrote it; dy bf16 [M][d]; dab bf16 [M][nab] (nab even; rows
+ * [0, nab / 2) and [nab / 2, nab) of wab are two projections); dx fp32 [M][d]; d <= 1024. */
+int camx_block_entry_bwd(const float * x, const float * nw, const float * rstd, const uint16_t * wab, int nab, const uint16_t * dy,
+                         const uint16_t * dab, float * dx, int d, float clip, int qmax, int M, camx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

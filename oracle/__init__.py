@@ -382,3 +382,35 @@ def block_entry_fwd(x, nw, wab, eps, clip=1.0, qmax=7):
     lib().orc_block_entry_fwd(_p(x), _p(_c(nw, np.float32)), _p(wab), I(nab), F(eps), _p(y), _p(s), _p(c), _p(ab), _p(rstd),
                               I(M), I(d), F(clip), I(qmax))
     return y, s, c, ab[:, :nab], rstd
+
+
+def actq_rotate(x):
+    """u = bf16(H128 . bf16 x) per 128-chunk, bf16 bits [M, K] (the forward's first stage; also the backward's last)"""
+    x = _c(x, np.uint16); M, K = x.shape
+    u = np.empty((M, K), np.uint16)
+    lib().orc_actq_rotate(_p(x), _p(u), I(M), I(K)); return u
+
+
+def actq_bwd(x, g, clip=1.0, qmax=7, bf16=False):
+    """-> dx [M, K]: fp32, or bf16 bits when x is bf16 bits"""
+    x = _c(x, np.uint16 if bf16 else np.float32); M, K = x.shape
+    dx = np.empty((M, K), np.uint16 if bf16 else np.float32); g = _c(g, np.uint16)
+    lib().orc_actq_bwd(_p(x), I(int(bf16)), _p(g), _p(dx), I(M), I(K), F(clip), I(qmax)); return dx
+
+
+def silu_mul_actq_bwd(gu, g, clip=1.0, qmax=7):
+    """-> dgu bf16 bits [M, 2F]"""
+    gu = _c(gu, np.uint16); M, F2 = gu.shape
+    dgu = np.empty((M, F2), np.uint16); g = _c(g, np.uint16)
+    lib().orc_silu_mul_actq_bwd(_p(gu), I(F2), I(F2 // 2), _p(g), _p(dgu), I(M), F(clip), I(qmax)); return dgu
+
+
+def block_entry_bwd(x, nw, rstd, wab, dy, dab, clip=1.0, qmax=7):
+    """-> dx fp32 [M, d]"""
+    x = _c(x, np.float32); M, d = x.shape
+    nab = 0 if wab is None else wab.shape[0]
+    nw = _c(nw, np.float32); rstd = _c(rstd, np.float32); dy = _c(dy, np.uint16)
+    wab = _c(wab, np.uint16) if nab else None; dab = _c(dab, np.uint16) if nab else None
+    dx = np.empty((M, d), np.float32)
+    lib().orc_block_entry_bwd(_p(x), _p(nw), _p(rstd), _p(wab), I(nab), _p(dy), _p(dab), _p(dx), I(M), I(d), F(clip), I(qmax))
+    return dx

@@ -22,7 +22,10 @@
  * (oracle/_ref), scalar per-value format definitions (tests/io/test_own_formats.py:31-68), the float64 Sylvester
  * Hadamard (tests/engine/test_q3moe_kvq8_cpu.py:153-173), the YaRN table expectations
  * (tests/engine/test_q3m_yarn_rope.py:57-62), q8_host (tests/engine/golden_util.py:101-110) and float64 closed forms.
- * Parity unpinned beyond its own text and invariants: orc_actq_* (the reference's tests need its private trainer).
+ * orc_actq_* / orc_silu_mul_actq_* / orc_block_entry_* (forward and backward): the reference's own tests compare with torch
+ * ops under bf16 autocast (tests/train/test_silu_mul_actq.py:29-37, tests/train/test_block_entry.py:17-33) through its
+ * private trainer's fq_act, which is not in the tree; the same graph, written from the kernel file's statement of it
+ * (kernels/actq.hip:1-12), is evaluated and differentiated by torch on the CPU in tests/test_oracle_actq_autograd.py.
  */
 #include <math.h>
 #include <stddef.h>
@@ -648,7 +651,7 @@ ORC_API void orc_emb_q8_0(const uint8_t * W, int rb, int vocab, const int32_t * 
     }
 }
 
-/* ---- activation fake-quant (kernels/actq.hip:40-53, 96-132, 247-274, 307-310). Parity unpinned (see header). --------- */
+/* ---- activation fake-quant (kernels/actq.hip:40-53, 96-132, 247-274, 307-310). Pinned against a torch graph (see header). - */
 #define HSCALE 0.08837890625f
 static void fwht128_actq(float * v) {   /* chunk element e = 4 lane + r: stages inside a lane's 4, then lanes by m = 1..16 */
     for (int l = 0; l < 32; l++) {
@@ -724,6 +727,112 @@ ORC_API void orc_block_entry_fwd(const float * x, const float * nw, const uint16
             for (int g = 0; g < 8; g++) tot += bfly32_sum(part + 32 * g);
             ab[(size_t)r * nab + j] = orc_f2bf(tot);
         }
+    }
+}
+
+/* ---- activation fake-quant, backward (kernels/actq.hip:134-218, 275-313). Pinned against autograd (see header). ---------
+ * Sum tree: logical thread (w = chunk % 8, l = element / 4 % 32) adds its terms in chunk order with fmaf; the 32 threads
+ * of a w combine by xor 16 .. 1; the eight w sums are added in order. out: the bf16-valued gradient of the bf16 source. */
+static float tree8x32(const float * part /* [8][32] */) {
+    float r = bfly32_sum(part);
+    for (int w = 1; w < 8; w++) r += bfly32_sum(part + 32 * w);
+    return r;
+}
+static void actq_bwd_row(const float * src, const uint16_t * g, int K, float clip, int qmax, float * out) {
+    float u[8192];
+    float amax = 0.0f;
+    for (int ch = 0; ch < K / 128; ch++) {
+        float * c = u + ch * 128;
+        for (int e = 0; e < 128; e++) c[e] = rbf(src[ch * 128 + e]);
+        fwht128_actq(c);
+        for (int e = 0; e < 128; e++) { c[e] = rbf(c[e] * HSCALE); amax = fmaxf(amax, fabsf(c[e])); }
+    }
+    const float s_raw = amax * clip / (float)qmax, s = fmaxf(s_raw, 1e-8f);
+    const float lo = (float)(-qmax - 1), hi = (float)qmax;
+    float dl[256], ti[256];
+    for (int t = 0; t < 256; t++) dl[t] = ti[t] = 0.0f;
+    for (int ch = 0; ch < K / 128; ch++)
+        for (int e = 0; e < 128; e++) {
+            const int k = ch * 128 + e, th = 32 * (ch % 8) + e / 4;
+            const float t = u[k] / s, r = rintf(t), q = fminf(fmaxf(r, lo), hi);
+            const int m = r > lo && r < hi;
+            dl[th] = fmaf(orc_bf2f(g[k]), m ? q - t : q, dl[th]);
+            ti[th] += fabsf(u[k]) == amax ? 1.0f : 0.0f;
+        }
+    const float dlds = tree8x32(dl), ties = tree8x32(ti);
+    const float coef = s_raw >= 1e-8f ? dlds * clip / (float)qmax / ties : 0.0f;
+    for (int ch = 0; ch < K / 128; ch++) {
+        float d[128];
+        for (int e = 0; e < 128; e++) {
+            const int k = ch * 128 + e;
+            const float t = u[k] / s, r = rintf(t);
+            float v = orc_bf2f(g[k]) * (r > lo && r < hi ? 1.0f : 0.0f);
+            if (fabsf(u[k]) == amax && u[k] != 0.0f) v += u[k] > 0.0f ? coef : -coef;
+            d[e] = rbf(v);
+        }
+        fwht128_actq(d);
+        for (int e = 0; e < 128; e++) out[ch * 128 + e] = rbf(d[e] * HSCALE);
+    }
+}
+ORC_API void orc_actq_rotate(const uint16_t * x, uint16_t * u, int M, int K) {
+    for (int r = 0; r < M; r++)
+        for (int ch = 0; ch < K / 128; ch++) {
+            float c[128];
+            for (int e = 0; e < 128; e++) c[e] = orc_bf2f(x[(size_t)r * K + ch * 128 + e]);
+            fwht128_actq(c);
+            for (int e = 0; e < 128; e++) u[(size_t)r * K + ch * 128 + e] = orc_f2bf(c[e] * HSCALE);
+        }
+}
+ORC_API void orc_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, int M, int K, float clip, int qmax) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < M; r++) {
+        float src[8192], out[8192];
+        for (int k = 0; k < K; k++) src[k] = is_bf16 ? orc_bf2f(((const uint16_t *)x)[(size_t)r * K + k]) : ((const float *)x)[(size_t)r * K + k];
+        actq_bwd_row(src, g + (size_t)r * K, K, clip, qmax, out);
+        for (int k = 0; k < K; k++) { if (is_bf16) ((uint16_t *)dx)[(size_t)r * K + k] = orc_f2bf(out[k]); else ((float *)dx)[(size_t)r * K + k] = out[k]; }
+    }
+}
+/* silu_mul_actq_bwd (actq.hip:140-153, 311-314): dgu [M][2F] = [dg | du] */
+ORC_API void orc_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, int M, float clip, int qmax) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < M; r++) {
+        float src[8192], out[8192];
+        const uint16_t * row = gu + (size_t)r * ld;
+        for (int k = 0; k < F; k++) { const float gg = orc_bf2f(row[k]); src[k] = rbf(rbf(gg / (1.0f + expf(-gg))) * orc_bf2f(row[F + k])); }
+        actq_bwd_row(src, g + (size_t)r * F, F, clip, qmax, out);
+        for (int k = 0; k < F; k++) {
+            const float dact = out[k], gg = orc_bf2f(row[k]), uu = orc_bf2f(row[F + k]);
+            const float ex = expf(-gg), sl = rbf(gg / (1.0f + ex)), sig = 1.0f / (1.0f + ex), ds = rbf(dact * uu);
+            dgu[(size_t)r * 2 * F + k] = orc_f2bf(ds * sig * fmaf(gg, 1.0f - sig, 1.0f));
+            dgu[(size_t)r * 2 * F + F + k] = orc_f2bf(dact * sl);
+        }
+    }
+}
+/* block_entry_bwd (actq.hip:275-304): thread t = k % 256 adds dot terms in k order with fmaf; 8 x 32 tree; d <= 1024 */
+ORC_API void orc_block_entry_bwd(const float * x, const float * nw, const float * rstd_in, const uint16_t * wab, int nab, const uint16_t * dy,
+                                 const uint16_t * dab, float * dx, int M, int d, float clip, int qmax) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < M; r++) {
+        const float * xr = x + (size_t)r * d;
+        const float rstd = rstd_in[r];
+        float src[1024], dh[1024], part[256];
+        for (int k = 0; k < d; k++) src[k] = xr[k] * rstd * nw[k];
+        actq_bwd_row(src, dy + (size_t)r * d, d, clip, qmax, dh);
+        for (int t = 0; t < 256; t++) part[t] = 0.0f;
+        const int half = nab / 2;
+        for (int k = 0; k < d; k++) {
+            float gk = dh[k];
+            if (nab) {
+                float pa = 0.0f, pb = 0.0f;
+                for (int j = 0; j < half; j++) pa = fmaf(orc_bf2f(dab[(size_t)r * nab + j]), orc_bf2f(wab[(size_t)j * d + k]), pa);
+                for (int j = half; j < nab; j++) pb = fmaf(orc_bf2f(dab[(size_t)r * nab + j]), orc_bf2f(wab[(size_t)j * d + k]), pb);
+                gk = (gk + rbf(pa)) + rbf(pb);
+            }
+            dh[k] = gk;
+            part[k & 255] = fmaf(gk * nw[k], xr[k] * rstd, part[k & 255]);
+        }
+        const float dot = tree8x32(part) / (float)d;
+        for (int k = 0; k < d; k++) dx[(size_t)r * d + k] = rstd * (dh[k] * nw[k] - (xr[k] * rstd) * dot);
     }
 }
 

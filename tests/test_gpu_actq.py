@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import oracle as O
-from gpu_util import F, I, L64, NULL, bits_equal, call, dev, host, outliers, ptr
+from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, dev, host, outliers, ptr
 
 pytestmark = pytest.mark.gpu
 
@@ -47,3 +47,95 @@ def test_silu_mul_actq_fwd():
     call('camx_silu_mul_bf16', ptr(gud), ptr(act), I(Fh), L64(M * Fh))
     ry, rs, rc = O.actq_fwd(host(act, np.uint16), bf16=True)
     assert bits_equal(host(s), rs) and bits_equal(host(c), rc) and bits_equal(host(y, np.uint16), ry)
+
+
+# ---- backward ----------------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('M,K,qmax', [(5, 896, 7), (3, 2048, 7), (2, 8192, 7), (4, 128, 3), (3, 768, 127), (300, 1024, 7), (7, 5120, 7)])
+def test_actq_bwd(M, K, qmax):
+    rng = np.random.default_rng(100 + K + qmax)
+    x = outliers(rng, (M, K)); x[0] = 0
+    if M > 2: x[2, :] = 0; x[2, 7] = 3.0                                   # rotates to a constant row: every element ties for the max
+    g = O.f2bf(rng.standard_normal((M, K)).astype(np.float32))
+    for bf in (False, True):
+        src = O.f2bf(x) if bf else x
+        want = O.actq_bwd(src, g, clip=0.9, qmax=qmax, bf16=bf)
+        dx = dev(np.zeros((M, K), np.uint16 if bf else np.float32))
+        call('camx_actq_bwd', ptr(dev(src)), I(int(bf)), ptr(dev(g)), ptr(dx), I(K), F(0.9), I(qmax), I(M))
+        assert bits_equal(host(dx, np.uint16) if bf else host(dx), want)
+
+
+@pytest.mark.parametrize('M,d,nab', [(6, 896, 14), (5, 1024, 0), (9, 256, 2), (130, 896, 16)])
+def test_block_entry_bwd(M, d, nab):
+    rng = np.random.default_rng(200 + d + nab)
+    x = outliers(rng, (M, d)); nw = (0.5 + rng.random(d)).astype(np.float32)
+    wab = O.f2bf((rng.standard_normal((max(nab, 2), d)) / 30).astype(np.float32))[:nab]
+    dy = O.f2bf(rng.standard_normal((M, d)).astype(np.float32)); dab = O.f2bf(rng.standard_normal((M, max(nab, 1))).astype(np.float32))[:, :nab]
+    rstd = O.block_entry_fwd(x, nw, wab if nab else None, 1e-6)[4]
+    want = O.block_entry_bwd(x, nw, rstd, wab if nab else None, dy, dab if nab else None)
+    dx = dev(np.zeros((M, d), np.float32))
+    call('camx_block_entry_bwd', ptr(dev(x)), ptr(dev(nw)), ptr(dev(rstd)), ptr(dev(wab)) if nab else NULL, I(nab), ptr(dev(dy)),
+         ptr(dev(np.ascontiguousarray(dab))) if nab else NULL, ptr(dx), I(d), F(1.0), I(7), I(M))
+    assert bits_equal(host(dx), want)
+
+
+@pytest.mark.parametrize('M,Fh,ld', [(24, 768, 1536), (12, 2048, 4608), (9, 256, 512)])
+def test_silu_mul_actq_bwd(M, Fh, ld):
+    """expf is the device's: rows whose activation the device computes to the oracle's bits are held to one bf16 step"""
+    rng = np.random.default_rng(300 + Fh)
+    base = O.f2bf((rng.standard_normal((M, ld)) * 2).astype(np.float32))
+    base[0, :8] = O.f2bf(np.array([30., -30., 0., -0.0, 1e-3, -88., 88., 3.], np.float32))
+    g = O.f2bf(rng.standard_normal((M, Fh)).astype(np.float32))
+    bd = dev(base)
+    dgu = dev(np.zeros((M, 2 * Fh), np.uint16))
+    call('camx_silu_mul_actq_bwd', ptr(bd), I(ld), I(Fh), ptr(dev(g)), ptr(dgu), F(1.0), I(7), I(M))
+    gu = np.ascontiguousarray(base[:, :2 * Fh])
+    act = dev(np.zeros((M, Fh), np.uint16))
+    call('camx_silu_mul_bf16', ptr(dev(gu)), ptr(act), I(Fh), L64(M * Fh))
+    ract = O.silu_mul_bf16(gu) if hasattr(O, 'silu_mul_bf16') else None
+    want = O.silu_mul_actq_bwd(gu, g)
+    got = host(dgu, np.uint16)
+    rows = np.ones(M, bool) if ract is None else (host(act, np.uint16) == ract.reshape(M, Fh)).all(1)
+    assert rows.sum() >= M // 2
+    assert close_16(got[rows], want[rows], 'bf16')
+    assert (got[rows] == want[rows]).mean() > 0.99
+
+
+def test_actq_autograd_wrappers():
+    """caminus_amd.train.actq end to end: values, codes, scales and every gradient equal the C entry points' results"""
+    import torch
+    from caminus_amd.train import actq as A
+    rng = np.random.default_rng(7)
+    M, K = 33, 1024
+    x = outliers(rng, (M, K)); gy = rng.standard_normal((M, K)).astype(np.float32)
+    for bf in (False, True):
+        xt = torch.from_numpy(x).to('cuda:0'); xt = (xt.bfloat16() if bf else xt).requires_grad_()
+        src = host(xt.detach().view(torch.int16), np.uint16) if bf else x
+        y, c, s = A.actq_codes(xt.view(3, 11, K), 4, 0.9)
+        ry, rs, rc = O.actq_fwd(src, clip=0.9, qmax=7, bf16=bf)
+        assert y.shape == (3, 11, K) and bits_equal(host(y.view(torch.int16), np.uint16).reshape(M, K), ry) and bits_equal(host(s), rs) and bits_equal(host(c), rc)
+        gt = torch.from_numpy(gy).to('cuda:0').view(3, 11, K)
+        y.backward(gt)
+        want = O.actq_bwd(src, O.f2bf(gy), clip=0.9, qmax=7, bf16=bf)
+        assert xt.grad.dtype == xt.dtype
+        assert bits_equal(host(xt.grad.view(torch.int16), np.uint16) if bf else host(xt.grad), want)
+        x2 = xt.detach().clone().requires_grad_()
+        A.actq(x2, 4, 0.9).backward(gt.view(M, K))
+        assert torch.equal(x2.grad, xt.grad)
+        assert torch.equal(A.scales(xt.detach(), 4, 0.9), s) and torch.equal(A.codes(xt.detach(), 4, 0.9)[0], c)
+    # block entry
+    d, nab = 896, 14
+    xb = outliers(rng, (M, d)); nw = (0.5 + rng.random(d)).astype(np.float32); wab = O.f2bf((rng.standard_normal((nab, d)) / 30).astype(np.float32))
+    dy = rng.standard_normal((M, d)).astype(np.float32); dab = rng.standard_normal((M, nab)).astype(np.float32)
+    xt = torch.from_numpy(xb).to('cuda:0').requires_grad_(); nwt = torch.from_numpy(nw).to('cuda:0'); wt = dev(wab).view(torch.bfloat16)
+    y, c, s, ab = A.block_entry(xt, nwt, wt, 1e-6)
+    ry, rs, rc, rab, rstd = O.block_entry_fwd(xb, nw, wab, 1e-6)
+    assert bits_equal(host(y.view(torch.int16), np.uint16), ry) and bits_equal(host(ab.view(torch.int16), np.uint16), rab) and bits_equal(host(c), rc)
+    torch.autograd.backward([y, ab], [torch.from_numpy(dy).to('cuda:0'), torch.from_numpy(dab).to('cuda:0')])
+    assert bits_equal(host(xt.grad), O.block_entry_bwd(xb, nw, rstd, wab, O.f2bf(dy), O.f2bf(dab)))
+    # silu-mul: gradient has gu's shape and dtype, strided input accepted
+    base = torch.randn(M, 4608, device='cuda:0').bfloat16()
+    gu = base[:, 256:256 + 2048].detach().requires_grad_()
+    yq, cq, sq = A.silu_mul_actq(gu)
+    yq.backward(torch.randn(M, 1024, device='cuda:0').bfloat16())
+    assert gu.grad.shape == (M, 2048) and gu.grad.dtype == torch.bfloat16 and torch.isfinite(gu.grad.float()).all()

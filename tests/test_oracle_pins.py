@@ -471,7 +471,7 @@ def test_core_elementwise_exact():
     assert np.array_equal(O.embedding_f32(tok, emb), emb[tok])
 
 
-# ---- actq: invariants only (the reference's tests need its private trainer): parity unpinned beyond these ------------------------------
+# ---- actq: invariants (the pins against a torch graph and autograd are in test_oracle_actq_autograd.py) --------------------------------
 
 def test_actq_invariants():
     rng = np.random.default_rng(10)
