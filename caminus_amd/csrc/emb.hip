@@ -1,14 +1,18 @@
-// Quantized embedding-row gather + dequant for gfx950: GGUF Q4_K (144 B / 256 values) and Q8_0 (34 B / 32 values) rows to
-// fp32 and / or bf16, optionally followed in the same wave by residual add + RMSNorm + q8_1 so the gathered row never
-// returns to HBM. Replaces q3p_emb / OP_OWN_EMB (kernels/q3m_prefill.hip:364-380, kernels/k3_own_ops.h:279-304); the Q8_0
+// Quantized embedding-row gather + dequant for gfx950: GGUF Q4_K (144 B / 256 values), Q8_0 (34 B / 32 values), IQ4_XS
+// (136 B / 256) and IQ2_S (82 B / 256) rows to fp32 and / or bf16, optionally followed in the same wave by residual add +
+// RMSNorm + q8_1 so the gathered row never returns to HBM; and the IQ4_NL rows (18 B / 32) of a per-layer-embedding feed.
+// Replaces q3p_emb / OP_OWN_EMB (kernels/q3m_prefill.hip:364-380, kernels/k3_own_ops.h:279-304), embd_rows_iq4xs and
+// ple_rows_iq4nl (kernels/prefill_feed.hip:24-54) and q35t_op_emb's IQ2_S rows (kernels/k3_q35t_ops.h:147-175); the Q8_0
 // arithmetic is the host decoder's (python/caminus/own_dequant.py:202-206).
 //
 // One wave per token row; slab j of 256 values = one Q4_K block or eight Q8_0 blocks; lane p decodes values 4p .. 4p + 3
 // of each slab: for Q4_K one dword of nibbles per lane (lanes 8 apart share it: low / high nibble) and the 16-byte block
 // header. y = (d * sc) * q - dmin * m with every product and the difference rounded separately.
 #include "common.cuh"
+#include "iq2s_grid.inc"
 
-enum { FMT_Q4_K = 0, FMT_Q8_0 = 1 };
+enum { FMT_Q4_K = 0, FMT_Q8_0 = 1, FMT_IQ4_XS = 2, FMT_IQ2_S = 3, FMT_COUNT = 4 };
+enum { ERR_PLE_INDEX = 1, ERR_TOKEN = 2 };
 
 CAMX_DEV f32x4 q4k_decode4(const uint8_t * blk, int lane) {
     const u32x4 hdr = *(const u32x4 *)blk;                       // d | dmin, then the 12 scale bytes
@@ -43,6 +47,58 @@ CAMX_DEV f32x4 q80_decode4(const uint8_t * slab, int lane) {     // slab: 8 bloc
     return y;
 }
 
+// the 16 values of IQ4_NL / IQ4_XS (-127 -104 -83 -65 -49 -35 -22 -10 1 13 25 38 53 69 89 113) for four 4-bit indices
+// held one per byte: two byte permutes over the table's halves, then a select on bit 3
+CAMX_DEV f32x4 iq4_values(uint32_t idx4) {
+    const uint32_t sel = idx4 & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(0xf6eaddcfu, 0xbfad9881u, sel), hi = __builtin_amdgcn_perm(0x71594535u, 0x26190d01u, sel);
+    const uint32_t top = ((idx4 >> 3) & 0x01010101u) * 0xffu;
+    const uint32_t v = (hi & top) | (lo & ~top);
+    f32x4 y;
+    y.x = (float)(int8_t)(v & 0xff); y.y = (float)(int8_t)((v >> 8) & 0xff); y.z = (float)(int8_t)((v >> 16) & 0xff); y.w = (float)(int8_t)(v >> 24);
+    return y;
+}
+
+// block_iq4_xs: f16 d, u16 scales_h, u8 scales_l[4], u8 qs[128]; sub-block ib (32 values): 6-bit scale ls, values
+// qs[16 ib ..] low nibbles then high; y = (d * (ls - 32)) * value
+CAMX_DEV f32x4 iq4xs_decode4(const uint8_t * blk, int lane) {
+    const u32x2 hdr = *(const u32x2 *)blk;
+    const int ib = lane >> 3;
+    const uint32_t sh = hdr.x >> 16, sl = (hdr.y >> (8 * (ib >> 1))) & 0xffu;
+    const int ls = (int)(((sl >> (4 * (ib & 1))) & 15u) | (((sh >> (2 * ib)) & 3u) << 4));
+    const float dl = h2f_bits((uint16_t)(hdr.x & 0xffffu)) * (float)(ls - 32);
+    const uint32_t qw = *(const uint32_t *)(blk + 8 + 16 * ib + 4 * (lane & 3)) >> (4 * ((lane >> 2) & 1));
+    const f32x4 k = iq4_values(qw & 0x0f0f0f0fu);
+    f32x4 y; y.x = dl * k.x; y.y = dl * k.y; y.z = dl * k.z; y.w = dl * k.w;
+    return y;
+}
+
+// block_iq2_s: f16 d, qs[32] (low 8 bits of a 10-bit grid index per 8 values), signs[32] (a bit per value), qh[8] (the
+// indices' high bits, four per byte), scales[8] (a nibble per 16 values); y = +-(((d * (0.5 + s)) * 0.25) * magnitude)
+CAMX_DEV f32x4 iq2s_decode4(const uint8_t * blk, int lane) {
+    const int ib = lane >> 3, g = (lane >> 1) & 3, h = lane & 1;
+    const float d = h2f_bits(*(const uint16_t *)blk);
+    const uint32_t idx = (uint32_t)blk[2 + 4 * ib + g] | ((((uint32_t)blk[66 + ib] >> (2 * g)) & 3u) << 8);
+    const uint32_t m4 = IQ2S_MAG[2 * idx + h];
+    const uint32_t sg = (uint32_t)blk[34 + 4 * ib + g] >> (4 * h);
+    const float sc = (float)(((uint32_t)blk[74 + ib] >> (4 * ((lane >> 2) & 1))) & 15u);
+    const float db = (d * (0.5f + sc)) * 0.25f;
+    f32x4 y;
+    y.x = db * (float)(m4 & 0xffu); y.y = db * (float)((m4 >> 8) & 0xffu); y.z = db * (float)((m4 >> 16) & 0xffu); y.w = db * (float)(m4 >> 24);
+    if (sg & 1u) y.x = -y.x;
+    if (sg & 2u) y.y = -y.y;
+    if (sg & 4u) y.z = -y.z;
+    if (sg & 8u) y.w = -y.w;
+    return y;
+}
+
+template <int FMT> CAMX_DEV f32x4 emb_decode4(const uint8_t * row, int j, int lane) {
+    if (FMT == FMT_Q4_K) return q4k_decode4(row + (size_t)j * 144, lane);
+    if (FMT == FMT_Q8_0) return q80_decode4(row + (size_t)j * 272, lane);
+    if (FMT == FMT_IQ4_XS) return iq4xs_decode4(row + (size_t)j * 136, lane);
+    return iq2s_decode4(row + (size_t)j * 82, lane);
+}
+
 struct EmbArgs {
     const uint8_t * W; long rb; int vocab;
     const int32_t * toks;
@@ -53,6 +109,7 @@ struct EmbArgs {
     const float * d;         // optional addend fp32 [n][N]
     const float * nw; float eps;
     float * h; uint16_t * h16; uint8_t * q8;
+    int * err;               // optional: bit ERR_TOKEN is set when an id lies outside [0, vocab) (the id is clamped either way)
 };
 
 // EXACT: the row has exactly NI_MAX slabs (straight-line loops: the loads are issued as one batch)
@@ -61,7 +118,9 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     const int lane = slot_of(threadIdx.x & 63);
     const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (t >= a.n) return;
-    int tok = a.toks[t]; tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;
+    int tok = a.toks[t];
+    if (a.err && (tok < 0 || tok >= a.vocab) && lane == 0) atomicOr(a.err, ERR_TOKEN);
+    tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;
     const uint8_t * row = a.W + (size_t)tok * a.rb;
     const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
     // short rows: the addend and gamma do not depend on the token id, so they are requested before the table row is decoded
@@ -81,7 +140,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     f32x4 xv[NI_MAX];
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) xv[j] = FMT == FMT_Q4_K ? q4k_decode4(row + (size_t)j * 144, lane) : q80_decode4(row + (size_t)j * 272, lane);
+        if (j < ni) xv[j] = emb_decode4<FMT>(row, j, lane);
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) {
@@ -135,37 +194,86 @@ static int launch_emb(const EmbArgs & a, hipStream_t st) {
 }
 
 static int emb_check(const EmbArgs & a, int fmt) {
+    static const int blk_bytes[FMT_COUNT] = {144, 272, 136, 82}, align[FMT_COUNT] = {16, 2, 8, 2};     // per 256 values
+    if (fmt < 0 || fmt >= FMT_COUNT) return CAMX_EINVAL;
     if (!a.W || !a.toks || a.N < 256 || a.N % 256 || a.N > 8192 || a.n < 0 || a.vocab < 1) return CAMX_EINVAL;
-    if (a.rb < (long)(fmt == FMT_Q4_K ? a.N / 256 * 144 : a.N / 32 * 34)) return CAMX_EINVAL;
-    if (fmt == FMT_Q4_K ? (((uintptr_t)a.W & 15) || (a.rb & 15)) : (((uintptr_t)a.W & 1) || (a.rb & 1))) return CAMX_EINVAL;
+    if (a.rb < (long)(a.N / 256 * blk_bytes[fmt])) return CAMX_EINVAL;
+    if (((uintptr_t)a.W & (align[fmt] - 1)) || (a.rb & (align[fmt] - 1))) return CAMX_EINVAL;
     if (((uintptr_t)a.x & 15) || ((uintptr_t)a.xbf & 7) || ((uintptr_t)a.d & 15) || ((uintptr_t)a.nw & 15) || ((uintptr_t)a.h & 15) ||
-        ((uintptr_t)a.h16 & 7) || ((uintptr_t)a.q8 & 3)) return CAMX_EINVAL;
+        ((uintptr_t)a.h16 & 7) || ((uintptr_t)a.q8 & 3) || ((uintptr_t)a.err & 3)) return CAMX_EINVAL;
     return CAMX_OK;
+}
+static int launch_emb_fmt(const EmbArgs & a, int fmt, hipStream_t st) {
+    switch (fmt) {
+        case FMT_Q4_K: return launch_emb<FMT_Q4_K>(a, st);
+        case FMT_Q8_0: return launch_emb<FMT_Q8_0>(a, st);
+        case FMT_IQ4_XS: return launch_emb<FMT_IQ4_XS>(a, st);
+        default: return launch_emb<FMT_IQ2_S>(a, st);
+    }
+}
+
+// IQ4_NL rows of a per-layer-embedding feed: out[r][k] = value k of raw row inv[r] (bpr blocks of 18 bytes: f16 d, 16 bytes
+// of nibbles, low nibble = value j, high = j + 16); y = d * value. One thread per four values.
+__global__ void __launch_bounds__(256) ple_rows_iq4nl_k(const uint8_t * __restrict__ raw, const int * __restrict__ inv, int nuniq, int nrows,
+                                                        int bpr, float * __restrict__ out, int * err) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    const int hq = bpr * 8;
+    if (q >= (long)nrows * hq) return;
+    const int r = (int)(q / hq), kq = (int)(q % hq), b = kq >> 3, j0 = (kq & 7) * 4;
+    int u = inv[r];
+    if (u < 0 || u >= nuniq) { atomicOr(err, ERR_PLE_INDEX); u = u < 0 ? 0 : nuniq - 1; }
+    const uint8_t * blk = raw + (size_t)u * (size_t)(bpr * 18) + (size_t)b * 18;
+    const float d = h2f_bits(*(const uint16_t *)blk);
+    const uint16_t * c = (const uint16_t *)(blk + 2 + (j0 & 15));
+    const uint32_t w = ((uint32_t)c[0] | ((uint32_t)c[1] << 16)) >> (j0 >= 16 ? 4 : 0);
+    const f32x4 k = iq4_values(w & 0x0f0f0f0fu);
+    f32x4 y; y.x = d * k.x; y.y = d * k.y; y.z = d * k.z; y.w = d * k.w;
+    *(f32x4 *)(out + 4 * q) = y;
 }
 
 extern "C" {
 
 // q3p_emb: x [n][N] fp32 = the Q4_K rows toks[i] (rb bytes per row), ids clamped to [0, vocab)
 int camx_q3p_emb(const uint8_t * W, int rb, int vocab, const int32_t * toks, float * x, int N, int n, hipStream_t st) {
-    EmbArgs a = {W, rb, vocab, toks, x, nullptr, N, n, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr};
+    EmbArgs a = {W, rb, vocab, toks, x, nullptr, N, n, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr, nullptr};
     if (!x || emb_check(a, FMT_Q4_K)) return CAMX_EINVAL;
     return launch_emb<FMT_Q4_K>(a, st);
 }
 
-// gather + dequant with fp32 and / or bf16 outputs; fmt 0 = Q4_K, 1 = Q8_0
+// gather + dequant with fp32 and / or bf16 outputs; fmt 0 = Q4_K, 1 = Q8_0, 2 = IQ4_XS, 3 = IQ2_S
 int camx_emb_gather(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int N, int n, int fmt, hipStream_t st) {
-    EmbArgs a = {W, rb, vocab, toks, x, xbf, N, n, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr};
-    if ((!x && !xbf) || (fmt != FMT_Q4_K && fmt != FMT_Q8_0) || emb_check(a, fmt)) return CAMX_EINVAL;
-    return fmt == FMT_Q4_K ? launch_emb<FMT_Q4_K>(a, st) : launch_emb<FMT_Q8_0>(a, st);
+    EmbArgs a = {W, rb, vocab, toks, x, xbf, N, n, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr, nullptr};
+    if ((!x && !xbf) || emb_check(a, fmt)) return CAMX_EINVAL;
+    return launch_emb_fmt(a, fmt, st);
 }
 
 // gather + dequant + (x += d) + RMSNorm * nw with h fp32 / fp16 / q8_1 copies, one pass per row (all outputs optional
 // except that at least one is given); x receives the residual row (after the add)
 int camx_emb_gather_add_rms(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, const float * d,
                             const float * nw, float eps, float * h, uint16_t * h16, void * q8, int N, int n, int fmt, hipStream_t st) {
-    EmbArgs a = {W, rb, vocab, toks, x, xbf, N, n, d, nw, eps, h, h16, (uint8_t *)q8};
-    if (!nw || (!x && !xbf && !h && !h16 && !q8) || (fmt != FMT_Q4_K && fmt != FMT_Q8_0) || emb_check(a, fmt)) return CAMX_EINVAL;
-    return fmt == FMT_Q4_K ? launch_emb<FMT_Q4_K>(a, st) : launch_emb<FMT_Q8_0>(a, st);
+    EmbArgs a = {W, rb, vocab, toks, x, xbf, N, n, d, nw, eps, h, h16, (uint8_t *)q8, nullptr};
+    if (!nw || (!x && !xbf && !h && !h16 && !q8) || emb_check(a, fmt)) return CAMX_EINVAL;
+    return launch_emb_fmt(a, fmt, st);
+}
+
+// embd_rows_iq4xs: out [n][256 nblk] fp32 = the IQ4_XS rows tok[i] of table ([nvocab][136 nblk]); an id outside [0, nvocab)
+// is clamped and reported as bit 1 of *err
+int camx_embd_rows_iq4xs(const uint8_t * table, const int32_t * tok, int nvocab, int n, int nblk, float * out, int * err, hipStream_t st) {
+    if (nblk < 1 || nblk > 32 || !out || !err) return CAMX_EINVAL;
+    EmbArgs a = {table, (long)nblk * 136, nvocab, tok, out, nullptr, nblk * 256, n, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr, err};
+    if (emb_check(a, FMT_IQ4_XS)) return CAMX_EINVAL;
+    return launch_emb<FMT_IQ4_XS>(a, st);
+}
+
+// ple_rows_iq4nl: out [nrows][32 bpr] fp32 = the IQ4_NL rows inv[r] of raw ([nuniq][18 bpr]); an index outside [0, nuniq)
+// is clamped and reported as bit 0 of *err
+int camx_ple_rows_iq4nl(const uint8_t * raw, const int32_t * inv, int nuniq, int nrows, int bpr, float * out, int * err, hipStream_t st) {
+    if (!raw || !inv || !out || !err || nuniq < 1 || nrows < 0 || bpr < 1 || bpr > (1 << 20) || ((uintptr_t)raw & 1) || ((uintptr_t)out & 15) ||
+        ((uintptr_t)err & 3) || (long)nrows * bpr * 8 > 0x7fffffffL * 256) return CAMX_EINVAL;
+    if (nrows == 0) return CAMX_OK;
+    const long quads = (long)nrows * bpr * 8;
+    ple_rows_iq4nl_k<<<dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st>>>(raw, inv, nuniq, nrows, bpr, out, err);
+    CAMX_LAUNCH_RET();
 }
 
 }   // extern "C"

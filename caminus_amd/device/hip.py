@@ -129,6 +129,17 @@ _ACTQ = {
     'silu_mul_actq_bwd': _rows('camx_silu_mul_actq_bwd'), 'block_entry_bwd': _rows('camx_block_entry_bwd'),
 }
 _KV = {'own_kv_q8_append': _rows('camx_own_kv_q8_append')}
+
+
+def _feed(name, rows_at, width_at, per_unit):
+    def ad(g, b, v):             # one thread per output value in the reference: the grid must cover them
+        need = _val(v[rows_at]) * _val(v[width_at]) * per_unit
+        _expect(g[0] * b[0] >= need, f'{name} covers {g[0] * b[0]} < {need} values')
+        return list(v)
+    return name, ad
+
+
+_FEED = {'ple_rows_iq4nl': _feed('camx_ple_rows_iq4nl', 3, 4, 32), 'embd_rows_iq4xs': _feed('camx_embd_rows_iq4xs', 3, 4, 256)}
 _GG = {'gg_quantize_q8_1': ('camx_gg_quantize_q8_1', _gg_q8_1), 'gg_silu_mul': _plain('camx_gg_silu_mul')}
 
 
@@ -152,7 +163,7 @@ _GDN = {'pf_gdn_l2': ('camx_pf_gdn_l2', _pf_gdn_l2)}
 _Q35 = {'q35p_add_rms16': _rows('camx_q35p_add_rms16'), 'q35p_gate_mul16': _gate(1)}
 
 SYMBOLS = {
-    'core': _CORE, 'fuse': _FUSE, 'actq': _ACTQ, 'kv_codec': _KV, 'k3_gguf': _GG, 'k3_gguf_swiglu': _GG,
+    'core': _CORE, 'fuse': _FUSE, 'actq': _ACTQ, 'kv_codec': _KV, 'prefill_feed': _FEED, 'k3_gguf': _GG, 'k3_gguf_swiglu': _GG,
     'q3m_prefill': _q3m(False, False), 'q3m_prefill_kvq8': _q3m(False, True), 'q3m_prefill_yarn': _q3m(True, False),
     'q3m_prefill_kvq8_yarn': _q3m(True, True), 'q35_prefill': _Q35,
     'prefill_glue': _glue(2560), 'prefill_glue_q35': _glue(2048), 'prefill_glue_q35d': _glue(5120),

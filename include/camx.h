@@ -165,7 +165,8 @@ int camx_hadamard128(const float * x, float * y, long heads, camx_stream_t strea
  * toks[i] of W (rb bytes per row), ids clamped to [0, vocab). */
 int camx_q3p_emb(const uint8_t * W, int rb, int vocab, const int32_t * toks, float * x, int N, int n, camx_stream_t stream);
 /* Gather + dequant to fp32 (x) and / or bf16 (xbf); fmt 0 = Q4_K (as q3p_emb), 1 = Q8_0 (the host decoder's arithmetic,
- * python/caminus/own_dequant.py:202-206). N = 256 NI <= 8192. */
+ * python/caminus/own_dequant.py:202-206), 2 = IQ4_XS (as embd_rows_iq4xs), 3 = IQ2_S (q35t_op_emb's rows,
+ * kernels/k3_q35t_ops.h:147-175; python/caminus/own_dequant.py:128-137). N = 256 NI <= 8192. W and rb aligned to 16 / 2 / 8 / 2. */
 int camx_emb_gather(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int N, int n, int fmt,
                     camx_stream_t stream);
 /* Gather + dequant + (x += d) + RMSNorm * nw with fp32 / fp16 / q8_1 copies of the normed row in one pass per row
@@ -173,6 +174,15 @@ int camx_emb_gather(const uint8_t * W, long rb, int vocab, const int32_t * toks,
 int camx_emb_gather_add_rms(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, const float * d,
                             const float * nw, float eps, float * h, uint16_t * h16, void * q8, int N, int n, int fmt,
                             camx_stream_t stream);
+
+/* embd_rows_iq4xs (kernels/prefill_feed.hip:40-54): out [n][256 nblk] fp32 = the IQ4_XS rows tok[i] of table ([nvocab][136 nblk]);
+ * an id outside [0, nvocab) is clamped and reported as bit 1 (value 2) of *err. */
+int camx_embd_rows_iq4xs(const uint8_t * table, const int32_t * tok, int nvocab, int n, int nblk, float * out, int * err,
+                         camx_stream_t stream);
+/* ple_rows_iq4nl (kernels/prefill_feed.hip:24-35): out [nrows][32 bpr] fp32 = the IQ4_NL rows inv[r] of raw ([nuniq][18 bpr]);
+ * an index outside [0, nuniq) is clamped and reported as bit 0 (value 1) of *err. */
+int camx_ple_rows_iq4nl(const uint8_t * raw, const int32_t * inv, int nuniq, int nrows, int bpr, float * out, int * err,
+                        camx_stream_t stream);
 
 /* ---- GDN short convolution and L2 norm ------------------------------------------------------------------------------------------ */
 /* pf_gdn_conv (kernels/prefill_glue.hip:314-332) = OP_GDN_CONV (kernels/k3_q35_ops.h:152-177): y[t][c] = silu(fma chain

@@ -357,6 +357,37 @@ def emb_q8_0(W, vocab, toks, N):
     lib().orc_emb_q8_0(_p(W), I(rb), I(vocab), _p(toks), _p(x), _p(xbf), I(N), I(toks.size)); return x, xbf
 
 
+def emb_iq4xs(W, vocab, toks, N):
+    """-> (x fp32 [n, N], xbf bf16 bits, err word)"""
+    W = _c(W, np.uint8); toks = _c(toks, np.int32)
+    x = np.empty((toks.size, N), np.float32); xbf = np.empty((toks.size, N), np.uint16); err = np.zeros(1, np.int32)
+    lib().orc_emb_iq4xs(_p(W), I(vocab), _p(toks), _p(x), _p(xbf), I(N // 256), I(toks.size), _p(err)); return x, xbf, int(err[0])
+
+
+def ple_rows_iq4nl(raw, inv, nuniq, bpr):
+    """-> (out fp32 [nrows, 32 bpr], err word)"""
+    raw = _c(raw, np.uint8); inv = _c(inv, np.int32)
+    out = np.empty((inv.size, 32 * bpr), np.float32); err = np.zeros(1, np.int32)
+    lib().orc_ple_rows_iq4nl(_p(raw), _p(inv), I(nuniq), I(inv.size), I(bpr), _p(out), _p(err)); return out, int(err[0])
+
+
+_IQ2S = None
+
+
+def iq2s_grid():
+    """the IQ2_S codebook, uint8 [1024, 8] (ggml's iq2s_grid as magnitude bytes; oracle/iq2s_grid.npy)"""
+    global _IQ2S
+    if _IQ2S is None:
+        _IQ2S = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'iq2s_grid.npy'))
+    return _IQ2S
+
+
+def emb_iq2s(W, vocab, toks, N):
+    W = _c(W, np.uint8); toks = _c(toks, np.int32); grid = _c(iq2s_grid(), np.uint8)
+    x = np.empty((toks.size, N), np.float32); xbf = np.empty((toks.size, N), np.uint16)
+    lib().orc_emb_iq2s(_p(W), I(vocab), _p(toks), _p(x), _p(xbf), I(N), I(toks.size), _p(grid)); return x, xbf
+
+
 # ---- actq -----------------------------------------------------------------------------------------------------------------------
 
 

@@ -651,6 +651,60 @@ ORC_API void orc_emb_q8_0(const uint8_t * W, int rb, int vocab, const int32_t * 
     }
 }
 
+/* IQ4_XS rows (kernels/prefill_feed.hip:40-54): one value at a time; err bit 1 for an id outside the table (clamped) */
+static const float KV_IQ4[16] = {-127.f, -104.f, -83.f, -65.f, -49.f, -35.f, -22.f, -10.f, 1.f, 13.f, 25.f, 38.f, 53.f, 69.f, 89.f, 113.f};
+ORC_API void orc_emb_iq4xs(const uint8_t * W, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int nblk, int n, int * err) {
+    const int D = nblk * 256;
+    for (int p = 0; p < n; p++) {
+        int t = toks[p];
+        if (t < 0 || t >= vocab) { if (err) *err |= 2; t = t < 0 ? 0 : vocab - 1; }
+        for (int k = 0; k < D; k++) {
+            const int bl = k >> 8, w = k & 255, ib = w >> 5, j = w & 31;
+            const uint8_t * b = W + (size_t)t * (size_t)(nblk * 136) + (size_t)bl * 136;
+            const int sh = b[2] | (b[3] << 8), sl = b[4 + (ib >> 1)];
+            const int ls = ((sl >> ((ib & 1) * 4)) & 15) | (((sh >> (2 * ib)) & 3) << 4);
+            const float dl = orc_h2f((uint16_t)(b[0] | (b[1] << 8))) * (float)(ls - 32);
+            const uint8_t q = b[8 + 16 * ib + (j & 15)];
+            const float v = dl * KV_IQ4[j < 16 ? (q & 15) : (q >> 4)];
+            if (x) x[(size_t)p * D + k] = v;
+            if (xbf) xbf[(size_t)p * D + k] = orc_f2bf(v);
+        }
+    }
+}
+/* IQ4_NL feed rows (kernels/prefill_feed.hip:24-35); err bit 0 for an index outside [0, nuniq) (clamped) */
+ORC_API void orc_ple_rows_iq4nl(const uint8_t * raw, const int32_t * inv, int nuniq, int nrows, int bpr, float * out, int * err) {
+    const int hd = bpr * 32;
+    for (int r = 0; r < nrows; r++) {
+        int u = inv[r];
+        if (u < 0 || u >= nuniq) { *err |= 1; u = u < 0 ? 0 : nuniq - 1; }
+        for (int k = 0; k < hd; k++) {
+            const int b = k >> 5, j = k & 31;
+            const uint8_t * blk = raw + (size_t)u * (size_t)(bpr * 18) + (size_t)b * 18;
+            const uint8_t q = blk[2 + (j & 15)];
+            out[(size_t)r * hd + k] = orc_h2f((uint16_t)(blk[0] | (blk[1] << 8))) * KV_IQ4[j < 16 ? (q & 15) : (q >> 4)];
+        }
+    }
+}
+/* IQ2_S rows (kernels/k3_q35t_ops.h:163-174); grid: [1024][8] magnitude bytes (the caller's copy of the format's codebook) */
+ORC_API void orc_emb_iq2s(const uint8_t * W, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int N, int n, const uint8_t * grid) {
+    for (int p = 0; p < n; p++) {
+        int t = toks[p]; t = t < 0 ? 0 : t; t = t > vocab - 1 ? vocab - 1 : t;
+        const uint8_t * row = W + (size_t)t * (size_t)(N / 256 * 82);
+        for (int i = 0; i < N; i++) {
+            const uint8_t * blk = row + (size_t)(i >> 8) * 82;
+            const int j = i & 255, ib = j >> 5, g = (j >> 3) & 3, k = j & 7;
+            const float d = orc_h2f((uint16_t)(blk[0] | (blk[1] << 8)));
+            const uint32_t idx = blk[2 + 4 * ib + g] | (((uint32_t)(blk[66 + ib] >> (2 * g)) & 3u) << 8);
+            const float mag = (float)grid[idx * 8 + k];
+            const float sc = (float)((blk[74 + ib] >> (4 * ((j >> 4) & 1))) & 15);
+            const float db = (d * (0.5f + sc)) * 0.25f;
+            const float v0 = db * mag, v = ((blk[34 + (j >> 3)] >> k) & 1) ? -v0 : v0;
+            if (x) x[(size_t)p * N + i] = v;
+            if (xbf) xbf[(size_t)p * N + i] = orc_f2bf(v);
+        }
+    }
+}
+
 /* ---- activation fake-quant (kernels/actq.hip:40-53, 96-132, 247-274, 307-310). Pinned against a torch graph (see header). - */
 #define HSCALE 0.08837890625f
 static void fwht128_actq(float * v) {   /* chunk element e = 4 lane + r: stages inside a lane's 4, then lanes by m = 1..16 */

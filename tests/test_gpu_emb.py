@@ -45,3 +45,73 @@ def test_gather_add_rms_q8_1(fmt, with_add):
     assert bits_equal(host(xbf, np.uint16), gbf)
     assert bits_equal(host(x), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
     assert bits_equal(host(q8), ref['q8'])
+
+
+# ---- IQ4_XS / IQ2_S token rows, IQ4_NL feed rows ------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('N,vocab,n', [(2048, 500, 256), (256, 9, 5), (5120, 40, 7), (8192, 12, 33), (1536, 30, 64)])
+def test_gather_iq4xs_iq2s(N, vocab, n):
+    from vectors import iq_table
+    rng = np.random.default_rng(2002 + N)
+    toks = rng.integers(0, vocab, n).astype(np.int32); toks[:3] = [-5, vocab + 7, vocab - 1][:min(3, n)]
+    for fmt, name in ((2, 'IQ4_XS'), (3, 'IQ2_S')):
+        table = iq_table(rng, vocab, N, name)
+        if fmt == 2: ref_x, ref_bf, _ = O.emb_iq4xs(table, vocab, toks, N)
+        else: ref_x, ref_bf = O.emb_iq2s(table, vocab, toks, N)
+        Wd, td = dev(table), dev(toks)
+        x = dev(np.zeros((n, N), np.float32)); xbf = dev(np.zeros((n, N), np.uint16))
+        call('camx_emb_gather', ptr(Wd), L64(table.shape[1]), I(vocab), ptr(td), ptr(x), ptr(xbf), I(N), I(n), I(fmt))
+        assert bits_equal(host(x), ref_x) and bits_equal(host(xbf, np.uint16), ref_bf)
+        if fmt == 2:                                                    # the reference's own entry point, with its error word
+            x2 = dev(np.zeros((n, N), np.float32)); err = dev(np.zeros(1, np.int32))
+            call('camx_embd_rows_iq4xs', ptr(Wd), ptr(td), I(vocab), I(n), I(N // 256), ptr(x2), ptr(err))
+            assert bits_equal(host(x2), ref_x) and int(host(err)[0]) == 2
+            good = dev(np.clip(toks, 0, vocab - 1)); err.zero_()
+            call('camx_embd_rows_iq4xs', ptr(Wd), ptr(good), I(vocab), I(n), I(N // 256), ptr(x2), ptr(err))
+            assert bits_equal(host(x2), ref_x) and int(host(err)[0]) == 0
+
+
+@pytest.mark.parametrize('fmt', [2, 3])
+def test_gather_add_rms_q8_1_iq(fmt):
+    from vectors import iq_table
+    rng = np.random.default_rng(2100 + fmt)
+    N, vocab, n = 2048, 300, 64
+    table = iq_table(rng, vocab, N, 'IQ4_XS' if fmt == 2 else 'IQ2_S')
+    toks = rng.integers(0, vocab, n).astype(np.int32)
+    nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    d = outliers(rng, (n, 1, N)) * np.float32(0.01)
+    gx, gbf = O.emb_iq4xs(table, vocab, toks, N)[:2] if fmt == 2 else O.emb_iq2s(table, vocab, toks, N)
+    ref = O.add_rms16(gx, nw, 1e-6, d=d, S=1, want_q8=True)
+    x = dev(np.zeros((n, N), np.float32)); xbf = dev(np.zeros((n, N), np.uint16)); h = dev(np.zeros((n, N), np.float32))
+    h16 = dev(np.zeros((n, N), np.uint16)); q8 = dev(np.zeros((n, N // 32, 36), np.uint8))
+    call('camx_emb_gather_add_rms', ptr(dev(table)), L64(table.shape[1]), I(vocab), ptr(dev(toks)), ptr(x), ptr(xbf), ptr(dev(d)), ptr(dev(nw)),
+         F(1e-6), ptr(h), ptr(h16), ptr(q8), I(N), I(n), I(fmt))
+    assert bits_equal(host(xbf, np.uint16), gbf) and bits_equal(host(x), ref['x']) and bits_equal(host(h), ref['h'])
+    assert bits_equal(host(h16, np.uint16), ref['h16']) and bits_equal(host(q8), ref['q8'])
+
+
+@pytest.mark.parametrize('nuniq,nrows,bpr', [(40, 2048 * 2, 5), (3, 7, 1), (64, 300, 8)])
+def test_ple_rows_iq4nl(nuniq, nrows, bpr):
+    """the feed's IQ4_NL rows through the reference's launcher surface, with its negative controls (tests/prefill/test_prefill_feed.py:189-199)"""
+    import ctypes
+    import torch
+    from caminus_amd.device.hip import Module
+    from vectors import iq_table
+    rng = np.random.default_rng(2200 + bpr)
+    raw = iq_table(rng, nuniq, 32 * bpr, 'IQ4_NL'); inv = rng.integers(0, nuniq, nrows).astype(np.int32)
+    want, e0 = O.ple_rows_iq4nl(raw, inv, nuniq, bpr)
+    out = dev(np.zeros((nrows, 32 * bpr), np.float32)); err = dev(np.zeros(1, np.int32))
+    mod = Module('prefill_feed')
+    N = nrows * 32 * bpr
+    rawd, invd = dev(raw), dev(inv)
+    mod.ple_rows_iq4nl(((N + 255) // 256,), (256,), rawd, invd, ctypes.c_int(nuniq), ctypes.c_int(nrows), ctypes.c_int(bpr), out, err)
+    torch.cuda.synchronize()
+    assert e0 == 0 and int(host(err)[0]) == 0 and bits_equal(host(out), want)
+    bad = inv.copy(); bad[min(3, nrows - 1)] = nuniq; bad[min(5, nrows - 1)] = -7
+    want, e1 = O.ple_rows_iq4nl(raw, bad, nuniq, bpr)
+    badd = dev(bad)
+    mod.ple_rows_iq4nl(((N + 255) // 256,), (256,), rawd, badd, ctypes.c_int(nuniq), ctypes.c_int(nrows), ctypes.c_int(bpr), out, err)
+    torch.cuda.synchronize()
+    assert e1 == 1 and int(host(err)[0]) == 1 and bits_equal(host(out), want)
+    with pytest.raises(ValueError):
+        mod.ple_rows_iq4nl((1,), (256,), rawd, invd, ctypes.c_int(nuniq), ctypes.c_int(nrows + 300), ctypes.c_int(bpr), out, err)

@@ -3,6 +3,7 @@ vectors and seeded generators, the reference's own header compiled for the host 
 independent numpy implementations written from the format definitions, float64 closed forms, and invariants chosen so that
 a dropped term, a wrong index or a transposed operand fails. CPU only."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -10,7 +11,7 @@ import pytest
 import oracle as O
 from caminus_amd import rope
 from oracle import np_dequant as own_dequant, np_kv as ref_kv
-from vectors import kv_invalid_blocks, kv_valid_blocks, q4k_table, q80_table, qk_par
+from vectors import iq_table, kv_invalid_blocks, kv_valid_blocks, q4k_table, q80_table, qk_par
 
 f32 = np.float32
 
@@ -226,6 +227,74 @@ def test_gguf_rows_against_scalar_definitions():
         want = np.array([_def_q8_0(row[(i // 32) * 34:(i // 32 + 1) * 34], i % 32) for i in range(N)], f32)
         assert np.array_equal(y[r].view(np.uint32), want.view(np.uint32))
     assert np.array_equal(ybf, O.f2bf(y))
+
+
+KV_IQ4 = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]      # ggml's kvalues_iq4nl (kernels/prefill_feed.hip:15)
+
+
+def test_iq2s_codebook_file():
+    """the codebook is format data that cannot be derived: its bytes are held to a digest and to the entries the format's
+    published table starts with; every entry is 8 magnitudes out of {8, 25, 43} and no entry repeats"""
+    import hashlib
+    g = O.iq2s_grid()
+    assert g.shape == (1024, 8) and g.dtype == np.uint8
+    assert hashlib.sha256(g.tobytes()).hexdigest() == 'e1aa1473412b0552c2174c30ef22ab4073f6a181b85a17056e8249bd2932fd88'
+    assert g[0].tolist() == [8] * 8 and g[1].tolist() == [43] + [8] * 7 and g[2].tolist() == [25, 25] + [8] * 6
+    assert set(np.unique(g).tolist()) == {8, 25, 43} and len({bytes(r) for r in g}) == 1024
+    # the product's copy (little-endian words of four magnitudes) holds the same bytes
+    import re
+    txt = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'caminus_amd', 'csrc', 'iq2s_grid.inc')).read()
+    words = np.array([int(w, 16) for w in re.findall(r'0x([0-9a-f]{8})u', txt)], np.uint32)
+    assert np.array_equal(words.view(np.uint8).reshape(1024, 8), g)
+
+
+def test_iq_rows_known_answers():
+    """hand-built blocks whose values are known without any decoder"""
+    h = lambda v: np.array([v], np.float16).view(np.uint8)
+    # IQ4_NL, d = 1: byte i holds index i (low nibble) and 15 - i (high): values 0-15 ascend through the table, 16-31 descend
+    blk = np.zeros(18, np.uint8); blk[0:2] = h(1.0); blk[2:18] = np.arange(16) | ((15 - np.arange(16)) << 4)
+    out, err = O.ple_rows_iq4nl(blk[None], np.array([0], np.int32), 1, 1)
+    assert err == 0 and out[0].tolist() == KV_IQ4 + KV_IQ4[::-1]
+    assert np.array_equal(own_dequant.iq4_nl(blk), out[0])
+    # IQ4_XS, d = 2, sub-block ib has the 6-bit scale 33 + ib (low nibble 1 + ib, high bits 2), every index 8 (value 1) but two
+    blk = np.zeros(136, np.uint8); blk[0:2] = h(2.0)
+    blk[2:4] = np.array([sum(2 << (2 * ib) for ib in range(8))], np.uint16).view(np.uint8)
+    blk[4:8] = [(1 + 2 * k) | ((2 + 2 * k) << 4) for k in range(4)]
+    blk[8:136] = 0x88
+    blk[8 + 16 * 3 + 5] = 0x0F                                           # sub-block 3: value 5 -> index 15, value 21 -> index 0
+    x, _, err = O.emb_iq4xs(blk[None], 1, np.array([0], np.int32), 256)
+    want = np.repeat(2.0 * (1 + np.arange(8)), 32).astype(f32); want[3 * 32 + 5] *= 113; want[3 * 32 + 21] *= -127
+    assert err == 0 and np.array_equal(x[0], want)
+    # IQ2_S, d = 4: db = 0.5 + s; sub-block 2 / group 1 (values 72-79) points at codebook entry 0x101 + signs 0b10000001
+    g = O.iq2s_grid()
+    blk = np.zeros(82, np.uint8); blk[0:2] = h(4.0)
+    blk[2 + 4 * 2 + 1] = 0x01; blk[66 + 2] = 1 << 2; blk[34 + 9] = 0x81
+    blk[74:82] = [0x10 * (k + 1) | k for k in range(8)]                 # 16-value halves of sub-block k: scales k and k + 1
+    x, _ = O.emb_iq2s(blk[None], 1, np.array([0], np.int32), 256)
+    want = np.repeat(0.5 + np.stack([np.arange(8), np.arange(8) + 1], 1).reshape(-1), 16).astype(f32) * 8       # entry 0: all 8
+    want[72:80] = 2.5 * g[0x101].astype(f32) * np.array([-1, 1, 1, 1, 1, 1, 1, -1], f32)
+    assert np.array_equal(x[0], want)
+
+
+def test_iq_rows_against_block_decoders():
+    """the one-value-at-a-time C statements against the block-wise numpy decoders on random blocks (both signs of d, every bit
+    pattern), with clamped ids and the error word"""
+    rng = np.random.default_rng(15)
+    vocab, toks = 7, np.array([3, 0, 6, 9, -2, 5], np.int32)
+    rows = np.clip(toks, 0, vocab - 1)
+    for N in (256, 768, 2048):
+        W = iq_table(rng, vocab, N, 'IQ4_XS')
+        x, xbf, err = O.emb_iq4xs(W, vocab, toks, N)
+        assert err == 2 and np.array_equal(x.view(np.uint32), own_dequant.iq4_xs(W.reshape(-1)).reshape(vocab, N)[rows].view(np.uint32))
+        assert np.array_equal(xbf, O.f2bf(x)) and O.emb_iq4xs(W, vocab, rows, N)[2] == 0
+        W = iq_table(rng, vocab, N, 'IQ2_S')
+        x, xbf = O.emb_iq2s(W, vocab, toks, N)
+        assert np.array_equal(x.view(np.uint32), own_dequant.iq2_s(W.reshape(-1), O.iq2s_grid()).reshape(vocab, N)[rows].view(np.uint32))
+        assert np.array_equal(xbf, O.f2bf(x))
+    for bpr in (1, 5, 8):
+        raw = iq_table(rng, 4, 32 * bpr, 'IQ4_NL'); inv = np.array([0, 3, 1, 4, -1, 2], np.int32)
+        out, err = O.ple_rows_iq4nl(raw, inv, 4, bpr)
+        assert err == 1 and np.array_equal(out.view(np.uint32), own_dequant.iq4_nl(raw.reshape(-1)).reshape(4, 32 * bpr)[np.clip(inv, 0, 3)].view(np.uint32))
 
 
 # ---- q8_1 -------------------------------------------------------------------------------------------------------------------------

@@ -58,6 +58,16 @@ def q80_table(rng, rows, N):
     return t.reshape(rows, nb * 34)
 
 
+def iq_table(rng, rows, N, fmt):
+    """random IQ4_XS / IQ2_S / IQ4_NL rows: every index, sign and scale pattern, fp16 d ~ N(0, 0.01) (either sign);
+    uint8 [rows, N / values * bytes]"""
+    qk, bs = {'IQ4_XS': (256, 136), 'IQ2_S': (256, 82), 'IQ4_NL': (32, 18)}[fmt]
+    nb = N // qk
+    t = rng.integers(0, 256, (rows, nb, bs), dtype=np.uint8)
+    t[:, :, 0:2] = (rng.standard_normal((rows, nb, 1)) * 0.01).astype(np.float16).view(np.uint8).reshape(rows, nb, 2)
+    return t.reshape(rows, nb * bs)
+
+
 def qk_par(rng, theta_base=1e6, eps=1e-6, yarn_table=None):
     """the own line's par block: q_norm[128] | k_norm[128] | theta_scale | eps (| freq[64] | mscale)"""
     qn = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32); kn = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32)
