@@ -323,7 +323,8 @@ def main():
     }
     if not a.no_extra and not a.only:
         ops = {}
-        for name, by, fn in extra_opsets(B):
+        sets = extra_opsets(B)
+        for name, by, fn in sets:
             if name == '_keep': continue
             med, mean = B.time_launch(fn, reps=50, warm=10, flush=True)
             med_hot, _ = B.time_launch(fn, reps=50, warm=10, flush=False)
@@ -337,6 +338,28 @@ def main():
         for k, ref_us in (('hc_post_rms_2048x4x2560_bf16_scale', 466.0), ('hc_mean_2048x4x2560_from_residual', 267.0)):
             if k in ops: ops[k]['reference_rx7900xtx_us'] = ref_us
         out['opsets'] = ops
+        # the launch-bound op-sets as they would run in a decode loop: each shape's launches captured once into a HIP graph
+        # and replayed (every entry point is stream-ordered, allocates nothing and keeps no host state per call)
+        graphs = {}
+        for prefix in ('c1_', 'c4_', 'c5_'):
+            fns = [fn for name, _, fn in sets if name.startswith(prefix)]
+            for fn in fns: fn()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            main_stream = B.stream
+            with torch.cuda.graph(gr):
+                B.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)      # the capture stream
+                for fn in fns: fn()
+            B.stream = main_stream
+            for _ in range(5): gr.replay()
+            torch.cuda.synchronize()
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            g0.record()
+            for _ in range(50): gr.replay()
+            g1.record(); g1.synchronize()
+            us = g0.elapsed_time(g1) * 1e3 / 50
+            graphs[prefix + 'opsets_as_one_graph'] = {'launches': len(fns), 'us_per_replay': round(us, 2), 'us_per_launch': round(us / len(fns), 2)}
+        out['opset_graphs'] = graphs
     if not a.no_cpu and not a.only:
         out['cpu_baseline'] = cpu_baseline(w)
     print(json.dumps(out))

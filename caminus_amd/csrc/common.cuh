@@ -130,6 +130,29 @@ CAMX_DEV uint32_t pack_round_i8x4(f32x4 v) {
     return round_i8(v.x) | (round_i8(v.y) << 8) | (round_i8(v.z) << 16) | (round_i8(v.w) << 24);
 }
 
+// the four codes roundf(x / d) of a lane (d > 0 or the block is all zero and never gets here), packed. The IEEE quotient
+// t = fl(x / d) is only needed to decide on which side of a half-integer it falls. p = x * rcp(d) is within 3.8e-5 of the
+// exact quotient for |x / d| <= 127 (rcp: 1 ulp; one more rounding), t within 4e-6 of it, and half-integers are floats, so
+// whenever p is farther than 2^-13 from every half-integer, roundf(t) = roundf(p). Lanes that hold a closer value (about
+// one in a thousand), an infinity or a NaN, or whose d is too small for rcp, divide.
+CAMX_DEV uint32_t q8_codes4(f32x4 v, float d) {
+    const float r = __builtin_amdgcn_rcpf(d);
+    float p[4] = {v.x * r, v.y * r, v.z * r, v.w * r};
+    int c[4];
+    bool safe = true;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        c[k] = (int)(p[k] + __builtin_copysignf(0.49999997f, p[k]));
+        safe &= fabsf(p[k] - (float)c[k]) <= 0.4998f;               // (exact difference; false for NaN and for an infinite p)
+    }
+    if (!safe) {
+        p[0] = v.x / d; p[1] = v.y / d; p[2] = v.z / d; p[3] = v.w / d;
+#pragma unroll
+        for (int k = 0; k < 4; k++) c[k] = (int)(p[k] + __builtin_copysignf(0.49999997f, p[k]));
+    }
+    return ((uint32_t)c[0] & 0xffu) | (((uint32_t)c[1] & 0xffu) << 8) | (((uint32_t)c[2] & 0xffu) << 16) | ((uint32_t)c[3] << 24);
+}
+
 // ---- q8_1 (ggml 36-byte block) of 32 values held by 8 lanes x 4 registers; sub = lane & 7 -------------------------------
 // d = amax / 127, q = amax == 0 ? 0 : roundf(x / d), header half2(d, sum) with the butterfly sum. blk: the block's base.
 CAMX_DEV void q8_1_emit(f32x4 v, uint8_t * blk, int sub) {
@@ -137,7 +160,7 @@ CAMX_DEV void q8_1_emit(f32x4 v, uint8_t * blk, int sub) {
     const float sum = group32_sum(v);
     const float d = amax / 127.0f;
     uint32_t q = 0;
-    if (amax != 0.0f) { f32x4 t; t.x = v.x / d; t.y = v.y / d; t.z = v.z / d; t.w = v.w / d; q = pack_round_i8x4(t); }
+    if (amax != 0.0f) q = q8_codes4(v, d);
     *(uint32_t *)(blk + 4 + 4 * sub) = q;
     if (sub == 0) *(uint32_t *)blk = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
 }

@@ -261,25 +261,37 @@ __global__ void __launch_bounds__(256) gdn_l2_k(const void * __restrict__ x, voi
     }
 }
 
-// K = 128 (the GDN key heads): a half-wave per head, two heads per wave, 128-bit accesses. The logical threads past 128
-// hold zeros in the reference's tree, so the four group sums of the head added in order are the whole sum.
-template <bool BF16>
+// K = 128 (the GDN key heads): a half-wave per head, two heads per wave, 128-bit accesses, U heads per half-wave with all
+// their loads issued first (a head is only 256 - 512 bytes). The logical threads past 128 hold zeros in the reference's
+// tree, so the four group sums of the head added in order are the whole sum.
+template <bool BF16, int U>
 __global__ void __launch_bounds__(256) gdn_l2_128(const void * __restrict__ x, void * __restrict__ y, int heads, int ldx, float rs, int total) {
     const int lane = slot_of(threadIdx.x & 63), l = lane & 31;
-    const int t = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
-    const bool active = t < total;
-    const int tc = active ? t : 0;
-    const int tt = tc / heads, hh = tc - tt * heads;
-    const size_t xo = (size_t)tt * ldx + (size_t)hh * 128 + 4 * l, yo = (size_t)tc * 128 + 4 * l;
-    const f32x4 v = BF16 ? unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)((const uint16_t *)x + xo)))
-                         : __builtin_nontemporal_load((const f32x4 *)((const float *)x + xo));
-    f32x4 ss;
-    ss.x = __builtin_fmaf(v.x, v.x, 0.0f); ss.y = __builtin_fmaf(v.y, v.y, 0.0f); ss.z = __builtin_fmaf(v.z, v.z, 0.0f); ss.w = __builtin_fmaf(v.w, v.w, 0.0f);
-    const float tot = half_groups_in_order<4>(group32_sum(ss), lane & 32);
-    const float scale = rsqrt_exact(tot / 128.0f + rs), s2 = 1.0f / sqrtf(128.0f);
-    f32x4 o;
-    o.x = (scale * v.x) * s2; o.y = (scale * v.y) * s2; o.z = (scale * v.z) * s2; o.w = (scale * v.w) * s2;
-    if (active) { if (BF16) *(u32x2 *)((uint16_t *)y + yo) = pack_bf16x4_rne(o); else *(f32x4 *)((float *)y + yo) = o; }
+    const int span = gridDim.x * 8;                                  // heads per pass of the grid
+    const int t0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+    f32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int t = t0 + u * span, tc = t < total ? t : 0;
+        const int tt = tc / heads, hh = tc - tt * heads;
+        const size_t xo = (size_t)tt * ldx + (size_t)hh * 128 + 4 * l;
+        v[u] = BF16 ? unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)((const uint16_t *)x + xo)))
+                    : __builtin_nontemporal_load((const f32x4 *)((const float *)x + xo));
+    }
+    const float s2 = 1.0f / sqrtf(128.0f);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int t = t0 + u * span;
+        f32x4 ss;
+        ss.x = __builtin_fmaf(v[u].x, v[u].x, 0.0f); ss.y = __builtin_fmaf(v[u].y, v[u].y, 0.0f);
+        ss.z = __builtin_fmaf(v[u].z, v[u].z, 0.0f); ss.w = __builtin_fmaf(v[u].w, v[u].w, 0.0f);
+        const float tot = half_groups_in_order<4>(group32_sum(ss), lane & 32);
+        const float scale = rsqrt_exact(tot / 128.0f + rs);
+        f32x4 o;
+        o.x = (scale * v[u].x) * s2; o.y = (scale * v[u].y) * s2; o.z = (scale * v[u].z) * s2; o.w = (scale * v[u].w) * s2;
+        const size_t yo = (size_t)t * 128 + 4 * l;
+        if (t < total) { if (BF16) *(u32x2 *)((uint16_t *)y + yo) = pack_bf16x4_rne(o); else *(f32x4 *)((float *)y + yo) = o; }
+    }
 }
 
 // ---- hyper-connection glue (kernels/prefill_glue.hip:172-206) -----------------------------------------------------------------
@@ -363,9 +375,27 @@ __global__ void __launch_bounds__(256) residual3_k(const float * __restrict__ x,
     const long step = (long)gridDim.x * 256;
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += step) out[i] = (x[i] + bf2f(m[i])) + bf2f(y[i]);
 }
+// four values per thread (16-byte x / out, 8-byte m / y); every stream is read once
+__global__ void __launch_bounds__(256) residual3_vec(const float * __restrict__ x, const uint16_t * __restrict__ m, const uint16_t * __restrict__ y,
+                                                     float * __restrict__ out, long n4) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    if (q >= n4) return;
+    const f32x4 xv = __builtin_nontemporal_load((const f32x4 *)x + q);
+    const f32x4 mv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)m + q)), yv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)y + q));
+    f32x4 o; o.x = (xv.x + mv.x) + yv.x; o.y = (xv.y + mv.y) + yv.y; o.z = (xv.z + mv.z) + yv.z; o.w = (xv.w + mv.w) + yv.w;
+    ((f32x4 *)out)[q] = o;
+}
 __global__ void __launch_bounds__(256) cast_bf16_k(const float * __restrict__ x, uint16_t * __restrict__ out, long n) {
     const long step = (long)gridDim.x * 256;
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += step) out[i] = f2bf(x[i]);
+}
+// eight values per thread: two 16-byte loads, one 16-byte store
+__global__ void __launch_bounds__(256) cast_bf16_vec(const float * __restrict__ x, uint16_t * __restrict__ out, long n8) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    if (q >= n8) return;
+    const f32x4 a = __builtin_nontemporal_load((const f32x4 *)x + 2 * q), b = __builtin_nontemporal_load((const f32x4 *)x + 2 * q + 1);
+    const u32x2 lo = pack_f2bf_x4(a), hi = pack_f2bf_x4(b);
+    ((u32x4 *)out)[q] = (u32x4){lo.x, lo.y, hi.x, hi.y};
 }
 __global__ void __launch_bounds__(256) copy_cols_bf16_k(const uint16_t * __restrict__ in, int ld_in, int c_in, uint16_t * __restrict__ out, int ld_out,
                                                         int c_out, int n, long rows) {
@@ -374,6 +404,14 @@ __global__ void __launch_bounds__(256) copy_cols_bf16_k(const uint16_t * __restr
         const long r = i / n, c = i - r * n;
         out[r * ld_out + c_out + c] = in[r * ld_in + c_in + c];
     }
+}
+// every offset and width a multiple of 8 values: 16-byte units
+__global__ void __launch_bounds__(256) copy_cols_bf16_vec(const u32x4 * __restrict__ in, int ld_in, int c_in, u32x4 * __restrict__ out, int ld_out,
+                                                          int c_out, int n, long rows) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * n) return;
+    const long r = i / n, c = i - r * n;
+    out[r * ld_out + c_out + c] = __builtin_nontemporal_load(in + r * ld_in + c_in + c);
 }
 // out = ((x + m) + mlp) + (pos[r] >= 0 ? ys[pos[r]] : 0), four columns per thread (d % 4 == 0)
 __global__ void __launch_bounds__(256) residual_slices_fwd_k(const float * __restrict__ x, const uint16_t * __restrict__ m, const uint16_t * __restrict__ mlp,
@@ -391,6 +429,8 @@ __global__ void __launch_bounds__(256) residual_slices_fwd_k(const float * __res
     o.z = ((xv.z + mv.z) + lv.z) + sv.z; o.w = ((xv.w + mv.w) + lv.w) + sv.w;
     *(f32x4 *)(out + e) = o;
 }
+
+__attribute__((visibility("hidden"))) int silu_mul_bf16_wide(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st);   // quant.hip
 
 extern "C" {
 
@@ -411,6 +451,8 @@ int camx_gg_silu_mul(const float * g, const float * u, float * h, int n, hipStre
 int camx_silu_mul_bf16(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st) {
     if (!gu || !act || H < 1 || n < 0 || n % H) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
+    const int wide = silu_mul_bf16_wide(gu, act, H, n, st);      // large inputs: bf16(silu g) from a table in LDS
+    if (wide != CAMX_EINVAL) return wide;
     const int vec = H % 4 == 0 && !(((uintptr_t)gu | (uintptr_t)act) & 7);
     silu_mul_bf16_k<<<GRID_1D((n + 3) / 4), dim3(256), 0, st>>>(gu, act, H, n, vec);
     CAMX_LAUNCH_RET();
@@ -463,8 +505,13 @@ int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs
     const dim3 grid((total + 3) / 4), block(256);
     const bool vec = K % 4 == 0 && ldx % 4 == 0 && !((uintptr_t)x & (bf16 ? 7 : 15)) && !((uintptr_t)y & (bf16 ? 7 : 15));
     if (vec && K == 128) {
-        const dim3 g2((total + 7) / 8);
-        if (bf16) gdn_l2_128<true><<<g2, block, 0, st>>>(x, y, heads, ldx, rs, total); else gdn_l2_128<false><<<g2, block, 0, st>>>(x, y, heads, ldx, rs, total);
+        if (total >= 32768) {                                         // enough heads to fill the chip four times over: four heads per half-wave
+            const dim3 g4((total + 31) / 32);
+            if (bf16) gdn_l2_128<true, 4><<<g4, block, 0, st>>>(x, y, heads, ldx, rs, total); else gdn_l2_128<false, 4><<<g4, block, 0, st>>>(x, y, heads, ldx, rs, total);
+        } else {
+            const dim3 g2((total + 7) / 8);
+            if (bf16) gdn_l2_128<true, 1><<<g2, block, 0, st>>>(x, y, heads, ldx, rs, total); else gdn_l2_128<false, 1><<<g2, block, 0, st>>>(x, y, heads, ldx, rs, total);
+        }
         CAMX_LAUNCH_RET();
     }
     if (bf16) { if (vec) gdn_l2_k<true, true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); else gdn_l2_k<true, false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); }
@@ -496,19 +543,26 @@ int camx_embedding_f32(const int * tok, const float * emb, float * out, int D, i
 int camx_residual3(const float * x, const uint16_t * m, const uint16_t * y, float * out, long n, hipStream_t st) {
     if (!x || !m || !y || !out || n < 0) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
-    residual3_k<<<GRID_1D(n), dim3(256), 0, st>>>(x, m, y, out, n);
+    if (n % 4 == 0 && n / 4 < 0x7fffffffL * 256 && !(((uintptr_t)x | (uintptr_t)out) & 15) && !(((uintptr_t)m | (uintptr_t)y) & 7))
+        residual3_vec<<<dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, st>>>(x, m, y, out, n / 4);
+    else residual3_k<<<GRID_1D(n), dim3(256), 0, st>>>(x, m, y, out, n);
     CAMX_LAUNCH_RET();
 }
 int camx_cast_bf16(const float * x, uint16_t * out, long n, hipStream_t st) {
     if (!x || !out || n < 0) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
-    cast_bf16_k<<<GRID_1D(n), dim3(256), 0, st>>>(x, out, n);
+    if (n % 8 == 0 && n / 8 < 0x7fffffffL * 256 && !(((uintptr_t)x | (uintptr_t)out) & 15))
+        cast_bf16_vec<<<dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, st>>>(x, out, n / 8);
+    else cast_bf16_k<<<GRID_1D(n), dim3(256), 0, st>>>(x, out, n);
     CAMX_LAUNCH_RET();
 }
 int camx_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out, int ld_out, int c_out, int n, long rows, hipStream_t st) {
     if (!in || !out || n < 0 || rows < 0 || c_in < 0 || c_out < 0 || c_in + n > ld_in || c_out + n > ld_out) return CAMX_EINVAL;
     if (n == 0 || rows == 0) return CAMX_OK;
-    copy_cols_bf16_k<<<GRID_1D(rows * n), dim3(256), 0, st>>>(in, ld_in, c_in, out, ld_out, c_out, n, rows);
+    if (!((ld_in | c_in | ld_out | c_out | n) & 7) && !(((uintptr_t)in | (uintptr_t)out) & 15) && rows * (n / 8) < 0x7fffffffL * 256)
+        copy_cols_bf16_vec<<<dim3((unsigned)((rows * (n / 8) + 255) / 256)), dim3(256), 0, st>>>((const u32x4 *)in, ld_in / 8, c_in / 8, (u32x4 *)out, ld_out / 8,
+                                                                                                c_out / 8, n / 8, rows);
+    else copy_cols_bf16_k<<<GRID_1D(rows * n), dim3(256), 0, st>>>(in, ld_in, c_in, out, ld_out, c_out, n, rows);
     CAMX_LAUNCH_RET();
 }
 // residual_slices_bwd (kernels/fuse.hip:35-47): dm = dmlp = bf16(dout) (f2bf), dys[pos[r]] = bf16(dout[r]) for the routed rows

@@ -68,7 +68,7 @@ __global__ void __launch_bounds__(256) q8_1_flat(const float * __restrict__ x, u
                 const float sum = group32_sum(q);
                 const float d = amax / 127.0f;
                 uint32_t codes = 0;
-                if (amax != 0.0f) { f32x4 t; t.x = q.x / d; t.y = q.y / d; t.z = q.z / d; t.w = q.w / d; codes = pack_round_i8x4(t); }
+                if (amax != 0.0f) codes = q8_codes4(q, d);
                 uint32_t * blk = stage[wv] + (8 * j + (lane >> 3)) * 9;
                 blk[1 + (lane & 7)] = codes;
                 if ((lane & 7) == 0) blk[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
@@ -365,6 +365,65 @@ static int silu_lut_ready(hipStream_t st) {
         done[dev] = true;
     }
     return CAMX_OK;
+}
+
+// act = bf16(bf16(silu g) * u) of wide bf16 rows [g (H) | u (H)] with the same table: persistent workgroups, a lane takes 8
+// values at a time (16 bytes of g, of u, of act) and keeps the next unit's loads in flight across the current one's lookups.
+// The products are rounded by the packed hardware convert; a unit that holds a NaN is redone with the canonical NaN.
+__global__ void __launch_bounds__(1024) silu_mul_lut(const uint16_t * __restrict__ gu, uint16_t * __restrict__ act, unsigned H8, unsigned n8) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    const unsigned S = gridDim.x * 1024u, dr = S / H8, dc = S % H8;
+    unsigned q = blockIdx.x * 1024u + threadIdx.x, r = q / H8, c = q % H8;
+    auto addr = [&](bool ok) { return ok ? (const u32x4 *)(gu + ((size_t)r * 2 * H8 + c) * 8) : (const u32x4 *)g_zero16; };
+    const u32x4 * p = addr(q < n8);
+    u32x4 g = __builtin_nontemporal_load(p), u = __builtin_nontemporal_load(q < n8 ? p + H8 : p);
+    for (unsigned i = threadIdx.x; i < 8192; i += 1024) ((u32x4 *)lut)[i] = ((const u32x4 *)g_silu_lut)[i];
+    __syncthreads();
+    while (q < n8) {
+        const size_t o = ((size_t)r * H8 + c) * 8;
+        const unsigned qn = q + S;
+        c += dc; r += dr;
+        if (c >= H8) { c -= H8; r++; }
+        const u32x4 * pn = addr(qn < n8);
+        const u32x4 gn = __builtin_nontemporal_load(pn), un = __builtin_nontemporal_load(qn < n8 ? pn + H8 : pn);
+        uint32_t pk[4];
+        bool nan = false;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t gw = g[k], uw = u[k];
+            const float a0 = __builtin_bit_cast(float, (uint32_t)lut[gw & 0xffffu] << 16) * __builtin_bit_cast(float, uw << 16);
+            const float a1 = __builtin_bit_cast(float, (uint32_t)lut[gw >> 16] << 16) * __builtin_bit_cast(float, uw & 0xffff0000u);
+            nan |= (a0 != a0) | (a1 != a1);
+            pk[k] = cvt_pk_bf16(a0, a1);
+        }
+        if (nan) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t gw = g[k], uw = u[k];
+                const float a0 = __builtin_bit_cast(float, (uint32_t)lut[gw & 0xffffu] << 16) * __builtin_bit_cast(float, uw << 16);
+                const float a1 = __builtin_bit_cast(float, (uint32_t)lut[gw >> 16] << 16) * __builtin_bit_cast(float, uw & 0xffff0000u);
+                pk[k] = (uint32_t)f2bf(a0) | ((uint32_t)f2bf(a1) << 16);
+            }
+        }
+        *(u32x4 *)(act + o) = (u32x4){pk[0], pk[1], pk[2], pk[3]};
+        g = gn; u = un; q = qn;
+    }
+}
+
+// the wide form of silu_mul_bf16 (rows of H = 8 k values, 16-byte aligned, at least 2^22 values); CAMX_EINVAL: not applicable
+__attribute__((visibility("hidden"))) int silu_mul_bf16_wide(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st) {
+    if (H % 8 || n < (1L << 22) || n / 8 >= 0x7fffffffL || (((uintptr_t)gu | (uintptr_t)act) & 15)) return CAMX_EINVAL;
+    static bool attr[64] = {false};
+    int dev = 0, ncu = 256;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return CAMX_EINVAL;
+    const int e = silu_lut_ready(st);
+    if (e) return e;
+    if (!attr[dev]) {
+        if (hipFuncSetAttribute((const void *)silu_mul_lut, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return CAMX_EINVAL;
+        attr[dev] = true;
+    }
+    silu_mul_lut<<<dim3((unsigned)ncu), dim3(1024), 131072, st>>>(gu, act, (unsigned)(H / 8), (unsigned)(n / 8));
+    return (int)hipGetLastError();
 }
 
 extern "C" {

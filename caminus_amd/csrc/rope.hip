@@ -8,6 +8,7 @@
 //
 // The frequency of pair j is powf(theta_scale, j) in the reference; here it is (float)pow((double)theta_scale, j), the
 // correctly rounded single-precision power, so a CPU libm that rounds powf correctly gives the same angle bits.
+#include <type_traits>
 #include "common.cuh"
 
 CAMX_DEV float rope_freq(float theta_scale, int j) { return (float)pow((double)theta_scale, (double)j); }
@@ -470,9 +471,87 @@ __global__ void __launch_bounds__(256) qk_nr_tokens_vec(NrArgs a) {
     }
 }
 
+// Prefill-sized batches of heads of at most 256 dims whose rotated width is a power of two (8 .. 256): the partner of
+// element i (i + nrot / 2 or i - nrot / 2) sits nrot / 8 lanes away, so the rotation is a lane exchange and nothing goes
+// through LDS but the token's cos / sin row. Lane p holds dims 4p .. 4p + 3; sin carries the sign of its half. A wave walks
+// heads wave, wave + 4, ..; two heads ahead are in flight.
+template <int XL> CAMX_DEV float nr_partner(float v) {
+    if (XL == 1) return lane_xor1(v);
+    if (XL == 2) return lane_xor2(v);
+    if (XL == 4) return lane_xor4(v);
+    if (XL == 8) return lane_xor8(v);
+    if (XL == 16) return lane_xor16(v);
+    return __shfl_xor(v, 32, 64);
+}
+template <bool BF16, int XL>
+__global__ void __launch_bounds__(256) qk_nr_tokens_fast(NrArgs a) {
+    __shared__ __attribute__((aligned(16))) float rc[128], rs[128];
+    typedef typename std::conditional<BF16, u32x2, f32x4>::type Raw;
+    const int tok = blockIdx.x, tid = threadIdx.x, lane = slot_of(tid & 63), wave = tid >> 6, nrot = 8 * XL, half = nrot / 2;
+    const int i0 = 4 * lane;
+    const bool on = i0 < a.D, rot = i0 < nrot;
+    auto load = [&](int h) {
+        Raw v = {};
+        if (h < a.heads && on) {
+            const size_t xo = ((size_t)tok * a.heads + h) * a.head_stride + i0;
+            if constexpr (BF16) v = __builtin_nontemporal_load((const u32x2 *)((const uint16_t *)a.x + xo));
+            else v = __builtin_nontemporal_load((const f32x4 *)((const float *)a.x + xo));
+        }
+        return v;
+    };
+    Raw r0 = load(wave), r1 = load(wave + 4);
+    f32x4 wv = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (on) wv = *(const f32x4 *)(a.w + i0);
+    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    if (tid < half) {
+        const float theta = pos * rope_freq(a.theta_scale, tid);
+        rc[tid] = cosf(theta); rs[tid] = sinf(theta);
+    }
+    __syncthreads();
+    f32x4 c4 = {1.0f, 1.0f, 1.0f, 1.0f}, s4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (rot) {
+        const int jj = i0 & (half - 1);
+        c4 = *(const f32x4 *)(rc + jj); s4 = *(const f32x4 *)(rs + jj);
+        if (i0 < half) { s4.x = -s4.x; s4.y = -s4.y; s4.z = -s4.z; s4.w = -s4.w; }
+    }
+    for (int h = wave; h < a.heads; h += 8) {
+        const Raw n0 = load(h + 8), n1 = load(h + 12);
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int hh = h + 4 * u;
+            if (hh < a.heads) {                                 // uniform per wave
+                const Raw raw = u ? r1 : r0;
+                f32x4 x;
+                if constexpr (BF16) x = unpack_bf16x4(raw); else x = raw;
+                f32x4 ss;
+                ss.x = __builtin_fmaf(x.x, x.x, 0.0f); ss.y = __builtin_fmaf(x.y, x.y, 0.0f); ss.z = __builtin_fmaf(x.z, x.z, 0.0f); ss.w = __builtin_fmaf(x.w, x.w, 0.0f);
+                const float tot = wave_groups_in_order(group32_sum(ss));
+                const float scale = rsqrt_exact(tot / (float)a.D + a.eps);
+                x.x = (scale * x.x) * wv.x; x.y = (scale * x.y) * wv.y; x.z = (scale * x.z) * wv.z; x.w = (scale * x.w) * wv.w;
+                f32x4 pr;
+                pr.x = nr_partner<XL>(x.x); pr.y = nr_partner<XL>(x.y); pr.z = nr_partner<XL>(x.z); pr.w = nr_partner<XL>(x.w);
+                f32x4 y = x;
+                if (rot) { y.x = x.x * c4.x + pr.x * s4.x; y.y = x.y * c4.y + pr.y * s4.y; y.z = x.z * c4.z + pr.z * s4.z; y.w = x.w * c4.w + pr.w * s4.w; }
+                if (on) {
+                    const size_t yo = ((size_t)tok * a.heads + hh) * a.D + i0;
+                    if (BF16) *(u32x2 *)((uint16_t *)a.out + yo) = pack_bf16x4_rne(y); else *(f32x4 *)((float *)a.out + yo) = y;
+                }
+            }
+        }
+        r0 = n0; r1 = n1;
+    }
+}
+
 static void launch_nr(const NrArgs & a, int io, hipStream_t st) {
     const int es = io ? 2 : 4;
     const bool vec = (a.D & 3) == 0 && (a.head_stride & 3) == 0 && ((uintptr_t)a.x & (4 * es - 1)) == 0 && ((uintptr_t)a.out & (4 * es - 1)) == 0;
+    if (vec && a.heads >= 8 && (long)a.T * a.heads >= 4096 && a.D <= 256 && a.nrot >= 8 && a.nrot <= a.D && (a.nrot & (a.nrot - 1)) == 0) {
+#define NR_FAST(XL) (io ? qk_nr_tokens_fast<true, XL><<<dim3(a.T), dim3(256), 0, st>>>(a) : qk_nr_tokens_fast<false, XL><<<dim3(a.T), dim3(256), 0, st>>>(a))
+        switch (a.nrot) { case 8: NR_FAST(1); break; case 16: NR_FAST(2); break; case 32: NR_FAST(4); break; case 64: NR_FAST(8); break;
+                          case 128: NR_FAST(16); break; default: NR_FAST(32); break; }
+#undef NR_FAST
+        return;
+    }
     if (vec && a.heads >= 8 && (long)a.T * a.heads >= 4096) {          // a prefill chunk: share the token's cos / sin among its heads
         if (io) qk_nr_tokens_vec<true><<<dim3(a.T), dim3(256), 0, st>>>(a); else qk_nr_tokens_vec<false><<<dim3(a.T), dim3(256), 0, st>>>(a);
         return;

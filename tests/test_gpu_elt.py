@@ -21,13 +21,20 @@ def test_swiglu(n):
     assert close_fp32(host(y32), O.silu_mul_f32(g, u))
 
 
-@pytest.mark.parametrize('R,H', [(4, 17408), (3, 7)])
+@pytest.mark.parametrize('R,H', [(4, 17408), (3, 7), (256, 17408), (1100, 4096)])
 def test_silu_mul_bf16(R, H):
+    """small inputs: the device's expf (one bf16 step); from 2^22 values on: the table of correctly rounded bf16(silu g), bit-equal
+    to the oracle wherever the host's expf is correctly rounded too, NaN and infinities included"""
     rng = np.random.default_rng(H)
-    gu = O.f2bf(outliers(rng, (R, 2 * H)))
+    gu = O.f2bf(outliers(rng, (R, 2 * H)) * np.float32(2))
+    gu[0, :6] = [0x7fc0, 0xffc1, 0x7f80, 0xff80, 0x0000, 0x8000]; gu[0, H:H + 6] = [0x3f80, 0x3f80, 0x0000, 0x3f80, 0x7f80, 0x7fa5]
     act = dev(np.zeros((R, H), np.uint16))
     call('camx_silu_mul_bf16', ptr(dev(gu)), ptr(act), I(H), L64(R * H))
-    assert close_16(host(act, np.uint16), O.silu_mul_bf16(gu), 'bf16')
+    want = O.silu_mul_bf16(gu); got = host(act, np.uint16)
+    fin = np.isfinite(O.bf2f(want))
+    assert np.array_equal(got[~fin], want[~fin])                   # NaN (canonical) and infinities exactly
+    assert close_16(got[fin], want[fin], 'bf16')
+    if R * H >= 1 << 22: assert (got == want).mean() > 0.9999
 
 
 def test_gate_mul():
@@ -58,14 +65,19 @@ def test_gdn_conv(T, C):
     assert close_fp32(host(y), ref_y) and bits_equal(host(sd), ref_st)
 
 
-@pytest.mark.parametrize('T,heads,K', [(16, 32, 128), (16, 48, 128), (3, 5, 256), (2, 3, 96)])
+@pytest.mark.parametrize('T,heads,K', [(16, 32, 128), (16, 48, 128), (3, 5, 256), (2, 3, 96), (1030, 32, 128), (683, 48, 128)])
 def test_gdn_l2(T, heads, K):
     rng = np.random.default_rng(K + heads)
     ldx = heads * K + 64
     x = outliers(rng, (T, ldx))
     y = dev(np.zeros((T * heads, K), np.float32))
     call('camx_pf_gdn_l2', ptr(dev(x)), ptr(y), I(heads), I(K), I(ldx), F(np.float32(1e-6 / K)), I(T), I(0))
-    assert bits_equal(host(y), O.gdn_l2(x, T, heads, K, 1e-6, ldx=ldx))
+    ref = O.gdn_l2(x, T, heads, K, 1e-6, ldx=ldx)
+    assert bits_equal(host(y), ref)
+    if K == 128:                                                       # bf16 in / out (a prefill chunk's form)
+        xb = O.f2bf(x); yb = dev(np.zeros((T * heads, K), np.uint16))
+        call('camx_pf_gdn_l2', ptr(dev(xb)), ptr(yb), I(heads), I(K), I(ldx), F(np.float32(1e-6 / K)), I(T), I(1))
+        assert bits_equal(host(yb, np.uint16), O.f2bf(O.gdn_l2(O.bf2f(xb), T, heads, K, 1e-6, ldx=ldx)))
 
 
 def test_core_and_fuse():
@@ -80,13 +92,22 @@ def test_core_and_fuse():
     o = dev(np.zeros((T, D), np.float32))
     call('camx_residual3', ptr(dev(x)), ptr(dev(m)), ptr(dev(y)), ptr(o), L64(T * D))
     assert bits_equal(host(o), O.residual3(x, m, y))
+    o1 = dev(np.zeros(T * D - 3, np.float32))                          # a length that is no multiple of four: the element-wise form
+    call('camx_residual3', ptr(dev(x)), ptr(dev(m)), ptr(dev(y)), ptr(o1), L64(T * D - 3))
+    assert bits_equal(host(o1), O.residual3(x, m, y).reshape(-1)[:T * D - 3])
     x[0, :6] = [np.nan, np.inf, -np.inf, 1e-40, -np.nan, 3.3895314e38]
     c = dev(np.zeros((T, D), np.uint16))
     call('camx_cast_bf16', ptr(dev(x)), ptr(c), L64(T * D))
     assert bits_equal(host(c, np.uint16), O.f2bf(x))
+    c1 = dev(np.zeros(T * D - 5, np.uint16))
+    call('camx_cast_bf16', ptr(dev(x)), ptr(c1), L64(T * D - 5))
+    assert bits_equal(host(c1, np.uint16), O.f2bf(x).reshape(-1)[:T * D - 5])
     dst = rng.integers(0, 65536, (T, 64)).astype(np.uint16); dd = dev(dst)
     call('camx_copy_cols_bf16', ptr(dev(m)), I(D), I(5), ptr(dd), I(64), I(3), I(40), L64(T))
     assert bits_equal(host(dd, np.uint16), O.copy_cols_bf16(m, 5, dst, 3, 40))
+    dd2 = dev(dst)                                                     # offsets and width in whole 16-byte units
+    call('camx_copy_cols_bf16', ptr(dev(m)), I(D), I(8), ptr(dd2), I(64), I(16), I(40), L64(T))
+    assert bits_equal(host(dd2, np.uint16), O.copy_cols_bf16(m, 8, dst, 16, 40))
     ys = O.f2bf(outliers(rng, (4, D))); pos = np.array([-1, 0, 3, -1, 2, 1, -1, -1, 0], np.int32)
     x2 = outliers(rng, (T, D))
     for has in (True, False):
