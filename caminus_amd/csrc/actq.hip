@@ -14,9 +14,10 @@
 
 #define HSCALE 0.08837890625f      // bf16(1 / sqrt(128))
 
-struct PlainF32 { const float * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); } };
-struct PlainBF16 { const uint16_t * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); } };
+struct PlainF32 { static constexpr bool bf16_valued = false; const float * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); } };
+struct PlainBF16 { static constexpr bool bf16_valued = true; const uint16_t * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); } };
 struct SiluMulSrc {
+    static constexpr bool bf16_valued = true;      // the activation is rounded to bf16 as it is formed
     const uint16_t * gu; int ld, F;
     CAMX_DEV f32x4 operator()(int row, int k) const {
         const uint16_t * r = gu + (size_t)row * ld;
@@ -28,6 +29,7 @@ struct SiluMulSrc {
     }
 };
 struct RmsSrc {
+    static constexpr bool bf16_valued = false;
     const float * x; const float * w; float rstd; int d;
     CAMX_DEV f32x4 operator()(int row, int k) const {
         const f32x4 xv = *(const f32x4 *)(x + (size_t)row * d + k), wv = *(const f32x4 *)(w + k);
@@ -38,8 +40,17 @@ struct RmsSrc {
 
 #define CAMX_EACH4(OP) OP(x) OP(y) OP(z) OP(w)
 
-CAMX_DEV f32x4 rbf4(f32x4 v) { v.x = rbf(v.x); v.y = rbf(v.y); v.z = rbf(v.z); v.w = rbf(v.w); return v; }
-CAMX_DEV f32x4 rbf4_scaled(f32x4 v) { v.x = rbf(v.x * HSCALE); v.y = rbf(v.y * HSCALE); v.z = rbf(v.z * HSCALE); v.w = rbf(v.w * HSCALE); return v; }
+// fp32 -> bf16 -> fp32. _any: a NaN stays a NaN but its sign and payload are the hardware's (for values that only feed further
+// arithmetic, where nothing but NaN-ness survives); _canon: a NaN becomes 0x7fc00000, as the stored bf16 tensors have it
+CAMX_DEV f32x4 rbf4_any(f32x4 v) {
+    const uint32_t a = hw_pk_bf16(v.x, v.y), b = hw_pk_bf16(v.z, v.w);
+    f32x4 r;
+    r.x = __builtin_bit_cast(float, a << 16); r.y = __builtin_bit_cast(float, a & 0xffff0000u);
+    r.z = __builtin_bit_cast(float, b << 16); r.w = __builtin_bit_cast(float, b & 0xffff0000u);
+    return r;
+}
+CAMX_DEV f32x4 rbf4_canon(f32x4 v) { return unpack_bf16x4(pack_f2bf_x4(v)); }
+CAMX_DEV f32x4 scaled4(f32x4 v) { v.x *= HSCALE; v.y *= HSCALE; v.z *= HSCALE; v.w *= HSCALE; return v; }
 
 // u = bf16(H128 . bf16(source)) for the NR rounds of this half-wave; returns the lane's max |u| over its active chunks
 template <int NR, typename Src>
@@ -54,11 +65,26 @@ CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[
     float amax = 0.0f;
 #pragma unroll
     for (int c = 0; c < NR; c++) {
-        const f32x4 v = rbf4_scaled(hadamard128_l4(rbf4(u[c]), l, false));      // rbf4: autocast's bf16 input
+        const f32x4 in = Src::bf16_valued ? u[c] : rbf4_any(u[c]);                // autocast's bf16 input
+        const f32x4 v = rbf4_any(scaled4(hadamard128_l4(in, l, false)));
         u[c] = v;
         if (hw + 8 * c < nch) amax = fmaxf(amax, absmax4(v));
     }
     return amax;
+}
+
+// rintf(u / s) for a lane's four values. p = u * rcp(s) is within 8e-5 of the exact quotient while |p| < 256 (rcp: 1 ulp; one
+// more rounding), the IEEE quotient within 1.6e-5 of it, and half-integers are floats: when p is farther than 3e-4 from every
+// half-integer, rintf of the two agree. Other lanes (about one value in 1600, and infinities / NaN) divide.
+CAMX_DEV f32x4 rint_div4(f32x4 u, float s, float s_rcp) {
+    f32x4 p = {u.x * s_rcp, u.y * s_rcp, u.z * s_rcp, u.w * s_rcp};
+    f32x4 r = {rintf(p.x), rintf(p.y), rintf(p.z), rintf(p.w)};
+    bool safe = true;
+#define S_(e) safe &= (fabsf(p.e - r.e) <= 0.4997f) & (fabsf(p.e) < 256.0f);
+    CAMX_EACH4(S_)
+#undef S_
+    if (!safe) { r.x = rintf(u.x / s); r.y = rintf(u.y / s); r.z = rintf(u.z / s); r.w = rintf(u.w / s); }
+    return r;
 }
 
 // row-wide max (order-free); lds: 4 floats
@@ -78,7 +104,7 @@ CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * 
     const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
     f32x4 u[NR];
     const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u), lds);
-    const float s = fmaxf(amax * clip / (float)qmax, 1e-8f);
+    const float s = fmaxf(amax * clip / (float)qmax, 1e-8f), s_rcp = __builtin_amdgcn_rcpf(s);
     if (tid == 0 && s_out) s_out[row] = s;
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
 #pragma unroll
@@ -86,7 +112,8 @@ CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * 
         const int ch = hw + 8 * c;
         if (ch < nch) {
             f32x4 q;
-#define Q_(e) q.e = fminf(fmaxf(rintf(u[c].e / s), lo), hi);
+            f32x4 r = rint_div4(u[c], s, s_rcp);
+#define Q_(e) q.e = fminf(fmaxf(r.e, lo), hi);
             CAMX_EACH4(Q_)
 #undef Q_
             if (y) { f32x4 d; d.x = q.x * s; d.y = q.y * s; d.z = q.z * s; d.w = q.w * s; *(u32x2 *)(y + (size_t)row * K + ch * 128 + 4 * l) = pack_f2bf_x4(d); }
@@ -179,10 +206,10 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
             f32x4 d;
             int bit = 4 * c;
 #define V_(e) { float v = gv[c].e * ((inside >> bit) & 1u ? 1.0f : 0.0f); bit++; \
-                if (fabsf(u[c].e) == amax && u[c].e != 0.0f) v += u[c].e > 0.0f ? coef : -coef; d.e = rbf(v); }
+                if (fabsf(u[c].e) == amax && u[c].e != 0.0f) v += u[c].e > 0.0f ? coef : -coef; d.e = v; }
             CAMX_EACH4(V_)
 #undef V_
-            sink(row, ch * 128 + 4 * l, rbf4_scaled(hadamard128_l4(d, l, false)));
+            sink(row, ch * 128 + 4 * l, rbf4_canon(scaled4(hadamard128_l4(rbf4_any(d), l, false))));      // rbf4_any: the gradient of the bf16 tensor u
         }
     }
 }

@@ -98,16 +98,27 @@ CAMX_DEV float h2f_bits(uint16_t h) { return (float)__builtin_bit_cast(_Float16,
 // producing fma and the convert into one mixed-precision instruction (one rounding instead of two)
 CAMX_DEV float f16r(float x) { asm volatile("" : "+v"(x)); return (float)(_Float16)x; }
 
+// two fp32 -> packed bf16 by the hardware convert (round to nearest even, denormals kept); a NaN comes out quiet with its
+// payload, which is neither of the two software conventions above, so callers route NaN through those
+CAMX_DEV uint32_t hw_pk_bf16(float lo, float hi) {
+    const f32x2 in = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, bf16x2));
+}
+CAMX_DEV bool any_nan4(f32x4 v) { return (v.x != v.x) | (v.y != v.y) | (v.z != v.z) | (v.w != v.w); }
 CAMX_DEV u32x2 pack_bf16x4_rne(f32x4 v) {  // to_bf16 of four values, packed little-endian
     u32x2 r;
-    r.x = (uint32_t)to_bf16(v.x) | ((uint32_t)to_bf16(v.y) << 16);
-    r.y = (uint32_t)to_bf16(v.z) | ((uint32_t)to_bf16(v.w) << 16);
+    if (__builtin_expect(any_nan4(v), 0)) {
+        r.x = (uint32_t)to_bf16(v.x) | ((uint32_t)to_bf16(v.y) << 16);
+        r.y = (uint32_t)to_bf16(v.z) | ((uint32_t)to_bf16(v.w) << 16);
+    } else { r.x = hw_pk_bf16(v.x, v.y); r.y = hw_pk_bf16(v.z, v.w); }
     return r;
 }
-CAMX_DEV u32x2 pack_f2bf_x4(f32x4 v) {
+CAMX_DEV u32x2 pack_f2bf_x4(f32x4 v) {     // f2bf of four values (NaN -> 0x7fc0), packed little-endian
     u32x2 r;
-    r.x = (uint32_t)f2bf(v.x) | ((uint32_t)f2bf(v.y) << 16);
-    r.y = (uint32_t)f2bf(v.z) | ((uint32_t)f2bf(v.w) << 16);
+    if (__builtin_expect(any_nan4(v), 0)) {
+        r.x = (uint32_t)f2bf(v.x) | ((uint32_t)f2bf(v.y) << 16);
+        r.y = (uint32_t)f2bf(v.z) | ((uint32_t)f2bf(v.w) << 16);
+    } else { r.x = hw_pk_bf16(v.x, v.y); r.y = hw_pk_bf16(v.z, v.w); }
     return r;
 }
 CAMX_DEV u32x2 pack_f16x4(f32x4 v) {
@@ -196,15 +207,27 @@ CAMX_DEV f32x4 hadamard128_l4(f32x4 v, int lane, bool scale) {
     a = v.z; b = v.w; v.z = a + b; v.w = a - b;
     a = v.x; b = v.z; v.x = a + b; v.z = a - b;
     a = v.y; b = v.w; v.y = a + b; v.w = a - b;
-#define CAMX_HSTAGE(BIT, XOR)                                                                         \
-    {                                                                                                 \
-        const bool hi = (lane & BIT) != 0;                                                            \
-        const float p0 = XOR(v.x), p1 = XOR(v.y), p2 = XOR(v.z), p3 = XOR(v.w);                        \
-        v.x = hi ? p0 - v.x : v.x + p0; v.y = hi ? p1 - v.y : v.y + p1;                               \
-        v.z = hi ? p2 - v.z : v.z + p2; v.w = hi ? p3 - v.w : v.w + p3;                               \
+    // a cross-lane stage is (own + partner) in the lower lane and (partner - own) in the upper one: the upper lane's sign is
+    // flipped first (exact), then both add the partner's value, which rides on the add as a DPP source where a row move does it.
+    // (The elements are copied to scalars first: a bit cast applied straight to a vector element reads element 0.)
+    float e[4] = {v.x, v.y, v.z, v.w};
+#define CAMX_HSTAGE_DPP(BIT, CTRL)                                                                                  \
+    {                                                                                                                 \
+        const uint32_t m = (lane & BIT) ? 0x80000000u : 0u;                                                           \
+        _Pragma("unroll") for (int k = 0; k < 4; k++) {                                                               \
+            const float own = e[k];                                                                                   \
+            const float p = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, own), CTRL, 0xf, 0xf, true));  \
+            e[k] = p + __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, own) ^ m);                              \
+        }                                                                                                             \
     }
-    CAMX_HSTAGE(1, lane_xor1) CAMX_HSTAGE(2, lane_xor2) CAMX_HSTAGE(4, lane_xor4) CAMX_HSTAGE(8, lane_xor8) CAMX_HSTAGE(16, lane_xor16)
-#undef CAMX_HSTAGE
+    CAMX_HSTAGE_DPP(1, 0xB1) CAMX_HSTAGE_DPP(2, 0x4E) CAMX_HSTAGE_DPP(4, 0x141) CAMX_HSTAGE_DPP(8, 0x128)
+#undef CAMX_HSTAGE_DPP
+    {
+        const uint32_t m = (lane & 16) ? 0x80000000u : 0u;
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const float own = e[k]; e[k] = lane_xor16(own) + __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, own) ^ m); }
+    }
+    v.x = e[0]; v.y = e[1]; v.z = e[2]; v.w = e[3];
     if (scale) { v.x *= 0x1.6a09e6p-4f; v.y *= 0x1.6a09e6p-4f; v.z *= 0x1.6a09e6p-4f; v.w *= 0x1.6a09e6p-4f; }
     return v;
 }

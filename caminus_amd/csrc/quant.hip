@@ -196,10 +196,7 @@ __global__ void __launch_bounds__(256) silu_lut_fill() {
     g_silu_lut[i] = f2bf(g / (1.0f + e));
 }
 
-CAMX_DEV uint32_t cvt_pk_bf16(float lo, float hi) {
-    const f32x2 in = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, bf16x2));
-}
+CAMX_DEV uint32_t cvt_pk_bf16(float lo, float hi) { return hw_pk_bf16(lo, hi); }
 CAMX_DEV int round_i32(float v) { return (int)(v + __builtin_copysignf(0.49999997f, v)); }
 CAMX_DEV uint32_t pack_i8x4(int q0, int q1, int q2, int q3) {
     return __builtin_amdgcn_perm((uint32_t)q1, (uint32_t)q0, 0x0c0c0400u) | __builtin_amdgcn_perm((uint32_t)q3, (uint32_t)q2, 0x04000c0cu);

@@ -147,9 +147,8 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
 // wave instruction) and the fp16 results leave as 128-bit stores. Lane l (of 16) holds dims 8 l .. 8 l + 7: the 32-thread
 // butterfly of the norm sum is lane ^ 2, lane ^ 1 (quad permutes) and three in-register levels (the same pairs in the same
 // order as thread xor 16, 8, 4, 2, 1), the four group sums are fetched with bit-mask swizzles and added in order, and the
-// NeoX partner dim i ^ 64 sits in lane l ^ 8 (row_ror:8). Each wave issues the loads of all its heads (up to RB_STEPS
+// NeoX partner dim i ^ 64 sits in lane l ^ 8 (row_ror:8). Each wave issues the loads of all its heads (up to STEPS
 // wave steps) before the token's cos / sin row is computed, so the row's bytes are in flight during the trigonometry.
-#define RB_STEPS 5
 CAMX_DEV float swz_group(float v, int j) {        // every lane of a 16-lane row reads the row's lane 4 j + (lane & 3)
     const int i = __builtin_bit_cast(int, v);
     switch (j) {
@@ -183,8 +182,9 @@ template <int S> CAMX_DEV float row_lane_bcast(float v) {   // every lane of a 1
 // TPW tokens per workgroup. With four, wave w computes the cos / sin row of token w while every wave's first loads are in
 // flight, one barrier publishes the four rows, and then each wave walks the four tokens on its own, loading token i + 1's
 // heads before it does token i's arithmetic. With one (small batches), wave 0 computes the row.
-template <bool YARN, int TPW>
-__global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
+// F32IN: fp32 rows (two 128-bit loads per lane and step), else bf16 rows (one). STEPS wave steps of 16 heads per pass.
+template <bool YARN, int TPW, bool F32IN, int STEPS>
+__global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[TPW][64];
     __shared__ __attribute__((aligned(16))) float rs[TPW][64];
     __shared__ __attribute__((aligned(16))) float nrm[256];                  // q_norm | k_norm
@@ -192,15 +192,22 @@ __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
     const int items = a.nh + 2 * a.nkv, nqk = a.nh + a.nkv;
     const size_t M = (size_t)a.nkv * 128;
     const int lo = 128 * hq + 8 * l16;                                      // this lane's element offset inside a wave step
-    const int nchunk = (items + 16 * RB_STEPS - 1) / (16 * RB_STEPS);       // a row longer than 80 heads takes several passes
-    u32x4 xin[RB_STEPS], xnext[RB_STEPS];
-    auto load = [&](u32x4 (&buf)[RB_STEPS], int tok, int base) {
-        const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)tok * a.ldq;
+    const int nchunk = (items + 16 * STEPS - 1) / (16 * STEPS);       // a row longer than 80 heads takes several passes
+    constexpr int NW = F32IN ? 2 : 1;
+    u32x4 xin[STEPS][NW], xnext[STEPS][NW];
+    auto load = [&](u32x4 (&buf)[STEPS][NW], int tok, int base) {
 #pragma unroll
-        for (int s = 0; s < RB_STEPS; s++) {                                // wave step s: heads base + 16 s + 4 wave + (0 .. 3)
+        for (int s = 0; s < STEPS; s++) {                                // wave step s: heads base + 16 s + 4 wave + (0 .. 3)
             const int h0 = base + 16 * s + 4 * wave;
-            buf[s] = (u32x4){0u, 0u, 0u, 0u};
-            if (tok < a.n && h0 + hq < items) buf[s] = __builtin_nontemporal_load((const u32x4 *)(rowb + (size_t)h0 * 128 + lo));
+            const bool ok = tok < a.n && h0 + hq < items;
+#pragma unroll
+            for (int w = 0; w < NW; w++) buf[s][w] = (u32x4){0u, 0u, 0u, 0u};
+            if (ok) {
+                if (F32IN) {
+                    const float * p = (const float *)a.qkv + (size_t)tok * a.ldq + (size_t)h0 * 128 + lo;
+                    buf[s][0] = __builtin_nontemporal_load((const u32x4 *)p); buf[s][NW - 1] = __builtin_nontemporal_load((const u32x4 *)(p + 4));
+                } else buf[s][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)a.qkv + (size_t)tok * a.ldq + (size_t)h0 * 128 + lo));
+            }
         }
     };
     load(xin, t0, 0);
@@ -217,9 +224,9 @@ __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
     __syncthreads();
     const float eps = a.par[257];
     for (int it = 0; it < TPW * nchunk; it++) {
-        const int ti = it / nchunk, base = (it - ti * nchunk) * 16 * RB_STEPS, t = t0 + ti;
+        const int ti = it / nchunk, base = (it - ti * nchunk) * 16 * STEPS, t = t0 + ti;
         if (t >= a.n) break;
-        if (it + 1 < TPW * nchunk) { const int tn = (it + 1) / nchunk; load(xnext, t0 + tn, ((it + 1) - tn * nchunk) * 16 * RB_STEPS); }
+        if (it + 1 < TPW * nchunk) { const int tn = (it + 1) / nchunk; load(xnext, t0 + tn, ((it + 1) - tn * nchunk) * 16 * STEPS); }
         const int pos = a.pos ? a.pos[t] : a.pos0 + t;
         uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
         uint16_t * qw = a.q16 + (size_t)t * a.nh * 128;
@@ -229,11 +236,16 @@ __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
         s4[0] = *(const f32x4 *)(rs[ti] + j0); s4[1] = *(const f32x4 *)(rs[ti] + j0 + 4);
         if (l16 < 8) { s4[0] = -s4[0]; s4[1] = -s4[1]; }                    // dims below 64 take -(x1 s): the sign moves into s
         // phase 1: the sum of squares of every step's heads (V heads included: their sums are never used)
-        float x[RB_STEPS][8], tot[RB_STEPS];
+        float x[STEPS][8], tot[STEPS];
 #pragma unroll
-        for (int s = 0; s < RB_STEPS; s++) {
+        for (int s = 0; s < STEPS; s++) {
+            if (F32IN) {
 #pragma unroll
-            for (int p = 0; p < 4; p++) { x[s][2 * p] = __builtin_bit_cast(float, xin[s][p] << 16); x[s][2 * p + 1] = __builtin_bit_cast(float, xin[s][p] & 0xffff0000u); }
+                for (int p = 0; p < 4; p++) { const uint32_t b0 = xin[s][0][p], b1 = xin[s][NW - 1][p]; x[s][p] = __builtin_bit_cast(float, b0); x[s][4 + p] = __builtin_bit_cast(float, b1); }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 4; p++) { const uint32_t b = xin[s][0][p]; x[s][2 * p] = __builtin_bit_cast(float, b << 16); x[s][2 * p + 1] = __builtin_bit_cast(float, b & 0xffff0000u); }
+            }
             float sq[8];
 #pragma unroll
             for (int k = 0; k < 8; k++) sq[k] = x[s][k] * x[s][k];
@@ -249,15 +261,18 @@ __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
         // phase 2: one IEEE sqrt + divide per row for all steps: lane s of a row takes step s, the row reads it back
         float tv = tot[0];
 #pragma unroll
-        for (int s = 1; s < RB_STEPS; s++) tv = l16 == s ? tot[s] : tv;
+        for (int s = 1; s < STEPS; s++) tv = l16 == s ? tot[s] : tv;
         const float sc = rsqrt_exact(tv / 128 + eps);
-        float scale[RB_STEPS];
-        scale[0] = row_lane_bcast<0>(sc); scale[1] = row_lane_bcast<1>(sc); scale[2] = row_lane_bcast<2>(sc);
-        scale[3] = row_lane_bcast<3>(sc); scale[4] = row_lane_bcast<4>(sc);
-        static_assert(RB_STEPS == 5, "the broadcasts above are written out for five steps");
+        float scale[STEPS];
+        static_assert(STEPS <= 5, "the broadcasts below are written out for at most five steps");
+        scale[0] = row_lane_bcast<0>(sc);
+        if (STEPS > 1) scale[1 % STEPS] = row_lane_bcast<1>(sc);
+        if (STEPS > 2) scale[2 % STEPS] = row_lane_bcast<2>(sc);
+        if (STEPS > 3) scale[3 % STEPS] = row_lane_bcast<3>(sc);
+        if (STEPS > 4) scale[4 % STEPS] = row_lane_bcast<4>(sc);
         // phase 3: scale, rotate, convert, store
 #pragma unroll
-        for (int s = 0; s < RB_STEPS; s++) {
+        for (int s = 0; s < STEPS; s++) {
             const int h0 = base + 16 * s + 4 * wave;                        // wave-uniform
             if (h0 >= items) break;
             u32x4 out;
@@ -298,7 +313,9 @@ __global__ void __launch_bounds__(256) qk_rope_bf16_tokens(RopeArgs a) {
             }
         }
 #pragma unroll
-        for (int s = 0; s < RB_STEPS; s++) xin[s] = xnext[s];
+        for (int s = 0; s < STEPS; s++)
+#pragma unroll
+            for (int w = 0; w < NW; w++) xin[s][w] = xnext[s][w];
     }
 }
 
@@ -582,13 +599,17 @@ static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st)
 static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bool bf16in = false) {
     if (rope_check(a, q8, bf16in)) return CAMX_EINVAL;
     if (a.n == 0) return CAMX_OK;
-    const bool wide = bf16in && !q8 && !a.page_table && (a.ldq & 7) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
+    const bool wide = !q8 && !a.page_table && (a.ldq & (bf16in ? 7 : 3)) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
                       ((uintptr_t)a.cache & 15) == 0;
-    if (wide && a.n >= 2048) {          // enough tokens to fill the chip four to a workgroup
+    if (wide && bf16in && a.n >= 2048) {          // enough tokens to fill the chip four to a workgroup
         const dim3 g4((a.n + 3) / 4);
-        if (yarn) qk_rope_bf16_tokens<true, 4><<<g4, dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false, 4><<<g4, dim3(256), 0, st>>>(a);
+        if (yarn) qk_rope_wide_tokens<true, 4, false, 5><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, false, 5><<<g4, dim3(256), 0, st>>>(a);
     }
-    else if (wide) { if (yarn) qk_rope_bf16_tokens<true, 1><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_bf16_tokens<false, 1><<<dim3(a.n), dim3(256), 0, st>>>(a); }
+    else if (wide && bf16in) { if (yarn) qk_rope_wide_tokens<true, 1, false, 5><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 1, false, 5><<<dim3(a.n), dim3(256), 0, st>>>(a); }
+    else if (wide && a.n >= 2048) {               // fp32 rows of a prefill chunk: the same kernel, three wave steps (48 heads) per pass
+        const dim3 g4((a.n + 3) / 4);
+        if (yarn) qk_rope_wide_tokens<true, 4, true, 3><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, true, 3><<<g4, dim3(256), 0, st>>>(a);
+    }
     else if (bf16in) rope_dispatch<true, 1>(a, yarn, q8, st);
     else rope_dispatch<false, 1>(a, yarn, q8, st);
     CAMX_LAUNCH_RET();

@@ -141,3 +141,17 @@ def test_residual_slices_bwd_and_autograd():
     out.backward(go)
     assert torch.equal(x.grad, go) and torch.equal(m.grad, go.bfloat16()) and torch.equal(mlp.grad, go.bfloat16())
     assert torch.equal(ys.grad[pd[sel].long()], go[sel].bfloat16())
+
+
+def test_cast_bf16_every_upper_half_with_edge_lower_halves():
+    """fp32 -> bf16 over every sign / exponent / top-mantissa pattern combined with the lower halves where rounding decides
+    (ties, one off a tie, all ones), NaN payloads and denormals included: 0x7fc0 for every NaN, nearest-even elsewhere"""
+    hi = np.arange(65536, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x7fff, 0x8000, 0x8001, 0xffff, 0x4000, 0xc000, 0x8000 - 2, 0x1234, 0xfedc, 0x8002], np.uint32)
+    x = (hi[:, None] | lows[None, :]).reshape(-1).view(np.float32)
+    c = dev(np.zeros(x.size, np.uint16))
+    call('camx_cast_bf16', ptr(dev(x)), ptr(c), L64(x.size))
+    assert bits_equal(host(c, np.uint16), O.f2bf(x))
+    c1 = dev(np.zeros(x.size - 1, np.uint16))                             # the element-wise form
+    call('camx_cast_bf16', ptr(dev(x)), ptr(c1), L64(x.size - 1))
+    assert bits_equal(host(c1, np.uint16), O.f2bf(x)[:-1])
