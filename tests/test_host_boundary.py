@@ -206,3 +206,55 @@ def test_yarn_mode_surface():
     with pytest.raises(ValueError):
         rope.yarn_table(64, 1e6, 4, 32768)
     assert rope.mscale(1.0) == 1.0 and rope.mscale(0.5) == 1.0
+
+
+# ---- the C entry points' own argument checks (host code only: nothing reaches a GPU) -----------------------------------------
+
+P = ctypes.c_void_p(0x7f0000001000)          # a well-aligned address that is never dereferenced
+NUL = ctypes.c_void_p(None)
+ODD = ctypes.c_void_p(0x7f0000001002)          # two-byte aligned only
+ODD1 = ctypes.c_void_p(0x7f0000001001)
+Ci, Cf, Cl = ctypes.c_int, ctypes.c_float, ctypes.c_long
+ST = ctypes.c_void_p(None)
+
+# name -> (arguments of an empty batch: accepted, returns 0 and launches nothing; [(position, bad value), ...]: each refused with 1)
+ENTRY_CASES = {
+    'camx_q3p_add_rms16': ([P, P, NUL, Ci(1), P, Cf(1e-6), P, P, Ci(2048), Ci(0)], [(0, NUL), (8, Ci(2047)), (8, Ci(4096)), (3, Ci(9)), (9, Ci(-1)), (7, NUL)]),
+    'camx_q35p_add_rms16': ([P, P, P, Cf(1e-6), P, P, Ci(5120), Ci(0)], [(0, NUL), (6, Ci(100)), (7, Ci(-1))]),
+    'camx_add_rms_q8_1': ([P, P, NUL, Ci(1), P, Cf(1e-6), P, P, P, Ci(2048), Ci(0)], [(9, Ci(48)), (4, NUL), (3, Ci(-1))]),
+    'camx_add_rms_bf16': ([P, P, P, Cf(1e-6), P, P, Ci(5120), Ci(0)], [(0, NUL), (2, NUL), (6, Ci(0)), (7, Ci(-2))]),
+    'camx_rmsnorm_f32': ([P, P, P, Ci(896), Cf(1e-6), Ci(0)], [(0, NUL), (2, NUL), (3, Ci(0)), (5, Ci(-1))]),
+    'camx_gg_quantize_q8_1': ([P, P, Cl(0), Ci(0), Cf(0), NUL], [(0, NUL), (1, NUL), (3, Ci(3)), (3, Ci(2)), (1, ODD), (2, Cl(-1))]),
+    'camx_q3p_swiglu': ([P, P, P, Ci(0)], [(0, NUL), (2, NUL), (3, Ci(-1))]),
+    'camx_silu_mul_bf16': ([P, P, Ci(17408), Cl(0)], [(0, NUL), (2, Ci(0)), (3, Cl(5))]),
+    'camx_q3p_qk_rope': ([P, Ci(5120), Ci(32), Ci(4), P, Ci(0), P, P, Ci(0), Ci(0)], [(0, NUL), (4, NUL), (1, Ci(100)), (8, Ci(-1))]),
+    'camx_q3p_qk_rope_q8': ([P, Ci(5120), Ci(32), Ci(4), P, Ci(0), P, P, P, Ci(0), Ci(0)], [(8, NUL), (0, NUL)]),
+    'camx_pf_qk_nr': ([P, Ci(512), Ci(24), P, Ci(256), Ci(64), Cf(0.5), Cf(1e-6), Ci(0), P, Ci(0), Ci(1)], [(4, Ci(513)), (5, Ci(63)), (5, Ci(258)), (1, Ci(128)), (11, Ci(2))]),
+    'camx_q3p_emb': ([P, Ci(1152), Ci(1000), P, P, Ci(2048), Ci(0)], [(0, NUL), (1, Ci(1000)), (5, Ci(2000)), (2, Ci(0))]),
+    'camx_emb_gather': ([P, Cl(1152), Ci(1000), P, P, P, Ci(2048), Ci(0), Ci(0)], [(8, Ci(4)), (8, Ci(-1)), (0, NUL), (1, Cl(1151))]),
+    'camx_embd_rows_iq4xs': ([P, P, Ci(1000), Ci(0), Ci(8), P, P], [(4, Ci(0)), (4, Ci(33)), (6, NUL), (5, NUL)]),
+    'camx_ple_rows_iq4nl': ([P, P, Ci(4), Ci(0), Ci(5), P, P], [(0, ODD1), (2, Ci(0)), (4, Ci(0)), (6, NUL)]),
+    'camx_hadamard128': ([P, P, Cl(0)], [(0, NUL), (2, Cl(-1))]),
+    'camx_gate_mul': ([P, P, P, Cl(0), Ci(256), Ci(512), Ci(256), Ci(2)], [(7, Ci(3)), (6, Ci(257)), (4, Ci(0))]),
+    'camx_residual3': ([P, P, P, P, Cl(0)], [(0, NUL), (4, Cl(-1))]),
+    'camx_cast_bf16': ([P, P, Cl(0)], [(1, NUL), (2, Cl(-1))]),
+    'camx_actq_fwd': ([P, Ci(1), P, P, P, Ci(2048), Cf(1.0), Ci(7), Ci(0)], [(5, Ci(100)), (5, Ci(8320)), (7, Ci(0)), (0, NUL), (8, Ci(-1))]),
+    'camx_actq_bwd': ([P, Ci(1), P, P, Ci(2048), Cf(1.0), Ci(7), Ci(0)], [(2, NUL), (3, NUL), (4, Ci(64))]),
+    'camx_silu_mul_actq_bwd': ([P, Ci(4096), Ci(2048), P, P, Cf(1.0), Ci(7), Ci(0)], [(1, Ci(4095)), (1, Ci(4000)), (4, NUL)]),
+    'camx_block_entry_bwd': ([P, P, P, P, Ci(14), P, P, P, Ci(896), Cf(1.0), Ci(7), Ci(0)], [(8, Ci(2048)), (4, Ci(13)), (4, Ci(18)), (6, NUL)]),
+    'camx_pf_hc_mean': ([P, P, P, P, P, Ci(0), Ci(4), Ci(2560), Cf(0.25)], [(1, NUL), (6, Ci(0)), (3, NUL)]),
+}
+
+
+def test_entry_points_accept_empty_batches_and_refuse_bad_arguments():
+    path = kernels.library_path()
+    if not os.path.isfile(path):
+        pytest.skip('libcamx.so is not built in this checkout (python -m caminus_amd.build)')
+    lib = ctypes.CDLL(path)
+    for name, case in ENTRY_CASES.items():
+        good, bad = case
+        fn = getattr(lib, name)
+        assert fn(*good, ST) == 0, name
+        for pos, val in bad:
+            args = list(good); args[pos] = val
+            assert fn(*args, ST) == 1, (name, pos)
