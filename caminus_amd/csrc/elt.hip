@@ -155,7 +155,8 @@ __global__ void __launch_bounds__(256) gdn_conv_vec(const void * __restrict__ x,
         const int tj = t0 - 3 + j;
         raw[j] = (u32x4){0u, 0u, 0u, 0u};
         if (j < nt + 3 && tj >= 0)
-            raw[j] = BF16 ? *(const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0) : *(const u32x4 *)((const float *)x + (size_t)tj * ldx + c0);
+            raw[j] = BF16 ? __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0))
+                          : __builtin_nontemporal_load((const u32x4 *)((const float *)x + (size_t)tj * ldx + c0));
     }
     f32x4 w4[VW];
 #pragma unroll
@@ -189,10 +190,8 @@ __global__ void __launch_bounds__(256) gdn_conv_vec(const void * __restrict__ x,
             }
             const size_t o = (size_t)(t0 + j) * ldy + c0;
             if (BF16) {
-                u32x4 ov;
-#pragma unroll
-                for (int p = 0; p < 4; p++) ov[p] = (uint32_t)to_bf16(r[2 * p]) | ((uint32_t)to_bf16(r[2 * p + 1]) << 16);
-                *(u32x4 *)((uint16_t *)y + o) = ov;
+                const u32x2 lo = pack_bf16x4_rne((f32x4){r[0], r[1], r[2], r[3]}), hi = pack_bf16x4_rne((f32x4){r[4 % VW], r[5 % VW], r[6 % VW], r[7 % VW]});
+                *(u32x4 *)((uint16_t *)y + o) = (u32x4){lo.x, lo.y, hi.x, hi.y};
             } else *(f32x4 *)((float *)y + o) = (f32x4){r[0], r[1], r[2], r[3]};
         }
     }

@@ -179,11 +179,59 @@ template <int S> CAMX_DEV float row_lane_bcast(float v) {   // every lane of a 1
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x10 | (S << 5)));
 }
 
+// the orthonormal 128-point Walsh-Hadamard transform of a head held by 16 lanes x 8 registers (element 8 l + k): stages
+// h = 1, 2, 4 pair registers, h = 8 .. 64 pair lanes l ^ 1 .. l ^ 8, in that order (the order of hadamard128_l4: same sums,
+// same bits); the upper lane of a pair flips its sign and both add the partner's value; then times 0x1.6a09e6p-4f
+CAMX_DEV void hadamard128_w8(float (&e)[8], int l16) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if (!(k & h)) { const float a = e[k], b = e[k + h]; e[k] = a + b; e[k + h] = a - b; }
+#define W8_STAGE(BIT, PARTNER)                                                                                   \
+    {                                                                                                              \
+        const uint32_t m = (l16 & BIT) ? 0x80000000u : 0u;                                                         \
+        _Pragma("unroll") for (int k = 0; k < 8; k++) {                                                            \
+            const float own = e[k];                                                                                \
+            e[k] = PARTNER(own) + __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, own) ^ m);                \
+        }                                                                                                          \
+    }
+#define W8_XOR4(x) __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x101F))
+    W8_STAGE(1, dpp_full<0xB1>) W8_STAGE(2, dpp_full<0x4E>) W8_STAGE(4, W8_XOR4) W8_STAGE(8, dpp_full<0x128>)
+#undef W8_XOR4
+#undef W8_STAGE
+#pragma unroll
+    for (int k = 0; k < 8; k++) e[k] *= 0x1.6a09e6p-4f;
+}
+// kv_q8_emit for a block of 32 values held by 4 lanes x 8 registers (sub = lane & 3): the same decisions and bytes
+CAMX_DEV void kv_q8_emit_w8(const float (&v)[8], uint8_t * blk, int sub, int * err, bool active) {
+    bool fin = true;
+    float m = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) { fin = fin && __builtin_isfinite(v[k]); m = fmaxf(m, fabsf(v[k])); }
+    m = fin ? m : INFINITY;
+    m = fmaxf(m, dpp_xor1(m)); const float amax = fmaxf(m, dpp_xor2(m));
+    const float d = amax / 127.0f;
+    const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+    const _Float16 stored = (_Float16)d;
+    const bool refuse = !__builtin_isfinite(amax) ||
+                        (amax != 0.0f && (d == 0.0f || !__builtin_isfinite(d) || !__builtin_isfinite(inv) || !__builtin_isfinite((float)stored)));
+    if (!active) return;
+    if (refuse) { if (sub == 0) atomicOr(err, 2); return; }
+    const f32x4 t0 = {v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv}, t1 = {v[4] * inv, v[5] * inv, v[6] * inv, v[7] * inv};
+    const uint32_t q0 = pack_round_i8x4(t0), q1 = pack_round_i8x4(t1);
+    uint16_t * o = (uint16_t *)(blk + 2 + 8 * sub);
+    o[0] = (uint16_t)q0; o[1] = (uint16_t)(q0 >> 16); o[2] = (uint16_t)q1; o[3] = (uint16_t)(q1 >> 16);
+    if (sub == 0) *(uint16_t *)blk = __builtin_bit_cast(uint16_t, stored);
+}
+
 // TPW tokens per workgroup. With four, wave w computes the cos / sin row of token w while every wave's first loads are in
 // flight, one barrier publishes the four rows, and then each wave walks the four tokens on its own, loading token i + 1's
 // heads before it does token i's arithmetic. With one (small batches), wave 0 computes the row.
 // F32IN: fp32 rows (two 128-bit loads per lane and step), else bf16 rows (one). STEPS wave steps of 16 heads per pass.
-template <bool YARN, int TPW, bool F32IN, int STEPS>
+// Q8: the Q8 cache rows (K through the Hadamard transform, V unrotated, both from fp16-rounded values) and q16 = fp16 of
+// the transformed q, as in qk_rope_tokens.
+template <bool YARN, int TPW, bool F32IN, int STEPS, bool Q8>
 __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[TPW][64];
     __shared__ __attribute__((aligned(16))) float rs[TPW][64];
@@ -276,6 +324,34 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
             const int h0 = base + 16 * s + 4 * wave;                        // wave-uniform
             if (h0 >= items) break;
             u32x4 out;
+            if constexpr (Q8) {
+                const int h = h0 + hq;                                      // this row of 16 lanes: one head
+                const bool isq = h < a.nh, isv = h >= nqk, active = h < items;
+                uint8_t * cwb = (uint8_t *)a.cache + (size_t)pos * (2 * (M / 32) * 34);
+                float v8[8];
+                if (isv) {
+#pragma unroll
+                    for (int k = 0; k < 8; k++) v8[k] = f16r(x[s][k]);
+                } else {
+                    const float * wp = nrm + (isq ? 0 : 128) + 8 * l16;
+                    const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        const float y1 = (scale[s] * x[s][k]) * (k < 4 ? w0[k] : w1[k - 4]);
+                        v8[k] = f16r(__builtin_fmaf(y1, k < 4 ? c4[0][k] : c4[1][k - 4], mul_ror8(y1, k < 4 ? s4[0][k] : s4[1][k - 4])));
+                    }
+                    hadamard128_w8(v8, l16);
+                }
+                if (isq) {
+#pragma unroll
+                    for (int p = 0; p < 4; p++) out[p] = pack_f16x2(v8[2 * p], v8[2 * p + 1]);
+                    if (active) *(u32x4 *)(qw + (size_t)h * 128 + 8 * l16) = out;
+                } else {
+                    const size_t b = isv ? M / 32 + (size_t)(h - nqk) * 4 + (l16 >> 2) : (size_t)(h - a.nh) * 4 + (l16 >> 2);
+                    kv_q8_emit_w8(v8, cwb + b * 34, l16 & 3, a.err, active);
+                }
+                continue;
+            }
             if (h0 >= nqk) {                                                // V heads only: fp16 copy
 #pragma unroll
                 for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[s][2 * p], x[s][2 * p + 1]);
@@ -599,16 +675,17 @@ static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st)
 static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bool bf16in = false) {
     if (rope_check(a, q8, bf16in)) return CAMX_EINVAL;
     if (a.n == 0) return CAMX_OK;
-    const bool wide = !q8 && !a.page_table && (a.ldq & (bf16in ? 7 : 3)) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
+    const bool wide = (!q8 || !bf16in) && !a.page_table && (a.ldq & (bf16in ? 7 : 3)) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
                       ((uintptr_t)a.cache & 15) == 0;
     if (wide && bf16in && a.n >= 2048) {          // enough tokens to fill the chip four to a workgroup
         const dim3 g4((a.n + 3) / 4);
-        if (yarn) qk_rope_wide_tokens<true, 4, false, 5><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, false, 5><<<g4, dim3(256), 0, st>>>(a);
+        if (yarn) qk_rope_wide_tokens<true, 4, false, 5, false><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, false, 5, false><<<g4, dim3(256), 0, st>>>(a);
     }
-    else if (wide && bf16in) { if (yarn) qk_rope_wide_tokens<true, 1, false, 5><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 1, false, 5><<<dim3(a.n), dim3(256), 0, st>>>(a); }
+    else if (wide && bf16in) { if (yarn) qk_rope_wide_tokens<true, 1, false, 5, false><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 1, false, 5, false><<<dim3(a.n), dim3(256), 0, st>>>(a); }
     else if (wide && a.n >= 2048) {               // fp32 rows of a prefill chunk: the same kernel, three wave steps (48 heads) per pass
         const dim3 g4((a.n + 3) / 4);
-        if (yarn) qk_rope_wide_tokens<true, 4, true, 3><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, true, 3><<<g4, dim3(256), 0, st>>>(a);
+        if (q8) { if (yarn) qk_rope_wide_tokens<true, 4, true, 3, true><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, true, 3, true><<<g4, dim3(256), 0, st>>>(a); }
+        else { if (yarn) qk_rope_wide_tokens<true, 4, true, 3, false><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, true, 3, false><<<g4, dim3(256), 0, st>>>(a); }
     }
     else if (bf16in) rope_dispatch<true, 1>(a, yarn, q8, st);
     else rope_dispatch<false, 1>(a, yarn, q8, st);

@@ -148,3 +148,36 @@ def test_qk_rope_bf16(nh, nkv, n, pos0, yarn, pad):
     assert close_16(gq, rq, 'f16') and close_16(gc[pos0:pos0 + n, :M], rc[pos0:pos0 + n, :M], 'f16')
     assert bits_equal(gc[:, M:], rc[:, M:])                              # V: an exact conversion
     assert not gc[:pos0].any() and not gc[pos0 + n:].any()
+
+
+@pytest.mark.parametrize('nh,nkv,yarn', [(32, 4, False), (13, 3, True)])
+def test_prefill_sized_rope_equals_the_small_batch_kernel(nh, nkv, yarn):
+    """2048 tokens in one launch (the wide kernels) against the same tokens in launches of 1024 (the decode-sized kernels): the
+    same bytes in q16 and in the fp16 and Q8 rows, refused blocks and the error word included"""
+    rng = np.random.default_rng(31 + nh)
+    n, pos0 = 2048, 17
+    tab = rope.yarn_table(128, 1e6, 4.0, 32768) if yarn else None
+    par = qk_par(rng, yarn_table=tab)
+    ldq = (nh + 2 * nkv) * 128
+    qkv = (rng.standard_normal((n, ldq)) * 1.3).astype(np.float32)
+    qkv[7, nh * 128 + 5] = np.inf                                         # a K block of token 7 and a V block of token 9 are refused
+    qkv[9, (nh + nkv) * 128 + 40] = np.nan
+    M = nkv * 128; rb = 2 * (M // 32) * 34; rows = pos0 + n + 3
+    pd, qd = dev(par), dev(qkv)
+    outs = []
+    for parts in ((n,), (1024, 1024)):
+        q16 = dev(np.zeros((n, nh, 128), np.uint16)); c16 = dev(np.zeros((rows, 2 * M), np.uint16))
+        q16b = dev(np.zeros((n, nh, 128), np.uint16)); c8 = dev(np.full((rows, rb), 0xa5, np.uint8)); err = dev(np.zeros(1, np.int32))
+        t = 0
+        for m in parts:
+            call('camx_q3p_qk_rope', ptr(qd[t:]), I(ldq), I(nh), I(nkv), ptr(pd), I(pos0 + t), ptr(q16[t:]), ptr(c16), I(m), I(int(yarn)))
+            call('camx_q3p_qk_rope_q8', ptr(qd[t:]), I(ldq), I(nh), I(nkv), ptr(pd), I(pos0 + t), ptr(q16b[t:]), ptr(c8), ptr(err), I(m), I(int(yarn)))
+            t += m
+        outs.append([host(q16, np.uint16), host(c16, np.uint16), host(q16b, np.uint16), host(c8), int(host(err)[0])])
+    wide, small = outs
+    assert wide[4] == 2 and small[4] == 2
+    for a, b in zip(wide[:4], small[:4]):
+        assert bits_equal(a, b)
+    blocks = wide[3].reshape(rows, 2 * M // 32, 34)
+    assert (blocks[pos0 + 7, 0:4] == 0xa5).all() and (blocks[pos0 + 9, M // 32 + 1] == 0xa5).all()    # the rotation spreads the infinity over its head
+    assert not (blocks[pos0 + 7, 4:] == 0xa5).all(1).any() and not (blocks[pos0 + 9, M // 32] == 0xa5).all() and not (blocks[pos0 + 8] == 0xa5).all(1).any()
