@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of each kernel of the step, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file
 # (KiB per dispatch, scaled by what the same counters read for the 256 MiB copy of --only copy_ref: FETCH_SIZE reads half
 # the bytes moved, WRITE_SIZE reads them all); the summaries are kept under profiles/
-HBM_TRAFFIC = {'add_rms_bf16': 252313030, 'qk_rope_bf16': 167927724, 'swiglu_mmq_q8_1': 366612011}
+HBM_TRAFFIC = {'add_rms_bf16': 252379913, 'qk_rope_bf16': 167966684, 'swiglu_mmq_q8_1': 366622147}
 I, F, L64 = C.c_int, C.c_float, C.c_int64
 NULL = C.c_void_p(None)
 
@@ -218,6 +218,135 @@ def extra_opsets(B):
     return out
 
 
+def prefill_scale_sweep(B):
+    """every entry point at a prefill-scale size (bench.py --only sweep): name -> {us, bytes, GBps, frac_of_8TBps}. Each is launched
+    30 times back to back over three copies of its buffers in rotation (a launch never finds its own lines in the Infinity Cache);
+    bytes are algorithmic (inputs read once, outputs written once)."""
+    import numpy as np
+    torch = B.torch; dev = B.dev
+    res = {}
+
+    def timeit(name, by, fns, reps=30):
+        for f in fns: f()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for k in range(reps): fns[k % len(fns)]()
+        b.record(); b.synchronize()
+        us = a.elapsed_time(b) * 1e3 / reps
+        res[name] = {'us': round(us, 2), 'bytes': int(by), 'GBps': round(by / us / 1e3, 1), 'frac_of_8TBps': round(by / us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+    def sets(mk): return [mk(i) for i in range(3)]
+    T = 4096
+    N = 2048
+    def mk(i):
+        x = B.acts((T, N), torch.float32, i); d = B.acts((T, 1, N), torch.float32, i + 10); nw = B.gamma(N, 3); h = torch.empty((T, N), device=dev); h16 = torch.empty((T, N), dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_q3p_add_rms16', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), _p(h), _p(h16), I(N), I(T))
+    timeit('q3p_add_rms16 4096x2048 S=1', T * N * (4 + 4 + 4 + 4 + 2), sets(mk))
+    def mk(i):
+        x = B.acts((T, N), torch.float32, i); d = B.acts((T, 8, N), torch.float32, i + 10); w = torch.rand((T, 8), device=dev); nw = B.gamma(N, 3); h16 = torch.empty((T, N), dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_q3p_add_rms16', _p(x), _p(d), _p(w), I(8), _p(nw), F(1e-6), NULL, _p(h16), I(N), I(T))
+    timeit('q3p_add_rms16 4096x2048 S=8 weighted', T * N * (4 + 32 + 4 + 2), sets(mk))
+    def mk(i):
+        x = B.acts((T, N), torch.float32, i); d = B.acts((T, 1, N), torch.float32, i + 10); nw = B.gamma(N, 3); q8 = torch.empty(T * N // 32 * 36, dtype=torch.uint8, device=dev)
+        return lambda: B.call('camx_add_rms_q8_1', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), NULL, NULL, _p(q8), I(N), I(T))
+    timeit('add_rms_q8_1 4096x2048', T * N * (4 + 4 + 4 + 1.125), sets(mk))
+    H = 5120
+    def mk(i):
+        x = B.acts((T, H), torch.float32, i); d = B.acts((T, H), torch.float32, i + 10); nw = B.gamma(H, 3); h = torch.empty((T, H), device=dev); h16 = torch.empty((T, H), dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_q35p_add_rms16', _p(x), _p(d), _p(nw), F(1e-6), _p(h), _p(h16), I(H), I(T))
+    timeit('q35p_add_rms16 4096x5120', T * H * (4 + 4 + 4 + 4 + 2), sets(mk))
+    def mk(i):
+        x = B.acts((2048 * 4, 2560), torch.float32, i); w = B.gamma(4 * 2560, 3); ybf = torch.empty((8192, 2560), dtype=torch.bfloat16, device=dev); scl = torch.empty(8192, device=dev)
+        return lambda: B.call('camx_pf_rms_mul', _p(x), _p(w), NULL, _p(ybf), _p(scl), I(8192), I(4), F(1e-6), I(2560))
+    timeit('pf_rms_mul 8192x2560 -> bf16', 8192 * 2560 * 6, sets(mk))
+    n = T * 8 * 768
+    def mk(i):
+        g = B.acts((n,), torch.float32, i); u = B.acts((n,), torch.float32, i + 5); y = torch.empty(n, dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_q3p_swiglu', _p(g), _p(u), _p(y), I(n))
+    timeit('q3p_swiglu 4096x6144', n * 10, sets(mk))
+    def mk(i):
+        gu = B.acts((T, 2 * 17408), torch.bfloat16, i); act = torch.empty((T, 17408), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_silu_mul_bf16', _p(gu), _p(act), I(17408), L64(T * 17408))
+    timeit('silu_mul_bf16 4096x17408', T * 17408 * 6, sets(mk))
+    def mk(i):
+        x = B.acts((n,), torch.float32, i); y = torch.empty(n // 32 * 36, dtype=torch.uint8, device=dev)
+        return lambda: B.call('camx_gg_quantize_q8_1', _p(x), _p(y), L64(n), I(0), F(0), NULL)
+    timeit('gg_quantize_q8_1 25M', n * 5.125, sets(mk))
+    K = 6144
+    def mk(i):
+        x = B.acts((T, K), torch.float32, i); y = torch.empty(K // 128 * T * 144, dtype=torch.uint8, device=dev)
+        return lambda: B.call('camx_quantize_mmq_q8_1', _p(x), NULL, _p(y), L64(K), L64(K), L64(0), L64(0), L64(K), I(T), I(1), I(0), I(1))
+    timeit('quantize_mmq_q8_1 4096x6144 DS4', T * K * 5.125, sets(mk))
+    nh, nkv = 32, 4; ldq = (nh + 2 * nkv) * 128
+    par, _ = yarn_par(torch, dev, 15, yarn=False)
+    def mk(i):
+        qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev); cache = torch.empty((T, 2 * nkv * 128), dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_q3p_qk_rope', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(0), _p(q16), _p(cache), I(T), I(0))
+    timeit('q3p_qk_rope 4096 tok f32 -> f16', T * ldq * 6, sets(mk))
+    rbq = 2 * (nkv * 128 // 32) * 34
+    def mk(i):
+        qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev); cache = torch.empty(T * rbq, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_q3p_qk_rope_q8', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(0), _p(q16), _p(cache), _p(err), I(T), I(0))
+    timeit('q3p_qk_rope_q8 4096 tok', T * (ldq * 4 + nh * 256 + rbq), sets(mk))
+    D = 256
+    def mk(i):
+        qg = B.acts((T * 24, 2 * D), torch.bfloat16, i); w4 = B.gamma(D, 2); o = torch.empty((T * 24, D), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_pf_qk_nr', _p(qg), I(2 * D), I(24), _p(w4), I(D), I(64), F(0.6), F(1e-6), I(0), _p(o), I(T), I(1))
+    timeit('pf_qk_nr 4096x24x256 bf16', T * 24 * D * 4, sets(mk))
+    def mk(i):
+        a = B.acts((T * 24, D), torch.bfloat16, i); qg = B.acts((T * 24, 2 * D), torch.bfloat16, i + 3); o = torch.empty((T * 24, D), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_gate_mul', _p(a), _p(qg), _p(o), L64(T * 24 * D), I(D), I(2 * D), I(D), I(2))
+    timeit('gate_mul 4096x24x256 bf16', T * 24 * D * 6, sets(mk))
+    Cc = 10240
+    def mk(i):
+        xc = B.acts((T, Cc), torch.bfloat16, i); wc = B.acts((Cc, 4), torch.float32, 45, frac=0); st = B.acts((Cc, 3), torch.float32, 46, frac=0); yc = torch.empty((T, Cc), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_pf_gdn_conv', _p(xc), _p(wc), _p(st), _p(yc), I(Cc), I(T), I(Cc), I(Cc), I(1))
+    timeit('pf_gdn_conv 4096x10240 bf16', T * Cc * 4, sets(mk))
+    def mk(i):
+        xc = B.acts((T, Cc), torch.bfloat16, i); o = torch.empty((T * 32, 128), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_pf_gdn_l2', _p(xc), _p(o), I(32), I(128), I(Cc), F(1e-6 / 128), I(T), I(1))
+    timeit('pf_gdn_l2 4096x32x128 bf16', T * 32 * 128 * 4, sets(mk))
+    M = 512
+    def mk(i):
+        k = B.acts((T, M), torch.float32, i); v = B.acts((T, M), torch.float32, i + 2); cache = torch.empty(T * 1088, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_own_kv_q8_append', _p(k), I(M), _p(v), I(M), I(M), _p(cache), I(0), I(T), _p(err), I(T))
+    timeit('own_kv_q8_append 4096x512', T * (M * 8 + 1088), sets(mk))
+    def mk(i):
+        x = B.acts((T * 36, 128), torch.float32, i); y = torch.empty_like(x)
+        return lambda: B.call('camx_hadamard128', _p(x), _p(y), L64(T * 36))
+    timeit('hadamard128 147456 heads', T * 36 * 128 * 8, sets(mk))
+    V = 151936
+    tab = torch.randint(0, 256, (V, 1152), device=dev, dtype=torch.uint8)
+    tab.view(V, 8, 144)[:, :, :4] = (torch.rand((V, 8, 2), device=dev) * 9e-3 + 1e-3).to(torch.float16).view(torch.uint8).view(V, 8, 4)
+    def mk(i):
+        toks = torch.randint(0, V, (T,), device=dev, dtype=torch.int32); x = torch.empty((T, N), device=dev)
+        return lambda: B.call('camx_q3p_emb', _p(tab), I(1152), I(V), _p(toks), _p(x), I(N), I(T))
+    timeit('q3p_emb 4096 rows Q4_K -> f32', T * (1152 + N * 4), sets(mk))
+    Kq = 2048; Mr = 8192
+    def mk(i):
+        x = B.acts((Mr, Kq), torch.bfloat16, i); y = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev); s = torch.empty(Mr, device=dev)
+        return lambda: B.call('camx_actq_fwd', _p(x), I(1), _p(y), _p(s), NULL, I(Kq), F(1.0), I(7), I(Mr))
+    timeit('actq_fwd bf16 8192x2048', Mr * Kq * 4, sets(mk))
+    def mk(i):
+        x = B.acts((Mr, Kq), torch.bfloat16, i); g = B.acts((Mr, Kq), torch.bfloat16, i + 1); dx = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_actq_bwd', _p(x), I(1), _p(g), _p(dx), I(Kq), F(1.0), I(7), I(Mr))
+    timeit('actq_bwd bf16 8192x2048', Mr * Kq * 6, sets(mk))
+    def mk(i):
+        gu = B.acts((Mr, 2 * Kq), torch.bfloat16, i); y = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev); s = torch.empty(Mr, device=dev); c = torch.empty((Mr, Kq // 2), dtype=torch.uint8, device=dev)
+        return lambda: B.call('camx_silu_mul_actq_fwd', _p(gu), I(2 * Kq), I(Kq), _p(y), _p(s), _p(c), F(1.0), I(7), I(Mr))
+    timeit('silu_mul_actq_fwd 8192x2048', Mr * Kq * 6.5, sets(mk))
+    def mk(i):
+        gu = B.acts((Mr, 2 * Kq), torch.bfloat16, i); g = B.acts((Mr, Kq), torch.bfloat16, i + 1); d = torch.empty((Mr, 2 * Kq), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_silu_mul_actq_bwd', _p(gu), I(2 * Kq), I(Kq), _p(g), _p(d), F(1.0), I(7), I(Mr))
+    timeit('silu_mul_actq_bwd 8192x2048', Mr * Kq * 10, sets(mk))
+    def mk(i):
+        x = B.acts((Mr * Kq,), torch.float32, i); m = B.acts((Mr * Kq,), torch.bfloat16, i + 1); y = B.acts((Mr * Kq,), torch.bfloat16, i + 2); o = torch.empty(Mr * Kq, device=dev)
+        return lambda: B.call('camx_residual3', _p(x), _p(m), _p(y), _p(o), L64(Mr * Kq))
+    timeit('residual3 16M', Mr * Kq * 12, sets(mk))
+    return res
+
+
 def cpu_baseline(w, sample_tokens=2048, budget_s=12.0):
     """the CPU oracle on the first sample_tokens tokens of the same three op-sets, repeated for about budget_s seconds; GB/s of
     the best repetition by the same byte accounting"""
@@ -265,6 +394,10 @@ def main():
         sys.exit(2)
     B = Bench()
     torch = B.torch
+    if a.only == 'sweep':
+        print(json.dumps({'metric': 'fused-op HBM GB/s per entry point at prefill-scale sizes, 1 GPU', 'unit': 'GB/s', 'n_gpus': 1, 'data': 'synthetic',
+                          'peak_GBps': HBM_PEAK_GBPS, 'sweep': prefill_scale_sweep(B)}))
+        return
     if a.only == 'copy_ref':
         # a plain device copy of known size (256 MiB read + 256 MiB written per launch): the yardstick that FETCH_SIZE / WRITE_SIZE
         # counter readings of the kernels above are scaled by
