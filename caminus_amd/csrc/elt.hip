@@ -138,63 +138,72 @@ __global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, c
     const float r = silu_f(sumf);
     if (BF16) ((uint16_t *)y)[(size_t)t * ldy + c] = to_bf16(r); else ((float *)y)[(size_t)t * ldy + c] = r;
 }
-// the same with VW consecutive channels per thread (VW = 8 for bf16, 4 for fp32) and a sliding window over CONV_TT tokens:
-// every input is read once (plus a three-token halo per chunk) with 128-bit loads that are all issued before the first
-// output is computed; the loaded vectors stay packed (4 registers per token) and are widened as the window reaches them
-template <bool BF16, int CONV_TT>
-__global__ void __launch_bounds__(256) gdn_conv_vec(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
-                                                    void * __restrict__ y, int C, int T, int ldx, int ldy) {
-    constexpr int VW = BF16 ? 8 : 4;
-    const int cv = blockIdx.x * 256 + threadIdx.x;
+// Prefill chunks: a lane owns VW consecutive channels and walks TR consecutive tokens, with the rows of the next eight tokens
+// always in flight (a ring of eight 128-bit loads that is refilled as it is consumed) and the four-tap window in registers;
+// one wave per workgroup, so the grid's (channel groups x token ranges) waves spread evenly over the chip.
+template <bool BF16>
+__global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
+                                                      void * __restrict__ y, int C, int T, int ldx, int ldy, int TR) {
+    constexpr int VW = BF16 ? 8 : 4, P = 8;
+    const int cv = blockIdx.x * 64 + threadIdx.x;
     if (cv * VW >= C) return;
-    const int c0 = cv * VW, t0 = blockIdx.y * CONV_TT;
-    const int nt = T - t0 < CONV_TT ? T - t0 : CONV_TT;
-    u32x4 raw[CONV_TT + 3];                                  // tokens t0 - 3 .. t0 + nt - 1 (those at or after time 0)
+    const int c0 = cv * VW, t0 = blockIdx.y * TR, t1 = T < t0 + TR ? T : t0 + TR;
+    auto row = [&](int t) {                                            // (a row index past the range is clamped: the load is harmless and never used)
+        const int tc = t < T - 1 ? t : T - 1;
+        return BF16 ? __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + (size_t)tc * ldx + c0))
+                    : __builtin_nontemporal_load((const u32x4 *)((const float *)x + (size_t)tc * ldx + c0));
+    };
+    auto widen = [&](float (&o)[VW], u32x4 r) {
+        if (BF16) {
 #pragma unroll
-    for (int j = 0; j < CONV_TT + 3; j++) {
-        const int tj = t0 - 3 + j;
-        raw[j] = (u32x4){0u, 0u, 0u, 0u};
-        if (j < nt + 3 && tj >= 0)
-            raw[j] = BF16 ? __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0))
-                          : __builtin_nontemporal_load((const u32x4 *)((const float *)x + (size_t)tj * ldx + c0));
-    }
+            for (int p = 0; p < 4; p++) { const uint32_t b = r[p]; o[2 * p] = __builtin_bit_cast(float, b << 16); o[(2 * p + 1) % VW] = __builtin_bit_cast(float, b & 0xffff0000u); }
+        } else {
+#pragma unroll
+            for (int p = 0; p < 4; p++) { const uint32_t b = r[p]; o[p % VW] = __builtin_bit_cast(float, b); }
+        }
+    };
+    u32x4 ring[P];
+#pragma unroll
+    for (int u = 0; u < P; u++) ring[u] = row(t0 + u);
     f32x4 w4[VW];
 #pragma unroll
     for (int k = 0; k < VW; k++) w4[k] = *(const f32x4 *)(w + (size_t)(c0 + k) * 4);
-    auto widen = [&](float (&o)[VW], int j) {                 // the inputs of window slot j: from the state before time 0
+    float win[4][VW];                                                  // token t0 - 3 + j sits in slot j & 3
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
         const int tj = t0 - 3 + j;
         if (tj < 0) {
 #pragma unroll
-            for (int k = 0; k < VW; k++) o[k] = st[(size_t)(c0 + k) * 3 + 3 + tj];
-        } else if (BF16) {
+            for (int k = 0; k < VW; k++) win[j][k] = st[(size_t)(c0 + k) * 3 + 3 + tj];
+        } else widen(win[j], BF16 ? *(const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0) : *(const u32x4 *)((const float *)x + (size_t)tj * ldx + c0));
+    }
+    auto emit = [&](int tt, int u) {                                   // token tt's output from window slots u .. u + 3 (mod 4)
+        float r[VW];
 #pragma unroll
-            for (int p = 0; p < 4; p++) { o[2 * p] = __builtin_bit_cast(float, raw[j][p] << 16); o[2 * p + 1] = __builtin_bit_cast(float, raw[j][p] & 0xffff0000u); }
-        } else {
-            const f32x4 v = __builtin_bit_cast(f32x4, raw[j]);
-            o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+        for (int k = 0; k < VW; k++) {
+            float sumf = 0.0f;
+            sumf = __builtin_fmaf(win[u & 3][k], w4[k].x, sumf); sumf = __builtin_fmaf(win[(u + 1) & 3][k], w4[k].y, sumf);
+            sumf = __builtin_fmaf(win[(u + 2) & 3][k], w4[k].z, sumf); sumf = __builtin_fmaf(win[(u + 3) & 3][k], w4[k].w, sumf);
+            r[k] = BF16 ? silu_fast(sumf) : silu_f(sumf);
         }
+        const size_t o = (size_t)tt * ldy + c0;
+        if (BF16) {
+            const u32x2 lo = pack_bf16x4_rne((f32x4){r[0], r[1], r[2], r[3]}), hi = pack_bf16x4_rne((f32x4){r[4 % VW], r[5 % VW], r[6 % VW], r[7 % VW]});
+            *(u32x4 *)((uint16_t *)y + o) = (u32x4){lo.x, lo.y, hi.x, hi.y};
+        } else *(f32x4 *)((float *)y + o) = (f32x4){r[0], r[1], r[2], r[3]};
     };
-    float win[4][VW];
-    widen(win[0], 0); widen(win[1], 1); widen(win[2], 2);
+    int t = t0;
+    for (; t + P <= t1; t += P) {                                      // whole groups of eight tokens: no guards
 #pragma unroll
-    for (int j = 0; j < CONV_TT; j++) {
-        if (j < nt) {
-            widen(win[(j + 3) & 3], j + 3);
-            float r[VW];
-#pragma unroll
-            for (int k = 0; k < VW; k++) {
-                float sumf = 0.0f;
-                sumf = __builtin_fmaf(win[j & 3][k], w4[k].x, sumf); sumf = __builtin_fmaf(win[(j + 1) & 3][k], w4[k].y, sumf);
-                sumf = __builtin_fmaf(win[(j + 2) & 3][k], w4[k].z, sumf); sumf = __builtin_fmaf(win[(j + 3) & 3][k], w4[k].w, sumf);
-                r[k] = BF16 ? silu_fast(sumf) : silu_f(sumf);
-            }
-            const size_t o = (size_t)(t0 + j) * ldy + c0;
-            if (BF16) {
-                const u32x2 lo = pack_bf16x4_rne((f32x4){r[0], r[1], r[2], r[3]}), hi = pack_bf16x4_rne((f32x4){r[4 % VW], r[5 % VW], r[6 % VW], r[7 % VW]});
-                *(u32x4 *)((uint16_t *)y + o) = (u32x4){lo.x, lo.y, hi.x, hi.y};
-            } else *(f32x4 *)((float *)y + o) = (f32x4){r[0], r[1], r[2], r[3]};
+        for (int u = 0; u < P; u++) {
+            widen(win[(u + 3) & 3], ring[u]);
+            ring[u] = row(t + u + P);
+            emit(t + u, u);
         }
     }
+#pragma unroll
+    for (int u = 0; u < P; u++)                                        // the last, partial group
+        if (t + u < t1) { widen(win[(u + 3) & 3], ring[u]); emit(t + u, u); }
 }
 
 template <bool BF16>
@@ -480,9 +489,9 @@ int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void 
     if (!x || !w || !state || !y || C < 1 || T < 1 || ldx < C || ldy < C || ((uintptr_t)w & 15)) return CAMX_EINVAL;
     const int vw = bf16 ? 8 : 4;
     if ((long)T * C >= (1L << 20) && C % vw == 0 && ldx % vw == 0 && ldy % vw == 0 && !(((uintptr_t)x | (uintptr_t)y) & 15)) {
-        const int tt = 16;      // (a decode / verify batch takes the one-value-per-thread kernel below: it fills the chip, a 16-token window would not)
-        const dim3 gv((unsigned)((C / vw + 255) / 256), (unsigned)((T + tt - 1) / tt)), bv(256);
-        { if (bf16) gdn_conv_vec<true, 16><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy); else gdn_conv_vec<false, 16><<<gv, bv, 0, st>>>(x, w, state, y, C, T, ldx, ldy); }
+        const int tr = 32;       // tokens per wave: 16 and 64 measured 15 % slower (halo re-reads; too few waves) (a decode / verify batch takes the one-value-per-thread kernel below)
+        const dim3 gs((unsigned)((C / vw + 63) / 64), (unsigned)((T + tr - 1) / tr)), bs(64);
+        if (bf16) gdn_conv_stream<true><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr); else gdn_conv_stream<false><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr);
         CAMX_LAUNCH_RET();
     }
     const dim3 grid((unsigned)(((long)T * C + 255) / 256)), block(256);

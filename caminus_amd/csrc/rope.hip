@@ -635,9 +635,131 @@ __global__ void __launch_bounds__(256) qk_nr_tokens_fast(NrArgs a) {
     }
 }
 
+// Heads of exactly 256 dims at prefill sizes: 32 lanes per head (lane l holds dims 8 l .. 8 l + 7), two heads per wave
+// instruction, NS wave steps (2 NS heads) per wave with all their loads issued first and ONE IEEE sqrt + divide for all of them
+// (lane s of a half-wave takes step s). The 32-thread butterfly of the norm sum is lane ^ 2, lane ^ 1 and three in-register
+// levels (the pairs and order of thread xor 16, 8, 4, 2, 1); the eight group sums are fetched by swizzles and added in order.
+// The rotary partner (dim i +- nrot / 2) sits XL = nrot / 16 lanes away.
+template <int J> CAMX_DEV float swz_group32(float v) {       // every lane of a 32-lane half reads the half's lane 4 J + (lane & 3)
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x03 | ((4 * J) << 5)));
+}
+template <int S> CAMX_DEV float half32_lane_bcast(float v) { // every lane of a 32-lane half reads the half's lane S
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x00 | (S << 5)));
+}
+template <int XL> CAMX_DEV float nr8_partner(float v) {
+    if (XL == 1) return dpp_xor1(v);
+    if (XL == 2) return dpp_xor2(v);
+    if (XL == 4) return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x101F));
+    if (XL == 8) return dpp_ror8(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+template <bool BF16, int XL, int NS>
+__global__ void __launch_bounds__(256) qk_nr_tokens_w8(NrArgs a) {
+    __shared__ __attribute__((aligned(16))) float rc[128], rs[128];
+    constexpr int NW = BF16 ? 1 : 2;
+    const int tok = blockIdx.x, tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, hf = lane >> 5, wave = tid >> 6;
+    const int nrot = 16 * XL, half = nrot / 2, i0 = 8 * l32;
+    const bool rot = i0 < nrot;
+    const int per_pass = 8 * NS;                                        // heads per workgroup pass: wave w, step s, half hf -> head 8 s + 2 w + hf
+    u32x4 raw[NS][NW];
+    auto load = [&](int base) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const int h = base + 8 * s + 2 * wave + hf;
+#pragma unroll
+            for (int w = 0; w < NW; w++) raw[s][w] = (u32x4){0u, 0u, 0u, 0u};
+            if (h < a.heads) {
+                const size_t xo = ((size_t)tok * a.heads + h) * a.head_stride + i0;
+                if (BF16) raw[s][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)a.x + xo));
+                else { raw[s][0] = __builtin_nontemporal_load((const u32x4 *)((const float *)a.x + xo)); raw[s][NW - 1] = __builtin_nontemporal_load((const u32x4 *)((const float *)a.x + xo + 4)); }
+            }
+        }
+    };
+    load(0);
+    const f32x4 w0 = *(const f32x4 *)(a.w + i0), w1 = *(const f32x4 *)(a.w + i0 + 4);
+    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    if (tid < half) {
+        const float theta = pos * rope_freq(a.theta_scale, tid);
+        rc[tid] = cosf(theta); rs[tid] = sinf(theta);
+    }
+    __syncthreads();
+    f32x4 c4[2] = {{1.0f, 1.0f, 1.0f, 1.0f}, {1.0f, 1.0f, 1.0f, 1.0f}}, s4[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    if (rot) {
+        const int jj = i0 & (half - 1);
+        c4[0] = *(const f32x4 *)(rc + jj); c4[1] = *(const f32x4 *)(rc + jj + 4);
+        s4[0] = *(const f32x4 *)(rs + jj); s4[1] = *(const f32x4 *)(rs + jj + 4);
+        if (i0 < half) { s4[0] = -s4[0]; s4[1] = -s4[1]; }              // dims below nrot / 2 take -(partner * sin)
+    }
+    for (int base = 0; base < a.heads; base += per_pass) {
+        float x[NS][8], tot[NS];
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            if (BF16) {
+#pragma unroll
+                for (int p = 0; p < 4; p++) { const uint32_t b = raw[s][0][p]; x[s][2 * p] = __builtin_bit_cast(float, b << 16); x[s][2 * p + 1] = __builtin_bit_cast(float, b & 0xffff0000u); }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 4; p++) { const uint32_t b0 = raw[s][0][p], b1 = raw[s][NW - 1][p]; x[s][p] = __builtin_bit_cast(float, b0); x[s][4 + p] = __builtin_bit_cast(float, b1); }
+            }
+            float sq[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] = x[s][k] * x[s][k];
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] = add_xor2(sq[k]);            // thread ^ 16
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] = add_xor1(sq[k]);            // thread ^ 8
+            const float b0 = sq[0] + sq[4], b1 = sq[1] + sq[5], b2 = sq[2] + sq[6], b3 = sq[3] + sq[7];   // thread ^ 4
+            const float e0 = b0 + b2, e1 = b1 + b3;                         // thread ^ 2
+            const float g = e0 + e1;                                        // thread ^ 1
+            tot[s] = ((((((swz_group32<0>(g) + swz_group32<1>(g)) + swz_group32<2>(g)) + swz_group32<3>(g)) + swz_group32<4>(g)) + swz_group32<5>(g)) +
+                      swz_group32<6>(g)) + swz_group32<7>(g);
+        }
+        if (base + per_pass < a.heads) load(base + per_pass);               // the next pass's rows, in flight during this pass's arithmetic
+        float tv = tot[0];
+#pragma unroll
+        for (int s = 1; s < NS; s++) tv = l32 == s ? tot[s] : tv;
+        const float sc = rsqrt_exact(tv / 256.0f + a.eps);
+        float scale[NS];
+        static_assert(NS <= 4, "the broadcasts below are written out for at most four steps");
+        scale[0] = half32_lane_bcast<0>(sc);
+        if (NS > 1) scale[1 % NS] = half32_lane_bcast<1>(sc);
+        if (NS > 2) scale[2 % NS] = half32_lane_bcast<2>(sc);
+        if (NS > 3) scale[3 % NS] = half32_lane_bcast<3>(sc);
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            if (base + 8 * s + 2 * wave >= a.heads) break;                  // wave-uniform: neither half has a head
+            const int h = base + 8 * s + 2 * wave + hf;
+            float y[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float xn = (scale[s] * x[s][k]) * (k < 4 ? w0[k] : w1[k - 4]);
+                const float pr = nr8_partner<XL>(xn);
+                y[k] = rot ? xn * (k < 4 ? c4[0][k] : c4[1][k - 4]) + pr * (k < 4 ? s4[0][k] : s4[1][k - 4]) : xn;
+            }
+            if (h < a.heads) {
+                const size_t yo = ((size_t)tok * a.heads + h) * 256 + i0;
+                if (BF16) {
+                    const u32x2 lo = pack_bf16x4_rne((f32x4){y[0], y[1], y[2], y[3]}), hi = pack_bf16x4_rne((f32x4){y[4], y[5], y[6], y[7]});
+                    *(u32x4 *)((uint16_t *)a.out + yo) = (u32x4){lo.x, lo.y, hi.x, hi.y};
+                } else {
+                    *(f32x4 *)((float *)a.out + yo) = (f32x4){y[0], y[1], y[2], y[3]};
+                    *(f32x4 *)((float *)a.out + yo + 4) = (f32x4){y[4], y[5], y[6], y[7]};
+                }
+            }
+        }
+    }
+}
+
 static void launch_nr(const NrArgs & a, int io, hipStream_t st) {
     const int es = io ? 2 : 4;
     const bool vec = (a.D & 3) == 0 && (a.head_stride & 3) == 0 && ((uintptr_t)a.x & (4 * es - 1)) == 0 && ((uintptr_t)a.out & (4 * es - 1)) == 0;
+    const bool vec8 = (a.head_stride & 7) == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.out & 15) == 0 && ((uintptr_t)a.w & 15) == 0;
+    if (vec8 && a.D == 256 && a.heads >= 8 && (long)a.T * a.heads >= 4096 && a.nrot >= 16 && (a.nrot & (a.nrot - 1)) == 0) {
+#define NR_W8(XL) (io ? qk_nr_tokens_w8<true, XL, 3><<<dim3(a.T), dim3(256), 0, st>>>(a) : qk_nr_tokens_w8<false, XL, 3><<<dim3(a.T), dim3(256), 0, st>>>(a))
+        switch (a.nrot) { case 16: NR_W8(1); break; case 32: NR_W8(2); break; case 64: NR_W8(4); break; case 128: NR_W8(8); break; default: NR_W8(16); break; }
+#undef NR_W8
+        return;
+    }
     if (vec && a.heads >= 8 && (long)a.T * a.heads >= 4096 && a.D <= 256 && a.nrot >= 8 && a.nrot <= a.D && (a.nrot & (a.nrot - 1)) == 0) {
 #define NR_FAST(XL) (io ? qk_nr_tokens_fast<true, XL><<<dim3(a.T), dim3(256), 0, st>>>(a) : qk_nr_tokens_fast<false, XL><<<dim3(a.T), dim3(256), 0, st>>>(a))
         switch (a.nrot) { case 8: NR_FAST(1); break; case 16: NR_FAST(2); break; case 32: NR_FAST(4); break; case 64: NR_FAST(8); break;

@@ -110,7 +110,7 @@ def test_qk_rope_paged_decode_batch():
 @pytest.mark.parametrize('T,heads,D,n_rot,stride,base', [(16, 24, 256, 64, 512, 1e7), (16, 4, 256, 64, 256, 1e7), (3, 5, 128, 128, 128, 1e6),
                                                          (2, 3, 96, 32, 100, 1e4), (2, 2, 512, 128, 512, 1e6), (400, 24, 256, 64, 512, 1e7), (520, 8, 128, 128, 128, 1e6),
                                                          (512, 8, 256, 256, 256, 1e6), (512, 9, 64, 8, 64, 1e4), (600, 12, 128, 16, 128, 1e5), (512, 8, 256, 32, 320, 1e6),
-                                                         (512, 8, 200, 64, 200, 1e6), (512, 8, 256, 48, 256, 1e6)])
+                                                         (512, 8, 200, 64, 200, 1e6), (512, 8, 256, 48, 256, 1e6), (300, 28, 256, 16, 256, 1e6), (260, 17, 256, 128, 264, 1e7)])
 def test_pf_qk_nr(T, heads, D, n_rot, stride, base):
     rng = np.random.default_rng(1004 + D + heads)
     x = outliers(rng, (T * heads, stride)); w = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
