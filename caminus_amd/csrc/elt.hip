@@ -24,7 +24,7 @@ __global__ void __launch_bounds__(256) swiglu_f32(const float * __restrict__ g, 
         const long i = q * 4;
         float gv[4], uv[4], r[4];
         if (vec && i + 3 < n) {
-            const f32x4 a = *(const f32x4 *)(g + i), b = *(const f32x4 *)(u + i);
+            const f32x4 a = __builtin_nontemporal_load((const f32x4 *)(g + i)), b = __builtin_nontemporal_load((const f32x4 *)(u + i));
             gv[0] = a.x; gv[1] = a.y; gv[2] = a.z; gv[3] = a.w; uv[0] = b.x; uv[1] = b.y; uv[2] = b.z; uv[3] = b.w;
         } else {
 #pragma unroll
@@ -33,8 +33,8 @@ __global__ void __launch_bounds__(256) swiglu_f32(const float * __restrict__ g, 
 #pragma unroll
         for (int k = 0; k < 4; k++) r[k] = gv[k] / (1.0f + expf(-gv[k])) * uv[k];
         if (vec && i + 3 < n) {
-            if (F16OUT) *(u32x2 *)((uint16_t *)y + i) = pack_f16x4((f32x4){r[0], r[1], r[2], r[3]});
-            else *(f32x4 *)((float *)y + i) = (f32x4){r[0], r[1], r[2], r[3]};
+            if (F16OUT) __builtin_nontemporal_store(pack_f16x4((f32x4){r[0], r[1], r[2], r[3]}), (u32x2 *)((uint16_t *)y + i));
+            else __builtin_nontemporal_store((f32x4){r[0], r[1], r[2], r[3]}, (f32x4 *)((float *)y + i));
         } else {
 #pragma unroll
             for (int k = 0; k < 4; k++)
@@ -391,7 +391,7 @@ __global__ void __launch_bounds__(256) residual3_vec(const float * __restrict__ 
     const f32x4 xv = __builtin_nontemporal_load((const f32x4 *)x + q);
     const f32x4 mv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)m + q)), yv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)y + q));
     f32x4 o; o.x = (xv.x + mv.x) + yv.x; o.y = (xv.y + mv.y) + yv.y; o.z = (xv.z + mv.z) + yv.z; o.w = (xv.w + mv.w) + yv.w;
-    ((f32x4 *)out)[q] = o;
+    __builtin_nontemporal_store(o, (f32x4 *)out + q);
 }
 __global__ void __launch_bounds__(256) cast_bf16_k(const float * __restrict__ x, uint16_t * __restrict__ out, long n) {
     const long step = (long)gridDim.x * 256;

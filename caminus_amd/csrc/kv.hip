@@ -129,9 +129,9 @@ __global__ void __launch_bounds__(256) hadamard128_heads(const float * __restric
     const int l = lane & 31;
     const bool active = h < heads;
     f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (active) v = *(const f32x4 *)(x + h * 128 + 4 * l);
+    if (active) v = x == y ? *(const f32x4 *)(x + h * 128 + 4 * l) : __builtin_nontemporal_load((const f32x4 *)(x + h * 128 + 4 * l));
     v = hadamard128_l4(v, l, true);
-    if (active) *(f32x4 *)(y + h * 128 + 4 * l) = v;
+    if (active) __builtin_nontemporal_store(v, (f32x4 *)(y + h * 128 + 4 * l));
 }
 
 extern "C" {

@@ -6,6 +6,7 @@
 //
 // Numeric contract: sum of squares = fmaf chain per logical thread t over elements t + 256 j, the 32-lane butterfly, the
 // 8 group sums in order; scale = 1 / sqrt(tot / N + eps) with IEEE sqrt and divide; h = (x * scale) * w.
+#include <type_traits>
 #include "common.cuh"
 
 enum { ADD_NONE = 0, ADD_F32_SLOTS = 1, ADD_BF16 = 2, ADD_F32_DIRECT = 3, ADD_HC = 4 };   // DIRECT: x = x + d (no 0 + d first)
@@ -27,6 +28,7 @@ struct NormArgs {
     float * scl;             // optional row scale [rows]
     int N, rows;
     const float * inj; int HC; float rs;   // ADD_HC only
+    int stream;              // set by the launcher for large batches: h / h16 leave as non-temporal stores (the consumer of a decode-sized batch finds them in cache instead)
 };
 
 // EXACT: the row has exactly NI_MAX slabs, so every loop below is straight-line code: no scalar branch stands between the
@@ -59,7 +61,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
             f32x4 dv[NI_MAX];
 #pragma unroll
             for (int j = 0; j < NI_MAX; j++)
-                if (j < ni) dv[j] = *(const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane);
+                if (j < ni) dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane));
 #pragma unroll
             for (int j = 0; j < NI_MAX; j++)
                 if (j < ni) {
@@ -131,17 +133,25 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     const float tot = wave_groups_in_order(group32_sum(ss));
     const float scale = rsqrt_exact(tot / (float)N + a.eps);
     if (a.scl && lane == 0) a.scl[row] = scale;
+    // (two copies of the loop, chosen once: with the choice inside it the stores of a long row were no longer issued back to back)
+    auto emit = [&](auto nt) {
+        constexpr bool NT = decltype(nt)::value;
 #pragma unroll
-    for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) {
-            f32x4 v;
-            v.x = (xv[j].x * scale) * g[j].x; v.y = (xv[j].y * scale) * g[j].y; v.z = (xv[j].z * scale) * g[j].z; v.w = (xv[j].w * scale) * g[j].w;
-            const size_t o = (size_t)row * N + 256 * j + 4 * lane;
-            if (a.h) *(f32x4 *)(a.h + o) = v;
-            if (a.h16) *(u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane) = pack_f16x4(v);
-            if (a.hbf) __builtin_nontemporal_store(pack_bf16x4_rne(v), (u32x2 *)(a.hbf + o));
-            if (a.q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
-        }
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) {
+                f32x4 v;
+                v.x = (xv[j].x * scale) * g[j].x; v.y = (xv[j].y * scale) * g[j].y; v.z = (xv[j].z * scale) * g[j].z; v.w = (xv[j].w * scale) * g[j].w;
+                const size_t o = (size_t)row * N + 256 * j + 4 * lane;
+                if (a.h) { if (NT) __builtin_nontemporal_store(v, (f32x4 *)(a.h + o)); else *(f32x4 *)(a.h + o) = v; }
+                if (a.h16) {
+                    u32x2 * p16 = (u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane);
+                    if (NT) __builtin_nontemporal_store(pack_f16x4(v), p16); else *p16 = pack_f16x4(v);
+                }
+                if (a.hbf) __builtin_nontemporal_store(pack_bf16x4_rne(v), (u32x2 *)(a.hbf + o));
+                if (a.q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
+            }
+    };
+    if (a.stream) emit(std::true_type{}); else emit(std::false_type{});
 }
 
 // Any row length (N not a multiple of 256, or longer than the register forms hold): the same tree with scalar accesses,
@@ -205,8 +215,10 @@ __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
 }
 
 template <int ADD>
-static int launch_norm(const NormArgs & a, hipStream_t st) {
-    if (a.rows <= 0) return CAMX_OK;
+static int launch_norm(const NormArgs & a0, hipStream_t st) {
+    if (a0.rows <= 0) return CAMX_OK;
+    NormArgs a = a0;
+    a.stream = (long)a.rows * a.N >= (1L << 20);
     const dim3 grid((a.rows + 3) / 4), block(256);
     const int ni = a.N >> 8;
     const bool vec = (a.N & 255) == 0 && ni <= 32 && (a.ld16 & 3) == 0 &&

@@ -402,7 +402,7 @@ __global__ void __launch_bounds__(1024) silu_mul_lut(const uint16_t * __restrict
                 pk[k] = (uint32_t)f2bf(a0) | ((uint32_t)f2bf(a1) << 16);
             }
         }
-        *(u32x4 *)(act + o) = (u32x4){pk[0], pk[1], pk[2], pk[3]};
+        __builtin_nontemporal_store((u32x4){pk[0], pk[1], pk[2], pk[3]}, (u32x4 *)(act + o));
         g = gn; u = un; q = qn;
     }
 }
