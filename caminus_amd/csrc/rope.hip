@@ -740,10 +740,10 @@ __global__ void __launch_bounds__(256) qk_nr_tokens_w8(NrArgs a) {
                 const size_t yo = ((size_t)tok * a.heads + h) * 256 + i0;
                 if (BF16) {
                     const u32x2 lo = pack_bf16x4_rne((f32x4){y[0], y[1], y[2], y[3]}), hi = pack_bf16x4_rne((f32x4){y[4], y[5], y[6], y[7]});
-                    *(u32x4 *)((uint16_t *)a.out + yo) = (u32x4){lo.x, lo.y, hi.x, hi.y};
+                    __builtin_nontemporal_store((u32x4){lo.x, lo.y, hi.x, hi.y}, (u32x4 *)((uint16_t *)a.out + yo));
                 } else {
-                    *(f32x4 *)((float *)a.out + yo) = (f32x4){y[0], y[1], y[2], y[3]};
-                    *(f32x4 *)((float *)a.out + yo + 4) = (f32x4){y[4], y[5], y[6], y[7]};
+                    __builtin_nontemporal_store((f32x4){y[0], y[1], y[2], y[3]}, (f32x4 *)((float *)a.out + yo));
+                    __builtin_nontemporal_store((f32x4){y[4], y[5], y[6], y[7]}, (f32x4 *)((float *)a.out + yo + 4));
                 }
             }
         }
