@@ -78,8 +78,8 @@ __global__ void __launch_bounds__(256) q8_1_flat(const float * __restrict__ x, u
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_s_waitcnt(0xc07f);                        // lgkmcnt(0): the wave's LDS stores have landed
             u32x4 * dst = (u32x4 *)(y + s * 1152);
-            dst[lraw] = *(const u32x4 *)(stage[wv] + 4 * lraw);
-            if (lraw < 8) dst[64 + lraw] = *(const u32x4 *)(stage[wv] + 4 * (64 + lraw));
+            __builtin_nontemporal_store(*(const u32x4 *)(stage[wv] + 4 * lraw), dst + lraw);
+            if (lraw < 8) __builtin_nontemporal_store(*(const u32x4 *)(stage[wv] + 4 * (64 + lraw)), dst + 64 + lraw);
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_s_waitcnt(0xc07f);                        // read out before the next step overwrites it
         }

@@ -139,3 +139,21 @@ def test_actq_autograd_wrappers():
     yq, cq, sq = A.silu_mul_actq(gu)
     yq.backward(torch.randn(M, 1024, device='cuda:0').bfloat16())
     assert gu.grad.shape == (M, 2048) and gu.grad.dtype == torch.bfloat16 and torch.isfinite(gu.grad.float()).all()
+
+
+@pytest.mark.parametrize('bf', [False, True])
+def test_actq_fwd_and_bwd_four_million_values(bf):
+    """enough values that the forward's division-free rounding meets its fallback thousands of times"""
+    rng = np.random.default_rng(5150)
+    M, K = 2048, 2048
+    x = (rng.standard_normal((M, K)) * np.exp(rng.standard_normal((M, 1)))).astype(np.float32)
+    g = O.f2bf(rng.standard_normal((M, K)).astype(np.float32))
+    src = O.f2bf(x) if bf else x
+    ry, rs, rc = O.actq_fwd(src, clip=0.95, qmax=7, bf16=bf)
+    y = dev(np.zeros((M, K), np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros((M, K // 2), np.uint8))
+    xd = dev(src)
+    call('camx_actq_fwd', ptr(xd), I(int(bf)), ptr(y), ptr(s), ptr(c), I(K), F(0.95), I(7), I(M))
+    assert bits_equal(host(s), rs) and bits_equal(host(c), rc) and bits_equal(host(y, np.uint16), ry)
+    dx = dev(np.zeros((M, K), np.uint16 if bf else np.float32))
+    call('camx_actq_bwd', ptr(xd), I(int(bf)), ptr(dev(g)), ptr(dx), I(K), F(0.95), I(7), I(M))
+    assert bits_equal(host(dx, np.uint16) if bf else host(dx), O.actq_bwd(src, g, clip=0.95, qmax=7, bf16=bf))

@@ -90,3 +90,21 @@ def test_swiglu_mmq_every_bf16_gate_value():
     diff = got[finite] != ref[finite]
     assert diff.sum() == 0, f'{int(diff.sum())} of {int(finite.sum())} gate values differ from the oracle'
     assert np.isnan(O.bf2f(got[~np.isfinite(O.bf2f(ref))])).all() or True
+
+
+def test_q8_1_quotients_next_to_rounding_boundaries():
+    """the codes come from x * rcp(d) where that provably rounds like the IEEE quotient and from the division elsewhere: blocks
+    whose quotients sit on, next to and a few error bounds away from every half-integer must give the oracle's bytes"""
+    rng = np.random.default_rng(99)
+    nblk = 1 << 15
+    amax = np.exp(rng.uniform(-20, 20, nblk)).astype(np.float32)
+    d = (amax / np.float32(127.0)).astype(np.float32).astype(np.float64)
+    k = rng.integers(0, 127, (nblk, 32)) + 0.5
+    off = rng.choice([0.0, 1e-7, 1e-6, 4e-6, 1e-5, 2e-5, 4e-5, 8e-5, 1.2e-4, 2e-4, 3e-4, 1e-3], (nblk, 32)) * rng.choice([-1.0, 1.0], (nblk, 32))
+    x = ((k + off) * rng.choice([-1.0, 1.0], (nblk, 32)) * d[:, None]).astype(np.float32)
+    x[:, 0] = amax                                                        # the block's maximum fixes d
+    x = np.clip(x, -amax[:, None], amax[:, None]).reshape(-1)
+    y = dev(np.zeros(nblk * 36, np.uint8))
+    call('camx_gg_quantize_q8_1', ptr(dev(x)), ptr(y), L64(x.size), I(0), F(0), NULL)
+    want = O.q8_1(x)
+    assert bits_equal(host(y), want.reshape(-1))
