@@ -1,0 +1,293 @@
+// More row kernels of the batched prefill for gfx950: the gated RMSNorm of the GDN output, the GDN gates, the fp16 KV
+// append, the residual sums and bf16 operand copies of the glue, the hyper-connection average, and the per-layer-embedding
+// gate / dilated conv / history. Replaces pf_gdn_norm and pf_gdn_gates (kernels/prefill_gdn.hip:80-92, 385-407),
+// q35p_gdn_norm16 and q35p_kv_append16 (kernels/q35_prefill.hip:671-707), pf_ple_gate, pf_ple_conv, pf_ple_hist, pf_add_sum,
+// pf_silu_bf16 and pf_to_bf16 (kernels/prefill_glue.hip:343-423, 552-566) and pf_hc_avg (kernels/prefill_attn.hip:388-397).
+//
+// The reference compiles these with contraction off: a sum of products here is a multiply and an add, never an fma, except
+// where its source writes fmaf. Row sums follow the 256-thread tree of the other norms (thread t owns elements t, t + 256,
+// ..; xor 16 .. 1 inside each group of 32 threads; the eight group sums in order).
+#include "common.cuh"
+
+#define GRID_1D(n4) dim3((unsigned)((((n4) + 255) / 256) < 1048576 ? (((n4) + 255) / 256) : 1048576))
+
+// ---- gated RMSNorm of a GDN value head: y = ((o * rsqrt(mean(o^2) + eps)) * w) * (SILU ? silu(z) : sigmoid(z)) ------------
+// one wave per (token, head) row of K values (K % 4 == 0, K <= 1024); lane p holds elements 256 j + 4 p + k
+template <bool SILU, bool F16OUT, int NI>
+__global__ void __launch_bounds__(256) gdn_norm_rows(const float * __restrict__ o, const float * __restrict__ w, const float * __restrict__ z,
+                                                     void * __restrict__ y, int K, float eps, long rows) {
+    const int lane = slot_of(threadIdx.x & 63);
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    f32x4 ov[NI], zv[NI], wv[NI];
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const int i0 = 256 * j + 4 * lane;
+        ov[j] = zv[j] = wv[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        if (i0 < K) {
+            ov[j] = __builtin_nontemporal_load((const f32x4 *)(o + row * K + i0));
+            zv[j] = __builtin_nontemporal_load((const f32x4 *)(z + row * K + i0));
+            wv[j] = *(const f32x4 *)(w + i0);
+        }
+    }
+    f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NI; j++) {                             // ss += o * o: a product, then a sum
+        ss.x = ss.x + ov[j].x * ov[j].x; ss.y = ss.y + ov[j].y * ov[j].y; ss.z = ss.z + ov[j].z * ov[j].z; ss.w = ss.w + ov[j].w * ov[j].w;
+    }
+    const float tot = wave_groups_in_order(group32_sum(ss));
+    const float scale = rsqrt_exact(tot / (float)K + eps);
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const int i0 = 256 * j + 4 * lane;
+        if (i0 < K) {
+            f32x4 r;
+#define G_(e) { const float nrm = (scale * ov[j].e) * wv[j].e; r.e = SILU ? nrm * (zv[j].e / (1.0f + expf(-zv[j].e))) : nrm * (1.0f / (1.0f + expf(-zv[j].e))); }
+            G_(x) G_(y) G_(z) G_(w)
+#undef G_
+            if (F16OUT) *(u32x2 *)((uint16_t *)y + row * K + i0) = pack_f16x4(r); else *(f32x4 *)((float *)y + row * K + i0) = r;
+        }
+    }
+}
+
+// ---- GDN gates: gate = softplus(alpha + dt) * a, beta_sig = sigmoid(beta); y [T][2H] = gate | beta_sig -----------------------
+__global__ void __launch_bounds__(256) gdn_gates_k(const float * __restrict__ al, int lda, const float * __restrict__ be, int ldb,
+                                                   const float * __restrict__ dt, const float * __restrict__ A, float * __restrict__ y, int H, int T) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    if (q >= (long)T * H) return;
+    const int tt = (int)(q / H), h = (int)(q - (long)tt * H);
+    const float ab = al[(size_t)tt * lda + h] + dt[h];
+    const float sp = ab > 20.0f ? ab : logf(1.0f + expf(ab));
+    y[(size_t)tt * 2 * H + h] = sp * A[h];
+    y[(size_t)tt * 2 * H + H + h] = 1.0f / (1.0f + expf(-be[(size_t)tt * ldb + h]));
+}
+
+// ---- fp16 KV append: cache[pos0 + t] = fp16(k[t]) | fp16(v[t]) -----------------------------------------------------------------
+__global__ void __launch_bounds__(256) kv_append16_k(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv,
+                                                     uint16_t * __restrict__ cache, int M, int pos0, int rows, int * __restrict__ err, int vec) {
+    const int tt = blockIdx.x;
+    const long pos = (long)pos0 + tt;
+    if (pos < 0 || pos >= rows) { if (threadIdx.x == 0) atomicOr(err, 1); return; }
+    uint16_t * c = cache + (size_t)pos * 2 * M;
+    if (vec) {
+        for (int i = 4 * threadIdx.x; i < M; i += 1024) {
+            const f32x4 kv = __builtin_nontemporal_load((const f32x4 *)(k + (size_t)tt * ldk + i)), vv = __builtin_nontemporal_load((const f32x4 *)(v + (size_t)tt * ldv + i));
+            *(u32x2 *)(c + i) = pack_f16x4(kv); *(u32x2 *)(c + M + i) = pack_f16x4(vv);
+        }
+    } else {
+        for (int i = threadIdx.x; i < M; i += 256) { c[i] = f2h_bits(k[(size_t)tt * ldk + i]); c[M + i] = f2h_bits(v[(size_t)tt * ldv + i]); }
+    }
+}
+
+// ---- y = y + (a + b) ------------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) add_sum_k(const float * __restrict__ a, const float * __restrict__ b, float * __restrict__ y, long n, int vec) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        if (q * 4 >= n) return;
+        const f32x4 av = __builtin_nontemporal_load((const f32x4 *)a + q), bv = __builtin_nontemporal_load((const f32x4 *)b + q), yv = ((const f32x4 *)y)[q];
+        f32x4 r; r.x = yv.x + (av.x + bv.x); r.y = yv.y + (av.y + bv.y); r.z = yv.z + (av.z + bv.z); r.w = yv.w + (av.w + bv.w);
+        __builtin_nontemporal_store(r, (f32x4 *)y + q);
+    } else {
+        for (long i = q; i < n; i += (long)gridDim.x * 256) y[i] = y[i] + (a[i] + b[i]);
+    }
+}
+
+// ---- bf16 operand copies with zero rows up to Tpad: y[t][j] = bf16(SILU ? silu(fma(rs, x, 0)) : x) ---------------------------
+template <bool SILU>
+__global__ void __launch_bounds__(256) to_bf16_rows(const float * __restrict__ x, int ldx, uint16_t * __restrict__ y, int T, int Tpad, int K, float rs, int vec) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    const int VW = vec ? 4 : 1;
+    const long i = q * VW;
+    if (i >= (long)Tpad * K) return;
+    const int t = (int)(i / K), j = (int)(i - (long)t * K);
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (t < T) {
+        if (vec) { const f32x4 xv = __builtin_nontemporal_load((const f32x4 *)(x + (size_t)t * ldx + j)); v[0] = xv.x; v[1] = xv.y; v[2] = xv.z; v[3] = xv.w; }
+        else v[0] = x[(size_t)t * ldx + j];
+        if (SILU) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) { const float s = __builtin_fmaf(rs, v[k], 0.0f); v[k] = s / (1.0f + expf(-s)); }
+        }
+    }
+    if (vec) *(u32x2 *)(y + i) = t < T ? pack_bf16x4_rne((f32x4){v[0], v[1], v[2], v[3]}) : (u32x2){0u, 0u};
+    else y[i] = t < T ? to_bf16(v[0]) : (uint16_t)0;
+}
+
+// ---- hyper-connection average: y[t][i] = (((r0 + r1) + r2) + ..) * (1 / hc) of r [T][hc][D], y rows at ldo -------------------
+__global__ void __launch_bounds__(256) hc_avg_k(const float * __restrict__ r, float * __restrict__ y, int T, int hc, int D, int ldo, int vec) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    const int VW = vec ? 4 : 1;
+    const long i = q * VW;
+    if (i >= (long)T * D) return;
+    const int tt = (int)(i / D), ii = (int)(i - (long)tt * D);
+    const float inv = 1.0f / (float)hc;
+    if (vec) {
+        f32x4 acc = __builtin_nontemporal_load((const f32x4 *)(r + (size_t)(tt * hc) * D + ii));
+        for (int h = 1; h < hc; h++) acc = acc + __builtin_nontemporal_load((const f32x4 *)(r + (size_t)(tt * hc + h) * D + ii));
+        acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+        *(f32x4 *)(y + (size_t)tt * ldo + ii) = acc;
+    } else {
+        float acc = r[(size_t)(tt * hc) * D + ii];
+        for (int h = 1; h < hc; h++) acc = acc + r[(size_t)(tt * hc + h) * D + ii];
+        y[(size_t)tt * ldo + ii] = acc * inv;
+    }
+}
+
+// ---- per-layer-embedding gate: per token and stream st, s = (kn . qn) / sqrt(D), gate = sigmoid(sgn(s) sqrt(max(|s|, 1e-6))),
+// gated[t][st][i] = val[t][i] * gate. qn given, or recomputed from the residual as (q * qscl[t * HC + st]) * qw[st][i].
+// One workgroup per token; the dot product is the 256-thread tree with a product and a sum per element; HC <= 8.
+__global__ void __launch_bounds__(256) ple_gate_k(const float * kn, const float * q, const float * qscl, const float * qw, const float * val, int ldv,
+                                                  float * gated, float * gate_out, int HC, int D) {
+    __shared__ float part[8];
+    __shared__ float gate[8];
+    const int tid = threadIdx.x, t = slot_of(tid), tt = blockIdx.x;
+    const float * k_ = kn + (size_t)tt * HC * D, * q_ = q + (size_t)tt * HC * D, * v_ = val + (size_t)tt * ldv;
+    for (int st = 0; st < HC; st++) {
+        float acc = 0.0f;
+        for (int i = t; i < D; i += 256) {
+            const float qv = qscl ? (q_[(size_t)st * D + i] * qscl[tt * HC + st]) * qw[(size_t)st * D + i] : q_[(size_t)st * D + i];
+            acc = acc + k_[(size_t)st * D + i] * qv;
+        }
+        acc += lane_xor16(acc); acc += lane_xor8(acc); acc += lane_xor4(acc); acc += lane_xor2(acc); acc += lane_xor1(acc);
+        __syncthreads();
+        if ((tid & 31) == 0) part[tid >> 5] = acc;
+        __syncthreads();
+        if (tid == 0) {
+            float sum = 0.0f;
+            for (int w = 0; w < 8; w++) sum += part[w];
+            const float s = sum * (1.0f / sqrtf((float)D));
+            const float mag = sqrtf(fmaxf(fabsf(s), 1e-6f));
+            const float sgn = s > 0.0f ? 1.0f : (s < 0.0f ? -1.0f : 0.0f);
+            const float gv = 1.0f / (1.0f + expf(-(sgn * mag)));
+            gate[st] = gv; gate_out[tt * HC + st] = gv;
+        }
+        __syncthreads();
+    }
+    // (gated may alias kn: every read of this token's kn rows is behind the barriers above)
+    for (int c = tid; c < HC * D; c += 256) gated[(size_t)tt * HC * D + c] = v_[c % D] * gate[c / D];
+}
+
+// ---- per-layer-embedding conv: taps at t - 3 dil, t - 2 dil, t - dil, t with fp16 weights, every product and sum rounded
+// separately, silu; inputs before the chunk from hist[c] = [x(-3 dil) .. x(-1)]; x given or recomputed as (x * xscl) * xw.
+// y (optional) = conv; res (optional): res = res + (a + conv).
+CAMX_DEV float ple_x(const float * x, const float * xscl, const float * xw, int tb, int c, int C, int D) {
+    return xscl ? (x[(size_t)tb * C + c] * xscl[tb * (C / D) + c / D]) * xw[c] : x[(size_t)tb * C + c];
+}
+__global__ void __launch_bounds__(256) ple_conv_k(const float * __restrict__ x, const float * __restrict__ xscl, const float * __restrict__ xw,
+                                                  const uint16_t * __restrict__ w, const float * __restrict__ hist, float * __restrict__ y,
+                                                  const float * __restrict__ a, float * __restrict__ res, int C, int T, int D, int dil) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)T * C) return;
+    const int t = (int)(i / C), c = (int)(i - (long)t * C), hl = 3 * dil;
+    float conv = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int back = (3 - k) * dil;
+        const float xv = back <= t ? ple_x(x, xscl, xw, t - back, c, C, D) : hist[(size_t)c * hl + hl - (back - t)];
+        const float term = xv * h2f_bits(w[(size_t)c * 4 + k]);
+        conv = k == 0 ? term : conv + term;
+    }
+    const float o = conv / (1.0f + expf(-conv));
+    if (y) y[i] = o;
+    if (res) { const float ab = a[i] + o; res[i] = res[i] + ab; }
+}
+// hist[c] = the last 3 dil inputs of [hist[c], x[0 .. T - 1][c]]; 3 dil <= 32
+__global__ void __launch_bounds__(256) ple_hist_k(const float * __restrict__ x, const float * __restrict__ xscl, const float * __restrict__ xw,
+                                                  float * __restrict__ hist, int C, int T, int D, int dil) {
+    const int c = blockIdx.x * 256 + threadIdx.x, hl = 3 * dil;
+    if (c >= C) return;
+    float h[32];
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+        h[j] = 0.0f;
+        if (j < hl) { const int tj = T - hl + j; h[j] = tj < 0 ? hist[(size_t)c * hl + hl + tj] : ple_x(x, xscl, xw, tj, c, C, D); }
+    }
+#pragma unroll
+    for (int j = 0; j < 32; j++) if (j < hl) hist[(size_t)c * hl + j] = h[j];
+}
+
+extern "C" {
+
+// pf_gdn_norm (silu = 0: sigmoid gate; 1: silu gate, the reference's PF_GDN_SILU build) and q35p_gdn_norm16 (f16 = 1, silu gate)
+static int gdn_norm_launch(const float * o, const float * w, const float * z, void * y, int K, float eps, long rows, int silu, int f16, hipStream_t st) {
+    if (!o || !w || !z || !y || K < 4 || K % 4 || K > 1024 || rows < 0 || (((uintptr_t)o | (uintptr_t)w | (uintptr_t)z) & 15) || ((uintptr_t)y & (f16 ? 7 : 15)))
+        return CAMX_EINVAL;
+    if (rows == 0) return CAMX_OK;
+    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    const int ni = (K + 255) / 256;
+#define GN(S, F, N) gdn_norm_rows<S, F, N><<<grid, block, 0, st>>>(o, w, z, y, K, eps, rows)
+#define GN_NI(S, F) { if (ni == 1) GN(S, F, 1); else if (ni == 2) GN(S, F, 2); else GN(S, F, 4); }
+    if (f16) GN_NI(true, true) else if (silu) GN_NI(true, false) else GN_NI(false, false)
+#undef GN_NI
+#undef GN
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_gdn_norm(const float * o, const float * w, const float * z, float * y, int K, float eps, long rows, int silu, hipStream_t st) {
+    return gdn_norm_launch(o, w, z, y, K, eps, rows, silu, 0, st);
+}
+int camx_q35p_gdn_norm16(const float * o, const float * w, const float * z, uint16_t * y16, int K, float eps, long rows, hipStream_t st) {
+    return gdn_norm_launch(o, w, z, y16, K, eps, rows, 1, 1, st);
+}
+int camx_pf_gdn_gates(const float * al, int lda, const float * be, int ldb, const float * dt, const float * A, float * y, int H, int T, hipStream_t st) {
+    if (!al || !be || !dt || !A || !y || H < 1 || T < 0 || lda < H || ldb < H) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    if ((long)T * H >= 0x7fffffffL * 256) return CAMX_EINVAL;
+    gdn_gates_k<<<dim3((unsigned)(((long)T * H + 255) / 256)), dim3(256), 0, st>>>(al, lda, be, ldb, dt, A, y, H, T);
+    CAMX_LAUNCH_RET();
+}
+int camx_q35p_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, int rows, int * err, int T, hipStream_t st) {
+    if (!k || !v || !cache || !err || M < 1 || ldk < M || ldv < M || T < 0 || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    const int vec = !((M | ldk | ldv) & 3) && !(((uintptr_t)k | (uintptr_t)v) & 15) && !((uintptr_t)cache & 7);
+    kv_append16_k<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, cache, M, pos0, rows, err, vec);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_add_sum(const float * a, const float * b, float * y, long n, hipStream_t st) {
+    if (!a || !b || !y || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const int vec = n % 4 == 0 && !(((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15) && n / 4 < 0x7fffffffL * 256;
+    add_sum_k<<<vec ? dim3((unsigned)((n / 4 + 255) / 256)) : GRID_1D(n), dim3(256), 0, st>>>(a, b, y, n, vec);
+    CAMX_LAUNCH_RET();
+}
+static int to_bf16_launch(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, bool silu, hipStream_t st) {
+    if (!x || !y || T < 0 || Tpad < T || K < 1 || ldx < K) return CAMX_EINVAL;
+    if (Tpad == 0) return CAMX_OK;
+    const int vec = !((K | ldx) & 3) && !((uintptr_t)x & 15) && !((uintptr_t)y & 7);
+    const long n = (long)Tpad * K / (vec ? 4 : 1);
+    if (n >= 0x7fffffffL * 256) return CAMX_EINVAL;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (silu) to_bf16_rows<true><<<grid, block, 0, st>>>(x, ldx, y, T, Tpad, K, rs, vec); else to_bf16_rows<false><<<grid, block, 0, st>>>(x, ldx, y, T, Tpad, K, rs, vec);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_silu_bf16(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, hipStream_t st) { return to_bf16_launch(x, ldx, y, T, Tpad, K, rs, true, st); }
+int camx_pf_to_bf16(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, hipStream_t st) { return to_bf16_launch(x, ldx, y, T, Tpad, K, 0.0f, false, st); }
+int camx_pf_hc_avg(const float * r, float * y, int T, int hc, int D, int ldo, hipStream_t st) {
+    if (!r || !y || T < 0 || hc < 1 || D < 1 || ldo < D) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    const int vec = !((D | ldo) & 3) && !(((uintptr_t)r | (uintptr_t)y) & 15);
+    const long n = (long)T * D / (vec ? 4 : 1);
+    hc_avg_k<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(r, y, T, hc, D, ldo, vec);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_ple_gate(const float * kn, const float * q, const float * qscl, const float * qw, const float * val, int ldv, float * gated, float * gate_out,
+                     int HC, int D, int T, hipStream_t st) {
+    if (!kn || !q || !val || !gated || !gate_out || HC < 1 || HC > 8 || D < 1 || ldv < D || T < 0 || ((qscl == nullptr) != (qw == nullptr))) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    ple_gate_k<<<dim3(T), dim3(256), 0, st>>>(kn, q, qscl, qw, val, ldv, gated, gate_out, HC, D);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_ple_conv(const float * x, const float * xscl, const float * xw, const uint16_t * w, const float * hist, float * y, const float * a, float * res,
+                     int C, int T, int D, int dil, hipStream_t st) {
+    if (!x || !w || !hist || (!y && !res) || (res && !a) || C < 1 || T < 0 || D < 1 || C % D || dil < 1 || ((xscl == nullptr) != (xw == nullptr))) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    if ((long)T * C >= 0x7fffffffL * 256) return CAMX_EINVAL;
+    ple_conv_k<<<dim3((unsigned)(((long)T * C + 255) / 256)), dim3(256), 0, st>>>(x, xscl, xw, w, hist, y, a, res, C, T, D, dil);
+    CAMX_LAUNCH_RET();
+}
+int camx_pf_ple_hist(const float * x, const float * xscl, const float * xw, float * hist, int C, int T, int D, int dil, hipStream_t st) {
+    if (!x || !hist || C < 1 || T < 0 || D < 1 || C % D || dil < 1 || 3 * dil > 32 || ((xscl == nullptr) != (xw == nullptr))) return CAMX_EINVAL;
+    ple_hist_k<<<dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st>>>(x, xscl, xw, hist, C, T, D, dil);
+    CAMX_LAUNCH_RET();
+}
+
+}   // extern "C"

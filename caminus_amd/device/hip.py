@@ -154,20 +154,29 @@ def _glue(K):
             'pf_hc_post_rms': ('camx_pf_hc_post_rms', lambda g, b, v: list(v) + [I(K)]),
             'pf_hc_post': _plain('camx_pf_hc_post'), 'pf_hc_mean': _plain('camx_pf_hc_mean'),
             'pf_gdn_conv': ('camx_pf_gdn_conv', lambda g, b, v: list(v) + [I(0)]),
-            'pf_conv_state': ('camx_pf_conv_state', lambda g, b, v: list(v) + [I(0)])}
+            'pf_conv_state': ('camx_pf_conv_state', lambda g, b, v: list(v) + [I(0)]),
+            'pf_add_sum': ('camx_pf_add_sum', lambda g, b, v: [v[0], v[1], v[2], L64(_val(v[3]))]),
+            'pf_silu_bf16': _plain('camx_pf_silu_bf16'), 'pf_to_bf16': _plain('camx_pf_to_bf16'),
+            'pf_ple_gate': _rows('camx_pf_ple_gate'), 'pf_ple_conv': _plain('camx_pf_ple_conv'), 'pf_ple_hist': _plain('camx_pf_ple_hist')}
 
 
 _ATTN = {'pf_qk_nr': ('camx_pf_qk_nr', _pf_qk_nr), 'pf_hadamard': _plain('camx_pf_hadamard'), 'pf_kv_append': _rows('camx_pf_kv_append'),
-         'pf_gate_mul': _gate(0)}
-_GDN = {'pf_gdn_l2': ('camx_pf_gdn_l2', _pf_gdn_l2)}
-_Q35 = {'q35p_add_rms16': _rows('camx_q35p_add_rms16'), 'q35p_gate_mul16': _gate(1)}
+         'pf_gate_mul': _gate(0), 'pf_hc_avg': _plain('camx_pf_hc_avg')}
+def _gdn_norm(silu):
+    return 'camx_pf_gdn_norm', lambda g, b, v: list(v) + [L64(g[0]), I(silu)]     # one workgroup per (token, value head) in the reference
+
+
+_GDN = {'pf_gdn_l2': ('camx_pf_gdn_l2', _pf_gdn_l2), 'pf_gdn_gates': _plain('camx_pf_gdn_gates'), 'pf_gdn_norm': _gdn_norm(0)}
+_GDN_SILU = dict(_GDN, pf_gdn_norm=_gdn_norm(1))                                   # the code objects built with PF_GDN_SILU (qwen35moe / qwen3next)
+_Q35 = {'q35p_add_rms16': _rows('camx_q35p_add_rms16'), 'q35p_gate_mul16': _gate(1),
+        'q35p_gdn_norm16': ('camx_q35p_gdn_norm16', lambda g, b, v: list(v) + [L64(g[0])]), 'q35p_kv_append16': _rows('camx_q35p_kv_append16')}
 
 SYMBOLS = {
     'core': _CORE, 'fuse': _FUSE, 'actq': _ACTQ, 'kv_codec': _KV, 'prefill_feed': _FEED, 'k3_gguf': _GG, 'k3_gguf_swiglu': _GG,
     'q3m_prefill': _q3m(False, False), 'q3m_prefill_kvq8': _q3m(False, True), 'q3m_prefill_yarn': _q3m(True, False),
     'q3m_prefill_kvq8_yarn': _q3m(True, True), 'q35_prefill': _Q35,
     'prefill_glue': _glue(2560), 'prefill_glue_q35': _glue(2048), 'prefill_glue_q35d': _glue(5120),
-    'prefill_attn': _ATTN, 'prefill_attn_q35': _ATTN, 'prefill_attn_q35d': _ATTN, 'prefill_gdn': _GDN, 'prefill_gdn_q35': _GDN,
+    'prefill_attn': _ATTN, 'prefill_attn_q35': _ATTN, 'prefill_attn_q35d': _ATTN, 'prefill_gdn': _GDN, 'prefill_gdn_q35': _GDN_SILU,
     'prefill_mmq_glue': {},      # its quantizers are template instances in the reference: caminus_amd.prefill.mmq binds them
     'camx': {},                  # direct access to every C entry point by its own name (Module('camx').camx_...)
 }

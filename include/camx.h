@@ -210,6 +210,37 @@ int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t
 int camx_residual_slices_bwd(const float * dout, const int * pos, uint16_t * dm, uint16_t * dmlp, uint16_t * dys, int d, long n4,
                              camx_stream_t stream);
 
+/* ---- more row kernels of the batched prefill ------------------------------------------------------------------------------------------ */
+/* pf_gdn_norm (kernels/prefill_gdn.hip:385-407): per (token, value head) row of K values, y = ((o * rsqrt(mean(o^2) + eps)) * w) *
+ * sigmoid(z) (silu = 0) or * silu(z) (silu = 1: the reference's PF_GDN_SILU build). K % 4 == 0, K <= 1024. */
+int camx_pf_gdn_norm(const float * o, const float * w, const float * z, float * y, int K, float eps, long rows, int silu, camx_stream_t stream);
+/* q35p_gdn_norm16 (kernels/q35_prefill.hip:671-692): the silu form with fp16 output. */
+int camx_q35p_gdn_norm16(const float * o, const float * w, const float * z, uint16_t * y16, int K, float eps, long rows, camx_stream_t stream);
+/* pf_gdn_gates (kernels/prefill_gdn.hip:80-92): y [T][2H] = softplus(alpha + dt) * a | sigmoid(beta); alpha / beta rows at lda / ldb. */
+int camx_pf_gdn_gates(const float * alpha, int lda, const float * beta, int ldb, const float * dt, const float * a, float * y, int H, int T,
+                      camx_stream_t stream);
+/* q35p_kv_append16 (kernels/q35_prefill.hip:694-707): cache[pos0 + t] = fp16(k[t]) | fp16(v[t]) (2 M halves per position); a row at
+ * or past `rows` is not written and sets bit 0 of *err. */
+int camx_q35p_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, int rows, int * err, int T,
+                          camx_stream_t stream);
+/* pf_add_sum (kernels/prefill_glue.hip:416-423): y = y + (a + b). */
+int camx_pf_add_sum(const float * a, const float * b, float * y, long n, camx_stream_t stream);
+/* pf_silu_bf16 / pf_to_bf16 (kernels/prefill_glue.hip:552-566): y [Tpad][K] = bf16(silu(fma(rs, x, 0))) / bf16(x) for rows < T (x rows
+ * at ldx), zero rows from T to Tpad. */
+int camx_pf_silu_bf16(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, camx_stream_t stream);
+int camx_pf_to_bf16(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, camx_stream_t stream);
+/* pf_hc_avg (kernels/prefill_attn.hip:388-397): y[t][i] = (((r0 + r1) + r2) + ..) * (1 / hc) of r [T][hc][D]; y rows at ldo. */
+int camx_pf_hc_avg(const float * r, float * y, int T, int hc, int D, int ldo, camx_stream_t stream);
+/* pf_ple_gate (kernels/prefill_glue.hip:343-372): per token and stream, gate = sigmoid(sgn(s) sqrt(max(|s|, 1e-6))), s = (kn . qn) /
+ * sqrt(D); gated = val * gate. qn = q, or (q * qscl) * qw when qscl / qw are given. gated may alias kn. HC <= 8. */
+int camx_pf_ple_gate(const float * kn, const float * q, const float * qscl, const float * qw, const float * val, int ldv, float * gated,
+                     float * gate_out, int HC, int D, int T, camx_stream_t stream);
+/* pf_ple_conv / pf_ple_hist (kernels/prefill_glue.hip:374-414): dilated 4-tap conv with fp16 weights + silu over a chunk, optionally
+ * fused with res = res + (a + conv); the history of the last 3 dil inputs per channel (3 dil <= 32). */
+int camx_pf_ple_conv(const float * x, const float * xscl, const float * xw, const uint16_t * w, const float * hist, float * y, const float * a,
+                     float * res, int C, int T, int D, int dil, camx_stream_t stream);
+int camx_pf_ple_hist(const float * x, const float * xscl, const float * xw, float * hist, int C, int T, int D, int dil, camx_stream_t stream);
+
 /* ---- activation fake-quant, forward (kernels/actq.hip) ------------------------------------------------------------------------------ */
 /* actq_fwd_{f32,bf16} and actq_fwd_codes_{f32,bf16} (kernels/actq.hip:96-132, 315-326): M rows of K values (K % 128 == 0,
  * K <= 8192); y bf16 [M][K] (optional when codes are written), s [M] (optional), codes [M][K / 2] bytes (optional). */

@@ -388,6 +388,68 @@ def emb_iq2s(W, vocab, toks, N):
     lib().orc_emb_iq2s(_p(W), I(vocab), _p(toks), _p(x), _p(xbf), I(N), I(toks.size), _p(grid)); return x, xbf
 
 
+# ---- more row kernels of the batched prefill ---------------------------------------------------------------------------------
+
+
+def gdn_norm(o, w, z, eps, silu=False):
+    """-> (y fp32 [rows, K], y16 fp16 bits)"""
+    o = _c(o, np.float32); rows, K = o.shape; w = _c(w, np.float32); z = _c(z, np.float32)
+    y = np.empty((rows, K), np.float32); y16 = np.empty((rows, K), np.uint16)
+    lib().orc_gdn_norm(_p(o), _p(w), _p(z), _p(y), _p(y16), I(K), F(eps), C.c_long(rows), I(int(silu))); return y, y16
+
+
+def gdn_gates(al, be, dt, A):
+    al = _c(al, np.float32); be = _c(be, np.float32); T, H = al.shape[0], dt.size
+    dt = _c(dt, np.float32); A = _c(A, np.float32); y = np.empty((T, 2 * H), np.float32)
+    lib().orc_gdn_gates(_p(al), I(al.shape[1]), _p(be), I(be.shape[1]), _p(dt), _p(A), _p(y), I(H), I(T)); return y
+
+
+def kv_append16(k, v, M, cache, pos0):
+    """-> (cache fp16 bits [rows, 2 M] after the append, err word)"""
+    k = _c(k, np.float32); v = _c(v, np.float32); cache = _c(cache, np.uint16).copy(); err = np.zeros(1, np.int32)
+    lib().orc_kv_append16(_p(k), I(k.shape[1]), _p(v), I(v.shape[1]), _p(cache), I(M), I(pos0), I(cache.shape[0]), _p(err), I(k.shape[0]))
+    return cache, int(err[0])
+
+
+def add_sum(a, b, y):
+    a = _c(a, np.float32); b = _c(b, np.float32); y = _c(y, np.float32).copy()
+    lib().orc_add_sum(_p(a), _p(b), _p(y), C.c_long(y.size)); return y
+
+
+def to_bf16_rows(x, T, Tpad, K, rs=0.0, silu=False):
+    x = _c(x, np.float32); y = np.empty((Tpad, K), np.uint16)
+    lib().orc_to_bf16_rows(_p(x), I(x.shape[1]), _p(y), I(T), I(Tpad), I(K), F(rs), I(int(silu))); return y
+
+
+def hc_avg(r, ldo=None):
+    r = _c(r, np.float32); T, hc, D = r.shape; ldo = ldo or D
+    y = np.zeros((T, ldo), np.float32)
+    lib().orc_hc_avg(_p(r), _p(y), I(T), I(hc), I(D), I(ldo)); return y
+
+
+def ple_gate(kn, q, val, qscl=None, qw=None):
+    """-> (gated [T, HC, D], gate [T, HC])"""
+    kn = _c(kn, np.float32); q = _c(q, np.float32); val = _c(val, np.float32); T, HC, D = kn.shape
+    qscl = _c(qscl, np.float32) if qscl is not None else None; qw = _c(qw, np.float32) if qw is not None else None
+    gated = np.empty((T, HC, D), np.float32); gate = np.empty((T, HC), np.float32)
+    lib().orc_ple_gate(_p(kn), _p(q), _p(qscl), _p(qw), _p(val), I(val.shape[1]), _p(gated), _p(gate), I(HC), I(D), I(T)); return gated, gate
+
+
+def ple_conv(x, w16, hist, D, dil, xscl=None, xw=None, a=None, res=None):
+    """-> (y [T, C], res after the fused add or None); w16: fp16 bits [C, 4]"""
+    x = _c(x, np.float32); T, Cc = x.shape; w16 = _c(w16, np.uint16); hist = _c(hist, np.float32)
+    xscl = _c(xscl, np.float32) if xscl is not None else None; xw = _c(xw, np.float32) if xw is not None else None
+    a = _c(a, np.float32) if a is not None else None; res = _c(res, np.float32).copy() if res is not None else None
+    y = np.empty((T, Cc), np.float32)
+    lib().orc_ple_conv(_p(x), _p(xscl), _p(xw), _p(w16), _p(hist), _p(y), _p(a), _p(res), I(Cc), I(T), I(D), I(dil)); return y, res
+
+
+def ple_hist(x, hist, D, dil, xscl=None, xw=None):
+    x = _c(x, np.float32); T, Cc = x.shape; hist = _c(hist, np.float32).copy()
+    xscl = _c(xscl, np.float32) if xscl is not None else None; xw = _c(xw, np.float32) if xw is not None else None
+    lib().orc_ple_hist(_p(x), _p(xscl), _p(xw), _p(hist), I(Cc), I(T), I(D), I(dil)); return hist
+
+
 # ---- actq -----------------------------------------------------------------------------------------------------------------------
 
 

@@ -890,4 +890,120 @@ ORC_API void orc_block_entry_bwd(const float * x, const float * nw, const float 
     }
 }
 
+/* ---- more row kernels of the batched prefill -----------------------------------------------------------------------------
+ * pf_gdn_norm / q35p_gdn_norm16 (prefill_gdn.hip:385-407, q35_prefill.hip:671-692): contraction off, so the row sum is a
+ * product and a sum per element in thread t = i % 256's chain; the 8 x 32 tree; rsqrtf -> 1 / sqrt. */
+ORC_API void orc_gdn_norm(const float * o, const float * w, const float * z, float * y, uint16_t * y16, int K, float eps, long rows, int silu) {
+    for (long r = 0; r < rows; r++) {
+        const float * orow = o + r * K, * zr = z + r * K;
+        float part[256];
+        for (int t = 0; t < 256; t++) part[t] = 0.0f;
+        for (int i = 0; i < K; i++) { const float p = orow[i] * orow[i]; part[i & 255] = part[i & 255] + p; }
+        float tot = 0.0f;
+        for (int g = 0; g < 8; g++) tot += bfly32_sum(part + 32 * g);
+        const float scale = rsqrt_c(tot / (float)K + eps);
+        for (int i = 0; i < K; i++) {
+            const float a = scale * orow[i], nrm = a * w[i];
+            float gate;
+            if (silu) { const float e = 1.0f + expf(-zr[i]); gate = zr[i] / e; } else { const float e = 1.0f + expf(-zr[i]); gate = 1.0f / e; }
+            const float v = nrm * gate;
+            if (y) y[r * K + i] = v;
+            if (y16) y16[r * K + i] = orc_f2h(v);
+        }
+    }
+}
+ORC_API void orc_gdn_gates(const float * al, int lda, const float * be, int ldb, const float * dt, const float * A, float * y, int H, int T) {
+    for (int tt = 0; tt < T; tt++)
+        for (int h = 0; h < H; h++) {
+            const float ab = al[(size_t)tt * lda + h] + dt[h];
+            const float sp = ab > 20.0f ? ab : logf(1.0f + expf(ab));
+            y[(size_t)tt * 2 * H + h] = sp * A[h];
+            y[(size_t)tt * 2 * H + H + h] = 1.0f / (1.0f + expf(-be[(size_t)tt * ldb + h]));
+        }
+}
+ORC_API void orc_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, int rows, int * err, int T) {
+    for (int tt = 0; tt < T; tt++) {
+        const long pos = (long)pos0 + tt;
+        if (pos < 0 || pos >= rows) { *err |= 1; continue; }
+        for (int i = 0; i < M; i++) { cache[(size_t)pos * 2 * M + i] = orc_f2h(k[(size_t)tt * ldk + i]); cache[(size_t)pos * 2 * M + M + i] = orc_f2h(v[(size_t)tt * ldv + i]); }
+    }
+}
+ORC_API void orc_add_sum(const float * a, const float * b, float * y, long n) { for (long i = 0; i < n; i++) { const float ab = a[i] + b[i]; y[i] = y[i] + ab; } }
+static inline uint16_t to_bf16_plain(float v) { const uint32_t u = f2u(v); return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16); }
+ORC_API void orc_to_bf16_rows(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, int silu) {
+    for (int t = 0; t < Tpad; t++)
+        for (int j = 0; j < K; j++) {
+            uint16_t o = 0;
+            if (t < T) {
+                float v = x[(size_t)t * ldx + j];
+                if (silu) { const float s = fmaf(rs, v, 0.0f); v = s / (1.0f + expf(-s)); }
+                o = to_bf16_plain(v);
+            }
+            y[(size_t)t * K + j] = o;
+        }
+}
+ORC_API void orc_hc_avg(const float * r, float * y, int T, int hc, int D, int ldo) {
+    for (int tt = 0; tt < T; tt++)
+        for (int i = 0; i < D; i++) {
+            float acc = r[(size_t)(tt * hc) * D + i];
+            for (int h = 1; h < hc; h++) acc = acc + r[(size_t)(tt * hc + h) * D + i];
+            y[(size_t)tt * ldo + i] = acc * (1.0f / (float)hc);
+        }
+}
+/* pf_ple_gate (prefill_glue.hip:343-372) */
+ORC_API void orc_ple_gate(const float * kn, const float * q, const float * qscl, const float * qw, const float * val, int ldv, float * gated,
+                          float * gate_out, int HC, int D, int T) {
+    for (int tt = 0; tt < T; tt++) {
+        float gate[8];
+        for (int st = 0; st < HC; st++) {
+            float part[256];
+            for (int t = 0; t < 256; t++) part[t] = 0.0f;
+            for (int i = 0; i < D; i++) {
+                const size_t o = ((size_t)tt * HC + st) * D + i;
+                const float qv = qscl ? (q[o] * qscl[tt * HC + st]) * qw[(size_t)st * D + i] : q[o];
+                const float p = kn[o] * qv;
+                part[i & 255] = part[i & 255] + p;
+            }
+            float sum = 0.0f;
+            for (int g = 0; g < 8; g++) sum += bfly32_sum(part + 32 * g);
+            const float s = sum * (1.0f / sqrtf((float)D));
+            const float mag = sqrtf(fmaxf(fabsf(s), 1e-6f));
+            const float sgn = s > 0.0f ? 1.0f : (s < 0.0f ? -1.0f : 0.0f);
+            gate[st] = 1.0f / (1.0f + expf(-(sgn * mag)));
+            gate_out[tt * HC + st] = gate[st];
+        }
+        for (int c = 0; c < HC * D; c++) gated[(size_t)tt * HC * D + c] = val[(size_t)tt * ldv + c % D] * gate[c / D];
+    }
+}
+/* pf_ple_conv / pf_ple_hist (prefill_glue.hip:374-414); w: fp16 bits [C][4] */
+static float ple_x_c(const float * x, const float * xscl, const float * xw, int tb, int c, int C, int D) {
+    return xscl ? (x[(size_t)tb * C + c] * xscl[tb * (C / D) + c / D]) * xw[c] : x[(size_t)tb * C + c];
+}
+ORC_API void orc_ple_conv(const float * x, const float * xscl, const float * xw, const uint16_t * w, const float * hist, float * y, const float * a,
+                          float * res, int C, int T, int D, int dil) {
+    const int hl = 3 * dil;
+    for (int t = 0; t < T; t++)
+        for (int c = 0; c < C; c++) {
+            float conv = 0.0f;
+            for (int k = 0; k < 4; k++) {
+                const int back = (3 - k) * dil;
+                const float xv = back <= t ? ple_x_c(x, xscl, xw, t - back, c, C, D) : hist[(size_t)c * hl + hl - (back - t)];
+                const float term = xv * orc_h2f(w[(size_t)c * 4 + k]);
+                conv = k == 0 ? term : conv + term;
+            }
+            const float o = conv / (1.0f + expf(-conv));
+            const size_t i = (size_t)t * C + c;
+            if (y) y[i] = o;
+            if (res) { const float ab = a[i] + o; res[i] = res[i] + ab; }
+        }
+}
+ORC_API void orc_ple_hist(const float * x, const float * xscl, const float * xw, float * hist, int C, int T, int D, int dil) {
+    const int hl = 3 * dil;
+    for (int c = 0; c < C; c++) {
+        float h[32];
+        for (int j = 0; j < hl; j++) { const int tj = T - hl + j; h[j] = tj < 0 ? hist[(size_t)c * hl + hl + tj] : ple_x_c(x, xscl, xw, tj, c, C, D); }
+        for (int j = 0; j < hl; j++) hist[(size_t)c * hl + j] = h[j];
+    }
+}
+
 ORC_API int orc_version(void) { return 1; }

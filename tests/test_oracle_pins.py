@@ -603,3 +603,79 @@ def test_kv_q8_reader_against_numpy_decoder_and_literals():
     hk, _, _ = O.kv_q8_read(blk, 32, 1, f16=True)
     assert np.array_equal(hk, lk.astype(np.float16).view(np.uint16))
     assert O.kv_q8_read(cache, M, 2, pos0=T - 1)[2] == 1 and O.kv_q8_read(cache, 48, 1)[2] == 4
+
+
+# ---- more row kernels of the batched prefill: numpy closed forms ---------------------------------------------------------------------
+
+def test_gdn_norm_gates_and_glue_against_numpy():
+    rng = np.random.default_rng(21)
+    rows, K = 37, 128
+    o = rng.standard_normal((rows, K)).astype(f32) * 3; z = rng.standard_normal((rows, K)).astype(f32) * 2; w = (1 + 0.1 * rng.standard_normal(K)).astype(f32)
+    o64, z64 = o.astype(np.float64), z.astype(np.float64)
+    scale = 1 / np.sqrt((o64 ** 2).mean(1, keepdims=True) + 1e-6)
+    for silu in (False, True):
+        y, y16 = O.gdn_norm(o, w, z, 1e-6, silu=silu)
+        gate = z64 / (1 + np.exp(-z64)) if silu else 1 / (1 + np.exp(-z64))
+        assert np.allclose(y, o64 * scale * w * gate, rtol=3e-6, atol=1e-7)
+        assert np.array_equal(y16, y.astype(np.float16).view(np.uint16))
+    # a row whose sum of squares is known exactly: 128 ones -> scale = 1 / sqrt(1 + eps)
+    y, _ = O.gdn_norm(np.ones((1, K), f32), np.ones(K, f32), np.zeros((1, K), f32), 0.0)
+    assert np.array_equal(y, np.full((1, K), 0.5, f32))
+    T, H = 9, 48
+    al = rng.standard_normal((T, H + 3)).astype(f32) * 8; be = rng.standard_normal((T, H)).astype(f32) * 4
+    dt = rng.standard_normal(H).astype(f32); A = -np.exp(rng.standard_normal(H)).astype(f32)
+    al[0, :2] = [30.0, -40.0]
+    g = O.gdn_gates(al, be, dt, A)
+    ab = (al[:, :H] + dt).astype(f32)                                     # the statement is fp32's: 1 + exp(ab) is rounded before the log
+    with np.errstate(over='ignore'):
+        sp = np.where(ab > 20, ab, np.log((f32(1) + np.exp(ab)).astype(f32))).astype(f32)
+    # (one ulp of 1 + exp(ab) is 6e-8 whatever ab is: the statement's own conditioning sets the absolute tolerance)
+    assert np.allclose(g[:, :H], sp * A, rtol=1e-5, atol=3e-7 * np.abs(A).max()) and g[0, 0] == ab[0, 0] * A[0] and g[0, 1] == 0
+    assert np.allclose(g[:, H:], 1 / (1 + np.exp(-be.astype(np.float64))), rtol=2e-6)
+    a = rng.standard_normal(1000).astype(f32); b = rng.standard_normal(1000).astype(f32); yv = rng.standard_normal(1000).astype(f32)
+    assert np.array_equal(O.add_sum(a, b, yv), yv + (a + b))
+    x = rng.standard_normal((5, 40)).astype(f32) * 4
+    assert np.array_equal(O.to_bf16_rows(x, 5, 8, 32)[:5], O.f2bf(x[:, :32])) and not O.to_bf16_rows(x, 5, 8, 32)[5:].any()
+    s = (np.float32(0.25) * x[:, :32]).astype(f32)
+    want = O.f2bf((s / (f32(1) + np.exp(-s.astype(np.float64)).astype(f32))).astype(f32))
+    got = O.to_bf16_rows(x, 5, 8, 32, rs=0.25, silu=True)[:5]
+    assert (np.abs(got.astype(np.int32) - want.astype(np.int32)) <= 1).all() and (got == want).mean() > 0.97
+    r = rng.standard_normal((6, 4, 20)).astype(f32)
+    assert np.array_equal(O.hc_avg(r, ldo=24)[:, :20], (((r[:, 0] + r[:, 1]) + r[:, 2]) + r[:, 3]) * f32(0.25))
+    k = rng.standard_normal((4, 70)).astype(f32) * 100; v = rng.standard_normal((4, 66)).astype(f32)
+    cache0 = np.full((7, 128), 0x1234, np.uint16)
+    c, err = O.kv_append16(k, v, 64, cache0, 2)
+    assert err == 0 and np.array_equal(c[2:6, :64], k[:, :64].astype(np.float16).view(np.uint16)) and np.array_equal(c[2:6, 64:], v[:, :64].astype(np.float16).view(np.uint16))
+    assert (c[:2] == 0x1234).all() and (c[6:] == 0x1234).all()
+    c, err = O.kv_append16(k, v, 64, cache0, 5)
+    assert err == 1 and (c[:5] == 0x1234).all() and np.array_equal(c[5, :64], k[0, :64].astype(np.float16).view(np.uint16))
+
+
+def test_ple_gate_conv_hist_against_numpy():
+    rng = np.random.default_rng(22)
+    T, HC, D, dil = 11, 4, 96, 3
+    kn = rng.standard_normal((T, HC, D)).astype(f32); q = rng.standard_normal((T, HC, D)).astype(f32); val = rng.standard_normal((T, D + 8)).astype(f32)
+    qscl = (0.5 + rng.random(T * HC)).astype(f32); qw = (1 + 0.1 * rng.standard_normal((HC, D))).astype(f32)
+    for recompute in (False, True):
+        gated, gate = O.ple_gate(kn, q, val, qscl if recompute else None, qw if recompute else None)
+        qn = (q * qscl.reshape(T, HC, 1)) * qw if recompute else q
+        s = (kn.astype(np.float64) * qn.astype(np.float64)).sum(-1) / np.sqrt(D)
+        gref = 1 / (1 + np.exp(-np.sign(s) * np.sqrt(np.maximum(np.abs(s), 1e-6))))
+        assert np.allclose(gate, gref, rtol=1e-5) and np.array_equal(gated, val[:, None, :D] * gate[:, :, None])
+    kz = np.zeros((1, 1, D), f32)
+    assert O.ple_gate(kz, kz, np.ones((1, D), f32))[1][0, 0] == f32(0.5)          # s = 0: sgn 0, gate exactly 1 / 2
+    # conv: taps at t - 9, t - 6, t - 3, t
+    C = HC * D
+    x = rng.standard_normal((T, C)).astype(f32); w16 = (rng.standard_normal((C, 4)) * 0.5).astype(np.float16); hist = rng.standard_normal((C, 3 * dil)).astype(f32)
+    xscl = (0.5 + rng.random(T * HC)).astype(f32); xw = (1 + 0.1 * rng.standard_normal(C)).astype(f32)
+    a = rng.standard_normal((T, C)).astype(f32); res = rng.standard_normal((T, C)).astype(f32)
+    for recompute in (False, True):
+        xn = ((x.reshape(T, HC, D) * xscl.reshape(T, HC, 1)).reshape(T, C) * xw).astype(f32) if recompute else x
+        full = np.concatenate([hist.T, xn], 0)                              # time -9 .. T - 1
+        wf = w16.astype(f32)
+        conv = (((full[0:T] * wf[:, 0] + full[3:T + 3] * wf[:, 1]) + full[6:T + 6] * wf[:, 2]) + full[9:T + 9] * wf[:, 3]).astype(f32)
+        y, r2 = O.ple_conv(x, w16.view(np.uint16), hist, D, dil, xscl if recompute else None, xw if recompute else None, a=a, res=res)
+        want = conv.astype(np.float64) / (1 + np.exp(-conv.astype(np.float64)))
+        assert np.allclose(y, want, rtol=3e-6, atol=1e-7) and np.array_equal(r2, res + (a + y))
+        assert np.array_equal(O.ple_hist(x, hist, D, dil, xscl if recompute else None, xw if recompute else None), full[-9:].T)
+    assert np.array_equal(O.ple_hist(x[:4], hist, D, dil), np.concatenate([hist.T, x[:4]], 0)[-9:].T)      # a chunk shorter than the history
