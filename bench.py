@@ -344,6 +344,24 @@ def prefill_scale_sweep(B):
         x = B.acts((Mr * Kq,), torch.float32, i); m = B.acts((Mr * Kq,), torch.bfloat16, i + 1); y = B.acts((Mr * Kq,), torch.bfloat16, i + 2); o = torch.empty(Mr * Kq, device=dev)
         return lambda: B.call('camx_residual3', _p(x), _p(m), _p(y), _p(o), L64(Mr * Kq))
     timeit('residual3 16M', Mr * Kq * 12, sets(mk))
+    rows_g, Kg = T * 48, 128
+    def mk(i):
+        o = B.acts((rows_g, Kg), torch.float32, i); z = B.acts((rows_g, Kg), torch.float32, i + 1, frac=0); wg = B.gamma(Kg, 5); y16 = torch.empty((rows_g, Kg), dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_q35p_gdn_norm16', _p(o), _p(wg), _p(z), _p(y16), I(Kg), F(1e-6), C.c_long(rows_g))
+    timeit('q35p_gdn_norm16 4096x48x128', rows_g * Kg * 10, sets(mk))
+    Dh = 2560
+    def mk(i):
+        r = B.acts((2048, 4, Dh), torch.float32, i); y = torch.empty((2048, Dh), device=dev)
+        return lambda: B.call('camx_pf_hc_avg', _p(r), _p(y), I(2048), I(4), I(Dh), I(Dh))
+    timeit('pf_hc_avg 2048x4x2560', 2048 * Dh * 20, sets(mk))
+    def mk(i):
+        a = B.acts((Mr * Kq,), torch.float32, i); b = B.acts((Mr * Kq,), torch.float32, i + 1); y = B.acts((Mr * Kq,), torch.float32, i + 2)
+        return lambda: B.call('camx_pf_add_sum', _p(a), _p(b), _p(y), L64(Mr * Kq))
+    timeit('pf_add_sum 16M', Mr * Kq * 16, sets(mk))
+    def mk(i):
+        x = B.acts((4096, 5120), torch.float32, i); y = torch.empty((4096, 5120), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_pf_to_bf16', _p(x), I(5120), _p(y), I(4096), I(4096), I(5120))
+    timeit('pf_to_bf16 4096x5120', 4096 * 5120 * 6, sets(mk))
     return res
 
 

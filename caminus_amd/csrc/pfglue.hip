@@ -50,6 +50,43 @@ __global__ void __launch_bounds__(256) gdn_norm_rows(const float * __restrict__ 
     }
 }
 
+// K = 128 (the GDN value heads) at prefill sizes: a half-wave per row, two rows per wave instruction, U rows per half-wave
+// with all their loads issued first. The logical threads past 128 hold zeros in the tree, so the four group sums of the row
+// added in order are the whole sum. FAST (fp16 output only): silu from v_exp / v_rcp, rounded to 16 bits at once.
+CAMX_DEV float silu_fast16(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.442695041f)); }
+template <bool SILU, bool F16OUT, int U>
+__global__ void __launch_bounds__(256) gdn_norm_128(const float * __restrict__ o, const float * __restrict__ w, const float * __restrict__ z,
+                                                    void * __restrict__ y, float eps, long rows) {
+    const int lane = slot_of(threadIdx.x & 63), l = lane & 31;
+    const long span = (long)gridDim.x * 8;
+    const long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+    f32x4 ov[U], zv[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const long r = r0 + u * span, rc = r < rows ? r : 0;
+        ov[u] = __builtin_nontemporal_load((const f32x4 *)(o + rc * 128 + 4 * l));
+        zv[u] = __builtin_nontemporal_load((const f32x4 *)(z + rc * 128 + 4 * l));
+    }
+    const f32x4 wv = *(const f32x4 *)(w + 4 * l);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const long r = r0 + u * span;
+        f32x4 ss;
+        ss.x = 0.0f + ov[u].x * ov[u].x; ss.y = 0.0f + ov[u].y * ov[u].y; ss.z = 0.0f + ov[u].z * ov[u].z; ss.w = 0.0f + ov[u].w * ov[u].w;
+        const float tot = half_groups_in_order<4>(group32_sum(ss), lane & 32);
+        const float scale = rsqrt_exact(tot / 128.0f + eps);
+        f32x4 rr;
+#define G_(e) { const float nrm = (scale * ov[u].e) * wv.e; const float zz = zv[u].e; \
+                rr.e = F16OUT ? nrm * silu_fast16(zz) : (SILU ? nrm * (zz / (1.0f + expf(-zz))) : nrm * (1.0f / (1.0f + expf(-zz)))); }
+        G_(x) G_(y) G_(z) G_(w)
+#undef G_
+        if (r < rows) {
+            if (F16OUT) __builtin_nontemporal_store(pack_f16x4(rr), (u32x2 *)((uint16_t *)y + r * 128 + 4 * l));
+            else __builtin_nontemporal_store(rr, (f32x4 *)((float *)y + r * 128 + 4 * l));
+        }
+    }
+}
+
 // ---- GDN gates: gate = softplus(alpha + dt) * a, beta_sig = sigmoid(beta); y [T][2H] = gate | beta_sig -----------------------
 __global__ void __launch_bounds__(256) gdn_gates_k(const float * __restrict__ al, int lda, const float * __restrict__ be, int ldb,
                                                    const float * __restrict__ dt, const float * __restrict__ A, float * __restrict__ y, int H, int T) {
@@ -93,6 +130,25 @@ __global__ void __launch_bounds__(256) add_sum_k(const float * __restrict__ a, c
 }
 
 // ---- bf16 operand copies with zero rows up to Tpad: y[t][j] = bf16(SILU ? silu(fma(rs, x, 0)) : x) ---------------------------
+// eight values per thread (K % 8 == 0, aligned): two 128-bit loads, one 128-bit non-temporal store
+template <bool SILU>
+__global__ void __launch_bounds__(256) to_bf16_rows8(const float * __restrict__ x, int ldx, uint16_t * __restrict__ y, int T, int Tpad, int K, float rs) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x, i = q * 8;
+    if (i >= (long)Tpad * K) return;
+    const int t = (int)(i / K), j = (int)(i - (long)t * K);
+    u32x4 out = {0u, 0u, 0u, 0u};
+    if (t < T) {
+        f32x4 a = __builtin_nontemporal_load((const f32x4 *)(x + (size_t)t * ldx + j)), b = __builtin_nontemporal_load((const f32x4 *)(x + (size_t)t * ldx + j + 4));
+        if (SILU) {
+#define S_(v) { const float s = __builtin_fmaf(rs, v, 0.0f); v = s / (1.0f + expf(-s)); }
+            S_(a.x) S_(a.y) S_(a.z) S_(a.w) S_(b.x) S_(b.y) S_(b.z) S_(b.w)
+#undef S_
+        }
+        const u32x2 lo = pack_bf16x4_rne(a), hi = pack_bf16x4_rne(b);
+        out = (u32x4){lo.x, lo.y, hi.x, hi.y};
+    }
+    __builtin_nontemporal_store(out, (u32x4 *)(y + i));
+}
 template <bool SILU>
 __global__ void __launch_bounds__(256) to_bf16_rows(const float * __restrict__ x, int ldx, uint16_t * __restrict__ y, int T, int Tpad, int K, float rs, int vec) {
     const long q = (long)blockIdx.x * 256 + threadIdx.x;
@@ -214,6 +270,13 @@ static int gdn_norm_launch(const float * o, const float * w, const float * z, vo
         return CAMX_EINVAL;
     if (rows == 0) return CAMX_OK;
     const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    if (K == 128 && rows >= 32768) {                                     // a prefill chunk: four rows per half-wave
+        const dim3 g4((unsigned)((rows + 31) / 32));
+        if (f16) gdn_norm_128<true, true, 4><<<g4, block, 0, st>>>(o, w, z, y, eps, rows);
+        else if (silu) gdn_norm_128<true, false, 4><<<g4, block, 0, st>>>(o, w, z, y, eps, rows);
+        else gdn_norm_128<false, false, 4><<<g4, block, 0, st>>>(o, w, z, y, eps, rows);
+        CAMX_LAUNCH_RET();
+    }
     const int ni = (K + 255) / 256;
 #define GN(S, F, N) gdn_norm_rows<S, F, N><<<grid, block, 0, st>>>(o, w, z, y, K, eps, rows)
 #define GN_NI(S, F) { if (ni == 1) GN(S, F, 1); else if (ni == 2) GN(S, F, 2); else GN(S, F, 4); }
@@ -252,6 +315,11 @@ int camx_pf_add_sum(const float * a, const float * b, float * y, long n, hipStre
 static int to_bf16_launch(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, bool silu, hipStream_t st) {
     if (!x || !y || T < 0 || Tpad < T || K < 1 || ldx < K) return CAMX_EINVAL;
     if (Tpad == 0) return CAMX_OK;
+    if (!((K | ldx) & 7) && !(((uintptr_t)x | (uintptr_t)y) & 15) && (long)Tpad * K / 8 < 0x7fffffffL * 256) {
+        const dim3 g8((unsigned)(((long)Tpad * K / 8 + 255) / 256));
+        if (silu) to_bf16_rows8<true><<<g8, dim3(256), 0, st>>>(x, ldx, y, T, Tpad, K, rs); else to_bf16_rows8<false><<<g8, dim3(256), 0, st>>>(x, ldx, y, T, Tpad, K, rs);
+        CAMX_LAUNCH_RET();
+    }
     const int vec = !((K | ldx) & 3) && !((uintptr_t)x & 15) && !((uintptr_t)y & 7);
     const long n = (long)Tpad * K / (vec ? 4 : 1);
     if (n >= 0x7fffffffL * 256) return CAMX_EINVAL;

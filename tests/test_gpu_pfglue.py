@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-@pytest.mark.parametrize('rows,K', [(16 * 48, 128), (5, 256), (3, 96), (7, 640), (4096 * 4, 128), (2, 1024)])
+@pytest.mark.parametrize('rows,K', [(16 * 48, 128), (5, 256), (3, 96), (7, 640), (4096 * 9 + 3, 128), (2, 1024)])
 def test_gdn_norm(rows, K):
     rng = np.random.default_rng(K + rows)
     o = outliers(rng, (rows, K)); z = (rng.standard_normal((rows, K)) * 3).astype(f32); w = (1 + 0.1 * rng.standard_normal(K)).astype(f32)
