@@ -679,3 +679,14 @@ def test_ple_gate_conv_hist_against_numpy():
         assert np.allclose(y, want, rtol=3e-6, atol=1e-7) and np.array_equal(r2, res + (a + y))
         assert np.array_equal(O.ple_hist(x, hist, D, dil, xscl if recompute else None, xw if recompute else None), full[-9:].T)
     assert np.array_equal(O.ple_hist(x[:4], hist, D, dil), np.concatenate([hist.T, x[:4]], 0)[-9:].T)      # a chunk shorter than the history
+
+
+def test_yarn_table_bits_against_the_reference_fixture():
+    """caminus_amd.rope's tables against the reference's own outputs, bit for bit (tests/golden/yarn_tables.npz, written once from the
+    reference's numpy-only python/caminus/rope.py by tests/golden/make_yarn_table_golden.py)"""
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'yarn_tables.npz'))
+    for case, want, corr, ms in zip(g['cases'], g['tables'], g['corr'], g['mscale']):
+        n_rot, base, factor, ctx = int(case[0]), float(case[1]), float(case[2]), int(case[3])
+        got = rope.yarn_table(n_rot, base, factor, ctx)
+        assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32)), case
+        assert rope.mscale(factor) == ms and tuple(rope.corr_dims(n_rot, ctx, base)) == tuple(corr)
