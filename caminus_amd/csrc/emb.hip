@@ -110,6 +110,7 @@ struct EmbArgs {
     const float * nw; float eps;
     float * h; uint16_t * h16; uint8_t * q8;
     int * err;               // optional: bit ERR_TOKEN is set when an id lies outside [0, vocab) (the id is clamped either way)
+    int stream;              // set by the launcher for large batches: the gathered rows leave as non-temporal stores
 };
 
 // EXACT: the row has exactly NI_MAX slabs (straight-line loops: the loads are issued as one batch)
@@ -145,8 +146,13 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) {
             const size_t o = (size_t)t * N + 256 * j + 4 * lane;
-            if (!TAIL || !a.d) { if (a.x) *(f32x4 *)(a.x + o) = xv[j]; }
-            if (a.xbf) *(u32x2 *)(a.xbf + o) = pack_f2bf_x4(xv[j]);
+            if (!TAIL && a.stream) {
+                if (a.x) __builtin_nontemporal_store(xv[j], (f32x4 *)(a.x + o));
+                if (a.xbf) __builtin_nontemporal_store(pack_f2bf_x4(xv[j]), (u32x2 *)(a.xbf + o));
+            } else {
+                if (!TAIL || !a.d) { if (a.x) *(f32x4 *)(a.x + o) = xv[j]; }
+                if (a.xbf) *(u32x2 *)(a.xbf + o) = pack_f2bf_x4(xv[j]);
+            }
         }
     if (!TAIL) return;
     if (a.d) {
@@ -181,8 +187,10 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
 }
 
 template <int FMT>
-static int launch_emb(const EmbArgs & a, hipStream_t st) {
-    if (a.n <= 0) return CAMX_OK;
+static int launch_emb(const EmbArgs & a0, hipStream_t st) {
+    if (a0.n <= 0) return CAMX_OK;
+    EmbArgs a = a0;
+    a.stream = (long)a.n * a.N >= (1L << 20);
     const dim3 grid((a.n + 3) / 4), block(256);
     const int ni = a.N >> 8;
     const bool tail = a.nw != nullptr;
