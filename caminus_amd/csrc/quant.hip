@@ -168,22 +168,21 @@ static int launch_mmq(const MmqArgs & a, int layout, hipStream_t st) {
 // off the VALU. The table itself is computed once per device ((float)exp in double, then the reference's fp32 statement
 // g / (1 + e), then round-to-nearest-even to bf16).
 //
-// A workgroup step is 16 tokens x one 1024-value slab (8 blocks of 128 values); wave w takes token w as two fully
-// coalesced 128-bit loads of g and of u: load i gives lane l the 8 consecutive values of 16-byte chunk 64 i + l. A
-// 32-value quantization group is the 4 lanes of a quad (for each i), a 128-value block 16 lanes. The reference's 8 threads
-// of a group are (lane & 3, half): thread 2 (lane & 3) + h holds values 4h .. 4h + 3 of the lane, so its xor 4 / 2 / 1
-// butterfly is lane ^ 2, lane ^ 1 (quad permutes) and the lane's two halves. Lane (l & 3) == i does group i's two IEEE
-// divisions (127 / amax, 1 / d_inv); the quad reads d_inv back through a DPP broadcast.
+// A wave's work item is 8 tokens x one 128-value block column: lane l takes the 8 consecutive values 8 (l & 15) .. + 7 of
+// tokens (l >> 4) and (l >> 4) + 4 (load i = token half i), so that one 128-bit load instruction of g (and of u) fetches
+// four 256-byte row pieces, and the 16 waves of a workgroup, on neighbouring columns of the same 8 tokens, 4 KiB of each
+// row. A 32-value quantization group is the 4 lanes of a quad (for each i), a 128-value block 16 lanes. The reference's
+// 8 threads of a group are (lane & 3, half): thread 2 (lane & 3) + h holds values 4h .. 4h + 3 of the lane, so its
+// xor 4 / 2 / 1 butterfly is lane ^ 2, lane ^ 1 (quad permutes) and the lane's two halves. Lane (l & 3) == i does
+// group i's two IEEE divisions (127 / amax, 1 / d_inv); the quad reads d_inv back through a DPP broadcast.
 //
-// Output: the 144-byte blocks of the step's 16 tokens are contiguous per block row (2304 B, a multiple of 64). Written
-// straight from the lanes they would leave as 8-byte pieces that straddle 64-byte boundaries (3.3 write requests per
-// block instead of 2.25, each costing a full 64-byte slot on the way to HBM), so the waves stage their blocks in LDS and
-// the workgroup writes each block row out as whole aligned 16-byte-per-lane runs.
-// Workgroups of one XCD (ids round-robin over the 8 XCDs) walk neighbouring token groups.
-#define SWM_TOK 16
-#define SWM_SLAB 1024
-#define SWM_KB (SWM_SLAB / 128)                  // block rows per step
-#define SWM_STAGE (SWM_KB * SWM_TOK * 144)       // 18432 bytes
+// Output: the 144-byte blocks of the item's 8 tokens are contiguous in the block row (1152 B = 9 whole 128-byte lines).
+// Written straight from the lanes they would leave as 8-byte pieces that straddle 64-byte boundaries (3.3 write requests
+// per block instead of 2.25, each costing a full 64-byte slot on the way to HBM), so a wave stages its blocks in its own
+// 1152 bytes of LDS and writes them out as one aligned run of 16 bytes per lane. Nothing but the table is shared
+// between waves: no barrier after the table copy, every wave runs its own pipeline (two items of loads in flight).
+#define SWM_TOK 8
+#define SWM_STAGE (16 * SWM_TOK * 144)           // 16 waves x 1152 bytes
 #define SWM_LDS (131072 + SWM_STAGE)
 
 __device__ uint16_t g_silu_lut[65536];
@@ -208,39 +207,40 @@ CAMX_DEV float max3_abs(float a, float b, float c) { return fmaxf(fmaxf(fabsf(a)
 
 struct SwmItem { u32x4 gw[2], uw[2]; };
 
-// issue the four 128-bit loads of work item (token t, slab). Every lane always issues all four (a lane past the row's
-// end, or a whole wave without work, reads 16 zero bytes instead): with a fixed number of loads in flight the compiler
-// can wait for exactly the older item's data and leave this item's loads outstanding across the other item's arithmetic.
+// issue the four 128-bit loads of work item (tokens tg .. tg + 7, block column unit). Every lane always issues all four
+// (a lane past the row's end or past the last token, or a whole wave without work, reads 16 zero bytes instead): with a
+// fixed number of loads in flight the compiler can wait for exactly the older item's data and leave this item's loads
+// outstanding across the other item's arithmetic.
 template <int SRC>
-CAMX_DEV void swm_load(SwmItem & it, const void * __restrict__ src, const int32_t * __restrict__ ids, long ld, long F, int t, int slab, int lane, bool valid) {
-    const long e0 = (long)slab * SWM_SLAB + 8 * lane;           // load i covers elements e0 + 512 i .. + 7
-    if (SRC == SRC_SWIGLU_BF16) {
-        const uint16_t * r = (const uint16_t *)src + (size_t)(valid ? t : 0) * ld + e0;
+CAMX_DEV void swm_load(SwmItem & it, const void * __restrict__ src, const int32_t * __restrict__ ids, long ld, long F, int T, long tg, long unit,
+                       int lane, bool valid) {
+    const long e0 = unit * 128 + 8 * (lane & 15);
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const bool ok = valid && e0 + 512 * i < F;
-            const u32x4 * pg = ok ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
-            const u32x4 * pu = ok ? (const u32x4 *)(r + F + 512 * i) : (const u32x4 *)g_zero16;
+    for (int i = 0; i < 2; i++) {
+        const long t = tg + (lane >> 4) + 4 * i;
+        const bool tok = valid && t < T;
+        if (SRC == SRC_SWIGLU_BF16) {
+            const bool ok = tok && e0 < F;
+            const uint16_t * r = (const uint16_t *)src + (size_t)(ok ? t : 0) * ld + e0;
+            const u32x4 * pg = ok ? (const u32x4 *)r : (const u32x4 *)g_zero16;
+            const u32x4 * pu = ok ? (const u32x4 *)(r + F) : (const u32x4 *)g_zero16;
             it.gw[i] = __builtin_nontemporal_load(pg); it.uw[i] = __builtin_nontemporal_load(pu);     // read once, never written: +15 % over plain loads
-        }
-    } else {                                                    // fp32 rows: gw[i] = values 0 .. 3, uw[i] = values 4 .. 7 of the lane's eight
-        const long row = valid ? (ids ? ids[t] : t) : 0;
-        const float * r = (const float *)src + (size_t)row * ld + e0;
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const u32x4 * p0 = valid && e0 + 512 * i < F ? (const u32x4 *)(r + 512 * i) : (const u32x4 *)g_zero16;
-            const u32x4 * p1 = valid && e0 + 512 * i + 4 < F ? (const u32x4 *)(r + 512 * i + 4) : (const u32x4 *)g_zero16;
+        } else {                                                // fp32 rows: gw[i] = values 0 .. 3, uw[i] = values 4 .. 7 of the lane's eight
+            const long row = tok ? (ids ? ids[t] : t) : 0;
+            const float * r = (const float *)src + (size_t)row * ld + e0;
+            const u32x4 * p0 = tok && e0 < F ? (const u32x4 *)r : (const u32x4 *)g_zero16;
+            const u32x4 * p1 = tok && e0 + 4 < F ? (const u32x4 *)(r + 4) : (const u32x4 *)g_zero16;
             it.gw[i] = __builtin_nontemporal_load(p0); it.uw[i] = __builtin_nontemporal_load(p1);
         }
     }
 }
 
-// the item's arithmetic; the wave's 8 blocks go to stage[kb][token slot][144]
+// the item's arithmetic; the wave's 8 blocks go to stage[token slot][144] (the wave's own 1152 bytes)
 template <int LAYOUT, int SRC>
-CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int t, int slab,
-                          int lane, int wave) {
+CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int T, long tg, long unit,
+                          int lane) {
     const int lq = lane & 3;
-    const long e0 = (long)slab * SWM_SLAB + 8 * lane;
+    const long e0 = unit * 128 + 8 * (lane & 15);
     float val[2][8];                                                   // the lane's eight values of each half, as quantized
     float amax[2], sum[2];
 #pragma unroll
@@ -267,7 +267,8 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
                 if (p == 0) s0 = v0 + v1; else if (p == 1) s0 = (s0 + v0) + v1; else if (p == 2) s1 = v0 + v1; else s1 = (s1 + v0) + v1;
             }
         }
-        if (SRC == SRC_SWIGLU_BF16 && act && e0 + 512 * i < F) *(u32x4 *)(act + (size_t)t * F + e0 + 512 * i) = (u32x4){pk[0], pk[1], pk[2], pk[3]};
+        const long t = tg + (lane >> 4) + 4 * i;
+        if (SRC == SRC_SWIGLU_BF16 && act && t < T && e0 < F) *(u32x4 *)(act + (size_t)t * F + e0) = (u32x4){pk[0], pk[1], pk[2], pk[3]};
         m = fmaxf(m, lane_xor2(m)); amax[i] = fmaxf(m, lane_xor1(m));
         sum[i] = 0.0f;
         if (LAYOUT == MMQ_DS4) {
@@ -282,69 +283,65 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
     float d_inv = 0.0f, d = 0.0f;
     if (am != 0.0f) { d_inv = 127.0f / am; d = 1.0f / d_inv; }
     const float di[2] = {quad_bcast<0>(d_inv), quad_bcast<1>(d_inv)};
-    uint8_t * blk0 = stage + ((lane >> 4) * SWM_TOK + wave) * 144;         // block row (lane >> 4) + 4 i, this wave's token slot
+    uint8_t * blk0 = stage + (lane >> 4) * 144;                            // token slot (lane >> 4) + 4 i
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         int q[8];
 #pragma unroll
         for (int p = 0; p < 8; p++) q[p] = round_i32(val[i][p] * di[i]);
-        *(u32x2 *)(blk0 + i * (4 * SWM_TOK * 144) + 16 + 8 * (lane & 15)) = (u32x2){pack_i8x4(q[0], q[1], q[2], q[3]), pack_i8x4(q[4], q[5], q[6], q[7])};
+        *(u32x2 *)(blk0 + i * (4 * 144) + 16 + 8 * (lane & 15)) = (u32x2){pack_i8x4(q[0], q[1], q[2], q[3]), pack_i8x4(q[4], q[5], q[6], q[7])};
     }
     if (lq < 2)
-        *(uint32_t *)(blk0 + lq * (4 * SWM_TOK * 144) + 4 * ((lane & 15) >> 2)) =
+        *(uint32_t *)(blk0 + lq * (4 * 144) + 4 * ((lane & 15) >> 2)) =
             LAYOUT == MMQ_DS4 ? ((uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sm) << 16)) : __builtin_bit_cast(uint32_t, d);
 }
 
 // SRC_F32 (quantize_mmq_q8_1 without scatter): the same work split and copy-out on fp32 rows (column c = row ids[c] or c), no table
 template <int LAYOUT, int SRC>
-__global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__ gu, const int32_t * __restrict__ ids, long ld, long F, long Kp,
-                                                       uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T, int ngroups, int nslab) {
+__global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__ gu, const int32_t * __restrict__ ids, long ld, long F,
+                                                       uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T, unsigned ncol, unsigned nitems) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
-    uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 131072 : 0);
-    const int xcd = blockIdx.x & 7, wgx = blockIdx.x >> 3, nwgx = gridDim.x >> 3;
-    const int per = (ngroups + 7) >> 3, lim = per * nslab;       // token groups per XCD, work items per XCD
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // work item j of this XCD: token group xcd * per + j / nslab, slab j % nslab; this wave's token inside the group: wave
-#define SWM_G(j) (xcd * per + (j) / nslab)
-#define SWM_T(j) (SWM_G(j) * SWM_TOK + wave)
-#define SWM_OK(j) ((j) < lim && SWM_G(j) < ngroups && SWM_T(j) < T)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 131072 : 0) + wave * (SWM_TOK * 144);
+    // item id -> token group id / ncol, block column id % ncol: the waves of a workgroup sit on neighbouring columns
+    const unsigned stride = gridDim.x * 16;                                   // (ids stay below 2^31: checked by the launcher)
+    unsigned j = blockIdx.x * 16 + wave;
+#define SWM_TG(id) ((long)((id) / ncol) * SWM_TOK)
+#define SWM_UNIT(id) ((long)((id) % ncol))
     SwmItem A, B, C;                                                          // three items in rotation: two steps of loads in flight
-    int j = wgx;
-    swm_load<SRC>(A, gu, ids, ld, F, SWM_T(j), j % nslab, lane, SWM_OK(j));             // in flight while the table is copied
-    swm_load<SRC>(B, gu, ids, ld, F, SWM_T(j + nwgx), (j + nwgx) % nslab, lane, SWM_OK(j + nwgx));
+    swm_load<SRC>(A, gu, ids, ld, F, T, SWM_TG(j), SWM_UNIT(j), lane, j < nitems);                  // in flight while the table is copied
+    swm_load<SRC>(B, gu, ids, ld, F, T, SWM_TG(j + stride), SWM_UNIT(j + stride), lane, j + stride < nitems);
     if (SRC == SRC_SWIGLU_BF16) {
         for (int i = threadIdx.x; i < 8192; i += 1024) ((u32x4 *)lut)[i] = ((const u32x4 *)g_silu_lut)[i];
         __syncthreads();
     }
-    // copy-out of a finished step: block row kb of the step = 2304 contiguous bytes = 144 lanes x 16 B
-    auto flush = [&](int jj) {
-        const int grp = SWM_G(jj), slab = jj % nslab;
-        const int ntok = min(SWM_TOK, T - grp * SWM_TOK);                     // tokens of the group that exist
-        for (int u = threadIdx.x; u < SWM_KB * 144; u += 1024) {
-            const int kb = u / 144, o = u - kb * 144;                           // o: 16-byte unit inside the row
-            const long kbg = (long)slab * SWM_KB + kb;
-            if (kbg * 128 < Kp && o < ntok * 9)
-                *(u32x4 *)(y + ((size_t)kbg * T + (size_t)grp * SWM_TOK) * 144 + 16 * o) = *(const u32x4 *)(stage + kb * (SWM_TOK * 144) + 16 * o);
-        }
+    // copy-out of a finished item: 1152 contiguous bytes = 72 lanes' worth of 16 B (lanes 0 .. 7 take a second unit)
+    auto flush = [&](unsigned id) {
+        const long tg = SWM_TG(id), unit = SWM_UNIT(id);
+        const int nunits = (int)min((long)SWM_TOK, T - tg) * 9;               // tokens of the group that exist
+        uint8_t * dst = y + ((size_t)unit * T + (size_t)tg) * 144;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // the wave's own LDS writes, in order
+        if (lane < nunits) *(u32x4 *)(dst + 16 * lane) = *(const u32x4 *)(stage + 16 * lane);
+        if (lane < 8 && 64 + lane < nunits) *(u32x4 *)(dst + 1024 + 16 * lane) = *(const u32x4 *)(stage + 1024 + 16 * lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
     };
 #define SWM_STEP(CUR, NXT2, jc)                                                                                              \
     {                                                                                                                        \
-        const int jn = (jc) + 2 * nwgx;                                                                                      \
-        swm_load<SRC>(NXT2, gu, ids, ld, F, SWM_T(jn), jn % nslab, lane, SWM_OK(jn));                                        \
-        if (SWM_OK(jc)) swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, SWM_T(jc), (jc) % nslab, lane, wave);              \
-        __syncthreads();                                                                                                     \
-        if ((jc) < lim && SWM_G(jc) < ngroups) flush(jc);                                                                    \
-        __syncthreads();                                                                                                     \
+        const unsigned jn = (jc) + 2 * stride;                                                                                  \
+        swm_load<SRC>(NXT2, gu, ids, ld, F, T, SWM_TG(jn), SWM_UNIT(jn), lane, jn < nitems);                                 \
+        if ((jc) < nitems) {                                                                                                 \
+            swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane);                            \
+            flush(jc);                                                                                                       \
+        }                                                                                                                    \
     }
-    for (; j < lim; j += 3 * nwgx) {
+    for (; j < nitems; j += 3 * stride) {
         SWM_STEP(A, C, j)
-        SWM_STEP(B, A, j + nwgx)
-        SWM_STEP(C, B, j + 2 * nwgx)
+        SWM_STEP(B, A, j + stride)
+        SWM_STEP(C, B, j + 2 * stride)
     }
 #undef SWM_STEP
-#undef SWM_G
-#undef SWM_T
-#undef SWM_OK
+#undef SWM_TG
+#undef SWM_UNIT
 }
 
 // the table is filled once per device, in stream order before its first reader
@@ -444,13 +441,13 @@ int camx_quantize_mmq_q8_1(const float * x, const int32_t * ids, void * vy, long
     (void)s02; (void)s03; (void)n_expert_used;
     if (!x || !vy || ne00 < 4 || ne00 % 4 || s01 < ne00 || s01 % 4 || ne0 % 512 || ne0 < ne00 || ne0 >= ne00 + 512 || ne1 < 0 || ne2 != 1 ||
         (layout != MMQ_D4 && layout != MMQ_DS4) || ((uintptr_t)x & 15) || ((uintptr_t)vy & 15)) return CAMX_EINVAL;
-    if (ne1 >= 256 && ne00 % 4 == 0) {       // enough columns to fill the chip: persistent workgroups, block rows stored as whole aligned runs
+    if (ne1 >= 256 && (long)((ne1 + SWM_TOK - 1) / SWM_TOK) * (ne0 / 128) < 0x7ff00000L) {       // enough columns to fill the chip: persistent workgroups, block rows stored as whole aligned runs
         int dev = 0, ncu = 256;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return CAMX_EINVAL;
-        const int ngroups = (ne1 + SWM_TOK - 1) / SWM_TOK, nslab = (int)((ne0 + SWM_SLAB - 1) / SWM_SLAB);
-        const dim3 grid((unsigned)((ncu + 7) / 8 * 8)), block(1024);
-        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, ne0, (uint8_t *)vy, nullptr, ne1, ngroups, nslab);
-        else swiglu_mmq_lut<MMQ_D4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, ne0, (uint8_t *)vy, nullptr, ne1, ngroups, nslab);
+        const long ncol = ne0 / 128, nitems = (long)((ne1 + SWM_TOK - 1) / SWM_TOK) * ncol;
+        const dim3 grid((unsigned)ncu), block(1024);
+        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, (uint8_t *)vy, nullptr, ne1, (unsigned)ncol, (unsigned)nitems);
+        else swiglu_mmq_lut<MMQ_D4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, (uint8_t *)vy, nullptr, ne1, (unsigned)ncol, (unsigned)nitems);
         CAMX_LAUNCH_RET();
     }
     MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s01, ne1, ne1, 0};
@@ -475,17 +472,18 @@ int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16
     if (!gu || !vy || F < 4 || F % 4 || ld < 2 * F || ld % 4 || T < 0 || (layout != MMQ_D4 && layout != MMQ_DS4) ||
         ((uintptr_t)gu & 7) || ((uintptr_t)vy & 15) || ((uintptr_t)act & 7)) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
-    if (F % 8 == 0 && ld % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)act & 15)) {
+    if (F % 8 == 0 && ld % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)act & 15) &&
+        (long)((T + SWM_TOK - 1) / SWM_TOK) * ((F + 511) / 512 * 4) < 0x7ff00000L) {
         const int rc = silu_lut_ready(st);
         if (rc) return rc;
         int dev = 0, ncu = 256;
         hipGetDevice(&dev);
         hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev);
         const long Kp = (F + 511) / 512 * 512;
-        const int ngroups = (T + SWM_TOK - 1) / SWM_TOK, nslab = (int)((Kp + SWM_SLAB - 1) / SWM_SLAB);
-        const dim3 grid((unsigned)((ncu + 7) / 8 * 8)), block(1024);
-        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
-        else swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, Kp, (uint8_t *)vy, act, T, ngroups, nslab);
+        const long ncol = Kp / 128, nitems = (long)((T + SWM_TOK - 1) / SWM_TOK) * ncol;
+        const dim3 grid((unsigned)ncu), block(1024);
+        if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol, (unsigned)nitems);
+        else swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol, (unsigned)nitems);
         CAMX_LAUNCH_RET();
     }
     MmqArgs a = {gu, nullptr, (uint8_t *)vy, act, F, (F + 511) / 512 * 512, ld, T, T, 0};
