@@ -5,6 +5,7 @@
 // Layout: 8 lanes x 4 consecutive floats = one 32-value quantization group; a wave covers 256 values per step with one
 // 128-bit load per lane and writes each group's 32 codes as 8 dwords.
 #include "common.cuh"
+#include <mutex>
 
 CAMX_DEV float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
@@ -344,23 +345,6 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
 #undef SWM_UNIT
 }
 
-// the table is filled once per device, in stream order before its first reader
-static int silu_lut_ready(hipStream_t st) {
-    static bool done[64] = {false};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
-    if (!done[dev]) {
-        silu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
-        const hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return (int)e;
-        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
-        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess) return CAMX_EINVAL;
-        if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
-        done[dev] = true;
-    }
-    return CAMX_OK;
-}
-
 // act = bf16(bf16(silu g) * u) of wide bf16 rows [g (H) | u (H)] with the same table: persistent workgroups, a lane takes 8
 // values at a time (16 bytes of g, of u, of act) and keeps the next unit's loads in flight across the current one's lookups.
 // The products are rounded by the packed hardware convert; a unit that holds a NaN is redone with the canonical NaN.
@@ -404,18 +388,37 @@ __global__ void __launch_bounds__(1024) silu_mul_lut(const uint16_t * __restrict
     }
 }
 
+// The table is filled once per device, in stream order before its first reader, and the kernels that hold it in LDS get their
+// dynamic LDS limit raised; callers on any host thread go through one lock. *ncu: the device's CU count.
+static std::mutex g_lut_mu;
+static struct { bool ready; int ncu; } g_lut_dev[64];
+static int silu_lut_ready(hipStream_t st, int * ncu) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
+    std::lock_guard<std::mutex> lock(g_lut_mu);
+    if (!g_lut_dev[dev].ready) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return CAMX_EINVAL;
+        silu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+        if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *)silu_mul_lut, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return CAMX_EINVAL;
+        if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
+        g_lut_dev[dev].ncu = n;
+        g_lut_dev[dev].ready = true;
+    }
+    *ncu = g_lut_dev[dev].ncu;
+    return CAMX_OK;
+}
+
 // the wide form of silu_mul_bf16 (rows of H = 8 k values, 16-byte aligned, at least 2^22 values); CAMX_EINVAL: not applicable
 __attribute__((visibility("hidden"))) int silu_mul_bf16_wide(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st) {
     if (H % 8 || n < (1L << 22) || n / 8 >= 0x7fffffffL || (((uintptr_t)gu | (uintptr_t)act) & 15)) return CAMX_EINVAL;
-    static bool attr[64] = {false};
-    int dev = 0, ncu = 256;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return CAMX_EINVAL;
-    const int e = silu_lut_ready(st);
+    int ncu = 0;
+    const int e = silu_lut_ready(st, &ncu);
     if (e) return e;
-    if (!attr[dev]) {
-        if (hipFuncSetAttribute((const void *)silu_mul_lut, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return CAMX_EINVAL;
-        attr[dev] = true;
-    }
     silu_mul_lut<<<dim3((unsigned)ncu), dim3(1024), 131072, st>>>(gu, act, (unsigned)(H / 8), (unsigned)(n / 8));
     return (int)hipGetLastError();
 }
@@ -474,11 +477,9 @@ int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16
     if (T == 0) return CAMX_OK;
     if (F % 8 == 0 && ld % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)act & 15) &&
         (long)((T + SWM_TOK - 1) / SWM_TOK) * ((F + 511) / 512 * 4) < 0x7ff00000L) {
-        const int rc = silu_lut_ready(st);
+        int ncu = 0;
+        const int rc = silu_lut_ready(st, &ncu);
         if (rc) return rc;
-        int dev = 0, ncu = 256;
-        hipGetDevice(&dev);
-        hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev);
         const long Kp = (F + 511) / 512 * 512;
         const long ncol = Kp / 128, nitems = (long)((T + SWM_TOK - 1) / SWM_TOK) * ncol;
         const dim3 grid((unsigned)ncu), block(1024);

@@ -72,6 +72,11 @@ def bf2f(h):
     return (_c(h, np.uint16).astype(np.uint32) << 16).view(np.float32)
 
 
+def set_threads(n):
+    """threads the row loops run on (timing only); returns the previous setting"""
+    return int(lib().orc_set_threads(C.c_int(n)))
+
+
 def row_ss(x):
     x = _c(x, np.float32); return np.float32(lib().orc_row_ss(_p(x), I(x.size)))
 

@@ -32,7 +32,23 @@
 #include <stdint.h>
 #include <string.h>
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 #define ORC_API __attribute__((visibility("default")))
+
+/* threads for the row loops (0: the runtime's default); returns the previous setting. Timing only: results do not depend on it */
+ORC_API int orc_set_threads(int n) {
+#ifdef _OPENMP
+    const int before = omp_get_max_threads();
+    omp_set_num_threads(n > 0 ? n : omp_get_num_procs());
+    return before;
+#else
+    (void)n;
+    return 1;
+#endif
+}
 
 /* ---- conversions (kernels/core.hip:14-21, kernels/prefill_glue.hip:77-80) ------------------------------------------ */
 static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
