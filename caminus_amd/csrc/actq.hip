@@ -19,12 +19,14 @@ struct PlainBF16 { static constexpr bool bf16_valued = true; const uint16_t * x;
 struct SiluMulSrc {
     static constexpr bool bf16_valued = true;      // the activation is rounded to bf16 as it is formed
     const uint16_t * gu; int ld, F;
+    const uint16_t * lut;                          // bf16(silu g) for every bf16 g (the table silu_mul_bf16 uses: the same activation bits)
     CAMX_DEV f32x4 operator()(int row, int k) const {
         const uint16_t * r = gu + (size_t)row * ld;
-        const f32x4 g = unpack_bf16x4(*(const u32x2 *)(r + k)), u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
+        const u32x2 gw = *(const u32x2 *)(r + k);
+        const f32x4 u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
         f32x4 a;
-        a.x = rbf(rbf(g.x / (1.0f + expf(-g.x))) * u.x); a.y = rbf(rbf(g.y / (1.0f + expf(-g.y))) * u.y);
-        a.z = rbf(rbf(g.z / (1.0f + expf(-g.z))) * u.z); a.w = rbf(rbf(g.w / (1.0f + expf(-g.w))) * u.w);
+        a.x = rbf(bf2f(lut[gw.x & 0xffffu]) * u.x); a.y = rbf(bf2f(lut[gw.x >> 16]) * u.y);
+        a.z = rbf(bf2f(lut[gw.y & 0xffffu]) * u.z); a.w = rbf(bf2f(lut[gw.y >> 16]) * u.w);
         return a;
     }
 };
@@ -154,13 +156,15 @@ struct SinkLds { float * buf; CAMX_DEV void operator()(int, int k, f32x4 v) cons
 // dact back through act = bf16(bf16(silu g) * u): each product rounded to bf16, then silu's derivative
 // ds * sig * fma(g, 1 - sig, 1), into dgu = [dg | du] rows of 2F
 struct SinkSiluMul {
-    const uint16_t * gu; int ld, F; uint16_t * dgu;
+    const uint16_t * gu; int ld, F; uint16_t * dgu; const uint16_t * lut;
     CAMX_DEV void operator()(int row, int k, f32x4 dact) const {
         const uint16_t * r = gu + (size_t)row * ld;
-        const f32x4 g = unpack_bf16x4(*(const u32x2 *)(r + k)), u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
+        const u32x2 gw = *(const u32x2 *)(r + k);
+        const f32x4 g = unpack_bf16x4(gw), u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
+        const f32x4 sl4 = {bf2f(lut[gw.x & 0xffffu]), bf2f(lut[gw.x >> 16]), bf2f(lut[gw.y & 0xffffu]), bf2f(lut[gw.y >> 16])};
         f32x4 dg, du;
-#define S_(e) { const float ex = expf(-g.e), sl = rbf(g.e / (1.0f + ex)), sig = 1.0f / (1.0f + ex), ds = rbf(dact.e * u.e); \
-                du.e = dact.e * sl; dg.e = ds * sig * __builtin_fmaf(g.e, 1.0f - sig, 1.0f); }
+#define S_(e) { const float ex = expf(-g.e), sig = 1.0f / (1.0f + ex), ds = rbf(dact.e * u.e); \
+                du.e = dact.e * sl4.e; dg.e = ds * sig * __builtin_fmaf(g.e, 1.0f - sig, 1.0f); }
         CAMX_EACH4(S_)
 #undef S_
         uint16_t * o = dgu + (size_t)row * (2 * F);
@@ -309,6 +313,8 @@ __global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const 
     }
 }
 
+__attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut);       // quant.hip
+
 static int actq_check(int K, int qmax, int M) { return (K < 128 || K % 128 || K > 8192 || qmax < 1 || M < 0) ? CAMX_EINVAL : CAMX_OK; }
 
 // one instance per number of rounds
@@ -334,7 +340,10 @@ int camx_actq_fwd(const void * x, int is_bf16, uint16_t * y, float * s, uint16_t
 int camx_silu_mul_actq_fwd(const uint16_t * gu, int ld, int F, uint16_t * y, float * s, uint16_t * codes, float clip, int qmax, int M, hipStream_t st) {
     if (!gu || (!y && !codes) || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    ACTQ_ROUNDS(F, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F}, y, s, codes, F, clip, qmax)))
+    const uint16_t * lut = nullptr;
+    const int rc = silu_lut_get(st, &lut);
+    if (rc) return rc;
+    ACTQ_ROUNDS(F, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut}, y, s, codes, F, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y, float * s, uint16_t * codes,
@@ -358,7 +367,10 @@ int camx_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, in
 int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, float clip, int qmax, int M, hipStream_t st) {
     if (!gu || !g || !dgu || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)g & 7) || ((uintptr_t)dgu & 7)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F}, g, SinkSiluMul{gu, ld, F, dgu}, F, clip, qmax)))
+    const uint16_t * lut = nullptr;
+    const int rc = silu_lut_get(st, &lut);
+    if (rc) return rc;
+    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut}, g, SinkSiluMul{gu, ld, F, dgu, lut}, F, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 // block_entry_bwd: dy bf16 [M][d], dab bf16 [M][nab] (needed when nab > 0), rstd [M] from the forward; dx fp32 [M][d]; d <= 1024

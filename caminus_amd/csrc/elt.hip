@@ -44,21 +44,25 @@ __global__ void __launch_bounds__(256) swiglu_f32(const float * __restrict__ g, 
 }
 
 // silu_mul_bf16: act[r][c] = bf16(bf16(silu(g)) * u), gu rows = [g (H) | u (H)]
-__global__ void __launch_bounds__(256) silu_mul_bf16_k(const uint16_t * __restrict__ gu, uint16_t * __restrict__ act, int H, long n, int vec) {
+// bf16(silu g) comes from the 65536-entry table in device memory (the one the wide form and the SwiGLU -> MMQ kernel hold in
+// LDS), so a row's result does not depend on which of them a batch size selects
+__global__ void __launch_bounds__(256) silu_mul_bf16_k(const uint16_t * __restrict__ gu, uint16_t * __restrict__ act, int H, long n, int vec,
+                                                       const uint16_t * __restrict__ lut) {
     const long stride = (long)gridDim.x * 256;
     for (long q = (long)blockIdx.x * 256 + threadIdx.x; q * 4 < n; q += stride) {
         const long i = q * 4;
         if (vec) {     // H % 4 == 0: the four elements share a row
             const long r = i / H, c = i - r * H;
-            const f32x4 g = unpack_bf16x4(*(const u32x2 *)(gu + r * 2 * H + c)), u = unpack_bf16x4(*(const u32x2 *)(gu + r * 2 * H + H + c));
+            const u32x2 gw = *(const u32x2 *)(gu + r * 2 * H + c);
+            const f32x4 u = unpack_bf16x4(*(const u32x2 *)(gu + r * 2 * H + H + c));
             f32x4 a;
-            a.x = rbf(silu_f(g.x)) * u.x; a.y = rbf(silu_f(g.y)) * u.y; a.z = rbf(silu_f(g.z)) * u.z; a.w = rbf(silu_f(g.w)) * u.w;
+            a.x = bf2f(lut[gw.x & 0xffffu]) * u.x; a.y = bf2f(lut[gw.x >> 16]) * u.y; a.z = bf2f(lut[gw.y & 0xffffu]) * u.z; a.w = bf2f(lut[gw.y >> 16]) * u.w;
             *(u32x2 *)(act + i) = pack_f2bf_x4(a);
         } else {
             for (int k = 0; k < 4 && i + k < n; k++) {
                 const long r = (i + k) / H, c = (i + k) - r * H;
-                const float g = bf2f(gu[r * 2 * H + c]), u = bf2f(gu[r * 2 * H + H + c]);
-                act[i + k] = f2bf(rbf(silu_f(g)) * u);
+                const float u = bf2f(gu[r * 2 * H + H + c]);
+                act[i + k] = f2bf(bf2f(lut[gu[r * 2 * H + c]]) * u);
             }
         }
     }
@@ -440,6 +444,7 @@ __global__ void __launch_bounds__(256) residual_slices_fwd_k(const float * __res
 }
 
 __attribute__((visibility("hidden"))) int silu_mul_bf16_wide(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st);   // quant.hip
+__attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut);                                        // quant.hip
 
 extern "C" {
 
@@ -460,10 +465,13 @@ int camx_gg_silu_mul(const float * g, const float * u, float * h, int n, hipStre
 int camx_silu_mul_bf16(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st) {
     if (!gu || !act || H < 1 || n < 0 || n % H) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
-    const int wide = silu_mul_bf16_wide(gu, act, H, n, st);      // large inputs: bf16(silu g) from a table in LDS
+    const uint16_t * lut = nullptr;
+    const int rc = silu_lut_get(st, &lut);                       // (a failure to set the table up is reported here, so CAMX_EINVAL below means "not applicable")
+    if (rc) return rc;
+    const int wide = silu_mul_bf16_wide(gu, act, H, n, st);      // large inputs: the table in LDS
     if (wide != CAMX_EINVAL) return wide;
     const int vec = H % 4 == 0 && !(((uintptr_t)gu | (uintptr_t)act) & 7);
-    silu_mul_bf16_k<<<GRID_1D((n + 3) / 4), dim3(256), 0, st>>>(gu, act, H, n, vec);
+    silu_mul_bf16_k<<<GRID_1D((n + 3) / 4), dim3(256), 0, st>>>(gu, act, H, n, vec, lut);
     CAMX_LAUNCH_RET();
 }
 // io: 0 fp32 -> fp32 (pf_gate_mul), 1 fp32 -> fp16 (q35p_gate_mul16), 2 bf16 -> bf16

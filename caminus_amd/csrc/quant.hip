@@ -100,13 +100,14 @@ struct MmqArgs {
     int ncols;               // destination columns
     int nsrc;                // source rows the grid walks (ncols, or ntok when scattering)
     int kexp;                // scatter: destination columns per source row (0: no scatter)
+    const uint16_t * lut;    // SRC_SWIGLU_BF16: the table of bf16(silu g) in device memory
 };
 
-CAMX_DEV f32x4 swiglu_bf16x4(u32x2 gw, u32x2 uw, u32x2 * packed) {
-    const f32x4 g = unpack_bf16x4(gw), u = unpack_bf16x4(uw);
+CAMX_DEV f32x4 swiglu_bf16x4(u32x2 gw, u32x2 uw, u32x2 * packed, const uint16_t * __restrict__ lut) {
+    const f32x4 u = unpack_bf16x4(uw);
     f32x4 a;
-    a.x = rbf(g.x / (1.0f + expf(-g.x))) * u.x; a.y = rbf(g.y / (1.0f + expf(-g.y))) * u.y;
-    a.z = rbf(g.z / (1.0f + expf(-g.z))) * u.z; a.w = rbf(g.w / (1.0f + expf(-g.w))) * u.w;
+    a.x = bf2f(lut[gw.x & 0xffffu]) * u.x; a.y = bf2f(lut[gw.x >> 16]) * u.y;
+    a.z = bf2f(lut[gw.y & 0xffffu]) * u.z; a.w = bf2f(lut[gw.y >> 16]) * u.w;
     const u32x2 p = pack_f2bf_x4(a);
     *packed = p;
     return unpack_bf16x4(p);
@@ -127,7 +128,7 @@ __global__ void __launch_bounds__(256) mmq_q8_1_rows(MmqArgs a) {
         else {
             const uint16_t * r = (const uint16_t *)a.x + srow * a.stride;
             u32x2 packed;
-            v = swiglu_bf16x4(*(const u32x2 *)(r + i0), *(const u32x2 *)(r + a.K + i0), &packed);
+            v = swiglu_bf16x4(*(const u32x2 *)(r + i0), *(const u32x2 *)(r + a.K + i0), &packed, a.lut);
             if (a.act) *(u32x2 *)(a.act + srow * a.K + i0) = packed;
         }
     }
@@ -391,8 +392,8 @@ __global__ void __launch_bounds__(1024) silu_mul_lut(const uint16_t * __restrict
 // The table is filled once per device, in stream order before its first reader, and the kernels that hold it in LDS get their
 // dynamic LDS limit raised; callers on any host thread go through one lock. *ncu: the device's CU count.
 static std::mutex g_lut_mu;
-static struct { bool ready; int ncu; } g_lut_dev[64];
-static int silu_lut_ready(hipStream_t st, int * ncu) {
+static struct { bool ready; int ncu; const uint16_t * lut; } g_lut_dev[64];
+static int silu_lut_ready(hipStream_t st, int * ncu, const uint16_t ** lut = nullptr) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
     std::lock_guard<std::mutex> lock(g_lut_mu);
@@ -405,12 +406,21 @@ static int silu_lut_ready(hipStream_t st, int * ncu) {
         if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void *)silu_mul_lut, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return CAMX_EINVAL;
+        void * sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_silu_lut)) != hipSuccess || !sym) return CAMX_EINVAL;
         if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
+        g_lut_dev[dev].lut = (const uint16_t *)sym;
         g_lut_dev[dev].ncu = n;
         g_lut_dev[dev].ready = true;
     }
     *ncu = g_lut_dev[dev].ncu;
+    if (lut) *lut = g_lut_dev[dev].lut;
     return CAMX_OK;
+}
+// the table's device address for kernels of other files (filled and synchronized on first use)
+__attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut) {
+    int ncu = 0;
+    return silu_lut_ready(st, &ncu, lut);
 }
 
 // the wide form of silu_mul_bf16 (rows of H = 8 k values, 16-byte aligned, at least 2^22 values); CAMX_EINVAL: not applicable
@@ -448,12 +458,13 @@ int camx_quantize_mmq_q8_1(const float * x, const int32_t * ids, void * vy, long
         int dev = 0, ncu = 256;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return CAMX_EINVAL;
         const long ncol = ne0 / 128, nitems = (long)((ne1 + SWM_TOK - 1) / SWM_TOK) * ncol;
-        const dim3 grid((unsigned)ncu), block(1024);
+        const long nwg = (nitems + 15) / 16;                                  // a small batch does not start workgroups that would only copy the table
+        const dim3 grid((unsigned)(nwg < ncu ? nwg : ncu)), block(1024);
         if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, (uint8_t *)vy, nullptr, ne1, (unsigned)ncol, (unsigned)nitems);
         else swiglu_mmq_lut<MMQ_D4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, (uint8_t *)vy, nullptr, ne1, (unsigned)ncol, (unsigned)nitems);
         CAMX_LAUNCH_RET();
     }
-    MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s01, ne1, ne1, 0};
+    MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s01, ne1, ne1, 0, nullptr};
     return launch_mmq<SRC_F32>(a, layout, st);
 }
 
@@ -465,7 +476,7 @@ int camx_quantize_mmq_q8_1_scatter(const float * x, const int32_t * ids, void * 
     if (!x || !vy || !ids || ne00 < 4 || ne00 % 4 || s02 < ne00 || s02 % 4 || ne0 % 512 || ne0 < ne00 || ne0 >= ne00 + 512 || ne2 != 1 ||
         n_expert_used < 1 || ntok < 0 || ne1 != ntok * n_expert_used || (layout != MMQ_D4 && layout != MMQ_DS4) ||
         ((uintptr_t)x & 15) || ((uintptr_t)vy & 15)) return CAMX_EINVAL;
-    MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s02, ne1, ntok, n_expert_used};
+    MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s02, ne1, ntok, n_expert_used, nullptr};
     return launch_mmq<SRC_F32>(a, layout, st);
 }
 
@@ -482,12 +493,16 @@ int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16
         if (rc) return rc;
         const long Kp = (F + 511) / 512 * 512;
         const long ncol = Kp / 128, nitems = (long)((T + SWM_TOK - 1) / SWM_TOK) * ncol;
-        const dim3 grid((unsigned)ncu), block(1024);
+        const long nwg = (nitems + 15) / 16;                                  // a small batch does not start workgroups that would only copy the table
+        const dim3 grid((unsigned)(nwg < ncu ? nwg : ncu)), block(1024);
         if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol, (unsigned)nitems);
         else swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol, (unsigned)nitems);
         CAMX_LAUNCH_RET();
     }
-    MmqArgs a = {gu, nullptr, (uint8_t *)vy, act, F, (F + 511) / 512 * 512, ld, T, T, 0};
+    const uint16_t * lut = nullptr;
+    const int rc = silu_lut_get(st, &lut);
+    if (rc) return rc;
+    MmqArgs a = {gu, nullptr, (uint8_t *)vy, act, F, (F + 511) / 512 * 512, ld, T, T, 0, lut};
     return launch_mmq<SRC_SWIGLU_BF16>(a, layout, st);
 }
 

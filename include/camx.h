@@ -5,8 +5,10 @@
  *   - Every entry point queues work on `stream` (a hipStream_t; NULL = the default stream) and returns at once:
  *     0, or a hipError_t value (1 = invalid value: a shape, alignment or pointer argument was refused and nothing was
  *     launched). camx_error_string() names the value.
- *   - The library allocates nothing per call and keeps no state between calls, except a 128 KiB lookup table that
- *     camx_swiglu_mmq_q8_1 fills once per device on its first call.
+ *   - The library allocates nothing per call and keeps no state between calls, except a 128 KiB lookup table of
+ *     bf16(silu(g)) for every bf16 g that camx_swiglu_mmq_q8_1, camx_silu_mul_bf16 and camx_silu_mul_actq_fwd / _bwd share and
+ *     the first of them to be called fills once per device (that call waits for its stream once: make it before any graph
+ *     capture). All four therefore produce the same activation bits for a row, whatever the batch size.
  *   - bf16 / fp16 values travel as uint16_t bit patterns. "rows" / "n" / "T" arguments that the reference kernels took
  *     from their launch grid are explicit trailing arguments here.
  *   - Device-side errors are sticky int32 words OR-ed by the kernels and never cleared by them; bit meanings are given at

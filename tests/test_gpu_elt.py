@@ -23,18 +23,15 @@ def test_swiglu(n):
 
 @pytest.mark.parametrize('R,H', [(4, 17408), (3, 7), (256, 17408), (1100, 4096)])
 def test_silu_mul_bf16(R, H):
-    """small inputs: the device's expf (one bf16 step); from 2^22 values on: the table of correctly rounded bf16(silu g), bit-equal
-    to the oracle wherever the host's expf is correctly rounded too, NaN and infinities included"""
+    """bf16(silu g) comes from the table of the correctly rounded value at every size (in device memory for small inputs, in LDS
+    from 2^22 values on): bit-equal to the oracle, NaN (canonical) and infinities included"""
     rng = np.random.default_rng(H)
     gu = O.f2bf(outliers(rng, (R, 2 * H)) * np.float32(2))
     gu[0, :6] = [0x7fc0, 0xffc1, 0x7f80, 0xff80, 0x0000, 0x8000]; gu[0, H:H + 6] = [0x3f80, 0x3f80, 0x0000, 0x3f80, 0x7f80, 0x7fa5]
     act = dev(np.zeros((R, H), np.uint16))
     call('camx_silu_mul_bf16', ptr(dev(gu)), ptr(act), I(H), L64(R * H))
     want = O.silu_mul_bf16(gu); got = host(act, np.uint16)
-    fin = np.isfinite(O.bf2f(want))
-    assert np.array_equal(got[~fin], want[~fin])                   # NaN (canonical) and infinities exactly
-    assert close_16(got[fin], want[fin], 'bf16')
-    if R * H >= 1 << 22: assert (got == want).mean() > 0.9999
+    assert np.array_equal(got, want)
 
 
 def test_gate_mul():
