@@ -3,6 +3,8 @@
 // actq_fwd_codes_{f32,bf16}, actq_bwd_{f32,bf16}, silu_mul_actq_{fwd,bwd} and block_entry_{fwd,bwd} (kernels/actq.hip:40-53,
 // 96-218, 247-333).
 //
+// Forward of plain fp32 / bf16 rows of at most 2048 values: one wave per row (actq_fwd_wave_k below, 30 vector instructions per
+// value against 44). Everything else:
 // One 256-thread workgroup per row. A half-wave (32 lanes) transforms one 128-chunk: lane l holds elements 4l .. 4l + 3,
 // butterfly stages 1-2 in registers, 4 .. 64 across lanes; half-wave h takes chunks h, h + 8, ... (the reference's wave h of
 // 32), NR = ceil(K / 1024) rounds of them stay in registers across the row-wide reductions. Kernels are instantiated per
@@ -14,8 +16,37 @@
 
 #define HSCALE 0.08837890625f      // bf16(1 / sqrt(128))
 
-struct PlainF32 { static constexpr bool bf16_valued = false; const float * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); } };
-struct PlainBF16 { static constexpr bool bf16_valued = true; const uint16_t * x; int K; CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); } };
+#define CAMX_EACH4(OP) OP(x) OP(y) OP(z) OP(w)
+
+// fp32 -> bf16 -> fp32. _any: a NaN stays a NaN but its sign and payload are the hardware's (for values that only feed further
+// arithmetic, where nothing but NaN-ness survives); _canon: a NaN becomes 0x7fc00000, as the stored bf16 tensors have it
+CAMX_DEV f32x4 rbf4_any(f32x4 v) {
+    const uint32_t a = hw_pk_bf16(v.x, v.y), b = hw_pk_bf16(v.z, v.w);
+    f32x4 r;
+    r.x = __builtin_bit_cast(float, a << 16); r.y = __builtin_bit_cast(float, a & 0xffff0000u);
+    r.z = __builtin_bit_cast(float, b << 16); r.w = __builtin_bit_cast(float, b & 0xffff0000u);
+    return r;
+}
+CAMX_DEV f32x4 rbf4_canon(f32x4 v) { return unpack_bf16x4(pack_f2bf_x4(v)); }
+CAMX_DEV f32x4 scaled4(f32x4 v) { v.x *= HSCALE; v.y *= HSCALE; v.z *= HSCALE; v.w *= HSCALE; return v; }
+
+// A source gives four values at element k of a row (operator()), or, for the wave-per-row kernel, eight: fetch() issues the
+// loads (NW 128-bit words), value8() turns them into floats later, so that the next row's loads fly during this row's arithmetic.
+CAMX_DEV void unpack_bf16x8(u32x4 w, f32x4 & a, f32x4 & b) { a = unpack_bf16x4((u32x2){w.x, w.y}); b = unpack_bf16x4((u32x2){w.z, w.w}); }
+struct PlainF32 {
+    static constexpr bool bf16_valued = false; static constexpr int NW = 2;
+    const float * x; int K;
+    CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); }
+    CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { const u32x4 * p = (const u32x4 *)(x + (size_t)row * K + k); w[0] = p[0]; w[1] = p[1]; }
+    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b) const { a = __builtin_bit_cast(f32x4, w[0]); b = __builtin_bit_cast(f32x4, w[1]); }
+};
+struct PlainBF16 {
+    static constexpr bool bf16_valued = true; static constexpr int NW = 1;
+    const uint16_t * x; int K;
+    CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); }
+    CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { w[0] = *(const u32x4 *)(x + (size_t)row * K + k); }
+    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b) const { unpack_bf16x8(w[0], a, b); }
+};
 struct SiluMulSrc {
     static constexpr bool bf16_valued = true;      // the activation is rounded to bf16 as it is formed
     const uint16_t * gu; int ld, F;
@@ -39,20 +70,6 @@ struct RmsSrc {
         return a;
     }
 };
-
-#define CAMX_EACH4(OP) OP(x) OP(y) OP(z) OP(w)
-
-// fp32 -> bf16 -> fp32. _any: a NaN stays a NaN but its sign and payload are the hardware's (for values that only feed further
-// arithmetic, where nothing but NaN-ness survives); _canon: a NaN becomes 0x7fc00000, as the stored bf16 tensors have it
-CAMX_DEV f32x4 rbf4_any(f32x4 v) {
-    const uint32_t a = hw_pk_bf16(v.x, v.y), b = hw_pk_bf16(v.z, v.w);
-    f32x4 r;
-    r.x = __builtin_bit_cast(float, a << 16); r.y = __builtin_bit_cast(float, a & 0xffff0000u);
-    r.z = __builtin_bit_cast(float, b << 16); r.w = __builtin_bit_cast(float, b & 0xffff0000u);
-    return r;
-}
-CAMX_DEV f32x4 rbf4_canon(f32x4 v) { return unpack_bf16x4(pack_f2bf_x4(v)); }
-CAMX_DEV f32x4 scaled4(f32x4 v) { v.x *= HSCALE; v.y *= HSCALE; v.z *= HSCALE; v.w *= HSCALE; return v; }
 
 // u = bf16(H128 . bf16(source)) for the NR rounds of this half-wave; returns the lane's max |u| over its active chunks
 template <int NR, typename Src>
@@ -131,6 +148,115 @@ template <int NR, typename Src>
 __global__ void __launch_bounds__(256) actq_fwd_k(Src src, uint16_t * y, float * s, uint16_t * codes, int K, float clip, int qmax) {
     __shared__ float lds[4];
     actq_fwd_row<NR>(src, blockIdx.x, y, s, K, clip, qmax, codes, lds);
+}
+
+// ---- rows of at most 2048 values: one wave per row, no LDS, no barrier ------------------------------------------------------
+// Lane (c = lane >> 2, q = lane & 3) holds 32 values of chunk c: element 32 j + 8 q + k of the chunk is u[j][k]. Butterfly
+// stages 1, 2, 4 pair registers k, stages 8 and 16 pair lanes q ^ 1 and q ^ 2, stages 32 and 64 pair registers j: the same
+// pairs in the same order as above, five of the seven stages without a lane exchange.
+CAMX_DEV void bfly(float & a, float & b) { const float s = a + b, d = a - b; a = s; b = d; }
+
+template <int CTRL>
+CAMX_DEV void lane_stage_w(float (&u)[4][8], uint32_t sign) {      // (own + partner) in the lower lane, (partner - own) in the upper one
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float own = u[j][k];
+            const float p = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, own), CTRL, 0xf, 0xf, true));
+            u[j][k] = p + __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, own) ^ sign);
+        }
+}
+CAMX_DEV void hadamard128_w32(float (&u)[4][8], int q) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int k = 0; k < 8; k += 2) bfly(u[j][k], u[j][k + 1]);
+#pragma unroll
+        for (int k = 0; k < 8; k += 4) { bfly(u[j][k], u[j][k + 2]); bfly(u[j][k + 1], u[j][k + 3]); }
+#pragma unroll
+        for (int k = 0; k < 4; k++) bfly(u[j][k], u[j][k + 4]);
+    }
+    lane_stage_w<0xB1>(u, (q & 1) ? 0x80000000u : 0u);
+    lane_stage_w<0x4E>(u, (q & 2) ? 0x80000000u : 0u);
+#pragma unroll
+    for (int k = 0; k < 8; k++) { bfly(u[0][k], u[1][k]); bfly(u[2][k], u[3][k]); }
+#pragma unroll
+    for (int k = 0; k < 8; k++) { bfly(u[0][k], u[2][k]); bfly(u[1][k], u[3][k]); }
+}
+CAMX_DEV float wave_max64(float v) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+// u = bf16(H128 . bf16(source)) of the lane's 32 values from the fetched words; returns the row's max |u|
+template <typename Src>
+CAMX_DEV float actq_rotate_w(const Src & src, const u32x4 (&raw)[4][Src::NW], int q, float (&u)[4][8]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        f32x4 a, b;
+        src.value8(raw[j], a, b);
+        if (!Src::bf16_valued) { a = rbf4_any(a); b = rbf4_any(b); }              // autocast's bf16 input
+        u[j][0] = a.x; u[j][1] = a.y; u[j][2] = a.z; u[j][3] = a.w; u[j][4] = b.x; u[j][5] = b.y; u[j][6] = b.z; u[j][7] = b.w;
+    }
+    hadamard128_w32(u, q);
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int k = 0; k < 8; k += 4) {
+            const f32x4 v = rbf4_any(scaled4((f32x4){u[j][k], u[j][k + 1], u[j][k + 2], u[j][k + 3]}));
+            u[j][k] = v.x; u[j][k + 1] = v.y; u[j][k + 2] = v.z; u[j][k + 3] = v.w;
+            amax = fmaxf(amax, absmax4(v));                                        // (an absent chunk holds zeros)
+        }
+    return wave_max64(amax);
+}
+template <typename Src>
+CAMX_DEV void fetch_row_w(const Src & src, int row, int c, int q, bool on, u32x4 (&raw)[4][Src::NW]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int w = 0; w < Src::NW; w++) raw[j][w] = (u32x4){0u, 0u, 0u, 0u};
+        if (on) src.fetch(row, c * 128 + 32 * j + 8 * q, raw[j]);
+    }
+}
+
+// One row per wave, four rows per workgroup: with many more workgroups than the chip holds at once, the loads of the workgroups
+// that start overlap the arithmetic of those that run (walking several rows per wave with the next row's loads in flight
+// measured 15 % slower).
+template <typename Src>
+__global__ void __launch_bounds__(256) actq_fwd_wave_k(Src src, uint16_t * __restrict__ y, float * __restrict__ s_out, uint16_t * __restrict__ codes,
+                                                       int K, float clip, int qmax, int M) {
+    const int lane = threadIdx.x & 63, nch = K / 128, c = lane >> 2, q = lane & 3;
+    const bool on = c < nch;
+    const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (row >= M) return;
+    const float lo = (float)(-qmax - 1), hi = (float)qmax;
+    u32x4 raw[4][Src::NW];
+    fetch_row_w(src, row, c, q, on, raw);
+    float u[4][8];
+    const float amax = actq_rotate_w(src, raw, q, u);
+    const float s = fmaxf(amax * clip / (float)qmax, 1e-8f), s_rcp = __builtin_amdgcn_rcpf(s);
+    if (lane == 0 && s_out) s_out[row] = s;
+    if (!on) return;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        f32x4 qa = rint_div4((f32x4){u[j][0], u[j][1], u[j][2], u[j][3]}, s, s_rcp), qb = rint_div4((f32x4){u[j][4], u[j][5], u[j][6], u[j][7]}, s, s_rcp);
+#define Q_(e) qa.e = fminf(fmaxf(qa.e, lo), hi); qb.e = fminf(fmaxf(qb.e, lo), hi);
+        CAMX_EACH4(Q_)
+#undef Q_
+        const size_t e0 = (size_t)row * K + c * 128 + 32 * j + 8 * q;
+        if (y) {
+            const u32x2 pa = pack_f2bf_x4((f32x4){qa.x * s, qa.y * s, qa.z * s, qa.w * s}), pb = pack_f2bf_x4((f32x4){qb.x * s, qb.y * s, qb.z * s, qb.w * s});
+            *(u32x4 *)(y + e0) = (u32x4){pa.x, pa.y, pb.x, pb.y};
+        }
+        if (codes) {
+#define N_(v, sh) (((uint32_t)(int)(v) & 0xfu) << (sh))
+            const uint32_t pk = N_(qa.x, 0) | N_(qa.y, 4) | N_(qa.z, 8) | N_(qa.w, 12) | N_(qb.x, 16) | N_(qb.y, 20) | N_(qb.z, 24) | N_(qb.w, 28);
+#undef N_
+            *(uint32_t *)(codes + (e0 >> 2)) = pk;
+        }
+    }
 }
 
 // ---- backward ----------------------------------------------------------------------------------------------------------------
@@ -315,6 +441,9 @@ __global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const 
 
 __attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut);       // quant.hip
 
+// the wave-per-row forward kernel: rows of at most 2048 values, operands aligned for its 16-byte loads and 16- / 4-byte stores
+static bool actq_wave_ok(int K, const void * x, const void * y, const void * codes) { return K <= 2048 && !((uintptr_t)x & 15) && !((uintptr_t)y & 15) && !((uintptr_t)codes & 3); }
+
 static int actq_check(int K, int qmax, int M) { return (K < 128 || K % 128 || K > 8192 || qmax < 1 || M < 0) ? CAMX_EINVAL : CAMX_OK; }
 
 // one instance per number of rounds
@@ -333,6 +462,11 @@ extern "C" {
 int camx_actq_fwd(const void * x, int is_bf16, uint16_t * y, float * s, uint16_t * codes, int K, float clip, int qmax, int M, hipStream_t st) {
     if (!x || (!y && !codes) || actq_check(K, qmax, M) || ((uintptr_t)x & (is_bf16 ? 7 : 15)) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
+    if (actq_wave_ok(K, x, y, codes)) {
+        if (is_bf16) actq_fwd_wave_k<<<dim3((M + 3) / 4), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, y, s, codes, K, clip, qmax, M);
+        else actq_fwd_wave_k<<<dim3((M + 3) / 4), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, y, s, codes, K, clip, qmax, M);
+        CAMX_LAUNCH_RET();
+    }
     if (is_bf16) { ACTQ_ROUNDS(K, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, y, s, codes, K, clip, qmax))) }
     else { ACTQ_ROUNDS(K, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, y, s, codes, K, clip, qmax))) }
     CAMX_LAUNCH_RET();

@@ -9,17 +9,24 @@ from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, dev, host, out
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize('M,K,qmax', [(5, 896, 7), (3, 2048, 7), (2, 8192, 7), (4, 128, 3), (3, 768, 127)])
+@pytest.mark.parametrize('M,K,qmax', [(5, 896, 7), (3, 2048, 7), (2, 8192, 7), (4, 128, 3), (3, 768, 127), (9, 1152, 7), (6, 1920, 7), (301, 1024, 7),
+                                      (5, 2176, 7)])
 def test_actq_fwd(M, K, qmax):
+    """rows of at most 2048 values take the wave-per-row kernel when the outputs are 16-byte (values) and 4-byte (codes) aligned,
+    the workgroup-per-row kernel otherwise: both against the oracle"""
+    import ctypes
     rng = np.random.default_rng(K + qmax)
     x = outliers(rng, (M, K)); x[0] = 0
     for bf in (False, True):
         src = O.f2bf(x) if bf else x
         ry, rs, rc = O.actq_fwd(src, clip=0.9, qmax=qmax, bf16=bf)
-        y = dev(np.zeros((M, K), np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros((M, K // 2), np.uint8))
-        call('camx_actq_fwd', ptr(dev(src)), I(int(bf)), ptr(y), ptr(s), ptr(c) if qmax <= 7 else NULL, I(K), F(0.9), I(qmax), I(M))
-        assert bits_equal(host(s), rs) and bits_equal(host(y, np.uint16), ry)
-        if qmax <= 7: assert bits_equal(host(c), rc)
+        srcd = dev(src)
+        for shift in (0, 1):                                            # shift: outputs moved off their 16- / 4-byte alignment
+            y = dev(np.zeros(M * K + 8, np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros(M * K // 2 + 8, np.uint8))
+            yp = ctypes.c_void_p(y.data_ptr() + 8 * shift); cp = ctypes.c_void_p(c.data_ptr() + 2 * shift)
+            call('camx_actq_fwd', ptr(srcd), I(int(bf)), yp, ptr(s), cp if qmax <= 7 else NULL, I(K), F(0.9), I(qmax), I(M))
+            assert bits_equal(host(s), rs) and bits_equal(host(y, np.uint16)[4 * shift:4 * shift + M * K].reshape(M, K), ry)
+            if qmax <= 7: assert bits_equal(host(c)[2 * shift:2 * shift + M * K // 2].reshape(M, K // 2), rc)
 
 
 def test_block_entry_fwd():
@@ -54,7 +61,8 @@ def test_silu_mul_actq_fwd():
 
 # ---- backward ----------------------------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize('M,K,qmax', [(5, 896, 7), (3, 2048, 7), (2, 8192, 7), (4, 128, 3), (3, 768, 127), (300, 1024, 7), (7, 5120, 7)])
+@pytest.mark.parametrize('M,K,qmax', [(5, 896, 7), (3, 2048, 7), (2, 8192, 7), (4, 128, 3), (3, 768, 127), (300, 1024, 7), (7, 5120, 7), (9, 1152, 7), (6, 1920, 7),
+                                      (5, 1536, 15)])
 def test_actq_bwd(M, K, qmax):
     rng = np.random.default_rng(100 + K + qmax)
     x = outliers(rng, (M, K)); x[0] = 0
