@@ -1,0 +1,80 @@
+"""Randomized shapes through the bodies of the GPU parity tests: every case is one of the parametrized tests of the other files
+called with drawn sizes (row counts around the kernels' dispatch thresholds, widths that end inside blocks and slabs, padded
+strides, every layout flag), against the oracle at the same bar as the fixed cases. The draws are seeded: the same cases every run."""
+import random
+
+import pytest
+
+import test_gpu_actq as A
+import test_gpu_elt as E
+import test_gpu_emb as M
+import test_gpu_kv as KV
+import test_gpu_norm as N
+import test_gpu_pfglue as P
+import test_gpu_quant as Q
+import test_gpu_rope as RP
+
+pytestmark = pytest.mark.gpu
+
+
+def _generators(r):
+    ri, ch = r.randint, r.choice
+
+    def rows():
+        return ch([1, 2, 3, 5, 8, 17, 64, 255, 256, 257, 300, 515, 1030])
+
+    def silu_actq():
+        m, f = ri(2, 40), 128 * ri(1, 24)
+        return m, f, 2 * f + 8 * ri(0, 4)
+
+    def rms_mul():
+        wr = ch([1, 1, 2, 4])
+        return wr * ri(1, 150), ch([100, 256, 896, 2048, 2560, 3072, 5120, 4 * ri(1, 2000)]), wr
+
+    def qk_nr():
+        d, t = ch([64, 96, 128, 256, 512]), ch([1, 3, 16, 400, 600])
+        return t, ri(1, 24), d, ch([x for x in (8, 16, 32, 64, 128, 256) if x <= d]), d + 4 * ri(0, 64), ch([1e4, 1e6, 1e7])
+
+    return [
+        (A.test_actq_fwd, lambda: (ri(1, 400), 128 * ri(1, 64), ch([1, 3, 7, 7, 7, 15, 127]))),
+        (A.test_actq_bwd, lambda: (ri(1, 300), 128 * ri(1, 64), ch([1, 3, 7, 7, 15, 127]))),
+        (A.test_block_entry_bwd, lambda: (ri(1, 200), 128 * ri(1, 8), 2 * ri(0, 8))),
+        (A.test_silu_mul_actq_bwd, silu_actq),
+        (E.test_swiglu, lambda: (ri(1, 70000),)),
+        (E.test_silu_mul_bf16, lambda: (ri(1, 300), ri(6, 3000))),
+        (E.test_gdn_conv, lambda: (ri(1, 600), ch([6, 64, 100, 256, 512, 1000, 4096, 8200, 10240]))),
+        (E.test_gdn_l2, lambda: (ri(1, 1100), ri(1, 48), ch([32, 64, 96, 128, 128, 256]))),
+        (M.test_gather_q4k_q80, lambda: (256 * ri(1, 32), ri(4, 2000), ri(3, 600))),
+        (M.test_gather_iq4xs_iq2s, lambda: (256 * ri(1, 32), ri(4, 300), ri(3, 300))),
+        (M.test_ple_rows_iq4nl, lambda: (ri(1, 100), ri(7, 5000), ri(1, 12))),
+        (KV.test_pf_kv_append, lambda: (32 * ri(1, 40), ri(1, 40))),
+        (KV.test_kv_q8_read_round_trip, lambda: (32 * ri(1, 40), ri(1, 400), ch([False, True]))),
+        (N.test_q3p_add_rms16, lambda: (rows(), 256 * ri(1, 8), ri(0, 8), ch([False, True]))),
+        (N.test_q35p_add_rms16, lambda: (rows(), 256 * ri(1, 40))),
+        (N.test_add_rms_q8_1, lambda: (rows(), 256 * ri(1, 32))),
+        (N.test_add_rms_bf16, lambda: (rows(), 256 * ri(1, 32))),
+        (N.test_rms_mul_and_rmsnorm, rms_mul),
+        (N.test_hc_glue, lambda: (ri(1, 300), ri(1, 4), ch([100, 256, 2048, 2560, 5120, 4 * ri(1, 1500)]))),
+        (P.test_gdn_norm, lambda: (ri(1, 5000), 4 * ri(1, 256))),
+        (P.test_ple_gate_conv_hist, lambda: (ri(2, 400), ri(1, 4), 32 * ri(1, 24), ri(1, 10))),
+        (Q.test_q8_1_plain, lambda: (ri(1, 600000),)),
+        (Q.test_mmq_quantize, lambda: (4 * ri(1, 2500), ri(1, 700), ri(0, 1))),
+        (Q.test_mmq_quantize_scatter, lambda: (4 * ri(1, 1000), ri(1, 40), ri(1, 8))),
+        (Q.test_swiglu_mmq, lambda: (ri(1, 400), ch([4, 8]) * ri(1, 600), 8 * ri(0, 3), ri(0, 1))),
+        (RP.test_qk_rope_f16_and_q8, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 5, 33, 2048, 2051]), ri(0, 120000), ch([False, True]))),
+        (RP.test_pf_qk_nr, qk_nr),
+        (RP.test_qk_rope_bf16, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 7, 2049]), ri(0, 120000), ch([False, True]), 8 * ri(0, 3))),
+    ]
+
+
+@pytest.mark.parametrize('seed', [20260, 20261])
+def test_random_shapes(seed):
+    r = random.Random(seed)
+    gens = _generators(r)
+    for _ in range(250):
+        fn, draw = r.choice(gens)
+        args = draw()
+        try:
+            fn(*args)
+        except Exception as e:
+            raise AssertionError(f'{fn.__module__}.{fn.__name__}{args}: {type(e).__name__}: {e}') from e
