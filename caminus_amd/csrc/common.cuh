@@ -58,7 +58,8 @@ CAMX_DEV float group8_sum(float a) {   // xor 4, 2, 1 butterfly over 8 lanes (th
     a += lane_xor4(a); a += lane_xor2(a); a += lane_xor1(a);
     return a;
 }
-CAMX_DEV float absmax4(f32x4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
+// max |v| as a chain of fmaxf that starts from 0: a NaN is skipped, and four NaNs give 0 (the reference's amax of a block of NaNs), not NaN
+CAMX_DEV float absmax4(f32x4 v) { return fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f); }
 
 // the 8 group sums of a wave added in order from 0.0f (0 + p0 is p0 for the non-negative sums used here)
 CAMX_DEV float wave_groups_in_order(float g) {

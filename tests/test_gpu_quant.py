@@ -111,3 +111,25 @@ def test_q8_1_quotients_next_to_rounding_boundaries():
     call('camx_gg_quantize_q8_1', ptr(dev(x)), ptr(y), L64(x.size), I(0), F(0), NULL)
     want = O.q8_1(x)
     assert bits_equal(host(y), want.reshape(-1))
+
+
+def test_q8_1_blocks_of_nan():
+    """a block that holds only NaN has amax 0 under the reference's fmaxf chain (a NaN is skipped): scale 0 and codes 0, in the flat
+    layout and as the copy of a normalized row; a NaN among numbers leaves the block's scale to the numbers. (The sum is NaN; its
+    sign is the adder's and is not compared.)"""
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal(32 * 40).astype(np.float32)
+    x[64:96] = np.nan; x[200] = np.nan; x[320:352] = -np.nan; x[352:356] = np.nan
+    y = dev(np.zeros(40 * 36, np.uint8))
+    call('camx_gg_quantize_q8_1', ptr(dev(x)), ptr(y), L64(x.size), I(0), F(0), NULL)
+    got, want = host(y).reshape(40, 36), O.q8_1(x).reshape(40, 36)
+    assert bits_equal(got[:, :2], want[:, :2]) and bits_equal(got[:, 4:], want[:, 4:])
+    assert (got[2, :2] == 0).all() and (got[10, :2] == 0).all() and (got[6, :2] != 0).any()
+    N = 2048
+    xr = np.full((3, N), np.nan, np.float32); xr[1] = rng.standard_normal(N)
+    nw = np.ones(N, np.float32)
+    ref = O.add_rms16(xr.copy(), nw, 1e-6, want_q8=True)
+    q8 = dev(np.zeros((3, N // 32, 36), np.uint8)); h = dev(np.zeros((3, N), np.float32))
+    call('camx_add_rms_q8_1', ptr(dev(xr.copy())), NULL, NULL, I(0), ptr(dev(nw)), F(1e-6), ptr(h), NULL, ptr(q8), I(N), I(3))
+    g = host(q8)
+    assert bits_equal(g[..., :2], ref['q8'][..., :2]) and bits_equal(g[..., 4:], ref['q8'][..., 4:]) and bits_equal(g[1], ref['q8'][1])
