@@ -132,7 +132,17 @@ static inline float rsqrt_c(float v) { return 1.0f / sqrtf(v); }
 
 /* ---- q8_1 (36-byte ggml block): kernels/k3_gguf_ops.h:146-162, kernels/k3_gguf.hip:29-36 ---------------------------- */
 static inline float silu_f(float x) { return x / (1.0f + expf(-x)); }                  /* k3_gguf_ops.h:53 */
-static inline int8_t roundf_i8(float v) { return (int8_t)roundf(v); }
+/* (int8_t)roundf(v). In range (|v| <= 127: every block whose scale is a normal number) this is the C conversion. Out of range the
+ * C conversion is undefined; the reference's kernels run it as the GPU's float -> int32 conversion, which saturates (NaN -> 0), and
+ * then keep the low byte. That is what is stated here, so that blocks whose scale underflows (amax below 127 * FLT_TRUE_MIN for
+ * q8_1, 127 / amax = inf for the MMQ layout) have defined bytes: +inf -> 0x7fffffff -> -1, -inf -> 0x80000000 -> 0. */
+static inline int8_t roundf_i8(float v) {
+    const float r = roundf(v);
+    if (r != r) return 0;
+    if (r >= 2147483648.0f) return (int8_t)0xff;
+    if (r <= -2147483648.0f) return 0;
+    return (int8_t)(uint8_t)((uint32_t)(int32_t)r & 0xffu);
+}
 
 static void q8_1_block(const float * xi, uint8_t * blk) {
     float amax = 0.0f;

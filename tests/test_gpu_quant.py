@@ -133,3 +133,32 @@ def test_q8_1_blocks_of_nan():
     call('camx_add_rms_q8_1', ptr(dev(xr.copy())), NULL, NULL, I(0), ptr(dev(nw)), F(1e-6), ptr(h), NULL, ptr(q8), I(N), I(3))
     g = host(q8)
     assert bits_equal(g[..., :2], ref['q8'][..., :2]) and bits_equal(g[..., 4:], ref['q8'][..., 4:]) and bits_equal(g[1], ref['q8'][1])
+
+
+def test_q8_blocks_whose_scale_underflows():
+    """blocks of subnormal-sized values: d = amax / 127 loses bits or becomes 0 (q8_1), 127 / amax becomes inf (MMQ layout), and the
+    quotients leave the int8 range; the codes are then the saturating float -> int32 conversion's low byte, as on the reference's GPU"""
+    rng = np.random.default_rng(4242)
+    nblk = 2048
+    e = rng.uniform(-149, -118, (nblk, 1)) + rng.uniform(-3, 0, (nblk, 32))
+    x = (np.exp2(e) * rng.choice([-1.0, 1.0], (nblk, 32))).astype(np.float32)
+    x[::7, 3] = 0.0
+    flat = x.reshape(-1)
+    y = dev(np.zeros(nblk * 36, np.uint8))
+    call('camx_gg_quantize_q8_1', ptr(dev(flat)), ptr(y), L64(flat.size), I(0), F(0), NULL)
+    assert bits_equal(host(y), O.q8_1(flat).reshape(-1))
+    for ncols, K in ((16, 4096), (512, 128)):                                # the row kernel and the persistent one
+        xm = flat.reshape(ncols, K)
+        for layout in (0, 1):
+            ym = dev(np.zeros((O.k_pad(K) // 128, ncols, 144), np.uint8))
+            call('camx_quantize_mmq_q8_1', ptr(dev(xm)), NULL, ptr(ym), L64(K), L64(K), L64(0), L64(0), L64(O.k_pad(K)), I(ncols), I(1), I(0), I(layout))
+            assert bits_equal(host(ym), O.mmq_q8_1(xm, K, ncols, layout))
+    # the fused form: bf16 gate / up values whose products are subnormal
+    T, Fh = 24, 1024
+    gu = O.f2bf((np.exp2(rng.uniform(-75, -55, (T, 2 * Fh))) * rng.choice([-1.0, 1.0], (T, 2 * Fh))).astype(np.float32))
+    want = O.silu_mul_bf16(gu)
+    for layout in (0, 1):
+        yf = dev(np.zeros((O.k_pad(Fh) // 128, T, 144), np.uint8)); act = dev(np.zeros((T, Fh), np.uint16))
+        call('camx_swiglu_mmq_q8_1', ptr(dev(gu)), L64(2 * Fh), L64(Fh), ptr(yf), ptr(act), I(T), I(layout))
+        assert bits_equal(host(act, np.uint16), want)
+        assert bits_equal(host(yf), O.mmq_q8_1(O.bf2f(want), Fh, T, layout))
