@@ -48,7 +48,7 @@ def _generators(r):
         (M.test_gather_iq4xs_iq2s, lambda: (256 * ri(1, 32), ri(4, 300), ri(3, 300))),
         (M.test_ple_rows_iq4nl, lambda: (ri(1, 100), ri(7, 5000), ri(1, 12))),
         (KV.test_pf_kv_append, lambda: (32 * ri(1, 40), ri(1, 40))),
-        (KV.test_kv_q8_read_round_trip, lambda: (32 * ri(1, 40), ri(1, 400), ch([False, True]))),
+        (KV.test_kv_q8_read_round_trip, lambda: (32 * ri(1, 40), ri(2, 400), ch([False, True]))),
         (N.test_q3p_add_rms16, lambda: (rows(), 256 * ri(1, 8), ri(0, 8), ch([False, True]))),
         (N.test_q35p_add_rms16, lambda: (rows(), 256 * ri(1, 40))),
         (N.test_add_rms_q8_1, lambda: (rows(), 256 * ri(1, 32))),
