@@ -137,7 +137,7 @@ __global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, c
     float sumf = 0.0f;
     sumf = __builtin_fmaf(in[0], w4.x, sumf); sumf = __builtin_fmaf(in[1], w4.y, sumf);
     sumf = __builtin_fmaf(in[2], w4.z, sumf); sumf = __builtin_fmaf(in[3], w4.w, sumf);
-    const float r = silu_f(sumf);
+    const float r = BF16 ? silu_fast(sumf) : silu_f(sumf);           // bf16 rows: the streaming kernel's form, so a token's bits do not depend on the chunk it came in
     if (BF16) ((uint16_t *)y)[(size_t)t * ldy + c] = to_bf16(r); else ((float *)y)[(size_t)t * ldy + c] = r;
 }
 // Prefill chunks: a lane owns VW consecutive channels and walks TR consecutive tokens, with the rows of the next eight tokens

@@ -12,6 +12,9 @@
 #define GRID_1D(n4) dim3((unsigned)((((n4) + 255) / 256) < 1048576 ? (((n4) + 255) / 256) : 1048576))
 
 // ---- gated RMSNorm of a GDN value head: y = ((o * rsqrt(mean(o^2) + eps)) * w) * (SILU ? silu(z) : sigmoid(z)) ------------
+// silu for fp16 outputs (both kernels below, so a row's bits do not depend on the batch it came in): v_exp / v_rcp, rounded to 16 bits at once
+CAMX_DEV float silu_fast16(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.442695041f)); }
+
 // one wave per (token, head) row of K values (K % 4 == 0, K <= 1024); lane p holds elements 256 j + 4 p + k
 template <bool SILU, bool F16OUT, int NI>
 __global__ void __launch_bounds__(256) gdn_norm_rows(const float * __restrict__ o, const float * __restrict__ w, const float * __restrict__ z,
@@ -42,7 +45,8 @@ __global__ void __launch_bounds__(256) gdn_norm_rows(const float * __restrict__ 
         const int i0 = 256 * j + 4 * lane;
         if (i0 < K) {
             f32x4 r;
-#define G_(e) { const float nrm = (scale * ov[j].e) * wv[j].e; r.e = SILU ? nrm * (zv[j].e / (1.0f + expf(-zv[j].e))) : nrm * (1.0f / (1.0f + expf(-zv[j].e))); }
+#define G_(e) { const float nrm = (scale * ov[j].e) * wv[j].e; \
+              r.e = F16OUT ? nrm * silu_fast16(zv[j].e) : (SILU ? nrm * (zv[j].e / (1.0f + expf(-zv[j].e))) : nrm * (1.0f / (1.0f + expf(-zv[j].e)))); }
             G_(x) G_(y) G_(z) G_(w)
 #undef G_
             if (F16OUT) *(u32x2 *)((uint16_t *)y + row * K + i0) = pack_f16x4(r); else *(f32x4 *)((float *)y + row * K + i0) = r;
@@ -53,7 +57,6 @@ __global__ void __launch_bounds__(256) gdn_norm_rows(const float * __restrict__ 
 // K = 128 (the GDN value heads) at prefill sizes: a half-wave per row, two rows per wave instruction, U rows per half-wave
 // with all their loads issued first. The logical threads past 128 hold zeros in the tree, so the four group sums of the row
 // added in order are the whole sum. FAST (fp16 output only): silu from v_exp / v_rcp, rounded to 16 bits at once.
-CAMX_DEV float silu_fast16(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.442695041f)); }
 template <bool SILU, bool F16OUT, int U>
 __global__ void __launch_bounds__(256) gdn_norm_128(const float * __restrict__ o, const float * __restrict__ w, const float * __restrict__ z,
                                                     void * __restrict__ y, float eps, long rows) {
