@@ -55,7 +55,7 @@ def test_gdn_norm_chunks():
         assert bits_equal(outs[0], outs[1]), name
 
 
-@pytest.mark.parametrize('io,D,n_rot', [(0, 256, 64), (1, 256, 64), (1, 128, 128), (0, 96, 32)])
+@pytest.mark.parametrize('io,D,n_rot', [(0, 256, 64), (1, 256, 64), (1, 128, 128), (0, 96, 32), (0, 512, 128), (1, 200, 48), (0, 256, 256)])
 def test_qk_nr_chunks(io, D, n_rot):
     """600 tokens x 8 heads at once (the per-token kernels) and in chunks of 100 (the per-head kernel)"""
     rng = np.random.default_rng(7 + D)
@@ -94,6 +94,12 @@ def test_qk_rope_bf16_chunks(yarn):
             call('camx_qk_rope_bf16', ptr(qd[t:]), I(ldq), I(nh), I(nkv), ptr(pd), I(pos0 + t), ptr(q16[t:]), ptr(c16), I(m), I(int(yarn)))
         outs.append((host(q16, np.uint16), host(c16, np.uint16)))
     assert bits_equal(outs[0][0], outs[1][0]) and bits_equal(outs[0][1], outs[1][1])
+    # the same rows at a stride that rules out 128-bit loads (the half-wave-per-head kernel)
+    ld2 = ldq + 4
+    wide = np.zeros((n, ld2), np.uint16); wide[:, :ldq] = qkv
+    q16 = dev(np.zeros((n, nh, 128), np.uint16)); c16 = dev(np.zeros((rows, 2 * M), np.uint16))
+    call('camx_qk_rope_bf16', ptr(dev(wide)), I(ld2), I(nh), I(nkv), ptr(pd), I(pos0), ptr(q16), ptr(c16), I(n), I(int(yarn)))
+    assert bits_equal(host(q16, np.uint16), outs[0][0]) and bits_equal(host(c16, np.uint16), outs[0][1])
 
 
 def test_elementwise_chunks():
