@@ -17,16 +17,11 @@ enum { ERR_PLE_INDEX = 1, ERR_TOKEN = 2 };
 CAMX_DEV f32x4 q4k_decode4(const uint8_t * blk, int lane) {
     const u32x4 hdr = *(const u32x4 *)blk;                       // d | dmin, then the 12 scale bytes
     const int sb = lane >> 3, is = sb >> 1, hi = sb & 1;
-    const uint64_t s03 = (uint64_t)hdr.y, s47 = (uint64_t)hdr.z, s8b = (uint64_t)hdr.w;
+    const uint32_t sh = 8 * (sb & 3);                                    // the sub-block's byte inside each scale word
+    const uint32_t b03 = (hdr.y >> sh) & 0xffu, b47 = (hdr.z >> sh) & 0xffu, b8b = (hdr.w >> sh) & 0xffu;
     uint32_t sc, m;
-    if (sb < 4) {
-        sc = (uint32_t)(s03 >> (8 * sb)) & 63u;
-        m = (uint32_t)(s47 >> (8 * sb)) & 63u;
-    } else {
-        const uint32_t hi8 = (uint32_t)(s8b >> (8 * (sb - 4))) & 0xffu;
-        sc = (hi8 & 0xfu) | ((((uint32_t)(s03 >> (8 * (sb - 4))) & 0xffu) >> 6) << 4);
-        m = (hi8 >> 4) | ((((uint32_t)(s47 >> (8 * (sb - 4))) & 0xffu) >> 6) << 4);
-    }
+    if (sb < 4) { sc = b03 & 63u; m = b47 & 63u; }
+    else { sc = (b8b & 0xfu) | ((b03 >> 6) << 4); m = (b8b >> 4) | ((b47 >> 6) << 4); }
     const float d = h2f_bits((uint16_t)(hdr.x & 0xffffu)), dm = h2f_bits((uint16_t)(hdr.x >> 16));
     const uint32_t qw = *(const uint32_t *)(blk + 16 + is * 32 + 4 * (lane & 7)) >> (4 * hi);
     const float dl = d * (float)sc, ml = dm * (float)m;
