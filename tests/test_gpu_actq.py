@@ -42,9 +42,9 @@ def test_block_entry_fwd():
     assert bits_equal(host(ab, np.uint16), rab)
 
 
-def test_silu_mul_actq_fwd():
-    rng = np.random.default_rng(12)
-    M, Fh = 5, 768
+@pytest.mark.parametrize('M,Fh', [(5, 768), (2100, 1024), (2050, 1920), (2049, 2176), (4099, 128)])
+def test_silu_mul_actq_fwd(M, Fh):
+    rng = np.random.default_rng(12 + M)
     gu = O.f2bf(outliers(rng, (M, 2 * Fh)))
     y = dev(np.zeros((M, Fh), np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros((M, Fh // 2), np.uint8))
     gud = dev(gu)
