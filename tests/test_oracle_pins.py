@@ -334,6 +334,27 @@ def test_q8_1_blocks():
     assert t.shape == (2, 36) and np.array_equal(t[0], y[0]) and not t[1, 4 + 8:].any()
 
 
+def test_q8_codes_when_the_scale_underflows_and_blocks_of_nan():
+    """known answers for the two statements that C leaves open: a quotient outside the int8 range takes the saturating
+    float -> int32 conversion's low byte (+inf -> 0x7fffffff -> -1, -inf -> 0x80000000 -> 0, NaN -> 0), and a block of NaNs has
+    amax 0 (fmaxf skips a NaN)"""
+    tiny = np.float32(1e-44)                                               # a subnormal: tiny / 127 rounds to 0, so x / d = +-inf
+    x = np.zeros(3 * 32, f32); x[0] = tiny; x[1] = -tiny; x[2] = tiny / 2
+    x[32:64] = np.nan
+    x[64] = np.nan; x[65] = 3.0; x[66] = -1.5
+    y = O.q8_1(x)
+    assert y[0, 0] == 0 and y[0, 1] == 0                                   # d = 0
+    assert y[0, 4:8].view(np.int8).tolist() == [-1, 0, -1, 0]              # +inf, -inf, +inf, 0 / 0 = NaN
+    assert not y[1, :2].any() and not y[1, 4:].any()                       # the block of NaNs: scale 0, codes 0
+    assert y[2, 0:2].copy().view(np.float16)[0] == np.float16(f32(3.0) / f32(127.0)) and y[2, 4:7].view(np.int8).tolist() == [0, 127, -64]
+    # MMQ layout: 127 / amax overflows for amax below 127 / FLT_MAX
+    K = 128
+    xm = np.zeros((1, K), f32); xm[0, 0] = f32(1e-38) / 64; xm[0, 1] = -xm[0, 0]
+    b = O.mmq_q8_1(xm, K, 1, 0)[0, 0]
+    assert b[:4].copy().view(f32)[0] == 0.0 and b[16:19].view(np.int8).tolist() == [-1, 0, 0]      # d = 1 / inf = 0; +inf, -inf, 0 * inf
+    assert O.set_threads(1) >= 1 and O.set_threads(0) == 1                 # (the thread control of the timing leg: previous setting returned)
+
+
 def test_mmq_q8_1_layout_and_invariants():
     rng = np.random.default_rng(4)
     K, ncols = 640, 5
