@@ -314,19 +314,23 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
     const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u), lds16);
     const float s_raw = amax * clip / (float)qmax, s = fmaxf(s_raw, 1e-8f);
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
-    // dL/ds = sum g (q - m t) and the number of max-|u| elements; m: the rounded value lies strictly inside (lo, hi)
-    float dlds = 0.0f, ties = 0.0f;
-    uint32_t inside = 0;
+    // dL/ds = sum g (q - m t) and the number of max-|u| elements; m: the rounded value lies strictly inside (lo, hi). The
+    // straight-through part g m is formed here (g is not needed afterwards); the ties are counted from the compares' lane masks
+    // on the scalar unit, one counter per half-wave (a count is exact in any order).
+    float dlds = 0.0f;
+    int ties_lo = 0, ties_hi = 0;
 #pragma unroll
     for (int c = 0; c < NR; c++) {
         if (hw + 8 * c < nch) {
-            int bit = 4 * c;
 #define D_(e) { const float t = u[c].e / s, r = rintf(t), q = fminf(fmaxf(r, lo), hi); const bool m = r > lo && r < hi; \
-                dlds = __builtin_fmaf(gv[c].e, m ? q - t : q, dlds); ties += fabsf(u[c].e) == amax ? 1.0f : 0.0f; inside |= (uint32_t)m << bit; bit++; }
+                dlds = __builtin_fmaf(gv[c].e, m ? q - t : q, dlds); gv[c].e = gv[c].e * (m ? 1.0f : 0.0f); \
+                const uint64_t tie = __builtin_amdgcn_ballot_w64(fabsf(u[c].e) == amax); \
+                ties_lo += __builtin_popcount((uint32_t)tie); ties_hi += __builtin_popcount((uint32_t)(tie >> 32)); }
             CAMX_EACH4(D_)
 #undef D_
         }
     }
+    float ties = (tid & 31) == 0 ? (float)((tid & 32) ? ties_hi : ties_lo) : 0.0f;
     block8_sum2(dlds, ties, lds16);
     const float coef = s_raw >= 1e-8f ? dlds * clip / (float)qmax / ties : 0.0f;
 #pragma unroll
@@ -334,8 +338,7 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
         const int ch = hw + 8 * c;
         if (ch < nch) {
             f32x4 d;
-            int bit = 4 * c;
-#define V_(e) { float v = gv[c].e * ((inside >> bit) & 1u ? 1.0f : 0.0f); bit++; \
+#define V_(e) { float v = gv[c].e; \
                 if (fabsf(u[c].e) == amax && u[c].e != 0.0f) v += u[c].e > 0.0f ? coef : -coef; d.e = v; }
             CAMX_EACH4(V_)
 #undef V_
