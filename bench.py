@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of each kernel of the step, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file
 # (KiB per dispatch, scaled by what the same counters read for the 256 MiB copy of --only copy_ref: FETCH_SIZE reads half
 # the bytes moved, WRITE_SIZE reads them all); the summaries are kept under profiles/
-HBM_TRAFFIC = {'add_rms_bf16': 252528878, 'qk_rope_bf16': 167960564, 'swiglu_mmq_q8_1': 366599510}
+HBM_TRAFFIC = {'add_rms_bf16': 252504188, 'qk_rope_bf16': 167965237, 'swiglu_mmq_q8_1': 366616250}
 I, F, L64 = C.c_int, C.c_float, C.c_int64
 NULL = C.c_void_p(None)
 
