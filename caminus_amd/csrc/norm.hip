@@ -42,9 +42,15 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
     float * xr = a.x + (size_t)row * N;
     f32x4 xv[NI_MAX];
+    if (a.stream) {        // a batch too large to be cache resident: its rows come from HBM once, past the caches
 #pragma unroll
-    for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) xv[j] = *(const f32x4 *)(xr + 256 * j + 4 * lane);
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) xv[j] = __builtin_nontemporal_load((const f32x4 *)(xr + 256 * j + 4 * lane));
+    } else {
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) xv[j] = *(const f32x4 *)(xr + 256 * j + 4 * lane);
+    }
     // Loads never sit behind a store they might alias: the compiler cannot prove that x, d, gamma and the outputs are
     // distinct, so a load written after a store waits for everything before it (one memory round trip per slab instead of
     // one per row). Hence: every addend load, then the x stores; gamma is requested before the reduction and arrives
@@ -116,8 +122,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
     if (ADD == ADD_HC || (ADD == ADD_F32_SLOTS && a.S > 0) || ((ADD == ADD_F32_DIRECT || ADD == ADD_BF16) && a.d)) {
-        // the updated residual goes back to the lines it was read from (plain loads above, nontemporal stores here: a
-        // nontemporal load followed by a store to the same line is slow on gfx950)
+        // the updated residual goes back to the lines it was read from
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
@@ -239,6 +244,82 @@ static int launch_norm(const NormArgs & a0, hipStream_t st) {
     CAMX_LAUNCH_RET();
 }
 
+// ---- the dense bf16 prefill form at chunk sizes: x += bf16 addend, RMSNorm, bf16 copy -------------------------------------------
+// One wave per row as above, written for this one job so that nothing stands between the loads: gamma goes straight to LDS
+// (one copy per workgroup, no registers, first in the queue), then every x and addend load of the row is issued, a short
+// pause apart, before the first dependent instruction; the residual goes back as soon as it is summed, and the bf16 rows are
+// packed by the hardware convert and stored without a branch in the loop (a row that produced a NaN is redone with the
+// reference's integer rounding, which has no NaN case). A wave's reads and writes are two separate bursts: HBM serves a read
+// burst and a write burst faster than an interleaved stream. rows % 4 == 0 (no partial workgroup).
+template <int NI>
+__global__ void __launch_bounds__(256) add_rms_bf16_chunk(float * __restrict__ x, const uint16_t * __restrict__ d, const float * __restrict__ nw, float eps,
+                                                          uint16_t * __restrict__ hbf) {
+    extern __shared__ __attribute__((aligned(16))) float gsh[];
+    constexpr int N = NI * 256;
+    const int lraw = threadIdx.x & 63, lane = slot_of(lraw), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t row = (size_t)blockIdx.x * 4 + wave;
+#pragma unroll
+    for (int j = wave; j < NI; j += 4)      // gamma piece j (1 KiB) -> LDS in lane order; read back in slot order below
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(nw + 256 * j + 4 * lraw), (__attribute__((address_space(3))) void *)(gsh + 256 * j), 16, 0, 0);
+    float * xr = x + row * N;
+    const uint16_t * dr = d + row * N;
+    f32x4 xv[NI]; u32x2 dv[NI];
+    // (the pause between requests: 4096 waves that each fire 40 requests at once measured 2 % slower than the same requests a few dozen cycles apart)
+#define CAMX_ISSUE_GAP() do { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_sleep(1); __builtin_amdgcn_sched_barrier(0); } while (0)
+#pragma unroll
+    for (int j = 0; j < NI; j++) { xv[j] = __builtin_nontemporal_load((const f32x4 *)(xr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
+#pragma unroll
+    for (int j = 0; j < NI; j++) { dv[j] = __builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
+#undef CAMX_ISSUE_GAP
+#pragma unroll
+    for (int j = 0; j < NI; j++) xv[j] = xv[j] + unpack_bf16x4(dv[j]);
+#pragma unroll
+    for (int j = 0; j < NI; j++) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
+    f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        ss.x = __builtin_fmaf(xv[j].x, xv[j].x, ss.x); ss.y = __builtin_fmaf(xv[j].y, xv[j].y, ss.y);
+        ss.z = __builtin_fmaf(xv[j].z, xv[j].z, ss.z); ss.w = __builtin_fmaf(xv[j].w, xv[j].w, ss.w);
+    }
+    const float tot = wave_groups_in_order(group32_sum(ss));
+    const float scale = rsqrt_exact(tot / (float)N + eps);
+    __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0): this wave's gamma pieces have landed in LDS (they were first in the queue)
+    __syncthreads();
+    uint16_t * hr = hbf + row * N;
+    bool nan = false;
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const f32x4 g = *(const f32x4 *)(gsh + 256 * j + 4 * lane);
+        f32x4 v;
+        v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
+        nan |= any_nan4(v);
+        const u32x2 pk = {hw_pk_bf16(v.x, v.y), hw_pk_bf16(v.z, v.w)};
+        __builtin_nontemporal_store(pk, (u32x2 *)(hr + 256 * j + 4 * lane));
+    }
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(nan) != 0, 0)) {
+#pragma unroll
+        for (int j = 0; j < NI; j++) {          // (unrolled: a register array cannot be indexed by a loop counter)
+            const f32x4 g = *(const f32x4 *)(gsh + 256 * j + 4 * lane);
+            f32x4 v;
+            v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
+            *(u32x2 *)(hr + 256 * j + 4 * lane) = pack_bf16x4_rne(v);
+        }
+    }
+}
+// Takes the first n - n % 4 rows when the chunk form applies (an addend, a bf16 copy and no fp32 copy, a chunk of at least 1024
+// rows of 256 NI values for the NI below, 16-byte aligned) and returns how many rows it took.
+static int launch_add_rms_bf16_chunk(float * x, const uint16_t * d, const float * nw, float eps, uint16_t * hbf, int N, int n, hipStream_t st) {
+    if (!d || !hbf || n < 1024 || (N & 255) || (((uintptr_t)x | (uintptr_t)d | (uintptr_t)nw | (uintptr_t)hbf) & 15)) return 0;
+    const int rows = n & ~3;
+    const dim3 grid(rows / 4), block(256);
+    switch (N >> 8) {
+#define CAMX_CHUNK(NI) case NI: add_rms_bf16_chunk<NI><<<grid, block, NI * 1024, st>>>(x, d, nw, eps, hbf); return rows;
+        CAMX_CHUNK(4) CAMX_CHUNK(6) CAMX_CHUNK(8) CAMX_CHUNK(10) CAMX_CHUNK(12) CAMX_CHUNK(14) CAMX_CHUNK(16) CAMX_CHUNK(20) CAMX_CHUNK(24) CAMX_CHUNK(28) CAMX_CHUNK(32)
+#undef CAMX_CHUNK
+    }
+    return 0;
+}
+
 extern "C" {
 
 int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
@@ -263,6 +344,14 @@ int camx_add_rms_q8_1(float * x, const float * d, const float * w, int S, const 
 
 int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps, float * h, uint16_t * hbf, int N, int n, hipStream_t st) {
     if (N < 1 || n < 0 || !x || !nw) return CAMX_EINVAL;
+    if (!h) {
+        const int done = launch_add_rms_bf16_chunk(x, d, nw, eps, hbf, N, n, st);
+        if (done) {
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess || done == n) return (int)e;
+            x += (size_t)done * N; d += (size_t)done * N; hbf += (size_t)done * N; n -= done;     // the last n % 4 rows
+        }
+    }
     NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, nullptr, N, hbf, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
     return launch_norm<ADD_BF16>(a, st);
 }

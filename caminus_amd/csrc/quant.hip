@@ -305,11 +305,13 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 131072 : 0) + wave * (SWM_TOK * 144);
-    // item id -> token group id / ncol, block column id % ncol: the waves of a workgroup sit on neighbouring columns
     const unsigned stride = gridDim.x * 16;                                   // (ids stay below 2^31: checked by the launcher)
     unsigned j = blockIdx.x * 16 + wave;
-#define SWM_TG(id) ((long)((id) / ncol) * SWM_TOK)
-#define SWM_UNIT(id) ((long)((id) % ncol))
+    // item id -> 4 neighbouring block columns x token groups, token groups fastest: the four waves of a SIMD row read 1 KiB of each token row
+    // and the workgroups that run side by side write neighbouring runs of the same block rows (ncol is a multiple of 4: K is padded to 512)
+    const unsigned ntg = (unsigned)((T + SWM_TOK - 1) / SWM_TOK);
+#define SWM_TG(id) ((long)((((id) >> 2) % ntg)) * SWM_TOK)
+#define SWM_UNIT(id) ((long)(((((id) >> 2) / ntg) << 2) + ((id) & 3)))
     SwmItem A, B, C;                                                          // three items in rotation: two steps of loads in flight
     swm_load<SRC>(A, gu, ids, ld, F, T, SWM_TG(j), SWM_UNIT(j), lane, j < nitems);                  // in flight while the table is copied
     swm_load<SRC>(B, gu, ids, ld, F, T, SWM_TG(j + stride), SWM_UNIT(j + stride), lane, j + stride < nitems);
@@ -323,8 +325,8 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
         const int nunits = (int)min((long)SWM_TOK, T - tg) * 9;               // tokens of the group that exist
         uint8_t * dst = y + ((size_t)unit * T + (size_t)tg) * 144;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // the wave's own LDS writes, in order
-        if (lane < nunits) *(u32x4 *)(dst + 16 * lane) = *(const u32x4 *)(stage + 16 * lane);
-        if (lane < 8 && 64 + lane < nunits) *(u32x4 *)(dst + 1024 + 16 * lane) = *(const u32x4 *)(stage + 1024 + 16 * lane);
+        if (lane < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 16 * lane), (u32x4 *)(dst + 16 * lane));
+        if (lane < 8 && 64 + lane < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 1024 + 16 * lane), (u32x4 *)(dst + 1024 + 16 * lane));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
     };
 #define SWM_STEP(CUR, NXT2, jc)                                                                                              \
