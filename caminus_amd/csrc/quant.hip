@@ -238,8 +238,11 @@ CAMX_DEV void swm_load(SwmItem & it, const void * __restrict__ src, const int32_
 }
 
 // the item's arithmetic; the wave's 8 blocks go to stage[token slot][144] (the wave's own 1152 bytes)
-template <int LAYOUT, int SRC>
-CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int T, long tg, long unit,
+// CANON: the activation is packed with f2bf (a NaN becomes 0x7fc0, as silu_mul_bf16 stores it) instead of the hardware convert, which
+// keeps a NaN's sign and payload. Returns whether a group sum of this lane's quad is a NaN: the callers run the item with the hardware
+// convert first and, in the rare wave that reports one (a NaN or infinite input), once more with CANON, which rewrites the same bytes.
+template <int LAYOUT, int SRC, bool CANON = false>
+CAMX_DEV bool swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int T, long tg, long unit,
                           int lane) {
     const int lq = lane & 3;
     const long e0 = unit * 128 + 8 * (lane & 15);
@@ -256,7 +259,7 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
                 const uint32_t sl = lut[it.gw[i][p] & 0xffffu], sh = lut[it.gw[i][p] >> 16];
                 const float u0 = __builtin_bit_cast(float, it.uw[i][p] << 16), u1 = __builtin_bit_cast(float, it.uw[i][p] & 0xffff0000u);
                 const float a0 = __builtin_bit_cast(float, sl << 16) * u0, a1 = __builtin_bit_cast(float, sh << 16) * u1;
-                pk[p] = cvt_pk_bf16(a0, a1);
+                pk[p] = CANON ? ((uint32_t)f2bf(a0) | ((uint32_t)f2bf(a1) << 16)) : cvt_pk_bf16(a0, a1);
                 v0 = __builtin_bit_cast(float, pk[p] << 16); v1 = __builtin_bit_cast(float, pk[p] & 0xffff0000u);
             } else {
                 const u32x4 w = p < 2 ? it.gw[i] : it.uw[i];
@@ -265,7 +268,7 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
             }
             val[i][2 * p] = v0; val[i][2 * p + 1] = v1;
             m = max3_abs(v0, v1, m);
-            if (LAYOUT == MMQ_DS4) {      // per thread ((x0 + x1) + x2) + x3: pairs p = 0, 1 are thread h = 0, pairs 2, 3 thread h = 1
+            if (LAYOUT == MMQ_DS4 || SRC == SRC_SWIGLU_BF16) {      // per thread ((x0 + x1) + x2) + x3: pairs p = 0, 1 are thread h = 0, pairs 2, 3 thread h = 1 (the bf16 source keeps the sums in the D4 layout too: a NaN shows in them)
                 if (p == 0) s0 = v0 + v1; else if (p == 1) s0 = (s0 + v0) + v1; else if (p == 2) s1 = v0 + v1; else s1 = (s1 + v0) + v1;
             }
         }
@@ -273,7 +276,7 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
         if (SRC == SRC_SWIGLU_BF16 && act && t < T && e0 < F) *(u32x4 *)(act + (size_t)t * F + e0) = (u32x4){pk[0], pk[1], pk[2], pk[3]};
         m = fmaxf(m, lane_xor2(m)); amax[i] = fmaxf(m, lane_xor1(m));
         sum[i] = 0.0f;
-        if (LAYOUT == MMQ_DS4) {
+        if (LAYOUT == MMQ_DS4 || SRC == SRC_SWIGLU_BF16) {
             s0 += lane_xor2(s0); s1 += lane_xor2(s1);          // thread ^ 4
             s0 += lane_xor1(s0); s1 += lane_xor1(s1);          // thread ^ 2
             sum[i] = s0 + s1;                                   // thread ^ 1
@@ -296,6 +299,7 @@ CAMX_DEV void swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
     if (lq < 2)
         *(uint32_t *)(blk0 + lq * (4 * 144) + 4 * ((lane & 15) >> 2)) =
             LAYOUT == MMQ_DS4 ? ((uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sm) << 16)) : __builtin_bit_cast(uint32_t, d);
+    return SRC == SRC_SWIGLU_BF16 && !CANON && ((sum[0] != sum[0]) | (sum[1] != sum[1]));
 }
 
 // SRC_F32 (quantize_mmq_q8_1 without scatter): the same work split and copy-out on fp32 rows (column c = row ids[c] or c), no table
@@ -334,7 +338,8 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
         const unsigned jn = (jc) + 2 * stride;                                                                                  \
         swm_load<SRC>(NXT2, gu, ids, ld, F, T, SWM_TG(jn), SWM_UNIT(jn), lane, jn < nitems);                                 \
         if ((jc) < nitems) {                                                                                                 \
-            swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane);                            \
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane)) != 0, 0))  \
+                swm_compute<LAYOUT, SRC, true>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane);                  \
             flush(jc);                                                                                                       \
         }                                                                                                                    \
     }

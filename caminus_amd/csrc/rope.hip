@@ -44,6 +44,7 @@ struct RopeArgs {
     int * err;
     const int32_t * page_table; int pt_stride, page, n_pages;   // paged addressing (null: row = position)
     int n;
+    int rows;                        // unpaged: rows of the cache when positions come from the caller's array (0: not checked here)
 };
 
 // TPW tokens per workgroup: 1 for decode-sized batches (wave 0 computes the token's cos / sin row); 4 for prefill chunks, where
@@ -99,7 +100,10 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         if (it_tp + 1 < TPW * npass) { const int tn = (it_tp + 1) / npass; load(xnext, t0 + tn, ((it_tp + 1) - tn * npass) * 8 * QR_STEPS); }
         const int pos = a.pos ? a.pos[t] : a.pos0 + t;
         uint8_t * cw = nullptr;
-        if (a.page_table) {
+        // a position outside the sequence's table row (paged) or outside the cache (unpaged): bit 1, that sequence's row is not written
+        const bool span = pos >= 0 && (a.page_table ? pos / a.page < a.pt_stride : (a.rows == 0 || pos < a.rows));
+        if (!span) { if (a.err && tid == 0 && base == 0) atomicOr(a.err, 1); }
+        else if (a.page_table) {
             const int pg = a.page_table[(size_t)t * a.pt_stride + pos / a.page];
             if (pg < 0 || pg >= a.n_pages) { if (tid == 0 && base == 0) atomicOr(a.err, 8); }
             else cw = (uint8_t *)a.cache + ((size_t)pg * a.page + (size_t)(pos % a.page)) * rb;
@@ -298,7 +302,9 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
         if (t >= a.n) break;
         if (it + 1 < TPW * nchunk) { const int tn = (it + 1) / nchunk; load(xnext, t0 + tn, ((it + 1) - tn * nchunk) * 16 * STEPS); }
         const int pos = a.pos ? a.pos[t] : a.pos0 + t;
-        uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
+        const bool span = pos >= 0 && (a.rows == 0 || pos < a.rows);          // (wave-uniform) outside the cache: bit 1, no row written
+        if (!span && a.err && tid == 0 && base == 0) atomicOr(a.err, 1);
+        uint16_t * cw = (uint16_t *)a.cache + (size_t)(span ? pos : 0) * 2 * M;
         uint16_t * qw = a.q16 + (size_t)t * a.nh * 128;
         const int j0 = 8 * (l16 & 7);
         f32x4 c4[2], s4[2];
@@ -349,7 +355,7 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
             if constexpr (Q8) {
                 const int h = h0 + hq;                                      // this row of 16 lanes: one head
                 const bool isq = h < a.nh, isv = h >= nqk, active = h < items;
-                uint8_t * cwb = (uint8_t *)a.cache + (size_t)pos * (2 * (M / 32) * 34);
+                uint8_t * cwb = (uint8_t *)a.cache + (size_t)(span ? pos : 0) * (2 * (M / 32) * 34);
                 float v8[8];
                 if (isv) {
 #pragma unroll
@@ -370,14 +376,14 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
                     if (active) *(u32x4 *)(qw + (size_t)h * 128 + 8 * l16) = out;
                 } else {
                     const size_t b = isv ? M / 32 + (size_t)(h - nqk) * 4 + (l16 >> 2) : (size_t)(h - a.nh) * 4 + (l16 >> 2);
-                    kv_q8_emit_w8(v8, cwb + b * 34, l16 & 3, a.err, active);
+                    kv_q8_emit_w8(v8, cwb + b * 34, l16 & 3, a.err, active && span);
                 }
                 continue;
             }
             if (h0 >= nqk) {                                                // V heads only: fp16 copy
 #pragma unroll
                 for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[s][2 * p], x[s][2 * p + 1]);
-                if (h0 + hq < items) RSTORE((u32x4 *)(cw + M + (size_t)(h0 - nqk) * 128 + lo), out);
+                if (h0 + hq < items && span) RSTORE((u32x4 *)(cw + M + (size_t)(h0 - nqk) * 128 + lo), out);
                 continue;
             }
             const bool allq = h0 + 3 < a.nh, allk = h0 >= a.nh && h0 + 3 < nqk;
@@ -398,13 +404,13 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
             } else if (allk) {
 #pragma unroll
                 for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
-                RSTORE((u32x4 *)(cw + (size_t)(h0 - a.nh) * 128 + lo), out);
+                if (span) RSTORE((u32x4 *)(cw + (size_t)(h0 - a.nh) * 128 + lo), out);
             } else {                                                        // a step that straddles q | k | v or the end of the row
 #pragma unroll
                 for (int k = 0; k < 8; k++) if (isv) y[k] = x[s][k];
 #pragma unroll
                 for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
-                if (h < items) {
+                if (h < items && (isq || span)) {
                     uint16_t * dst = isq ? qw + (size_t)h * 128 : (isv ? cw + M + (size_t)(h - nqk) * 128 : cw + (size_t)(h - a.nh) * 128);
                     RSTORE((u32x4 *)(dst + 8 * l16), out);
                 }
@@ -841,29 +847,30 @@ extern "C" {
 // q3p_qk_rope: n tokens at positions pos0 .. pos0 + n - 1; cache = fp16 rows [K | V] indexed by position
 int camx_q3p_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
                      int n, int yarn, hipStream_t st) {
-    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, nullptr, nullptr, 0, 0, 0, n};
+    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, nullptr, nullptr, 0, 0, 0, n, 0};
     return rope_launch(a, yarn, false, st);
 }
 // q3p_qk_rope_q8: the Q8 cache rows (K rotated by the 128-point Hadamard transform, V unrotated); err bit 2 on a refused block
 int camx_q3p_qk_rope_q8(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint8_t * cache,
                         int * err, int n, int yarn, hipStream_t st) {
-    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, err, nullptr, 0, 0, 0, n};
+    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, err, nullptr, 0, 0, 0, n, 0};
     return rope_launch(a, yarn, true, st);
 }
 // batched decode form: sequence t at its own position pos[t]; row address through a page table
-// (page_table[t * pt_stride + pos / page] * page + pos % page) when page_table is given, else row = pos[t].
-// err bit 8: a page id outside [0, n_pages) (that row is not written). q8 = 0 writes fp16 rows.
+// (page_table[t * pt_stride + pos / page] * page + pos % page) when page_table is given, else row = pos[t] of a cache of n_pages rows.
+// err bit 1: a position outside the sequence's table row (pos < 0 or pos / page >= pt_stride) or outside the unpaged cache;
+// err bit 8: a page id outside [0, n_pages). Either way that sequence's row is not written. q8 = 0 writes fp16 rows.
 int camx_qk_rope_paged(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16, void * cache,
                        int * err, const int32_t * page_table, int pt_stride, int page, int n_pages, int n, int yarn, int q8, hipStream_t st) {
-    if (!pos) return CAMX_EINVAL;
-    RopeArgs a = {qkv, ldq, nh, nkv, par, 0, pos, q16, cache, err, page_table, pt_stride, page, n_pages, n};
+    if (!pos || !err || (!page_table && n_pages < 1)) return CAMX_EINVAL;
+    RopeArgs a = {qkv, ldq, nh, nkv, par, 0, pos, q16, cache, err, page_table, pt_stride, page, n_pages, n, page_table ? 0 : n_pages};
     return rope_launch(a, yarn, q8 != 0, st);
 }
 
 // q3p_qk_rope on bf16 activations: qkv bf16 [n][ldq] widened exactly, then the same statements (a dense bf16 prefill chunk)
 int camx_qk_rope_bf16(const uint16_t * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
                       int n, int yarn, hipStream_t st) {
-    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, nullptr, nullptr, 0, 0, 0, n};
+    RopeArgs a = {qkv, ldq, nh, nkv, par, pos0, nullptr, q16, cache, nullptr, nullptr, 0, 0, 0, n, 0};
     return rope_launch(a, yarn, false, st, true);
 }
 

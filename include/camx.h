@@ -125,8 +125,9 @@ int camx_qk_rope_bf16(const uint16_t * qkv, int ldq, int nh, int nkv, const floa
                       int n, int yarn, camx_stream_t stream);
 /* Batched decode form of the two kernels above: sequence t at its own position pos[t]; with page_table the row address is
  * (page_table[t * pt_stride + pos / page] * page + pos % page) * row_bytes, else pos * row_bytes. q8 selects the row format.
- * err bit 8: a page id outside [0, n_pages) (that sequence's row is not written). Paging has no reference counterpart:
- * each row's bytes equal the unpaged kernel's. */
+ * With page_table NULL, n_pages is the number of rows of the cache. err (required) bit 1: a position outside the sequence's
+ * table row (pos < 0 or pos / page >= pt_stride) or outside the unpaged cache; bit 8: a page id outside [0, n_pages). Either way
+ * that sequence's row is not written (q16 is). Paging has no reference counterpart: each row's bytes equal the unpaged kernel's. */
 int camx_qk_rope_paged(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16,
                        void * cache, int * err, const int32_t * page_table, int pt_stride, int page, int n_pages, int n, int yarn,
                        int q8, camx_stream_t stream);

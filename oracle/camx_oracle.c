@@ -582,8 +582,9 @@ ORC_API void orc_pf_kv_append(const float * k, int ldk, const float * v, int ldv
  *   q8 = 0: q16 = fp16(rope(norm q)); cache row (fp16) = [K | V].
  *   q8 = 1: q16 = fp16(H f16r(rope)); cache row (bytes) = Q8 blocks of H f16r(rope(norm k)) | f16r(v).
  *   Row address: row_index(t) * row_bytes with row_index = position, or, paged (page_table != NULL):
- *   page_table[t * pt_stride + pos / page] * page + pos % page; a page id outside [0, n_pages) ORs 8 into err and the
- *   row is not written (paging has no reference counterpart: each row's bytes equal the unpaged row's). */
+ *   page_table[t * pt_stride + pos / page] * page + pos % page; a page id outside [0, n_pages) ORs 8 into err, a position outside
+ *   the table row (or, unpaged with n_pages given as the cache's row count, outside the cache) ORs 1, and the row is not written
+ *   (paging has no reference counterpart: each row's bytes equal the unpaged row's). */
 ORC_API void orc_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, const int32_t * pos,
                          uint16_t * q16, void * cache, int n, int yarn, int q8, int32_t * err,
                          const int32_t * page_table, int pt_stride, int page, int n_pages) {
@@ -600,7 +601,13 @@ ORC_API void orc_qk_rope(const float * qkv, int ldq, int nh, int nkv, const floa
             else { const float theta = (float)p * powf(par[256], (float)i); rc[i] = cosf(theta); rs[i] = sinf(theta); }
         }
         uint8_t * cw = NULL;
-        if (page_table) {
+        /* our addressing layer's span refusal: a position outside the sequence's table row, or (unpaged, n_pages = rows of the cache when
+         * given) outside the cache: bit 1, the row is not written */
+        const int span = p >= 0 && (page_table ? p / page < pt_stride : (n_pages == 0 || p < n_pages));
+        if (!span) {
+#pragma omp atomic
+            *err |= 1;
+        } else if (page_table) {
             const int pg = page_table[(size_t)t * pt_stride + p / page];
             if (pg < 0 || pg >= n_pages) {
 #pragma omp atomic

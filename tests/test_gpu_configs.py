@@ -221,7 +221,7 @@ def test_config5_batched_decode_paged_q8():
     del cache
     # the unpaged F16 form at the same positions: the stage boundary the Q8 bytes are defined from
     c16 = dev(np.zeros((131072, 2 * M), np.uint16)); q16f = dev(np.zeros((S, nh, 128), np.uint16)); e2 = dev(np.zeros(1, np.int32))
-    call('camx_qk_rope_paged', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16f), ptr(c16), ptr(e2), NULL, I(0), I(0), I(0), I(S), I(0), I(0))
+    call('camx_qk_rope_paged', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16f), ptr(c16), ptr(e2), NULL, I(0), I(0), I(131072), I(S), I(0), I(0))
     rows16 = host(c16, np.uint16)[pos]
     rq, rc, _ = O.qk_rope(qkv, nh, nkv, par, S, pos=pos, rows=131072)
     assert close_16(host(q16f, np.uint16), rq, 'f16') and close_16(rows16[:, :M], rc[pos][:, :M], 'f16') and bits_equal(rows16[:, M:], rc[pos][:, M:])

@@ -91,7 +91,7 @@ def test_qk_rope_paged_decode_batch():
     # the unpaged form at the same positions, one sequence per launch row, as the reference for the row bytes
     c_flat = dev(np.full((131072, rb), 0xa5, np.uint8)); q16f = dev(np.zeros((n, nh, 128), np.uint16)); err2 = dev(np.zeros(1, np.int32))
     call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16f), ptr(c_flat), ptr(err2), NULL, I(0),
-         I(0), I(0), I(n), I(0), I(1))
+         I(0), I(131072), I(n), I(0), I(1))
     assert int(host(err2)[0]) == 0
     g, flat = host(c8).reshape(n_pages, page, rb), host(c_flat)
     touched = np.zeros((n_pages, page), bool)
@@ -105,6 +105,40 @@ def test_qk_rope_paged_decode_batch():
     # the oracle on the same inputs: q16 within tolerance, and the same error word
     rq, _, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos, q8=True, rows=n_pages * page, page_table=table, page=page, n_pages=n_pages)
     assert oerr == 8 and close_16(host(q16, np.uint16), rq, 'f16')
+
+
+def test_qk_rope_paged_refuses_positions_outside_the_table_and_the_cache():
+    """a position past the sequence's table row, a negative one, and (unpaged) one past the cache: bit 1, that sequence's row is not
+    written, every other row has the oracle's bytes and nothing else is touched"""
+    rng = np.random.default_rng(77)
+    nh, nkv, n, page, n_pages, maxp = 8, 2, 12, 16, 64, 4
+    par = qk_par(rng); M = nkv * 128; rb = 2 * (M // 32) * 34
+    qkv = outliers(rng, (n, (nh + 2 * nkv) * 128))
+    pos = rng.integers(0, page * maxp, n).astype(np.int32)
+    pos[3] = page * maxp + 5                                               # past the table row: would read the next sequence's page ids
+    pos[7] = -2
+    table = rng.permutation(n_pages)[:n * maxp].reshape(n, maxp).astype(np.int32)
+    pd, qd, posd, td = dev(par), dev(qkv), dev(pos), dev(table)
+    for q8 in (1, 0):
+        fill = np.full((n_pages * page, rb if q8 else 2 * M), 0xa5 if q8 else 0xa5a5, np.uint8 if q8 else np.uint16)
+        cd = dev(fill); err = dev(np.zeros(1, np.int32)); q16 = dev(np.zeros((n, nh, 128), np.uint16))
+        call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(q16), ptr(cd), ptr(err), ptr(td), I(maxp),
+             I(page), I(n_pages), I(n), I(0), I(q8))
+        rq, rcache, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos, q8=bool(q8), cache=fill, page_table=table, page=page, n_pages=n_pages)
+        assert int(host(err)[0]) == oerr == 1
+        got = host(cd, None if q8 else np.uint16)
+        if q8: assert bits_equal(got, rcache)
+        else:
+            rows = [table[t, pos[t] // page] * page + pos[t] % page for t in range(n) if t not in (3, 7)]
+            untouched = np.ones(n_pages * page, bool); untouched[rows] = False
+            assert (got[untouched] == 0xa5a5).all() and close_16(got[rows][:, :M], rcache[rows][:, :M], 'f16') and bits_equal(got[rows][:, M:], rcache[rows][:, M:])
+        assert close_16(host(q16, np.uint16), rq, 'f16')
+    # unpaged: the cache has 40 rows, one sequence sits at row 40
+    pos2 = rng.permutation(40)[:n].astype(np.int32); pos2[5] = 40
+    fill = np.full((40, rb), 0xa5, np.uint8); cd = dev(fill); err = dev(np.zeros(1, np.int32)); q16 = dev(np.zeros((n, nh, 128), np.uint16))
+    call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(dev(pos2)), ptr(q16), ptr(cd), ptr(err), NULL, I(0), I(0), I(40), I(n), I(0), I(1))
+    _, rcache, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos2, q8=True, cache=fill, n_pages=40)
+    assert int(host(err)[0]) == oerr == 1 and bits_equal(host(cd), rcache)
 
 
 @pytest.mark.parametrize('T,heads,D,n_rot,stride,base', [(16, 24, 256, 64, 512, 1e7), (16, 4, 256, 64, 256, 1e7), (3, 5, 128, 128, 128, 1e6),

@@ -91,6 +91,35 @@ def test_kv_hadamard_actq_swiglu(seed):
         assert bits_equal(host(act, np.uint16), wa) and bits_equal(host(y), O.mmq_q8_1(O.bf2f(wa), Fh, T2, layout))
 
 
+@pytest.mark.parametrize('T2,layout', [(40, 1), (40, 0), (300, 1), (2100, 1), (2100, 0)])
+def test_swiglu_mmq_nonfinite_activations(T2, layout):
+    """+-inf and NaN gate / up values (and inf * 0 products): the activation is the canonical NaN 0x7fc0 that silu_mul_bf16 stores, in every
+    batch-size form of the fused kernel, and the blocks are the quantizer's of that activation (a block sum that is a NaN: a NaN)"""
+    rng = np.random.default_rng(4200 + T2 + layout)
+    Fh = 8 * 80
+    with np.errstate(all='ignore'):
+        gu = O.f2bf(values(rng, (T2, 2 * Fh), emin=-130.0, emax=60.0))
+        for pat in (0x7f80, 0xff80, 0x7fc0, 0xffc1, 0x7fff, 0x7f81):
+            gu[rng.random(gu.shape) < 2e-3] = pat
+        wa = O.silu_mul_bf16(gu)
+        want = O.mmq_q8_1(O.bf2f(wa), Fh, T2, layout)
+    assert (wa == 0x7fc0).any()
+    y = dev(np.zeros((O.k_pad(Fh) // 128, T2, 144), np.uint8)); act = dev(np.zeros((T2, Fh), np.uint16))
+    call('camx_swiglu_mmq_q8_1', ptr(dev(gu)), L64(2 * Fh), L64(Fh), ptr(y), ptr(act), I(T2), I(layout))
+    assert bits_equal(host(act, np.uint16), wa)
+    got = host(y)
+    if layout == 1:                                  # the half-precision sums: a NaN for a NaN, everything else bit for bit
+        gs = got[:, :, :16].copy().view(np.float16)[..., 1::2]; ws = want[:, :, :16].copy().view(np.float16)[..., 1::2]
+        nan = np.isnan(ws)
+        assert np.isnan(gs[nan]).all() and np.array_equal(gs[~nan].view(np.uint16), ws[~nan].view(np.uint16))
+        got = got.copy(); want = want.copy()
+        for k in range(4): got[:, :, 4 * k + 2:4 * k + 4] = 0; want[:, :, 4 * k + 2:4 * k + 4] = 0
+    assert bits_equal(got, want)
+    silu = dev(np.zeros((T2, Fh), np.uint16))
+    call('camx_silu_mul_bf16', ptr(dev(gu)), ptr(silu), I(Fh), L64(T2 * Fh))
+    assert bits_equal(host(silu, np.uint16), wa)
+
+
 @pytest.mark.parametrize('seed', range(6))
 def test_embedding_blocks_of_random_bytes(seed):
     """every scale pattern (negative, subnormal, infinite, NaN) and every code byte"""
