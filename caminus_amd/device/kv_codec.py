@@ -113,6 +113,8 @@ class Q8KVCodec:
             check_span(pos0, T, rows, what='own Q8 KV read')
         if not isinstance(k, torch.Tensor) or k.dtype not in (torch.float32, torch.float16):
             raise ValueError('kv_codec: k must be float32 or float16')
+        if k.dtype == torch.float16 and (ldk % 4 or ldv % 4):
+            raise ValueError('kv_codec: float16 rows need strides that are multiples of 4 (the rows are written 8 bytes at a time)')
         operands = {
             'cache': (cache, torch.uint8, rows * row_bytes, 2),
             'k': (k, k.dtype, (T - 1) * ldk + M, 8 if k.dtype == torch.float16 else 4),
