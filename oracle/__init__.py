@@ -14,12 +14,21 @@ _lib = None
 _ref = None
 
 
+_path = None
+
+
+def use_library(path):
+    """load the oracle from another build of the same source (the benchmark's -O3 -march=native build)"""
+    global _lib, _path
+    _lib, _path = None, path
+
+
 def lib():
     global _lib
     if _lib is None:
-        if not os.path.isfile(_build.ORC_SO):
+        if _path is None and not os.path.isfile(_build.ORC_SO):
             _build.build_oracle()
-        L = C.CDLL(_build.ORC_SO)
+        L = C.CDLL(_path or _build.ORC_SO)
         for n, r in (('orc_bf2f', C.c_float), ('orc_h2f', C.c_float), ('orc_row_ss', C.c_float), ('orc_bfly32_sum', C.c_float)):
             getattr(L, n).restype = r
         for n in ('orc_f2bf', 'orc_to_bf16', 'orc_f2h'):

@@ -26,13 +26,17 @@ extern "C" void ref_kv_q8_encode(const float * x, unsigned char * y, unsigned ch
 '''
 
 
-def build_oracle(fast=False):
-    """fast: -O3 -march=native for the benchmark's CPU-baseline leg (same source, same contraction setting)"""
+def build_oracle(fast=False, out=None):
+    """fast: -O3 -march=native for the benchmark's CPU-baseline leg (same source, same contraction setting), built on the host that
+    times it and written to `out` (the tests keep oracle/liborc.so, the -O2 build)"""
+    if fast and out is None:
+        raise ValueError('the -march=native build goes to a path of its own, never over oracle/liborc.so')
+    out = out or ORC_SO
     cmd = ['gcc', '-std=c11', '-O3' if fast else '-O2', '-ffp-contract=off', '-fno-fast-math', '-fopenmp', '-fvisibility=hidden',
-           '-shared', '-fPIC', os.path.join(HERE, 'camx_oracle.c'), '-o', ORC_SO, '-lm']
+           '-shared', '-fPIC', os.path.join(HERE, 'camx_oracle.c'), '-o', out, '-lm']
     if fast: cmd.insert(3, '-march=native')
     subprocess.run(cmd, check=True)
-    return ORC_SO
+    return out
 
 
 def build_ref():
@@ -50,5 +54,5 @@ def build_ref():
 
 
 if __name__ == '__main__':
-    print(build_oracle(fast='--fast' in sys.argv))
+    print(build_oracle())
     print(build_ref())
