@@ -423,6 +423,129 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
     }
 }
 
+// ---- the same arithmetic for the aligned shape of a dense bf16 prefill chunk, written straight-line -----------------------------
+// Rows of exactly 16 STEPS heads (STEPS <= 5) with nh and nkv multiples of 4, so a wave step of four heads is wholly q, k or v and
+// no lane is ever predicated; positions pos0 + t. TPW tokens per workgroup, all their loads issued before anything else (one
+// burst of reads per wave, then its arithmetic, then one burst of writes), the norm weights and the tokens' cos / sin rows in LDS.
+// The operations and their order are qk_rope_wide_tokens': same bits.
+template <bool YARN, int STEPS, int TPW>
+__global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
+    __shared__ __attribute__((aligned(16))) float rc[TPW][64];
+    __shared__ __attribute__((aligned(16))) float rs[TPW][64];
+    __shared__ __attribute__((aligned(16))) float nrm[256];                  // q_norm | k_norm
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, hq = lane >> 4;
+    const int t0 = blockIdx.x * TPW;
+    const int nqk = a.nh + a.nkv;
+    const size_t M = (size_t)a.nkv * 128;
+    const int lo = 128 * hq + 8 * l16;                                      // this lane's element offset inside a wave step
+    u32x4 xin[TPW][STEPS];
+#pragma unroll
+    for (int ti = 0; ti < TPW; ti++) {
+        const int tk = t0 + ti < a.n ? t0 + ti : a.n - 1;
+        const uint16_t * p = (const uint16_t *)a.qkv + (size_t)tk * a.ldq + 512 * wave + lo;      // heads 16 s + 4 wave .. + 3
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) xin[ti][s] = __builtin_nontemporal_load((const u32x4 *)(p + 2048 * s));
+    }
+    nrm[tid] = a.par[tid];
+    if (wave < TPW) {                                                       // wave w: the cos / sin row of token t0 + w
+        const int pos = a.pos0 + (t0 + wave < a.n ? t0 + wave : a.n - 1);
+        float c, sn;
+        if (YARN) { const float theta = (float)pos * a.par[258 + lane], ms = a.par[322]; c = cosf(theta) * ms; sn = sinf(theta) * ms; }
+        else { const float theta = (float)pos * rope_freq(a.par[256], lane); c = cosf(theta); sn = sinf(theta); }
+        rc[wave][lane] = c; rs[wave][lane] = sn;
+    }
+    __syncthreads();
+    const float eps = a.par[257];
+#pragma unroll
+    for (int ti = 0; ti < TPW; ti++) {
+        const int t = t0 + ti;
+        if (t >= a.n) break;
+        const int pos = a.pos0 + t;
+        uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
+        uint16_t * qw = a.q16 + (size_t)t * a.nh * 128;
+        const int j0 = 8 * (l16 & 7);
+        f32x4 c4[2], s4[2];
+        c4[0] = *(const f32x4 *)(rc[ti] + j0); c4[1] = *(const f32x4 *)(rc[ti] + j0 + 4);
+        s4[0] = *(const f32x4 *)(rs[ti] + j0); s4[1] = *(const f32x4 *)(rs[ti] + j0 + 4);
+        if (l16 < 8) { s4[0] = -s4[0]; s4[1] = -s4[1]; }                    // dims below 64 take -(x1 s): the sign moves into s
+        // phase 1: the sum of squares of every q / k step (thread ^ 16, ^ 8 across lanes, ^ 4, ^ 2, ^ 1 in registers, four groups in order)
+        float tot[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            tot[s] = 1.0f;
+            if (16 * s + 4 * wave >= nqk) continue;                         // (wave-uniform) V heads: no norm
+            float sq[8];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const uint32_t b = xin[ti][s][p];
+                const float x0 = __builtin_bit_cast(float, b << 16), x1 = __builtin_bit_cast(float, b & 0xffff0000u);
+                sq[2 * p] = x0 * x0; sq[2 * p + 1] = x1 * x1;
+            }
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] = add_xor2(sq[k]);
+#pragma unroll
+            for (int k = 0; k < 8; k++) sq[k] = add_xor1(sq[k]);
+            const float b0 = sq[0] + sq[4], b1 = sq[1] + sq[5], b2 = sq[2] + sq[6], b3 = sq[3] + sq[7];
+            const float e0 = b0 + b2, e1 = b1 + b3;
+            const float g = e0 + e1;
+            tot[s] = ((swz_group(g, 0) + swz_group(g, 1)) + swz_group(g, 2)) + swz_group(g, 3);
+        }
+        // phase 2: one IEEE sqrt + divide per row for all steps: lane s of a row takes step s, the row reads it back
+        float tv = tot[0];
+#pragma unroll
+        for (int s = 1; s < STEPS; s++) tv = l16 == s ? tot[s] : tv;
+        const float sc = rsqrt_exact(tv / 128 + eps);
+        float scale[STEPS];
+        static_assert(STEPS <= 5, "the broadcasts below are written out for at most five steps");
+        scale[0] = row_lane_bcast<0>(sc);
+        if (STEPS > 1) scale[1 % STEPS] = row_lane_bcast<1>(sc);
+        if (STEPS > 2) scale[2 % STEPS] = row_lane_bcast<2>(sc);
+        if (STEPS > 3) scale[3 % STEPS] = row_lane_bcast<3>(sc);
+        if (STEPS > 4) scale[4 % STEPS] = row_lane_bcast<4>(sc);
+        // phase 3: scale, rotate, convert, store
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const int h0 = 16 * s + 4 * wave;                               // wave-uniform
+            float x[8];
+#pragma unroll
+            for (int p = 0; p < 4; p++) { const uint32_t b = xin[ti][s][p]; x[2 * p] = __builtin_bit_cast(float, b << 16); x[2 * p + 1] = __builtin_bit_cast(float, b & 0xffff0000u); }
+            u32x4 out;
+            if (h0 >= nqk) {                                                // V heads: fp16 copy
+#pragma unroll
+                for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[2 * p], x[2 * p + 1]);
+                RSTORE((u32x4 *)(cw + M + (size_t)(h0 - nqk) * 128 + lo), out);
+                continue;
+            }
+            const bool isq = h0 < a.nh;
+            const float * wp = nrm + (isq ? 0 : 128) + 8 * l16;
+            const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
+            float y[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float y1 = (scale[s] * x[k]) * (k < 4 ? w0[k] : w1[k - 4]);
+                y[k] = __builtin_fmaf(y1, k < 4 ? c4[0][k] : c4[1][k - 4], mul_ror8(y1, k < 4 ? s4[0][k] : s4[1][k - 4]));
+            }
+#pragma unroll
+            for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
+            RSTORE((u32x4 *)((isq ? qw + (size_t)h0 * 128 : cw + (size_t)(h0 - a.nh) * 128) + lo), out);
+        }
+    }
+}
+template <bool YARN, int TPW>
+static bool rope_chunk_launch(const RopeArgs & a, hipStream_t st) {
+    const int items = a.nh + 2 * a.nkv;
+    if (a.pos || a.page_table || (items & 15) || items > 80 || (a.nh & 3) || (a.nkv & 3)) return false;
+    const dim3 grid((a.n + TPW - 1) / TPW), block(256);
+    switch (items >> 4) {
+    case 1: qk_rope_chunk<YARN, 1, TPW><<<grid, block, 0, st>>>(a); break;
+    case 2: qk_rope_chunk<YARN, 2, TPW><<<grid, block, 0, st>>>(a); break;
+    case 3: qk_rope_chunk<YARN, 3, TPW><<<grid, block, 0, st>>>(a); break;
+    case 4: qk_rope_chunk<YARN, 4, TPW><<<grid, block, 0, st>>>(a); break;
+    default: qk_rope_chunk<YARN, 5, TPW><<<grid, block, 0, st>>>(a); break;
+    }
+    return true;
+}
+
 // ---- pf_qk_nr: any head dim D <= 512, rotary on the first n_rot dims, input heads at head_stride ------------------------------
 struct NrArgs {
     const void * x; int head_stride, heads; const float * w; int D, nrot; float theta_scale, eps; int pos0; const int32_t * pos; void * out; int T;
@@ -827,7 +950,9 @@ static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bo
     if (a.n == 0) return CAMX_OK;
     const bool wide = (!q8 || !bf16in) && !a.page_table && (a.ldq & (bf16in ? 7 : 3)) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
                       ((uintptr_t)a.cache & 15) == 0;
-    if (wide && bf16in && a.n >= 2048) {          // enough tokens to fill the chip two to a workgroup (4096 tokens, every launch on cold lines: 32.2 us; four: 34.0, one: 33.7)
+    // one token per workgroup: 29.9 us for 4096 tokens x 80 heads on cold lines (two tokens: 32.4, four: 34.9; the general kernel below: 32.3)
+    if (wide && bf16in && a.n >= 2048 && (yarn ? rope_chunk_launch<true, 1>(a, st) : rope_chunk_launch<false, 1>(a, st))) {}
+    else if (wide && bf16in && a.n >= 2048) {          // enough tokens to fill the chip two to a workgroup (4096 tokens, every launch on cold lines: 32.2 us; four: 34.0, one: 33.7)
         const dim3 g2((a.n + 1) / 2);
         if (yarn) qk_rope_wide_tokens<true, 2, false, 5, false><<<g2, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 2, false, 5, false><<<g2, dim3(256), 0, st>>>(a);
     }
