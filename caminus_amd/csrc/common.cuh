@@ -128,6 +128,15 @@ CAMX_DEV u32x2 pack_f16x4(f32x4 v) {
     r.y = (uint32_t)f2h_bits(v.z) | ((uint32_t)f2h_bits(v.w) << 16);
     return r;
 }
+// fp16 of the products t * g rounded once (no intermediate fp32 rounding): the mixed-precision fma with a -0 addend (which keeps the
+// sign of a zero product), low then high half of one register
+CAMX_DEV uint32_t mul_pack_f16x2_once(float t0, float g0, float t1, float g1) {
+    uint32_t r = 0;
+    const float nz = -0.0f;
+    asm("v_fma_mixlo_f16 %0, %1, %2, %3" : "+v"(r) : "v"(t0), "v"(g0), "v"(nz));
+    asm("v_fma_mixhi_f16 %0, %1, %2, %3" : "+v"(r) : "v"(t1), "v"(g1), "v"(nz));
+    return r;
+}
 CAMX_DEV f32x4 unpack_bf16x4(u32x2 w) {
     f32x4 r;
     r.x = __builtin_bit_cast(float, w.x << 16); r.y = __builtin_bit_cast(float, w.x & 0xffff0000u);

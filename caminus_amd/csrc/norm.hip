@@ -144,13 +144,18 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) {
-                f32x4 v;
-                v.x = (xv[j].x * scale) * g[j].x; v.y = (xv[j].y * scale) * g[j].y; v.z = (xv[j].z * scale) * g[j].z; v.w = (xv[j].w * scale) * g[j].w;
+                f32x4 t, v;
+                t.x = xv[j].x * scale; t.y = xv[j].y * scale; t.z = xv[j].z * scale; t.w = xv[j].w * scale;
+                v.x = t.x * g[j].x; v.y = t.y * g[j].y; v.z = t.z * g[j].z; v.w = t.w * g[j].w;
                 const size_t o = (size_t)row * N + 256 * j + 4 * lane;
                 if (a.h) { if (NT) __builtin_nontemporal_store(v, (f32x4 *)(a.h + o)); else *(f32x4 *)(a.h + o) = v; }
                 if (a.h16) {
                     u32x2 * p16 = (u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane);
-                    if (NT) __builtin_nontemporal_store(pack_f16x4(v), p16); else *p16 = pack_f16x4(v);
+                    // the dense line (q35p_add_rms16) stores fp16 of the last product rounded once, as the reference's binary does
+                    // (kernels/q35_prefill.hip:630-635); the own line's statement is fp16 of the rounded fp32 value
+                    const u32x2 pk = ADD == ADD_F32_DIRECT ? (u32x2){mul_pack_f16x2_once(t.x, g[j].x, t.y, g[j].y), mul_pack_f16x2_once(t.z, g[j].z, t.w, g[j].w)}
+                                                           : pack_f16x4(v);
+                    if (NT) __builtin_nontemporal_store(pk, p16); else *p16 = pk;
                 }
                 if (a.hbf) __builtin_nontemporal_store(pack_bf16x4_rne(v), (u32x2 *)(a.hbf + o));
                 if (a.q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
@@ -209,7 +214,7 @@ __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
                 vk[k] = (xr[i] * scale) * gw[i];
                 const size_t o = (size_t)row * N + i;
                 if (a.h) a.h[o] = vk[k];
-                if (a.h16) a.h16[(size_t)row * a.ld16 + i] = f2h_bits(vk[k]);
+                if (a.h16) a.h16[(size_t)row * a.ld16 + i] = ADD == ADD_F32_DIRECT ? (uint16_t)mul_pack_f16x2_once(xr[i] * scale, gw[i], 0.0f, 0.0f) : f2h_bits(vk[k]);
                 if (a.hbf) a.hbf[o] = to_bf16(vk[k]);
             }
         }
@@ -326,6 +331,15 @@ int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const
                        uint16_t * h16, int N, int n, hipStream_t st) {
     if (N < 256 || N % 256 || N > 2048 || S < 0 || S > 8 || n < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
     NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
+    return launch_norm<ADD_F32_SLOTS>(a, st);
+}
+
+// OP_OWN_ADD_RMS16 with its Seg fields (python/caminus/engine/k3.py:881-902): W = nw, gs = w, a = d, asum = h, y = x, rs = eps, N,
+// K = the fp16 copy's token stride (elements, >= N), pad1 = S, aux = h16, tokens = the tape's T
+int camx_op_own_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h, uint16_t * h16,
+                          int N, int K, int tokens, hipStream_t st) {
+    if (N < 256 || N % 256 || N > 2048 || K < N || S < 0 || S > 8 || tokens < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
+    NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, K, nullptr, nullptr, nullptr, N, tokens, nullptr, 1, 0.0f};
     return launch_norm<ADD_F32_SLOTS>(a, st);
 }
 

@@ -454,6 +454,12 @@ int camx_gg_quantize_q8_1(const float * x, void * y, long n, int mode, float rs,
     CAMX_LAUNCH_RET();
 }
 
+// OP_GG_Q8_1 with its Seg fields in the tape's order (python/caminus/engine/k3.py:649-659): a = x, y, N = n, work = mode, rs = the SiLU
+// pre-scale of mode 1, gs = the multiplier of mode 2
+int camx_op_gg_q8_1(const float * x, void * y, int n, int work, float rs, const float * gs, hipStream_t st) {
+    return camx_gg_quantize_q8_1(x, y, (long)n, work, rs, gs, st);
+}
+
 // quantize_mmq_q8_1<layout, false>: column c = row (ids ? ids[c] : c) of x (row stride s01 floats); ne00 = K, ne0 = K
 // padded to 512, ne1 = ncols. The reference's s02 / s03 / ne2 (batch dims) must be 0 / 0 / 1.
 int camx_quantize_mmq_q8_1(const float * x, const int32_t * ids, void * vy, long ne00, long s01, long s02, long s03,

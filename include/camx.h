@@ -59,6 +59,14 @@ int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps
  * ybf (bf16 copy), scl (row scale [R]) each optional. The reference kernel is built for K = 2560; K is an argument here. */
 int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf, float * scl, int R, int wr, float eps, int K,
                     camx_stream_t stream);
+/* OP_OWN_ADD_RMS16 (kernels/k3_own_ops.h:326-383) with the tape's Seg fields (python/caminus/engine/k3.py:881-902): y = x, a = d,
+ * gs = w, pad1 = S, W = nw, rs = eps, asum = h, aux = h16, N, K = the token stride of h16 in elements (>= N), team = tokens.
+ * camx_q3p_add_rms16 is the same pass with K = N. */
+int camx_op_own_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h, uint16_t * h16,
+                          int N, int K, int tokens, camx_stream_t stream);
+/* OP_GG_Q8_1 (kernels/k3_gguf_ops.h:55-77) with the tape's Seg fields in their order (python/caminus/engine/k3.py:649-659):
+ * a = x, y, N = n, work = 0 plain / 1 silu(x * rs) / 2 silu(x) * gs[i], rs, gs. The same blocks as camx_gg_quantize_q8_1. */
+int camx_op_gg_q8_1(const float * x, void * y, int n, int work, float rs, const float * gs, camx_stream_t stream);
 /* OP_RMS_MUL (kernels/k3_gguf_ops.h:1233-1268; Seg fields: a = x, W = w, y, asum = q8, N = R, K, pad1 = wr, rs = eps). */
 int camx_op_rms_mul(const float * x, const float * w, float * y, void * q8, int R, int wr, int K, float eps, camx_stream_t stream);
 /* pf_hc_post_rms (kernels/prefill_glue.hip:130-170): row q = t * HC + h of N values: res[q] = fma(b[t], 2 sigmoid(inj[q] * rs),

@@ -258,6 +258,23 @@ ORC_API void orc_add_rms16(float * x, const float * d, const float * w, int S, c
     }
 }
 /* q35p_add_rms16 (kernels/q35_prefill.hip:636-660): x = x + d directly (d NULL: no add), any N = 256 NI */
+/* the product of two floats rounded ONCE to half: the product is exact in double (24 + 24 significant bits), the conversion below rounds it
+ * to nearest even. This is what the reference's q35p_add_rms16 binary stores in h16: its compiler rounds the fp16 copy straight from the
+ * last product (v_fma_mixlo_f16), and the reference keeps its source shaped so that it does (kernels/q35_prefill.hip:630-635). */
+static uint16_t d2h(double v) {
+    uint64_t u; memcpy(&u, &v, 8);
+    const uint16_t sign = (uint16_t)((u >> 48) & 0x8000u);
+    const double a = fabs(v);
+    if (a != a) return (uint16_t)(sign | 0x7e00u);
+    if (a >= 65520.0) return (uint16_t)(sign | 0x7c00u);                 /* rounds to 2^16: infinity */
+    if (a < 0x1p-14) return (uint16_t)(sign | (uint16_t)nearbyint(a * 0x1p24));       /* subnormal halves (and 2^-14 itself by carry) */
+    int e; const double m = frexp(a, &e);                                 /* a = m 2^e, m in [0.5, 1) */
+    uint32_t mant = (uint32_t)nearbyint(m * 2048.0);                      /* 11 bits, ties to even */
+    if (mant == 2048u) { mant = 1024u; e++; }
+    return (uint16_t)(sign | (uint32_t)((e - 1 + 15) << 10) | (mant - 1024u));
+}
+ORC_API uint16_t orc_mul_f2h_once(float a, float b) { return d2h((double)a * (double)b); }
+
 ORC_API void orc_add_rms16_q35(float * x, const float * d, const float * nw, float eps, float * h, uint16_t * h16, int N, int n) {
 #pragma omp parallel for schedule(static)
     for (int t = 0; t < n; t++) {
@@ -265,9 +282,9 @@ ORC_API void orc_add_rms16_q35(float * x, const float * d, const float * nw, flo
         if (d) for (int i = 0; i < N; i++) xr[i] = xr[i] + d[(size_t)t * N + i];
         const float scale = rsqrt_c(row_ss(xr, N) / (float)N + eps);
         for (int i = 0; i < N; i++) {
-            const float v = (xr[i] * scale) * nw[i];
-            h[(size_t)t * N + i] = v;
-            h16[(size_t)t * N + i] = orc_f2h(v);
+            const float tt = xr[i] * scale;
+            h[(size_t)t * N + i] = tt * nw[i];
+            h16[(size_t)t * N + i] = d2h((double)tt * (double)nw[i]);       /* one rounding from the last product, as the reference's binary */
         }
     }
 }

@@ -20,6 +20,12 @@ def test_q3p_add_rms16(n, N, S, weighted):
     assert bits_equal(host(xd), ref['x'])
     assert bits_equal(host(h), ref['h'])
     assert bits_equal(host(h16, np.uint16), ref['h16'])
+    # the tape's form: the fp16 copy at its own token stride (the Seg's K), the elements between the rows untouched
+    K = N + 64
+    xd = dev(x); h = dev(np.zeros((n, N), np.float32)); h16 = dev(np.full((n, K), 0x5a5a, np.uint16))
+    call('camx_op_own_add_rms16', ptr(xd), ptr(dd) if S else NULL, ptr(wd) if weighted else NULL, I(S), ptr(nwd), F(1e-6), ptr(h), ptr(h16), I(N), I(K), I(n))
+    got = host(h16, np.uint16)
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(got[:, :N], ref['h16']) and (got[:, N:] == 0x5a5a).all()
 
 
 @pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096), (520, 4096), (513, 8192), (600, 3072)])

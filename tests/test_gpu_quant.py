@@ -33,6 +33,12 @@ def test_q8_1_silu_modes(mode):
     d_g, d_r = got[:, 0:2].copy().view(np.float16).astype(np.float64), ref[:, 0:2].copy().view(np.float16).astype(np.float64)
     assert np.all(np.abs(d_g - d_r) <= np.abs(d_r) * 2.0 ** -9 + 1e-12)
     assert np.abs(got[:, 4:].view(np.int8).astype(int) - ref[:, 4:].view(np.int8).astype(int)).max() <= 1
+    y2 = dev(np.zeros((n // 32, 36), np.uint8))                           # the tape's field order: the same kernel, the same bytes
+    call('camx_op_gg_q8_1', ptr(xd), ptr(y2), I(n), I(mode), F(0.37), ptr(gd) if mode == 2 else NULL)
+    assert bits_equal(host(y2), got)
+    y0 = dev(np.zeros((n // 32, 36), np.uint8))
+    call('camx_op_gg_q8_1', ptr(xd), ptr(y0), I(n), I(0), F(0), NULL)
+    assert bits_equal(host(y0), O.q8_1(x))
 
 
 @pytest.mark.parametrize('K,ncols,layout', [(512, 3, 0), (2048, 17, 1), (17408, 5, 1), (896, 4, 0), (100 * 4, 2, 1), (2048, 300, 1), (900, 257, 0),

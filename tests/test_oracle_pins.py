@@ -384,7 +384,90 @@ def test_mmq_q8_1_layout_and_invariants():
         for s in range(2): assert np.array_equal(sc[:, inv[2 * t + s]], ys[:, t])
 
 
+def test_mmq_q8_1_bit_level_known_answers():
+    """what the vendored statement (kernels/ggml_mmq/quantize_mmq.cuh:78-112) fixes to the last bit and a plausible restatement would
+    get wrong: ties away from zero; codes from x * (127 / amax), not x / (amax / 127); d = 1 / (127 / amax), not amax / 127; and the
+    DS4 sum as ((x0 + x1) + x2) + x3 per thread, then thread xor 4, 2, 1"""
+    K = 128
+
+    def block(v32, layout):
+        x = np.zeros((1, K), f32); x[0, :32] = v32
+        b = O.mmq_q8_1(x, K, 1, layout)[0, 0]
+        hdr = b[:4].copy()
+        return (hdr.view(f32)[0] if layout == 0 else hdr.view(np.float16)), b[16:48].view(np.int8)
+
+    # amax = 127: 127 / amax = 1 exactly, the codes are roundf(x): halves go away from zero
+    v = np.zeros(32, f32); v[0] = 127; v[1:13] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.49999997, -0.49999997, 126.5, -126.5, 3.5, 4.5]
+    d, q = block(v, 0)
+    assert d == 1.0 and q[:13].tolist() == [127, 1, -1, 2, -2, 3, -3, 0, 0, 127, -127, 4, 5]
+    # a value whose product with fl(127 / amax) and whose quotient by fl(amax / 127) round to different codes: found by a seeded
+    # search over values next to a tie
+    rng = np.random.default_rng(12)
+    found = None
+    for _ in range(400):
+        amax = rng.uniform(1, 4, 20000).astype(f32); k = rng.integers(1, 126, 20000)
+        x = ((k + 0.5) * (amax.astype(np.float64) / 127.0)).astype(f32)                 # near a tie
+        pm = (x * (f32(127.0) / amax)).astype(f32); pd = (x / (amax / f32(127.0))).astype(f32)
+        rm = np.sign(pm) * np.floor(np.abs(pm.astype(np.float64)) + 0.5); rd = np.sign(pd) * np.floor(np.abs(pd.astype(np.float64)) + 0.5)
+        hit = np.nonzero((rm != rd) & (x <= amax))[0]
+        if hit.size: found = (amax[hit[0]], x[hit[0]], int(rm[hit[0]]), int(rd[hit[0]])); break
+    assert found is not None
+    amax, x, by_mul, by_div = found
+    v = np.zeros(32, f32); v[0] = amax; v[1] = x; v[2] = -x
+    d, q = block(v, 0)
+    assert by_mul != by_div and q[1] == by_mul and q[2] == -by_mul and q[0] == 127
+    # d is the reciprocal of the reciprocal: an amax where fl(1 / fl(127 / amax)) differs from fl(amax / 127)
+    cand = rng.uniform(0.5, 8, 200000).astype(f32)
+    two = (f32(1.0) / (f32(127.0) / cand)).astype(f32); one = (cand / f32(127.0)).astype(f32)
+    amax = cand[np.nonzero(two != one)[0][0]]
+    v = np.zeros(32, f32); v[5] = -amax
+    d, q = block(v, 0)
+    assert d == f32(1.0) / (f32(127.0) / amax) and d != amax / f32(127.0) and q[5] == -127
+    ds, _ = block(v, 1)
+    assert ds[0] == np.float16(d) and ds[1] == np.float16(-amax)
+    # the DS4 sum. Thread t holds values 4t .. 4t + 3. (a) inside a thread: ((2^24 + 1) + 1) + -2^24 = 0 (each 1 is lost), any other
+    # association gives 1 or 2
+    v = np.zeros(32, f32); v[0:4] = [2.0 ** 24, 1, 1, -2.0 ** 24]
+    assert block(v, 1)[0][1] == 0.0
+    v[0:4] = [2.0 ** 24, -2.0 ** 24, 1, 1]
+    assert block(v, 1)[0][1] == 2.0
+    # (b) across threads: partners are t ^ 4 first. Thread sums s0 = 2^24, s4 = 1, s2 = 1, s6 = -2^24:
+    # (s0 + s4) + (s2 + s6) = 2^24 + -(2^24 - 1) = 1; pairing neighbours first ((s0 + s2) + (s4 + s6)) would also lose a 1 but a
+    # running sum over threads 0 .. 7 gives 2^24 + 1 + 1 - 2^24 = 0
+    v = np.zeros(32, f32); v[0] = 2.0 ** 24; v[16] = 1; v[8] = 1; v[24] = -2.0 ** 24
+    assert block(v, 1)[0][1] == 1.0
+    # partners t ^ 4 then t ^ 2 then t ^ 1: s0 = 2^24, s1 = -2^24, s4 = 1, s5 = 1 -> ((s0 + s4) + 0) + ((s1 + s5) + 0) = 2^24 + -(2^24 - 1) = 1,
+    # where xor 1 first would give (s0 + s1) + (s4 + s5) = 2
+    v = np.zeros(32, f32); v[0] = 2.0 ** 24; v[4] = -2.0 ** 24; v[16] = 1; v[20] = 1
+    assert block(v, 1)[0][1] == 1.0
+
+
 # ---- RMSNorm family ---------------------------------------------------------------------------------------------------------------
+
+def test_dense_line_h16_is_the_last_product_rounded_once():
+    """q35p_add_rms16's fp16 copy: the reference's binary rounds it straight from the last product (kernels/q35_prefill.hip:630-635), so the
+    oracle rounds the exact product once. Known answer: (1 + 2^-12)^2 = 1 + 2^-11 + 2^-24 lies above the fp16 tie at 1 + 2^-11 and goes to
+    0x3c01, where fp32 first (ties to even: 1 + 2^-11) and fp16 second (ties to even: 1.0) give 0x3c00. The conversion itself against
+    numpy's double -> half on random products, subnormal and overflowing ones included."""
+    import ctypes as C
+    L = O.lib(); L.orc_mul_f2h_once.restype = C.c_uint16; L.orc_mul_f2h_once.argtypes = [C.c_float, C.c_float]
+    a = f32(1 + 2.0 ** -12)
+    assert L.orc_mul_f2h_once(a, a) == 0x3c01 and O.f2h(np.array([a * a], f32))[0] == 0x3c00
+    assert L.orc_mul_f2h_once(f32(-0.0), f32(3.0)) == 0x8000 and L.orc_mul_f2h_once(f32(300.0), f32(300.0)) == 0x7c00
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal(20000) * np.exp2(rng.integers(-20, 12, 20000))).astype(f32); y = (rng.standard_normal(20000) * np.exp2(rng.integers(-12, 8, 20000))).astype(f32)
+    with np.errstate(over='ignore'):
+        want = (x.astype(np.float64) * y.astype(np.float64)).astype(np.float16).view(np.uint16)
+    assert np.array_equal(np.array([L.orc_mul_f2h_once(float(p), float(q)) for p, q in zip(x, y)], np.uint16), want)
+    # the row function uses it: h16 = half(exact(fl(x scale) nw)), h = fl of the same product; the scale from the sibling pf_rms_mul
+    n, N = 3, 2560
+    xr = (rng.standard_normal((n, N)) * 3).astype(f32); nw = (1 + 0.1 * rng.standard_normal(N)).astype(f32)
+    r = O.add_rms16_q35(xr, nw, 1e-6)
+    t = (xr * O.rms_mul(xr, nw, 1e-6)['scale'][:, None]).astype(f32)
+    assert np.array_equal(r['h'], (t * nw).astype(f32))
+    assert np.array_equal(r['h16'], (t.astype(np.float64) * nw.astype(np.float64)).astype(np.float16).view(np.uint16))
+    assert (r['h16'] != O.f2h(r['h'])).sum() < n * N * 1e-3                # (one value in about 16000 differs from the twice-rounded one)
+
 
 def test_add_rms_closed_form_and_invariants():
     rng = np.random.default_rng(6)
