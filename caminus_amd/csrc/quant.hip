@@ -241,13 +241,21 @@ CAMX_DEV void swm_load(SwmItem & it, const void * __restrict__ src, const int32_
 // CANON: the activation is packed with f2bf (a NaN becomes 0x7fc0, as silu_mul_bf16 stores it) instead of the hardware convert, which
 // keeps a NaN's sign and payload. Returns whether a group sum of this lane's quad is a NaN: the callers run the item with the hardware
 // convert first and, in the rare wave that reports one (a NaN or infinite input), once more with CANON, which rewrites the same bytes.
-template <int LAYOUT, int SRC, bool CANON = false>
-CAMX_DEV bool swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int T, long tg, long unit,
-                          int lane) {
+// LUTMODE: where bf16(silu g) comes from. LUT_FULL: the 65536-entry table (in LDS for the persistent kernel, in device memory for the
+// rare redo of the one-shot kernel). LUT_SMALL: the 8192-entry table of the one-shot kernel, which holds the gates a model produces
+// (+-0 and 2^-24 <= |g| < 2^8 less two values); bit 1 of the result reports a gate outside it, and the caller redoes the item with the full table.
+enum { LUT_FULL = 0, LUT_SMALL = 1 };
+#define SWS_A0 0x3380u                 // bf16 bits of 2^-24: the small table's first magnitude
+#define SWS_SPAN 0x0fffu               // magnitudes per sign; index SWS_SPAN is the entry of +-0 (and the stand-in of every gate outside the table)
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+template <int LAYOUT, int SRC, bool CANON = false, int LUTMODE = LUT_FULL>
+CAMX_DEV int swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int T, long tg, long unit,
+                         int lane) {
     const int lq = lane & 3;
     const long e0 = unit * 128 + 8 * (lane & 15);
     float val[2][8];                                                   // the lane's eight values of each half, as quantized
     float amax[2], sum[2];
+    u16x2 gmin = {0xffff, 0xffff}, gmax = {0, 0};                      // LUT_SMALL: min of |g| - 1 (a zero wraps to 0xffff), max of |g|, per half
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         float m = 0.0f, s0 = 0.0f, s1 = 0.0f;
@@ -256,7 +264,15 @@ CAMX_DEV bool swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
         for (int p = 0; p < 4; p++) {
             float v0, v1;
             if (SRC == SRC_SWIGLU_BF16) {
-                const uint32_t sl = lut[it.gw[i][p] & 0xffffu], sh = lut[it.gw[i][p] >> 16];
+                uint32_t sl, sh;
+                if (LUTMODE == LUT_SMALL) {
+                    const uint32_t w = it.gw[i][p];
+                    const u16x2 a2 = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+                    const u16x2 i2 = __builtin_elementwise_min(a2 - (u16x2){SWS_A0, SWS_A0}, (u16x2){SWS_SPAN, SWS_SPAN});      // below the table: wraps, clamps
+                    const uint32_t idx = ((w >> 3) & 0x10001000u) | __builtin_bit_cast(uint32_t, i2);                            // the sign in bit 12
+                    gmin = __builtin_elementwise_min(gmin, a2 - (u16x2){1, 1}); gmax = __builtin_elementwise_max(gmax, a2);
+                    sl = lut[idx & 0xffffu]; sh = lut[idx >> 16];
+                } else { sl = lut[it.gw[i][p] & 0xffffu]; sh = lut[it.gw[i][p] >> 16]; }
                 const float u0 = __builtin_bit_cast(float, it.uw[i][p] << 16), u1 = __builtin_bit_cast(float, it.uw[i][p] & 0xffff0000u);
                 const float a0 = __builtin_bit_cast(float, sl << 16) * u0, a1 = __builtin_bit_cast(float, sh << 16) * u1;
                 pk[p] = CANON ? ((uint32_t)f2bf(a0) | ((uint32_t)f2bf(a1) << 16)) : cvt_pk_bf16(a0, a1);
@@ -299,7 +315,10 @@ CAMX_DEV bool swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * st
     if (lq < 2)
         *(uint32_t *)(blk0 + lq * (4 * 144) + 4 * ((lane & 15) >> 2)) =
             LAYOUT == MMQ_DS4 ? ((uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sm) << 16)) : __builtin_bit_cast(uint32_t, d);
-    return SRC == SRC_SWIGLU_BF16 && !CANON && ((sum[0] != sum[0]) | (sum[1] != sum[1]));
+    int flags = SRC == SRC_SWIGLU_BF16 && !CANON && ((sum[0] != sum[0]) | (sum[1] != sum[1]));
+    if (LUTMODE == LUT_SMALL)
+        flags |= ((gmin.x < SWS_A0 - 1) | (gmin.y < SWS_A0 - 1) | (gmax.x >= SWS_A0 + SWS_SPAN) | (gmax.y >= SWS_A0 + SWS_SPAN)) ? 2 : 0;
+    return flags;
 }
 
 // SRC_F32 (quantize_mmq_q8_1 without scatter): the same work split and copy-out on fp32 rows (column c = row ids[c] or c), no table
@@ -338,7 +357,7 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
         const unsigned jn = (jc) + 2 * stride;                                                                                  \
         swm_load<SRC>(NXT2, gu, ids, ld, F, T, SWM_TG(jn), SWM_UNIT(jn), lane, jn < nitems);                                 \
         if ((jc) < nitems) {                                                                                                 \
-            if (__builtin_expect(__builtin_amdgcn_ballot_w64(swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane)) != 0, 0))  \
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(swm_compute<LAYOUT, SRC>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane) & 1) != 0, 0))  \
                 swm_compute<LAYOUT, SRC, true>(CUR, lut, stage, F, act, T, SWM_TG(jc), SWM_UNIT(jc), lane);                  \
             flush(jc);                                                                                                       \
         }                                                                                                                    \
@@ -351,6 +370,74 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
 #undef SWM_STEP
 #undef SWM_TG
 #undef SWM_UNIT
+}
+
+// ---- the one-shot form for prefill chunks -----------------------------------------------------------------------------------------
+// A workgroup of SWS_WAVES waves takes SWS_WAVES neighbouring token groups of one block column and ends; the hardware hands the next
+// workgroup to whichever CU is free, which keeps the chip's accesses inside a narrow moving window of the inputs and makes neighbouring
+// waves write neighbouring runs of one block row (measured with every launch on cold lines, the same access pattern runs 12 % faster
+// than under persistent workgroups). Several workgroups share a CU, so the table they look gates up in must be small: the 8192
+// entries that cover +-0 and 2^-24 <= |g| < 2^8 (16 KiB, copied straight from device memory into LDS, no registers), index = the
+// magnitude's offset from 2^-24 clamped to the last entry, which holds +-0. A wave that meets a gate outside the table (2 in the
+// flags) redoes its item with the full table in device memory; one that meets a NaN redoes it with the canonical NaN.
+#define SWS_WAVES 4
+#define SWS_TAB (2 * (SWS_SPAN + 1))                                       // entries: positive gates, then negative ones
+__device__ __attribute__((aligned(16))) uint16_t g_silu_small[SWS_TAB];
+
+__global__ void __launch_bounds__(256) silu_small_fill() {             // after silu_lut_fill, on the same stream
+    const uint32_t e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= SWS_TAB) return;
+    const uint32_t sign = e >> 12, i = e & SWS_SPAN;
+    g_silu_small[e] = i == SWS_SPAN ? (uint16_t)(sign << 15) : g_silu_lut[(sign << 15) | (SWS_A0 + i)];
+}
+
+#define SWS_IPW 2                                                          // items (token groups) per wave, loaded together
+template <int LAYOUT, int SRC>
+__global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void * __restrict__ gu, const int32_t * __restrict__ ids, long ld, long F,
+                                                                    uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    const int lraw = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : 0) + wave * (SWM_TOK * 144);
+    if (SRC == SRC_SWIGLU_BF16) {
+#pragma unroll
+        for (int j = wave; j < 2 * SWS_TAB / 1024; j += SWS_WAVES)        // the table, 1 KiB per wave instruction
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g_silu_small + 512 * j + 8 * lraw),
+                                             (__attribute__((address_space(3))) void *)(lut + 512 * j), 16, 0, 0);
+    }
+    const long tg0 = ((long)blockIdx.x * SWS_WAVES + wave) * (SWM_TOK * SWS_IPW), unit = blockIdx.y;
+    SwmItem it[SWS_IPW];
+#pragma unroll
+    for (int k = 0; k < SWS_IPW; k++) swm_load<SRC>(it[k], gu, ids, ld, F, T, tg0 + SWM_TOK * k, unit, lraw, tg0 + SWM_TOK * k < T);
+    if (SRC == SRC_SWIGLU_BF16) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);                               // vmcnt(0): this wave's part of the table has landed (and its items)
+        __syncthreads();
+    }
+#pragma unroll
+    for (int k = 0; k < SWS_IPW; k++) {
+        const long tg = tg0 + SWM_TOK * k;
+        if (tg >= T) return;
+        int fl = swm_compute<LAYOUT, SRC, false, SRC == SRC_SWIGLU_BF16 ? LUT_SMALL : LUT_FULL>(it[k], lut, stage, F, act, T, tg, unit, lraw);
+        if (SRC == SRC_SWIGLU_BF16) {
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(fl & 2) != 0, 0))
+                fl = swm_compute<LAYOUT, SRC, false, LUT_FULL>(it[k], g_silu_lut, stage, F, act, T, tg, unit, lraw);
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(fl & 1) != 0, 0))
+                swm_compute<LAYOUT, SRC, true, LUT_FULL>(it[k], g_silu_lut, stage, F, act, T, tg, unit, lraw);
+        }
+        const int nunits = (int)min((long)SWM_TOK, T - tg) * 9;           // tokens of the group that exist
+        uint8_t * dst = y + ((size_t)unit * T + (size_t)tg) * 144;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // the wave's own LDS writes, in order
+        if (lraw < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 16 * lraw), (u32x4 *)(dst + 16 * lraw));
+        if (lraw < 8 && 64 + lraw < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 1024 + 16 * lraw), (u32x4 *)(dst + 1024 + 16 * lraw));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
+    }
+}
+template <int SRC>
+static void launch_oneshot(const void * src, const int32_t * ids, long ld, long F, void * vy, uint16_t * act, int T, long ncol, int layout, hipStream_t st) {
+    const int per = SWS_WAVES * SWM_TOK * SWS_IPW;
+    const dim3 grid((unsigned)((T + per - 1) / per), (unsigned)ncol), block(SWS_WAVES * 64);
+    const size_t lds = (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : 0) + SWS_WAVES * SWM_TOK * 144;
+    if (layout == MMQ_DS4) swiglu_mmq_oneshot<MMQ_DS4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T);
+    else swiglu_mmq_oneshot<MMQ_D4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T);
 }
 
 // act = bf16(bf16(silu g) * u) of wide bf16 rows [g (H) | u (H)] with the same table: persistent workgroups, a lane takes 8
@@ -408,6 +495,7 @@ static int silu_lut_ready(hipStream_t st, int * ncu, const uint16_t ** lut = nul
         int n = 0;
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return CAMX_EINVAL;
         silu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
+        silu_small_fill<<<dim3((SWS_TAB + 255) / 256), dim3(256), 0, st>>>();
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
         if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
@@ -471,6 +559,10 @@ int camx_quantize_mmq_q8_1(const float * x, const int32_t * ids, void * vy, long
         int dev = 0, ncu = 256;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return CAMX_EINVAL;
         const long ncol = ne0 / 128, nitems = (long)((ne1 + SWM_TOK - 1) / SWM_TOK) * ncol;
+        if (ne1 >= 2048 && ncol <= 65535) {                                   // a prefill chunk: the one-shot form (no table for fp32 rows)
+            launch_oneshot<SRC_F32>(x, ids, s01, ne00, vy, nullptr, ne1, ncol, layout, st);
+            CAMX_LAUNCH_RET();
+        }
         const long nwg = (nitems + 15) / 16;                                  // a small batch does not start workgroups that would only copy the table
         const dim3 grid((unsigned)(nwg < ncu ? nwg : ncu)), block(1024);
         if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_F32><<<grid, block, SWM_STAGE, st>>>(x, ids, s01, ne00, (uint8_t *)vy, nullptr, ne1, (unsigned)ncol, (unsigned)nitems);
@@ -508,6 +600,10 @@ int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16
         const long ncol = Kp / 128, nitems = (long)((T + SWM_TOK - 1) / SWM_TOK) * ncol;
         const long nwg = (nitems + 15) / 16;                                  // a small batch does not start workgroups that would only copy the table
         const dim3 grid((unsigned)(nwg < ncu ? nwg : ncu)), block(1024);
+        if (T >= 2048 && ncol <= 65535) {                                     // a prefill chunk: the one-shot form
+            launch_oneshot<SRC_SWIGLU_BF16>(gu, nullptr, ld, F, vy, act, T, ncol, layout, st);
+            CAMX_LAUNCH_RET();
+        }
         if (layout == MMQ_DS4) swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol, (unsigned)nitems);
         else swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16><<<grid, block, SWM_LDS, st>>>(gu, nullptr, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol, (unsigned)nitems);
         CAMX_LAUNCH_RET();
