@@ -234,15 +234,17 @@ def extra_opsets(B):
     return out
 
 
-def prefill_scale_sweep(B):
-    """every entry point at a prefill-scale size (bench.py --only sweep): name -> {us, bytes, GBps, frac_of_8TBps}. Each is launched
-    30 times back to back over three copies of its buffers in rotation (a launch never finds its own lines in the Infinity Cache);
-    bytes are algorithmic (inputs read once, outputs written once)."""
+def prefill_scale_sweep(B, T=4096):
+    """every entry point at a prefill-scale size (bench.py --only sweep [--sweep-tokens T]): name -> {us, bytes, GBps, frac_of_8TBps}. Each
+    is launched 30 times back to back over enough copies of its buffers, in rotation, that the rotation's footprint is at least 1.2 GB
+    (no launch finds its own lines in the 256 MB Infinity Cache); bytes are algorithmic (inputs read once, outputs written once)."""
     import numpy as np
     torch = B.torch; dev = B.dev
     res = {}
 
-    def timeit(name, by, fns, reps=30):
+    def timeit(name, by, mk, reps=30):
+        ncopy = max(3, min(16, -(-1_200_000_000 // int(by))))
+        fns = [mk(i) for i in range(ncopy)]
         for f in fns: f()
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -250,135 +252,215 @@ def prefill_scale_sweep(B):
         for k in range(reps): fns[k % len(fns)]()
         b.record(); b.synchronize()
         us = a.elapsed_time(b) * 1e3 / reps
-        res[name] = {'us': round(us, 2), 'bytes': int(by), 'GBps': round(by / us / 1e3, 1), 'frac_of_8TBps': round(by / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        res[name] = {'us': round(us, 2), 'bytes': int(by), 'copies': ncopy, 'GBps': round(by / us / 1e3, 1), 'frac_of_8TBps': round(by / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        del fns
+        torch.cuda.empty_cache()
 
-    def sets(mk): return [mk(i) for i in range(3)]
-    T = 4096
     N = 2048
     def mk(i):
         x = B.acts((T, N), torch.float32, i); d = B.acts((T, 1, N), torch.float32, i + 10); nw = B.gamma(N, 3); h = torch.empty((T, N), device=dev); h16 = torch.empty((T, N), dtype=torch.float16, device=dev)
         return lambda: B.call('camx_q3p_add_rms16', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), _p(h), _p(h16), I(N), I(T))
-    timeit('q3p_add_rms16 4096x2048 S=1', T * N * (4 + 4 + 4 + 4 + 2), sets(mk))
+    timeit(f'q3p_add_rms16 {T}x2048 S=1', T * N * (4 + 4 + 4 + 4 + 2), mk)
     def mk(i):
         x = B.acts((T, N), torch.float32, i); d = B.acts((T, 8, N), torch.float32, i + 10); w = torch.rand((T, 8), device=dev); nw = B.gamma(N, 3); h16 = torch.empty((T, N), dtype=torch.float16, device=dev)
         return lambda: B.call('camx_q3p_add_rms16', _p(x), _p(d), _p(w), I(8), _p(nw), F(1e-6), NULL, _p(h16), I(N), I(T))
-    timeit('q3p_add_rms16 4096x2048 S=8 weighted', T * N * (4 + 32 + 4 + 2), sets(mk))
+    timeit(f'q3p_add_rms16 {T}x2048 S=8 weighted', T * N * (4 + 32 + 4 + 2), mk)
     def mk(i):
         x = B.acts((T, N), torch.float32, i); d = B.acts((T, 1, N), torch.float32, i + 10); nw = B.gamma(N, 3); q8 = torch.empty(T * N // 32 * 36, dtype=torch.uint8, device=dev)
         return lambda: B.call('camx_add_rms_q8_1', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), NULL, NULL, _p(q8), I(N), I(T))
-    timeit('add_rms_q8_1 4096x2048', T * N * (4 + 4 + 4 + 1.125), sets(mk))
+    timeit(f'add_rms_q8_1 {T}x2048', T * N * (4 + 4 + 4 + 1.125), mk)
     H = 5120
     def mk(i):
         x = B.acts((T, H), torch.float32, i); d = B.acts((T, H), torch.float32, i + 10); nw = B.gamma(H, 3); h = torch.empty((T, H), device=dev); h16 = torch.empty((T, H), dtype=torch.float16, device=dev)
         return lambda: B.call('camx_q35p_add_rms16', _p(x), _p(d), _p(nw), F(1e-6), _p(h), _p(h16), I(H), I(T))
-    timeit('q35p_add_rms16 4096x5120', T * H * (4 + 4 + 4 + 4 + 2), sets(mk))
+    timeit(f'q35p_add_rms16 {T}x5120', T * H * (4 + 4 + 4 + 4 + 2), mk)
     def mk(i):
         x = B.acts((2048 * 4, 2560), torch.float32, i); w = B.gamma(4 * 2560, 3); ybf = torch.empty((8192, 2560), dtype=torch.bfloat16, device=dev); scl = torch.empty(8192, device=dev)
         return lambda: B.call('camx_pf_rms_mul', _p(x), _p(w), NULL, _p(ybf), _p(scl), I(8192), I(4), F(1e-6), I(2560))
-    timeit('pf_rms_mul 8192x2560 -> bf16', 8192 * 2560 * 6, sets(mk))
+    timeit('pf_rms_mul 8192x2560 -> bf16', 8192 * 2560 * 6, mk)
     n = T * 8 * 768
     def mk(i):
         g = B.acts((n,), torch.float32, i); u = B.acts((n,), torch.float32, i + 5); y = torch.empty(n, dtype=torch.float16, device=dev)
         return lambda: B.call('camx_q3p_swiglu', _p(g), _p(u), _p(y), I(n))
-    timeit('q3p_swiglu 4096x6144', n * 10, sets(mk))
+    timeit(f'q3p_swiglu {T}x6144', n * 10, mk)
     def mk(i):
         gu = B.acts((T, 2 * 17408), torch.bfloat16, i); act = torch.empty((T, 17408), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_silu_mul_bf16', _p(gu), _p(act), I(17408), L64(T * 17408))
-    timeit('silu_mul_bf16 4096x17408', T * 17408 * 6, sets(mk))
+    timeit(f'silu_mul_bf16 {T}x17408', T * 17408 * 6, mk)
     def mk(i):
         x = B.acts((n,), torch.float32, i); y = torch.empty(n // 32 * 36, dtype=torch.uint8, device=dev)
         return lambda: B.call('camx_gg_quantize_q8_1', _p(x), _p(y), L64(n), I(0), F(0), NULL)
-    timeit('gg_quantize_q8_1 25M', n * 5.125, sets(mk))
+    timeit(f'gg_quantize_q8_1 {T}x6144', n * 5.125, mk)
     K = 6144
     def mk(i):
         x = B.acts((T, K), torch.float32, i); y = torch.empty(K // 128 * T * 144, dtype=torch.uint8, device=dev)
         return lambda: B.call('camx_quantize_mmq_q8_1', _p(x), NULL, _p(y), L64(K), L64(K), L64(0), L64(0), L64(K), I(T), I(1), I(0), I(1))
-    timeit('quantize_mmq_q8_1 4096x6144 DS4', T * K * 5.125, sets(mk))
+    timeit(f'quantize_mmq_q8_1 {T}x6144 DS4', T * K * 5.125, mk)
     nh, nkv = 32, 4; ldq = (nh + 2 * nkv) * 128
     par, _ = yarn_par(torch, dev, 15, yarn=False)
     def mk(i):
         qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev); cache = torch.empty((T, 2 * nkv * 128), dtype=torch.float16, device=dev)
         return lambda: B.call('camx_q3p_qk_rope', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(0), _p(q16), _p(cache), I(T), I(0))
-    timeit('q3p_qk_rope 4096 tok f32 -> f16', T * ldq * 6, sets(mk))
+    timeit(f'q3p_qk_rope {T} tok f32 -> f16', T * ldq * 6, mk)
     rbq = 2 * (nkv * 128 // 32) * 34
     def mk(i):
         qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev); cache = torch.empty(T * rbq, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
         return lambda: B.call('camx_q3p_qk_rope_q8', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(0), _p(q16), _p(cache), _p(err), I(T), I(0))
-    timeit('q3p_qk_rope_q8 4096 tok', T * (ldq * 4 + nh * 256 + rbq), sets(mk))
+    timeit(f'q3p_qk_rope_q8 {T} tok', T * (ldq * 4 + nh * 256 + rbq), mk)
     D = 256
     def mk(i):
         qg = B.acts((T * 24, 2 * D), torch.bfloat16, i); w4 = B.gamma(D, 2); o = torch.empty((T * 24, D), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_pf_qk_nr', _p(qg), I(2 * D), I(24), _p(w4), I(D), I(64), F(0.6), F(1e-6), I(0), _p(o), I(T), I(1))
-    timeit('pf_qk_nr 4096x24x256 bf16', T * 24 * D * 4, sets(mk))
+    timeit(f'pf_qk_nr {T}x24x256 bf16', T * 24 * D * 4, mk)
     def mk(i):
         a = B.acts((T * 24, D), torch.bfloat16, i); qg = B.acts((T * 24, 2 * D), torch.bfloat16, i + 3); o = torch.empty((T * 24, D), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_gate_mul', _p(a), _p(qg), _p(o), L64(T * 24 * D), I(D), I(2 * D), I(D), I(2))
-    timeit('gate_mul 4096x24x256 bf16', T * 24 * D * 6, sets(mk))
+    timeit(f'gate_mul {T}x24x256 bf16', T * 24 * D * 6, mk)
     Cc = 10240
     def mk(i):
         xc = B.acts((T, Cc), torch.bfloat16, i); wc = B.acts((Cc, 4), torch.float32, 45, frac=0); st = B.acts((Cc, 3), torch.float32, 46, frac=0); yc = torch.empty((T, Cc), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_pf_gdn_conv', _p(xc), _p(wc), _p(st), _p(yc), I(Cc), I(T), I(Cc), I(Cc), I(1))
-    timeit('pf_gdn_conv 4096x10240 bf16', T * Cc * 4, sets(mk))
+    timeit(f'pf_gdn_conv {T}x10240 bf16', T * Cc * 4, mk)
     def mk(i):
         xc = B.acts((T, Cc), torch.bfloat16, i); o = torch.empty((T * 32, 128), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_pf_gdn_l2', _p(xc), _p(o), I(32), I(128), I(Cc), F(1e-6 / 128), I(T), I(1))
-    timeit('pf_gdn_l2 4096x32x128 bf16', T * 32 * 128 * 4, sets(mk))
+    timeit(f'pf_gdn_l2 {T}x32x128 bf16', T * 32 * 128 * 4, mk)
     M = 512
     def mk(i):
         k = B.acts((T, M), torch.float32, i); v = B.acts((T, M), torch.float32, i + 2); cache = torch.empty(T * 1088, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
         return lambda: B.call('camx_own_kv_q8_append', _p(k), I(M), _p(v), I(M), I(M), _p(cache), I(0), I(T), _p(err), I(T))
-    timeit('own_kv_q8_append 4096x512', T * (M * 8 + 1088), sets(mk))
+    timeit(f'own_kv_q8_append {T}x512', T * (M * 8 + 1088), mk)
     def mk(i):
         x = B.acts((T * 36, 128), torch.float32, i); y = torch.empty_like(x)
         return lambda: B.call('camx_hadamard128', _p(x), _p(y), L64(T * 36))
-    timeit('hadamard128 147456 heads', T * 36 * 128 * 8, sets(mk))
+    timeit(f'hadamard128 {T}x36 heads', T * 36 * 128 * 8, mk)
     V = 151936
     tab = torch.randint(0, 256, (V, 1152), device=dev, dtype=torch.uint8)
     tab.view(V, 8, 144)[:, :, :4] = (torch.rand((V, 8, 2), device=dev) * 9e-3 + 1e-3).to(torch.float16).view(torch.uint8).view(V, 8, 4)
     def mk(i):
         toks = torch.randint(0, V, (T,), device=dev, dtype=torch.int32); x = torch.empty((T, N), device=dev)
         return lambda: B.call('camx_q3p_emb', _p(tab), I(1152), I(V), _p(toks), _p(x), I(N), I(T))
-    timeit('q3p_emb 4096 rows Q4_K -> f32', T * (1152 + N * 4), sets(mk))
+    timeit(f'q3p_emb {T} rows Q4_K -> f32', T * (1152 + N * 4), mk)
     Kq = 2048; Mr = 8192
     def mk(i):
         x = B.acts((Mr, Kq), torch.bfloat16, i); y = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev); s = torch.empty(Mr, device=dev)
         return lambda: B.call('camx_actq_fwd', _p(x), I(1), _p(y), _p(s), NULL, I(Kq), F(1.0), I(7), I(Mr))
-    timeit('actq_fwd bf16 8192x2048', Mr * Kq * 4, sets(mk))
+    timeit('actq_fwd bf16 8192x2048', Mr * Kq * 4, mk)
     def mk(i):
         x = B.acts((Mr, Kq), torch.bfloat16, i); g = B.acts((Mr, Kq), torch.bfloat16, i + 1); dx = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_actq_bwd', _p(x), I(1), _p(g), _p(dx), I(Kq), F(1.0), I(7), I(Mr))
-    timeit('actq_bwd bf16 8192x2048', Mr * Kq * 6, sets(mk))
+    timeit('actq_bwd bf16 8192x2048', Mr * Kq * 6, mk)
     def mk(i):
         gu = B.acts((Mr, 2 * Kq), torch.bfloat16, i); y = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev); s = torch.empty(Mr, device=dev); c = torch.empty((Mr, Kq // 2), dtype=torch.uint8, device=dev)
         return lambda: B.call('camx_silu_mul_actq_fwd', _p(gu), I(2 * Kq), I(Kq), _p(y), _p(s), _p(c), F(1.0), I(7), I(Mr))
-    timeit('silu_mul_actq_fwd 8192x2048', Mr * Kq * 6.5, sets(mk))
+    timeit('silu_mul_actq_fwd 8192x2048', Mr * Kq * 6.5, mk)
     def mk(i):
         gu = B.acts((Mr, 2 * Kq), torch.bfloat16, i); g = B.acts((Mr, Kq), torch.bfloat16, i + 1); d = torch.empty((Mr, 2 * Kq), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_silu_mul_actq_bwd', _p(gu), I(2 * Kq), I(Kq), _p(g), _p(d), F(1.0), I(7), I(Mr))
-    timeit('silu_mul_actq_bwd 8192x2048', Mr * Kq * 10, sets(mk))
+    timeit('silu_mul_actq_bwd 8192x2048', Mr * Kq * 10, mk)
     def mk(i):
         x = B.acts((Mr * Kq,), torch.float32, i); m = B.acts((Mr * Kq,), torch.bfloat16, i + 1); y = B.acts((Mr * Kq,), torch.bfloat16, i + 2); o = torch.empty(Mr * Kq, device=dev)
         return lambda: B.call('camx_residual3', _p(x), _p(m), _p(y), _p(o), L64(Mr * Kq))
-    timeit('residual3 16M', Mr * Kq * 12, sets(mk))
+    timeit('residual3 16M', Mr * Kq * 12, mk)
     rows_g, Kg = T * 48, 128
     def mk(i):
         o = B.acts((rows_g, Kg), torch.float32, i); z = B.acts((rows_g, Kg), torch.float32, i + 1, frac=0); wg = B.gamma(Kg, 5); y16 = torch.empty((rows_g, Kg), dtype=torch.float16, device=dev)
         return lambda: B.call('camx_q35p_gdn_norm16', _p(o), _p(wg), _p(z), _p(y16), I(Kg), F(1e-6), C.c_long(rows_g))
-    timeit('q35p_gdn_norm16 4096x48x128', rows_g * Kg * 10, sets(mk))
+    timeit(f'q35p_gdn_norm16 {T}x48x128', rows_g * Kg * 10, mk)
     Dh = 2560
     def mk(i):
         r = B.acts((2048, 4, Dh), torch.float32, i); y = torch.empty((2048, Dh), device=dev)
         return lambda: B.call('camx_pf_hc_avg', _p(r), _p(y), I(2048), I(4), I(Dh), I(Dh))
-    timeit('pf_hc_avg 2048x4x2560', 2048 * Dh * 20, sets(mk))
+    timeit('pf_hc_avg 2048x4x2560', 2048 * Dh * 20, mk)
     def mk(i):
         a = B.acts((Mr * Kq,), torch.float32, i); b = B.acts((Mr * Kq,), torch.float32, i + 1); y = B.acts((Mr * Kq,), torch.float32, i + 2)
         return lambda: B.call('camx_pf_add_sum', _p(a), _p(b), _p(y), L64(Mr * Kq))
-    timeit('pf_add_sum 16M', Mr * Kq * 16, sets(mk))
+    timeit('pf_add_sum 16M', Mr * Kq * 16, mk)
     def mk(i):
         x = B.acts((4096, 5120), torch.float32, i); y = torch.empty((4096, 5120), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_pf_to_bf16', _p(x), I(5120), _p(y), I(4096), I(4096), I(5120))
-    timeit('pf_to_bf16 4096x5120', 4096 * 5120 * 6, sets(mk))
+    timeit('pf_to_bf16 4096x5120', 4096 * 5120 * 6, mk)
+    def mk(i):
+        cache = torch.randint(0, 256, (T * 1088,), device=dev, dtype=torch.uint8)
+        cache.view(T * 32, 34)[:, :2] = (torch.rand((T * 32, 1), device=dev) * 9e-3 + 1e-3).to(torch.float16).view(torch.uint8).view(T * 32, 2)
+        k = torch.empty((T, M), dtype=torch.float16, device=dev); v = torch.empty((T, M), dtype=torch.float16, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_own_kv_q8_read', _p(cache), NULL, I(0), I(T), I(M), _p(k), I(M), _p(v), I(M), _p(err), I(T), I(1))
+    timeit(f'own_kv_q8_read {T}x512 -> f16', T * (1088 + M * 4), mk)
+    page, n_pages = 256, max(64, T // 64)
+    def mk(i):
+        qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev)
+        cache = torch.empty(n_pages * page * rbq, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        perm = torch.randperm(n_pages * page, device=dev)[:T].to(torch.int32)            # every sequence at its own row: page = row / 256 through a one-column table
+        pos = (perm % page).contiguous(); pt = (perm // page).reshape(T, 1).contiguous()
+        return lambda: B.call('camx_qk_rope_paged', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), _p(pos), _p(q16), _p(cache), _p(err), _p(pt), I(1), I(page), I(n_pages), I(T), I(0), I(1))
+    timeit(f'qk_rope_paged {T} seq Q8', T * (ldq * 4 + 8 + nh * 256 + rbq), mk)
+    Th, HC, Nh = max(T // 2, 64), 4, 2560
+    def mk(i):
+        bh = B.acts((Th, Nh), torch.float32, i); injh = B.acts((Th, HC), torch.float32, i + 1, frac=0); resh = B.acts((Th, HC, Nh), torch.float32, i + 2)
+        wh = B.gamma(HC * Nh, 64); xnbf = torch.empty((Th, HC, Nh), dtype=torch.bfloat16, device=dev); sclh = torch.empty(Th * HC, device=dev)
+        return lambda: B.call('camx_pf_hc_post_rms', _p(bh), _p(injh), _p(resh), _p(wh), NULL, _p(xnbf), _p(sclh), I(Th), I(HC), F(0.25), F(1e-6), I(Nh))
+    timeit(f'pf_hc_post_rms {Th}x4x2560 -> bf16 + scale', Th * Nh * 4 + Th * HC * Nh * 10 + HC * Nh * 4 + Th * HC * 8, mk)
     return res
+
+
+def batch_ladder(B):
+    """the op-sets of the configs from a verify batch to a prefill chunk (bench.py --only ladder): us per launch and GB/s at 16 .. 4096
+    tokens, 30 launches back to back over copies in rotation (footprint >= 1.2 GB or 16 copies: the small batches stay cache-resident, as
+    they are in a decode loop). The launchers switch kernels with the batch size; this shows the switches as a curve."""
+    torch = B.torch; dev = B.dev
+    out = {}
+    nh, nkv = 32, 4; ldq = (nh + 2 * nkv) * 128; rbq = 2 * (nkv * 128 // 32) * 34; N = 2048
+    par, _ = yarn_par(torch, dev, 15, yarn=False)
+    parb, _ = yarn_par(torch, dev, 16)
+    nw = B.gamma(N, 3); nw5 = B.gamma(5120, 4)
+    V = 151936
+    tab = torch.randint(0, 256, (V, 1152), device=dev, dtype=torch.uint8)
+    tab.view(V, 8, 144)[:, :, :4] = (torch.rand((V, 8, 2), device=dev) * 9e-3 + 1e-3).to(torch.float16).view(torch.uint8).view(V, 8, 4)
+
+    def ops(T):
+        def add_rms16(i):
+            x = B.acts((T, N), torch.float32, i); d = B.acts((T, 1, N), torch.float32, i + 10); h = torch.empty((T, N), device=dev); h16 = torch.empty((T, N), dtype=torch.float16, device=dev)
+            return lambda: B.call('camx_q3p_add_rms16', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), _p(h), _p(h16), I(N), I(T))
+        def add_rms_q8(i):
+            x = B.acts((T, N), torch.float32, i); d = B.acts((T, 1, N), torch.float32, i + 10); q8 = torch.empty(T * N // 32 * 36, dtype=torch.uint8, device=dev)
+            return lambda: B.call('camx_add_rms_q8_1', _p(x), _p(d), NULL, I(1), _p(nw), F(1e-6), NULL, NULL, _p(q8), I(N), I(T))
+        def gather_norm(i):
+            toks = torch.randint(0, V, (T,), device=dev, dtype=torch.int32); x = torch.empty((T, N), device=dev); qq = torch.empty(T * (N // 32) * 36, dtype=torch.uint8, device=dev)
+            return lambda: B.call('camx_emb_gather_add_rms', _p(tab), L64(1152), I(V), _p(toks), _p(x), NULL, NULL, _p(nw), F(1e-6), NULL, NULL, _p(qq), I(N), I(T), I(0))
+        def rope_f32(i):
+            qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev); cache = torch.empty((T, 2 * nkv * 128), dtype=torch.float16, device=dev)
+            return lambda: B.call('camx_q3p_qk_rope', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(0), _p(q16), _p(cache), I(T), I(0))
+        def rope_q8(i):
+            qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev); cache = torch.empty(T * rbq, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+            return lambda: B.call('camx_q3p_qk_rope_q8', _p(qkv), I(ldq), I(nh), I(nkv), _p(par), I(0), _p(q16), _p(cache), _p(err), I(T), I(0))
+        def add_rms_bf16(i):
+            x = B.acts((T, 5120), torch.float32, i); d = B.acts((T, 5120), torch.bfloat16, i + 1); hb = torch.empty((T, 5120), dtype=torch.bfloat16, device=dev)
+            return lambda: B.call('camx_add_rms_bf16', _p(x), _p(d), _p(nw5), F(1e-6), NULL, _p(hb), I(5120), I(T))
+        def rope_bf16(i):
+            l = 80 * 128; qkv = B.acts((T, l), torch.bfloat16, i); q16 = torch.empty((T, 64, 128), dtype=torch.float16, device=dev); cache = torch.empty((T, 2048), dtype=torch.float16, device=dev)
+            return lambda: B.call('camx_qk_rope_bf16', _p(qkv), I(l), I(64), I(8), _p(parb), I(0), _p(q16), _p(cache), I(T), I(1))
+        def swiglu_mmq(i):
+            Fh = 17408; gu = B.acts((T, 2 * Fh), torch.bfloat16, i); y = torch.empty((Fh // 128, T, 144), dtype=torch.uint8, device=dev)
+            return lambda: B.call('camx_swiglu_mmq_q8_1', _p(gu), L64(2 * Fh), L64(Fh), _p(y), NULL, I(T), I(1))
+        return {'q3p_add_rms16 x2048': (T * N * 18, add_rms16), 'add_rms_q8_1 x2048': (T * N * 13.125, add_rms_q8), 'gather Q4_K + norm + q8_1': (T * (1152 + N * 5.125), gather_norm),
+                'q3p_qk_rope f32 40 heads': (T * ldq * 6, rope_f32), 'q3p_qk_rope_q8 40 heads': (T * (ldq * 4 + nh * 256 + rbq), rope_q8),
+                'add_rms_bf16 x5120': (T * 5120 * 12, add_rms_bf16), 'qk_rope_bf16 80 heads': (T * 80 * 128 * 4, rope_bf16), 'swiglu_mmq_q8_1 x17408': (T * 17408 * 5.125, swiglu_mmq)}
+
+    for T in (16, 64, 256, 512, 1024, 2048, 4096):
+        for name, (by, mk) in ops(T).items():
+            ncopy = max(3, min(16, -(-1_200_000_000 // int(by))))
+            fns = [mk(i) for i in range(ncopy)]
+            for f in fns: f()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for k in range(30): fns[k % ncopy]()
+            b.record(); b.synchronize()
+            us = a.elapsed_time(b) * 1e3 / 30
+            out.setdefault(name, {})[str(T)] = {'us': round(us, 2), 'GBps': round(by / us / 1e3, 1)}
+            del fns
+        torch.cuda.empty_cache()
+    return out
 
 
 def cpu_baseline(w, budget_s=15.0):
@@ -436,6 +518,7 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--copies', type=int, default=8, help='copies of the batch taken in rotation (8: no launch finds its lines in the Infinity Cache)')
+    ap.add_argument('--sweep-tokens', type=int, default=4096, help='rows of the --only sweep shapes')
     ap.add_argument('--no-cpu', action='store_true')
     ap.add_argument('--no-extra', action='store_true')
     ap.add_argument('--only', default=None, help='run a single kernel of the step (for profiling)')
@@ -448,7 +531,10 @@ def main():
     torch = B.torch
     if a.only == 'sweep':
         print(json.dumps({'metric': 'fused-op HBM GB/s per entry point at prefill-scale sizes, 1 GPU', 'unit': 'GB/s', 'n_gpus': 1, 'data': 'synthetic',
-                          'peak_GBps': HBM_PEAK_GBPS, 'sweep': prefill_scale_sweep(B)}))
+                          'peak_GBps': HBM_PEAK_GBPS, 'tokens': a.sweep_tokens, 'sweep': prefill_scale_sweep(B, a.sweep_tokens)}))
+        return
+    if a.only == 'ladder':
+        print(json.dumps({'metric': 'us per launch and GB/s of the configs\' op-sets from 16 to 4096 tokens, 1 GPU', 'n_gpus': 1, 'data': 'synthetic', 'ladder': batch_ladder(B)}))
         return
     if a.only == 'copy_ref':
         # a plain device copy of known size (256 MiB read + 256 MiB written per launch): the yardstick that FETCH_SIZE / WRITE_SIZE
