@@ -28,24 +28,44 @@ struct NormArgs {
     float * scl;             // optional row scale [rows]
     int N, rows;
     const float * inj; int HC; float rs;   // ADD_HC only
+    int row0;                // set by the launcher: first row of this launch (a batch may be split into a bulk launch and a tail)
     int stream;              // set by the launcher for large batches: h / h16 leave as non-temporal stores (the consumer of a decode-sized batch finds them in cache instead)
 };
 
 // EXACT: the row has exactly NI_MAX slabs, so every loop below is straight-line code: no scalar branch stands between the
 // loads, which the backend then issues as one batch (with a run-time slab count each `j < ni` is a branch that loads do
 // not cross, and a 4096 x 5120 launch loses 17 % to it).
-template <int NI_MAX, int ADD, bool EXACT>
+// OUT != 0 is the chunk form for batches that stream from HBM: the set of copies is fixed at compile time (NORM_* bits, so
+// no branch stands in the store loop either), every access is non-temporal, the requests of a row leave a short pause apart,
+// and gamma waits in LDS instead of registers: GL == 1 one copy per workgroup (one gamma row for all), GL == 2 one row per
+// wave (row r uses gamma row r % wr). The launcher gives these forms whole workgroups only.
+enum { NORM_H = 1, NORM_H16 = 2, NORM_HBF = 4, NORM_Q8 = 8, NORM_SCL = 16 };
+#define CAMX_ISSUE_GAP() do { if (OUT) { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_sleep(1); __builtin_amdgcn_sched_barrier(0); } } while (0)
+template <int NI_MAX, int ADD, bool EXACT, int OUT = 0, int GL = 0>
 __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
-    const int lane = slot_of(threadIdx.x & 63);
-    const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (row >= a.rows) return;
+    static_assert(OUT == 0 ? GL == 0 : EXACT, "the chunk form is straight-line code");
+    extern __shared__ __attribute__((aligned(16))) float gsh[];
+    const int lraw = threadIdx.x & 63, lane = slot_of(lraw), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int row = a.row0 + blockIdx.x * 4 + wave;
+    if (!OUT && row >= a.rows) return;
     const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
-    float * xr = a.x + (size_t)row * N;
-    f32x4 xv[NI_MAX];
-    if (a.stream) {        // a batch too large to be cache resident: its rows come from HBM once, past the caches
+    if (GL == 1) {
+#pragma unroll
+        for (int j = wave; j < NI_MAX; j += 4)      // gamma piece j (1 KiB) -> LDS in lane order; read back in slot order below
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(a.nw + 256 * j + 4 * lraw), (__attribute__((address_space(3))) void *)(gsh + 256 * j), 16, 0, 0);
+    }
+    if (GL == 2) {
+        const float * gw2 = a.nw + (size_t)(row % a.wr) * N;
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) xv[j] = __builtin_nontemporal_load((const f32x4 *)(xr + 256 * j + 4 * lane));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gw2 + 256 * j + 4 * lraw), (__attribute__((address_space(3))) void *)(gsh + wave * N + 256 * j), 16, 0, 0);
+    }
+    float * xr = a.x + (size_t)row * N;
+    f32x4 xv[NI_MAX];
+    if (OUT || a.stream) {        // a batch too large to be cache resident: its rows come from HBM once, past the caches
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) { xv[j] = __builtin_nontemporal_load((const f32x4 *)(xr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
     } else {
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
@@ -67,7 +87,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
             f32x4 dv[NI_MAX];
 #pragma unroll
             for (int j = 0; j < NI_MAX; j++)
-                if (j < ni) dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane));
+                if (j < ni) { dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + (size_t)s * N + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
 #pragma unroll
             for (int j = 0; j < NI_MAX; j++)
                 if (j < ni) {
@@ -86,7 +106,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         f32x4 dv[NI_MAX];
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + 256 * j + 4 * lane));
+            if (j < ni) { dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) xv[j] = xv[j] + dv[j];
@@ -96,7 +116,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         u32x2 dv[NI_MAX];
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) dv[j] = __builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane));
+            if (j < ni) { dv[j] = __builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) xv[j] = xv[j] + unpack_bf16x4(dv[j]);
@@ -106,7 +126,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         f32x4 dv[NI_MAX];
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) dv[j] = *(const f32x4 *)(dr + 256 * j + 4 * lane);       // (plain: the HC rows of a token share it)
+            if (j < ni) { dv[j] = *(const f32x4 *)(dr + 256 * j + 4 * lane); CAMX_ISSUE_GAP(); }       // (plain: the HC rows of a token share it)
         const float v = a.inj[row] * a.rs;
         const float sgm = 1.0f / (1.0f + expf(-v));
         const float p = sgm * 2.0f;
@@ -117,10 +137,12 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
                 xv[j].z = __builtin_fmaf(dv[j].z, p, xv[j].z); xv[j].w = __builtin_fmaf(dv[j].w, p, xv[j].w);
             }
     }
-    f32x4 g[NI_MAX];
+    f32x4 g[GL ? 1 : NI_MAX];
+    if (!GL) {
 #pragma unroll
-    for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+    }
     if (ADD == ADD_HC || (ADD == ADD_F32_SLOTS && a.S > 0) || ((ADD == ADD_F32_DIRECT || ADD == ADD_BF16) && a.d)) {
         // the updated residual goes back to the lines it was read from
 #pragma unroll
@@ -137,39 +159,57 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         }
     const float tot = wave_groups_in_order(group32_sum(ss));
     const float scale = rsqrt_exact(tot / (float)N + a.eps);
-    if (a.scl && lane == 0) a.scl[row] = scale;
+    if ((OUT ? (OUT & NORM_SCL) != 0 : a.scl != nullptr) && lane == 0) a.scl[row] = scale;
+    if (GL) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0): this wave's gamma pieces have landed in LDS (they were first in the queue)
+        if (GL == 1) __syncthreads();
+    }
+    const float * gl = gsh + (GL == 2 ? wave * N : 0);
     // (two copies of the loop, chosen once: with the choice inside it the stores of a long row were no longer issued back to back)
-    auto emit = [&](auto nt) {
-        constexpr bool NT = decltype(nt)::value;
+    auto emit = [&](auto nt, auto redo) {
+        constexpr bool NT = decltype(nt)::value, REDO = decltype(redo)::value;
+        bool nan = false;
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) {
+                const f32x4 gj = GL ? *(const f32x4 *)(gl + 256 * j + 4 * lane) : g[GL ? 0 : j];
                 f32x4 t, v;
                 t.x = xv[j].x * scale; t.y = xv[j].y * scale; t.z = xv[j].z * scale; t.w = xv[j].w * scale;
-                v.x = t.x * g[j].x; v.y = t.y * g[j].y; v.z = t.z * g[j].z; v.w = t.w * g[j].w;
+                v.x = t.x * gj.x; v.y = t.y * gj.y; v.z = t.z * gj.z; v.w = t.w * gj.w;
                 const size_t o = (size_t)row * N + 256 * j + 4 * lane;
-                if (a.h) { if (NT) __builtin_nontemporal_store(v, (f32x4 *)(a.h + o)); else *(f32x4 *)(a.h + o) = v; }
-                if (a.h16) {
+                if (REDO) { *(u32x2 *)(a.hbf + o) = pack_bf16x4_rne(v); continue; }
+                if (OUT ? (OUT & NORM_H) != 0 : a.h != nullptr) { if (NT) __builtin_nontemporal_store(v, (f32x4 *)(a.h + o)); else *(f32x4 *)(a.h + o) = v; }
+                if (OUT ? (OUT & NORM_H16) != 0 : a.h16 != nullptr) {
                     u32x2 * p16 = (u32x2 *)(a.h16 + (size_t)row * a.ld16 + 256 * j + 4 * lane);
                     // the dense line (q35p_add_rms16) stores fp16 of the last product rounded once, as the reference's binary does
                     // (kernels/q35_prefill.hip:630-635); the own line's statement is fp16 of the rounded fp32 value
-                    const u32x2 pk = ADD == ADD_F32_DIRECT ? (u32x2){mul_pack_f16x2_once(t.x, g[j].x, t.y, g[j].y), mul_pack_f16x2_once(t.z, g[j].z, t.w, g[j].w)}
+                    const u32x2 pk = ADD == ADD_F32_DIRECT ? (u32x2){mul_pack_f16x2_once(t.x, gj.x, t.y, gj.y), mul_pack_f16x2_once(t.z, gj.z, t.w, gj.w)}
                                                            : pack_f16x4(v);
                     if (NT) __builtin_nontemporal_store(pk, p16); else *p16 = pk;
                 }
-                if (a.hbf) __builtin_nontemporal_store(pack_bf16x4_rne(v), (u32x2 *)(a.hbf + o));
-                if (a.q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
+                if (OUT ? (OUT & NORM_HBF) != 0 : a.hbf != nullptr) {
+                    if (OUT) {     // the hardware convert, branch-free; a row that produced a NaN is redone below with the reference's integer rounding
+                        nan |= any_nan4(v);
+                        __builtin_nontemporal_store((u32x2){hw_pk_bf16(v.x, v.y), hw_pk_bf16(v.z, v.w)}, (u32x2 *)(a.hbf + o));
+                    } else __builtin_nontemporal_store(pack_bf16x4_rne(v), (u32x2 *)(a.hbf + o));
+                }
+                if (OUT ? (OUT & NORM_Q8) != 0 : a.q8 != nullptr) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
             }
+        return nan;
     };
-    if (a.stream) emit(std::true_type{}); else emit(std::false_type{});
+    if (OUT) {
+        const bool nan = emit(std::true_type{}, std::false_type{});
+        if ((OUT & NORM_HBF) && __builtin_expect(__builtin_amdgcn_ballot_w64(nan) != 0, 0)) emit(std::true_type{}, std::true_type{});
+    } else if (a.stream) emit(std::true_type{}, std::false_type{}); else emit(std::false_type{}, std::false_type{});
 }
+#undef CAMX_ISSUE_GAP
 
 // Any row length (N not a multiple of 256, or longer than the register forms hold): the same tree with scalar accesses,
 // x re-read for the second walk. One wave per row.
 template <int ADD>
 __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
     const int lane = slot_of(threadIdx.x & 63);
-    const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int row = a.row0 + blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (row >= a.rows) return;
     const int N = a.N;
     float * xr = a.x + (size_t)row * N;
@@ -224,16 +264,49 @@ __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
     }
 }
 
-template <int ADD>
+// The chunk form of add_rms_rows for one set of copies, if the launch fits it: returns the rows it took (whole workgroups).
+template <int ADD, int OUT>
+static int launch_norm_chunk(const NormArgs & a, hipStream_t st) {
+    const int rows = a.rows & ~3, ni = a.N >> 8, gl = a.wr == 1 ? 1 : 2;
+    if (gl == 2 && a.N > 2560) return 0;          // (a gamma row per wave: 4 N floats of LDS per workgroup)
+    const dim3 grid(rows / 4), block(256);
+    const size_t lds = (size_t)(gl == 1 ? 1 : 4) * a.N * sizeof(float);
+    NormArgs b = a; b.rows = rows;
+    switch (ni) {
+#define CAMX_NORM_CHUNK(NI) case NI: \
+        if (gl == 1) add_rms_rows<NI, ADD, true, OUT, 1><<<grid, block, lds, st>>>(b); \
+        else if constexpr (ADD == ADD_NONE || ADD == ADD_HC) { if constexpr (NI <= 10) add_rms_rows<NI, ADD, true, OUT, 2><<<grid, block, lds, st>>>(b); } \
+        else return 0; \
+        return rows;
+        CAMX_NORM_CHUNK(4) CAMX_NORM_CHUNK(8) CAMX_NORM_CHUNK(10) CAMX_NORM_CHUNK(16) CAMX_NORM_CHUNK(20)
+#undef CAMX_NORM_CHUNK
+    }
+    return 0;
+}
+
+// CHUNK_OUTS: the sets of copies (NORM_* masks) this entry point's prefill callers ask for; a batch that streams from HBM
+// with one of them runs the chunk form, anything else the general one.
+template <int ADD, int... CHUNK_OUTS>
 static int launch_norm(const NormArgs & a0, hipStream_t st) {
     if (a0.rows <= 0) return CAMX_OK;
     NormArgs a = a0;
+    a.row0 = 0;
     a.stream = (long)a.rows * a.N >= (1L << 20);
-    const dim3 grid((a.rows + 3) / 4), block(256);
     const int ni = a.N >> 8;
     const bool vec = (a.N & 255) == 0 && ni <= 32 && (a.ld16 & 3) == 0 &&
                      ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.nw & 15) == 0 && ((uintptr_t)a.d & 15) == 0 && ((uintptr_t)a.h & 15) == 0 &&
                      ((uintptr_t)a.h16 & 7) == 0 && ((uintptr_t)a.hbf & 7) == 0 && ((uintptr_t)a.q8 & 3) == 0;
+    if (vec && a.stream && a.rows >= 1024 && (ADD == ADD_NONE || ADD == ADD_HC || a.d)) {
+        const int mask = (a.h ? NORM_H : 0) | (a.h16 ? NORM_H16 : 0) | (a.hbf ? NORM_HBF : 0) | (a.q8 ? NORM_Q8 : 0) | (a.scl ? NORM_SCL : 0);
+        int done = 0;
+        (void)((mask == CHUNK_OUTS && ((done = launch_norm_chunk<ADD, CHUNK_OUTS>(a, st)), true)) || ...);
+        if (done) {
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess || done == a.rows) return (int)e;
+            a.row0 = done;                        // the last rows % 4 rows
+        }
+    }
+    const dim3 grid((a.rows - a.row0 + 3) / 4), block(256);
     if (!vec) add_rms_rows_any<ADD><<<grid, block, 0, st>>>(a);
     else switch (ni) {
 #define CAMX_NORM_EXACT(NI) case NI: add_rms_rows<NI, ADD, true><<<grid, block, 0, st>>>(a); break;
@@ -331,7 +404,7 @@ int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const
                        uint16_t * h16, int N, int n, hipStream_t st) {
     if (N < 256 || N % 256 || N > 2048 || S < 0 || S > 8 || n < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
     NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
-    return launch_norm<ADD_F32_SLOTS>(a, st);
+    return launch_norm<ADD_F32_SLOTS, NORM_H16, NORM_H | NORM_H16>(a, st);
 }
 
 // OP_OWN_ADD_RMS16 with its Seg fields (python/caminus/engine/k3.py:881-902): W = nw, gs = w, a = d, asum = h, y = x, rs = eps, N,
@@ -340,20 +413,20 @@ int camx_op_own_add_rms16(float * x, const float * d, const float * w, int S, co
                           int N, int K, int tokens, hipStream_t st) {
     if (N < 256 || N % 256 || N > 2048 || K < N || S < 0 || S > 8 || tokens < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
     NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, K, nullptr, nullptr, nullptr, N, tokens, nullptr, 1, 0.0f};
-    return launch_norm<ADD_F32_SLOTS>(a, st);
+    return launch_norm<ADD_F32_SLOTS, NORM_H16, NORM_H | NORM_H16>(a, st);
 }
 
 int camx_q35p_add_rms16(float * x, const float * d, const float * nw, float eps, float * h, uint16_t * h16, int N, int n, hipStream_t st) {
     if (N < 256 || N % 256 || N > 65536 || n < 0 || !x || !nw || !h || !h16) return CAMX_EINVAL;
     NormArgs a = {x, d, nullptr, 0, nw, 1, eps, h, h16, N, nullptr, nullptr, nullptr, N, n, nullptr, 1, 0.0f};
-    return launch_norm<ADD_F32_DIRECT>(a, st);
+    return launch_norm<ADD_F32_DIRECT, NORM_H | NORM_H16>(a, st);
 }
 
 int camx_add_rms_q8_1(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h,
                       uint16_t * h16, uint8_t * q8, int N, int n, hipStream_t st) {
     if (N < 32 || N % 32 || S < 0 || S > 8 || n < 0 || !x || !nw || (S > 0 && !d)) return CAMX_EINVAL;
     NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, N, nullptr, q8, nullptr, N, n, nullptr, 1, 0.0f};
-    return launch_norm<ADD_F32_SLOTS>(a, st);
+    return launch_norm<ADD_F32_SLOTS, NORM_Q8, NORM_H | NORM_Q8, NORM_H | NORM_H16 | NORM_Q8>(a, st);
 }
 
 int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps, float * h, uint16_t * hbf, int N, int n, hipStream_t st) {
@@ -373,7 +446,7 @@ int camx_add_rms_bf16(float * x, const uint16_t * d, const float * nw, float eps
 int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf, float * scl, int R, int wr, float eps, int K, hipStream_t st) {
     if (K < 1 || R < 0 || wr < 1 || !x || !w) return CAMX_EINVAL;
     NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, ybf, nullptr, scl, K, R, nullptr, 1, 0.0f};
-    return launch_norm<ADD_NONE>(a, st);
+    return launch_norm<ADD_NONE, NORM_H, NORM_HBF | NORM_SCL, NORM_HBF>(a, st);
 }
 
 int camx_op_rms_mul(const float * x, const float * w, float * y, uint8_t * q8, int R, int wr, int K, float eps, hipStream_t st) {
@@ -387,7 +460,7 @@ int camx_pf_hc_post_rms(const float * b, const float * inj, float * res, const f
                         float rs, float eps, int N, hipStream_t st) {
     if (!b || !inj || !res || !w || T < 0 || HC < 1 || N < 1 || (long)T * HC > 0x7fffffffL) return CAMX_EINVAL;
     NormArgs a = {res, b, nullptr, 0, w, HC, eps, xn, nullptr, N, xnbf, nullptr, scl, N, T * HC, inj, HC, rs};
-    return launch_norm<ADD_HC>(a, st);
+    return launch_norm<ADD_HC, NORM_HBF | NORM_SCL, NORM_HBF>(a, st);
 }
 
 int camx_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows, hipStream_t st) {

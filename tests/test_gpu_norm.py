@@ -8,7 +8,8 @@ from gpu_util import F, I, NULL, bits_equal, call, dev, host, outliers, ptr
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize('n,N,S,weighted', [(1, 2048, 1, False), (5, 2048, 8, True), (3, 256, 0, False), (7, 1024, 3, True), (256, 2048, 1, False)])
+@pytest.mark.parametrize('n,N,S,weighted', [(1, 2048, 1, False), (5, 2048, 8, True), (3, 256, 0, False), (7, 1024, 3, True), (256, 2048, 1, False),
+                                                (1027, 2048, 2, True), (1024, 1024, 1, False), (1030, 2048, 8, False)])
 def test_q3p_add_rms16(n, N, S, weighted):
     rng = np.random.default_rng(1001 + n + N + S)
     x = outliers(rng, (n, N)); d = outliers(rng, (n, max(S, 1), N)); w = rng.random((n, max(S, 1))).astype(np.float32)
@@ -20,6 +21,10 @@ def test_q3p_add_rms16(n, N, S, weighted):
     assert bits_equal(host(xd), ref['x'])
     assert bits_equal(host(h), ref['h'])
     assert bits_equal(host(h16, np.uint16), ref['h16'])
+    # without the fp32 copy (the layers whose consumer reads fp16 only)
+    xd = dev(x); h16 = dev(np.zeros((n, N), np.uint16))
+    call('camx_q3p_add_rms16', ptr(xd), ptr(dd) if S else NULL, ptr(wd) if weighted else NULL, I(S), ptr(nwd), F(1e-6), NULL, ptr(h16), I(N), I(n))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(h16, np.uint16), ref['h16'])
     # the tape's form: the fp16 copy at its own token stride (the Seg's K), the elements between the rows untouched
     K = N + 64
     xd = dev(x); h = dev(np.zeros((n, N), np.float32)); h16 = dev(np.full((n, K), 0x5a5a, np.uint16))
@@ -28,7 +33,7 @@ def test_q3p_add_rms16(n, N, S, weighted):
     assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(got[:, :N], ref['h16']) and (got[:, N:] == 0x5a5a).all()
 
 
-@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096), (520, 4096), (513, 8192), (600, 3072)])
+@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096), (520, 4096), (513, 8192), (600, 3072), (1030, 2560), (1025, 5120), (1024, 4096)])
 def test_q35p_add_rms16(n, N):
     rng = np.random.default_rng(7 + N)
     x = outliers(rng, (n, N)); d = outliers(rng, (n, N)); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
@@ -40,7 +45,7 @@ def test_q35p_add_rms16(n, N):
         assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
 
 
-@pytest.mark.parametrize('n,N', [(4, 2048), (256, 2048), (2, 5120)])
+@pytest.mark.parametrize('n,N', [(4, 2048), (256, 2048), (2, 5120), (1026, 2048), (1024, 4096)])
 def test_add_rms_q8_1(n, N):
     rng = np.random.default_rng(1002 + N)
     x = outliers(rng, (n, N)); d = outliers(rng, (n, 1, N)); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
@@ -50,6 +55,13 @@ def test_add_rms_q8_1(n, N):
     call('camx_add_rms_q8_1', ptr(xd), ptr(dd), NULL, I(1), ptr(nwd), F(1e-6), ptr(h), NULL, ptr(q8), I(N), I(n))
     assert bits_equal(host(h), ref['h'])
     assert bits_equal(host(q8), ref['q8'])
+    # the q8_1 copy alone, and with both float copies
+    xd = dev(x); q8 = dev(np.zeros((n, N // 32, 36), np.uint8))
+    call('camx_add_rms_q8_1', ptr(xd), ptr(dd), NULL, I(1), ptr(nwd), F(1e-6), NULL, NULL, ptr(q8), I(N), I(n))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(q8), ref['q8'])
+    xd = dev(x); q8 = dev(np.zeros((n, N // 32, 36), np.uint8)); h = dev(np.zeros((n, N), np.float32)); h16 = dev(np.zeros((n, N), np.uint16))
+    call('camx_add_rms_q8_1', ptr(xd), ptr(dd), NULL, I(1), ptr(nwd), F(1e-6), ptr(h), ptr(h16), ptr(q8), I(N), I(n))
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(q8), ref['q8']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
 
 
 @pytest.mark.parametrize('n,N', [(3, 5120), (64, 5120), (2, 2048), (600, 5120), (515, 6144), (512, 7168)])
@@ -63,7 +75,7 @@ def test_add_rms_bf16(n, N):
     assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(hbf, np.uint16), ref['hbf'])
 
 
-@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2), (516, 3072, 4), (512, 5120, 1)])
+@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2), (516, 3072, 4), (512, 5120, 1), (1028, 2560, 4), (1026, 2048, 1), (1024, 5120, 4)])
 def test_rms_mul_and_rmsnorm(R, K, wr):
     rng = np.random.default_rng(R * K)
     x = outliers(rng, (R, K)); w = (1 + 0.1 * rng.standard_normal((wr, K))).astype(np.float32)
@@ -73,6 +85,14 @@ def test_rms_mul_and_rmsnorm(R, K, wr):
     y = dev(np.zeros((R, K), np.float32)); ybf = dev(np.zeros((R, K), np.uint16)); scl = dev(np.zeros(R, np.float32))
     call('camx_pf_rms_mul', ptr(xd), ptr(wd), ptr(y), ptr(ybf), ptr(scl), I(R), I(wr), F(1e-6), I(K))
     assert bits_equal(host(y), ref['y']) and bits_equal(host(ybf, np.uint16), ref['ybf']) and bits_equal(host(scl), ref['scale'])
+    # each copy set the prefill callers ask for on its own (python/caminus/prefill/glue.py:153: absent copies are null)
+    ybf = dev(np.zeros((R, K), np.uint16)); scl = dev(np.zeros(R, np.float32)); y = dev(np.zeros((R, K), np.float32))
+    call('camx_pf_rms_mul', ptr(xd), ptr(wd), NULL, ptr(ybf), ptr(scl), I(R), I(wr), F(1e-6), I(K))
+    call('camx_pf_rms_mul', ptr(xd), ptr(wd), ptr(y), NULL, NULL, I(R), I(wr), F(1e-6), I(K))
+    assert bits_equal(host(y), ref['y']) and bits_equal(host(ybf, np.uint16), ref['ybf']) and bits_equal(host(scl), ref['scale'])
+    xnan = x.copy(); xnan[R // 2, 3] = np.nan; xnd = dev(xnan); ybf = dev(np.zeros((R, K), np.uint16))
+    call('camx_pf_rms_mul', ptr(xnd), ptr(wd), NULL, ptr(ybf), NULL, I(R), I(wr), F(1e-6), I(K))
+    assert bits_equal(host(ybf, np.uint16), O.rms_mul(xnan, w, 1e-6)['ybf'])         # a NaN row takes the reference's integer rounding
     if K % 32 == 0:
         q8 = dev(np.zeros((R, K // 32, 36), np.uint8)); y2 = dev(np.zeros((R, K), np.float32))
         call('camx_op_rms_mul', ptr(xd), ptr(wd), ptr(y2), ptr(q8), I(R), I(wr), I(K), F(1e-6))
@@ -83,7 +103,7 @@ def test_rms_mul_and_rmsnorm(R, K, wr):
         assert bits_equal(host(out), O.rmsnorm_f32(x, w[0], 1e-6))
 
 
-@pytest.mark.parametrize('T,HC,N', [(5, 4, 2560), (2048, 4, 2560), (3, 2, 2048), (7, 3, 100), (130, 4, 5120)])
+@pytest.mark.parametrize('T,HC,N', [(5, 4, 2560), (2048, 4, 2560), (3, 2, 2048), (7, 3, 100), (130, 4, 5120), (601, 2, 2048), (1100, 1, 2560)])
 def test_hc_glue(T, HC, N):
     """hyper-connection glue: the residual update passes expf (tolerance class: 1e-5 x max), everything behind it is exact given
     the updated residual; inj = 0 makes the gate exactly 1, so those rows are compared bit for bit"""
@@ -101,6 +121,10 @@ def test_hc_glue(T, HC, N):
     # exact given the device's own residual: the norm of it by the oracle's rms_mul
     again = O.rms_mul(gres.reshape(T * HC, N), w, 1e-6)
     assert bits_equal(gxn.reshape(T * HC, N), again['y']) and bits_equal(host(scl), again['scale']) and bits_equal(host(xnbf, np.uint16).reshape(T * HC, N), again['ybf'])
+    # the prefill caller's copy set (bf16 + row scale, no fp32 copy): the same bits
+    r3 = dev(res); xnbf3 = dev(np.zeros((T, HC, N), np.uint16)); scl3 = dev(np.zeros(T * HC, np.float32))
+    call('camx_pf_hc_post_rms', ptr(bd), ptr(injd), ptr(r3), ptr(wd), NULL, ptr(xnbf3), ptr(scl3), I(T), I(HC), F(0.25), F(1e-6), I(N))
+    assert bits_equal(host(r3), gres) and bits_equal(host(xnbf3, np.uint16), host(xnbf, np.uint16)) and bits_equal(host(scl3), host(scl))
     r2 = dev(res)
     call('camx_pf_hc_post', ptr(bd), ptr(injd), ptr(r2), I(T), I(HC), I(N), F(0.25))
     assert bits_equal(host(r2), gres)                                      # the same statements: the same bits as the fused kernel
