@@ -234,7 +234,7 @@ def extra_opsets(B):
     return out
 
 
-def prefill_scale_sweep(B, T=4096):
+def prefill_scale_sweep(B, T=4096, only=None):
     """every entry point at a prefill-scale size (bench.py --only sweep [--sweep-tokens T]): name -> {us, bytes, GBps, frac_of_8TBps}. Each
     is launched 30 times back to back over enough copies of its buffers, in rotation, that the rotation's footprint is at least 1.2 GB
     (no launch finds its own lines in the 256 MB Infinity Cache); bytes are algorithmic (inputs read once, outputs written once)."""
@@ -243,6 +243,7 @@ def prefill_scale_sweep(B, T=4096):
     res = {}
 
     def timeit(name, by, mk, reps=30):
+        if only and only not in name: return
         ncopy = max(3, min(16, -(-1_200_000_000 // int(by))))
         fns = [mk(i) for i in range(ncopy)]
         for f in fns: f()
@@ -519,6 +520,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--copies', type=int, default=8, help='copies of the batch taken in rotation (8: no launch finds its lines in the Infinity Cache)')
     ap.add_argument('--sweep-tokens', type=int, default=4096, help='rows of the --only sweep shapes')
+    ap.add_argument('--sweep-filter', default=None, help='--only sweep: entries whose name contains this text')
     ap.add_argument('--no-cpu', action='store_true')
     ap.add_argument('--no-extra', action='store_true')
     ap.add_argument('--only', default=None, help='run a single kernel of the step (for profiling)')
@@ -531,7 +533,7 @@ def main():
     torch = B.torch
     if a.only == 'sweep':
         print(json.dumps({'metric': 'fused-op HBM GB/s per entry point at prefill-scale sizes, 1 GPU', 'unit': 'GB/s', 'n_gpus': 1, 'data': 'synthetic',
-                          'peak_GBps': HBM_PEAK_GBPS, 'tokens': a.sweep_tokens, 'sweep': prefill_scale_sweep(B, a.sweep_tokens)}))
+                          'peak_GBps': HBM_PEAK_GBPS, 'tokens': a.sweep_tokens, 'sweep': prefill_scale_sweep(B, a.sweep_tokens, a.sweep_filter)}))
         return
     if a.only == 'ladder':
         print(json.dumps({'metric': 'us per launch and GB/s of the configs\' op-sets from 16 to 4096 tokens, 1 GPU', 'n_gpus': 1, 'data': 'synthetic', 'ladder': batch_ladder(B)}))

@@ -87,6 +87,76 @@ __global__ void __launch_bounds__(256) q8_1_flat(const float * __restrict__ x, u
     }
 }
 
+// The same blocks for a batch that streams from HBM (modes 0 and 1, whole steps of 2048 values, 16-byte aligned): one lane per
+// block. With four values per lane, as above, the eight lanes of a block each repeat the block's divide and walk two
+// butterflies, and the vector ALUs, not HBM, set the time. Here a wave's 2048 values go to its own LDS as they arrive (16 bytes
+// per lane, neighbouring lanes on neighbouring addresses, no registers held), lane l then reads block l whole, and everything
+// per block happens once. The sum keeps the 32-thread butterfly's tree (xor 16, 8, 4, 2, 1 over one value per thread): its
+// first three levels add the block's 4-value pieces c and c + 4, then c and c + 2, then the last two, its last two levels
+// the four sums left. A lane reads its pieces in the order l, l + 1, .. (mod 8), so that the lanes of a request fall on
+// different banks; each level pairs pieces half a period apart, so the rotation changes no operand pair, and max and the
+// codes do not depend on order. Codes: v * (1 / d) rounded to nearest is roundf(v / d) whenever it is farther than 2^-15
+// from a half-integer (|v / d| <= 127 and the refined reciprocal is within an ulp); a piece in which some lane's value
+// is closer, infinite or NaN (one in sixty) is redone with the division.
+template <int MODE>
+__global__ void __launch_bounds__(256) q8_1_blocks(const float * __restrict__ x, uint8_t * __restrict__ y, float rs) {
+    __shared__ __attribute__((aligned(16))) float in_all[4][2048];
+    __shared__ __attribute__((aligned(16))) uint32_t stage_all[4][576];
+    const int l = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t step = (size_t)blockIdx.x * 4 + wv;
+    float * in = in_all[wv];
+    uint32_t * stage = stage_all[wv];
+    const float * src = x + step * 2048;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + 256 * i + 4 * l), (__attribute__((address_space(3))) void *)(in + 256 * i), 16, 0, 2);
+    __builtin_amdgcn_s_waitcnt(0x0f70);                                    // vmcnt(0): the wave's own values have landed
+    f32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = *(const f32x4 *)(in + 32 * l + 4 * ((k + l) & 7));
+    if (MODE == 1) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) { v[k].x = silu_f(v[k].x * rs); v[k].y = silu_f(v[k].y * rs); v[k].z = silu_f(v[k].z * rs); v[k].w = silu_f(v[k].w * rs); }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) amax = fmaxf(amax, absmax4(v[k]));
+    const f32x4 s0 = v[0] + v[4], s1 = v[1] + v[5], s2 = v[2] + v[6], s3 = v[3] + v[7];
+    const f32x4 u0 = s0 + s2, u1 = s1 + s3;
+    const f32x4 w = u0 + u1;
+    const float w0 = w.x + w.z, w1 = w.y + w.w;
+    const float sum = w0 + w1;
+    const float d = amax / 127.0f;
+    uint32_t * blk = stage + 9 * l;
+    blk[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
+    float r = __builtin_amdgcn_rcpf(d);
+    r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        float p[4] = {v[k].x * r, v[k].y * r, v[k].z * r, v[k].w * r};
+        int c[4];
+        bool safe = true;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float n = __builtin_rintf(p[e]);
+            safe &= fabsf(p[e] - n) <= 0.49996948f;                        // (false for NaN and for an infinite p)
+            c[e] = (int)n;
+        }
+        if (__builtin_amdgcn_ballot_w64(!safe && amax != 0.0f) != 0) {
+            p[0] = v[k].x / d; p[1] = v[k].y / d; p[2] = v[k].z / d; p[3] = v[k].w / d;
+#pragma unroll
+            for (int e = 0; e < 4; e++) c[e] = (int)(p[e] + __builtin_copysignf(0.49999997f, p[e]));
+        }
+        const uint32_t codes = ((uint32_t)c[0] & 0xffu) | (((uint32_t)c[1] & 0xffu) << 8) | (((uint32_t)c[2] & 0xffu) << 16) | ((uint32_t)c[3] << 24);
+        blk[1 + ((k + l) & 7)] = amax != 0.0f ? codes : 0u;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // the wave's own LDS writes, in order
+    u32x4 * dst = (u32x4 *)(y + step * 2304);
+    __builtin_nontemporal_store(*(const u32x4 *)(stage + 4 * l), dst + l);
+    __builtin_nontemporal_store(*(const u32x4 *)(stage + 4 * (64 + l)), dst + 64 + l);
+    if (l < 16) __builtin_nontemporal_store(*(const u32x4 *)(stage + 4 * (128 + l)), dst + 128 + l);
+}
+
 // ---- q8_1 in the MMQ layout ---------------------------------------------------------------------------------------------------
 enum { MMQ_D4 = 0, MMQ_DS4 = 1 };
 enum { SRC_F32 = 0, SRC_SWIGLU_BF16 = 1 };
@@ -394,7 +464,7 @@ __global__ void __launch_bounds__(256) silu_small_fill() {             // after 
 #define SWS_IPW 2                                                          // items (token groups) per wave, loaded together
 template <int LAYOUT, int SRC>
 __global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void * __restrict__ gu, const int32_t * __restrict__ ids, long ld, long F,
-                                                                    uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T) {
+                                                                    uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T, unsigned ncolp) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
     const int lraw = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : 0) + wave * (SWM_TOK * 144);
@@ -404,11 +474,35 @@ __global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void 
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g_silu_small + 512 * j + 8 * lraw),
                                              (__attribute__((address_space(3))) void *)(lut + 512 * j), 16, 0, 0);
     }
-    const long tg0 = ((long)blockIdx.x * SWS_WAVES + wave) * (SWM_TOK * SWS_IPW), unit = blockIdx.y;
+    const unsigned ntb = gridDim.x / ncolp;                              // workgroups walk the token groups of a block column first
+    const long tg0 = ((long)(blockIdx.x % ntb) * SWS_WAVES + wave) * (SWM_TOK * SWS_IPW), unit = blockIdx.x / ntb;
     SwmItem it[SWS_IPW];
+    if (SRC == SRC_F32) {
+        // fp32 rows: a lane's eight values are 32 bytes, so loading them into its registers takes two requests that each use half of
+        // every line. The rows go to LDS instead, 16 bytes per lane with neighbouring lanes on neighbouring addresses (one request
+        // per line, no registers held while they fly), and each lane then reads its eight values from there.
+        float * in = (float *)((uint8_t *)lut + SWS_WAVES * (SWM_TOK * 144)) + wave * (SWS_IPW * SWM_TOK * 128);
 #pragma unroll
-    for (int k = 0; k < SWS_IPW; k++) swm_load<SRC>(it[k], gu, ids, ld, F, T, tg0 + SWM_TOK * k, unit, lraw, tg0 + SWM_TOK * k < T);
-    if (SRC == SRC_SWIGLU_BF16) {
+        for (int k = 0; k < SWS_IPW; k++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const long t = tg0 + SWM_TOK * k + 2 * i + (lraw >> 5), e = unit * 128 + 4 * (lraw & 31);
+                const bool ok = t < T && e < F;
+                const float * p = ok ? (const float *)gu + (size_t)(ids ? ids[t] : t) * ld + e : (const float *)g_zero16;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
+                                                 (__attribute__((address_space(3))) void *)(in + k * (SWM_TOK * 128) + i * 256), 16, 0, 2);
+            }
+        __builtin_amdgcn_s_waitcnt(0x0f70);                               // vmcnt(0): the wave's own rows have landed
+#pragma unroll
+        for (int k = 0; k < SWS_IPW; k++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const float * q = in + k * (SWM_TOK * 128) + ((lraw >> 4) + 4 * i) * 128 + 8 * (lraw & 15);
+                it[k].gw[i] = *(const u32x4 *)q; it[k].uw[i] = *(const u32x4 *)(q + 4);
+            }
+    } else {
+#pragma unroll
+        for (int k = 0; k < SWS_IPW; k++) swm_load<SRC>(it[k], gu, ids, ld, F, T, tg0 + SWM_TOK * k, unit, lraw, tg0 + SWM_TOK * k < T);
         __builtin_amdgcn_s_waitcnt(0x0f70);                               // vmcnt(0): this wave's part of the table has landed (and its items)
         __syncthreads();
     }
@@ -434,10 +528,10 @@ __global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void 
 template <int SRC>
 static void launch_oneshot(const void * src, const int32_t * ids, long ld, long F, void * vy, uint16_t * act, int T, long ncol, int layout, hipStream_t st) {
     const int per = SWS_WAVES * SWM_TOK * SWS_IPW;
-    const dim3 grid((unsigned)((T + per - 1) / per), (unsigned)ncol), block(SWS_WAVES * 64);
-    const size_t lds = (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : 0) + SWS_WAVES * SWM_TOK * 144;
-    if (layout == MMQ_DS4) swiglu_mmq_oneshot<MMQ_DS4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T);
-    else swiglu_mmq_oneshot<MMQ_D4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T);
+    const dim3 grid((unsigned)((T + per - 1) / per) * (unsigned)ncol), block(SWS_WAVES * 64);
+    const size_t lds = (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : SWS_WAVES * SWS_IPW * SWM_TOK * 512) + SWS_WAVES * SWM_TOK * 144;
+    if (layout == MMQ_DS4) swiglu_mmq_oneshot<MMQ_DS4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol);
+    else swiglu_mmq_oneshot<MMQ_D4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol);
 }
 
 // act = bf16(bf16(silu g) * u) of wide bf16 rows [g (H) | u (H)] with the same table: persistent workgroups, a lane takes 8
@@ -534,6 +628,15 @@ extern "C" {
 int camx_gg_quantize_q8_1(const float * x, void * y, long n, int mode, float rs, const float * g, hipStream_t st) {
     if (n < 0 || !x || !y || mode < 0 || mode > 2 || (mode == 2 && !g) || ((uintptr_t)y & 3)) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
+    if (mode != 2 && n >= (1L << 20) && (((uintptr_t)x | (uintptr_t)y) & 15) == 0) {       // a batch that streams from HBM: one lane per block
+        const long wgs = n / 8192;                                                           // whole workgroups of 4 x 2048 values
+        if (wgs > 0x7fffffffL) return CAMX_EINVAL;
+        if (mode == 0) q8_1_blocks<0><<<dim3((unsigned)wgs), dim3(256), 0, st>>>(x, (uint8_t *)y, rs);
+        else q8_1_blocks<1><<<dim3((unsigned)wgs), dim3(256), 0, st>>>(x, (uint8_t *)y, rs);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess || n == wgs * 8192) return (int)e;
+        x += wgs * 8192; y = (uint8_t *)y + wgs * (8192 / 32 * 36); n -= wgs * 8192;         // the rest: less than 8192 values
+    }
     const long nstep = (n + 1023) >> 10;
     const int vec = ((uintptr_t)x & 15) == 0 && (mode != 2 || ((uintptr_t)g & 15) == 0);
     const int vecst = ((uintptr_t)y & 15) == 0;

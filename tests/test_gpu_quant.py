@@ -122,6 +122,42 @@ def test_q8_1_quotients_next_to_rounding_boundaries():
     assert bits_equal(host(y), want.reshape(-1))
 
 
+def test_q8_1_streaming_form():
+    """2^20 values and more take the one-lane-per-block kernel for the whole workgroups (8192 values) and the general kernel for the
+    rest: every special block of the tests above inside one such batch, bit for bit against the oracle; mode 1 within its tolerance"""
+    rng = np.random.default_rng(2024)
+    n = (1 << 20) + 3 * 8192 + 1000
+    x = outliers(rng, n)
+    x[:32] = 0.0
+    x[64:96] = np.float32(127.0) * np.sign(rng.standard_normal(32)).astype(np.float32)
+    x[4096:4128] = np.nan; x[5000] = np.nan; x[6000] = np.inf; x[6100] = -np.inf; x[8192 + 320:8192 + 352] = -np.nan
+    e = rng.uniform(-149, -118, (256, 1)) + rng.uniform(-3, 0, (256, 32))
+    x[16384:16384 + 8192] = (np.exp2(e) * rng.choice([-1.0, 1.0], (256, 32))).astype(np.float32).reshape(-1)
+    nblk = 4096
+    amax = np.exp(rng.uniform(-20, 20, nblk)).astype(np.float32)
+    d = (amax / np.float32(127.0)).astype(np.float32).astype(np.float64)
+    k = rng.integers(0, 127, (nblk, 32)) + 0.5
+    off = rng.choice([0.0, 1e-7, 1e-6, 4e-6, 8e-6, 1.5e-5, 2e-5, 3e-5, 4e-5, 8e-5, 2e-4, 1e-3], (nblk, 32)) * rng.choice([-1.0, 1.0], (nblk, 32))
+    t = ((k + off) * rng.choice([-1.0, 1.0], (nblk, 32)) * d[:, None]).astype(np.float32)
+    t[:, 0] = amax
+    x[32768:32768 + nblk * 32] = np.clip(t, -amax[:, None], amax[:, None]).reshape(-1)
+    y = dev(np.full(((n + 31) // 32, 36), 0xa5, np.uint8))
+    call('camx_gg_quantize_q8_1', ptr(dev(x)), ptr(y), L64(n), I(0), F(0), NULL)
+    got, want = host(y), O.q8_1(x).reshape(-1, 36)
+    nanblk = np.isnan(x[:n // 32 * 32].reshape(-1, 32)).any(axis=1) | np.isinf(x[:n // 32 * 32].reshape(-1, 32)).any(axis=1)
+    nanblk = np.concatenate([nanblk, np.zeros(got.shape[0] - nanblk.size, bool)])
+    assert bits_equal(got[~nanblk], want[~nanblk])
+    assert bits_equal(got[nanblk][:, :2], want[nanblk][:, :2]) and bits_equal(got[nanblk][:, 4:], want[nanblk][:, 4:])     # (a NaN sum's sign is the adder's)
+    xs = x.copy(); xs[~np.isfinite(xs)] = 1.0
+    y1 = dev(np.zeros(((n + 31) // 32, 36), np.uint8))
+    call('camx_gg_quantize_q8_1', ptr(dev(xs)), ptr(y1), L64(n), I(1), F(0.37), NULL)
+    g1, r1 = host(y1), O.q8_1(xs, mode=1, rs=0.37).reshape(-1, 36)
+    d_g, d_r = g1[:, 0:2].copy().view(np.float16).astype(np.float64), r1[:, 0:2].copy().view(np.float16).astype(np.float64)
+    fin = np.isfinite(d_r)                                                # (a scale past the half range is inf on both sides)
+    assert np.array_equal(d_g[~fin], d_r[~fin]) and np.all(np.abs(d_g[fin] - d_r[fin]) <= np.abs(d_r[fin]) * 2.0 ** -9 + 1e-12)
+    assert np.abs(g1[:, 4:].view(np.int8).astype(int) - r1[:, 4:].view(np.int8).astype(int)).max() <= 1
+
+
 def test_q8_1_blocks_of_nan():
     """a block that holds only NaN has amax 0 under the reference's fmaxf chain (a NaN is skipped): scale 0 and codes 0, in the flat
     layout and as the copy of a normalized row; a NaN among numbers leaves the block's scale to the numbers. (The sum is NaN; its
