@@ -243,7 +243,7 @@ def prefill_scale_sweep(B, T=4096, only=None):
     res = {}
 
     def timeit(name, by, mk, reps=30):
-        if only and only not in name: return
+        if only and not any(o in name for o in only.split(',')): return
         ncopy = max(3, min(16, -(-1_200_000_000 // int(by))))
         fns = [mk(i) for i in range(ncopy)]
         for f in fns: f()
@@ -520,7 +520,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--copies', type=int, default=8, help='copies of the batch taken in rotation (8: no launch finds its lines in the Infinity Cache)')
     ap.add_argument('--sweep-tokens', type=int, default=4096, help='rows of the --only sweep shapes')
-    ap.add_argument('--sweep-filter', default=None, help='--only sweep: entries whose name contains this text')
+    ap.add_argument('--sweep-filter', default=None, help='--only sweep: entries whose name contains one of these comma-separated texts')
     ap.add_argument('--no-cpu', action='store_true')
     ap.add_argument('--no-extra', action='store_true')
     ap.add_argument('--only', default=None, help='run a single kernel of the step (for profiling)')

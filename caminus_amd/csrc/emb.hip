@@ -109,11 +109,15 @@ struct EmbArgs {
 };
 
 // EXACT: the row has exactly NI_MAX slabs (straight-line loops: the loads are issued as one batch)
-template <int FMT, int NI_MAX, bool TAIL, bool EXACT>
+// SPLIT (batches too small to fill the chip): a workgroup per row. Every wave decodes the row and, with a tail, walks the same
+// sum of squares (the same operations on the same values: the same bits in all four), but converts, quantizes and stores only
+// the slabs j = wave (mod 4): the serial part behind the reduction, eight q8_1 slabs for a 2048-wide row, is a quarter as long.
+template <int FMT, int NI_MAX, bool TAIL, bool EXACT, bool SPLIT = false>
 __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
-    const int lane = slot_of(threadIdx.x & 63);
-    const int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = slot_of(threadIdx.x & 63), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t = SPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
     if (t >= a.n) return;
+    auto mine = [&](int j) { return !SPLIT || (j & 3) == wave; };
     int tok = a.toks[t];
     if (a.err && (tok < 0 || tok >= a.vocab) && lane == 0) atomicOr(a.err, ERR_TOKEN);
     tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;
@@ -127,7 +131,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) {
-                gpre[j] = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
+                if (mine(j)) gpre[j] = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
                 if (a.d) dpre[j] = *(const f32x4 *)(a.d + (size_t)t * N + 256 * j + 4 * lane);
             }
     }
@@ -136,10 +140,10 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     f32x4 xv[NI_MAX];
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) xv[j] = emb_decode4<FMT>(row, j, lane);
+        if (j < ni && (TAIL || mine(j))) xv[j] = emb_decode4<FMT>(row, j, lane);
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) {
+        if (j < ni && mine(j)) {
             const size_t o = (size_t)t * N + 256 * j + 4 * lane;
             if (!TAIL && a.stream) {
                 if (a.x) __builtin_nontemporal_store(xv[j], (f32x4 *)(a.x + o));
@@ -156,7 +160,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
             if (j < ni) {
                 const size_t o = (size_t)t * N + 256 * j + 4 * lane;
                 xv[j] = xv[j] + (PRE ? dpre[j] : *(const f32x4 *)(a.d + o));
-                if (a.x) *(f32x4 *)(a.x + o) = xv[j];
+                if (a.x && mine(j)) *(f32x4 *)(a.x + o) = xv[j];
             }
     }
     f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -170,7 +174,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     const float scale = rsqrt_exact(tot / (float)N + a.eps);
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
-        if (j < ni) {
+        if (j < ni && mine(j)) {
             const f32x4 g = PRE ? gpre[j] : *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
             f32x4 v;
             v.x = (xv[j].x * scale) * g.x; v.y = (xv[j].y * scale) * g.y; v.z = (xv[j].z * scale) * g.z; v.w = (xv[j].w * scale) * g.w;
@@ -186,9 +190,17 @@ static int launch_emb(const EmbArgs & a0, hipStream_t st) {
     if (a0.n <= 0) return CAMX_OK;
     EmbArgs a = a0;
     a.stream = (long)a.n * a.N >= (1L << 20);
-    const dim3 grid((a.n + 3) / 4), block(256);
+    const dim3 block(256);
     const int ni = a.N >> 8;
     const bool tail = a.nw != nullptr;
+    if (a.n <= 1024 && (ni == 4 || ni == 8 || ni == 16 || ni == 20)) {          // a workgroup per row
+        const dim3 grid(a.n);
+#define CAMX_EMB_SPLIT(NI) (tail ? emb_rows<FMT, NI, true, true, true><<<grid, block, 0, st>>>(a) : emb_rows<FMT, NI, false, true, true><<<grid, block, 0, st>>>(a))
+        if (ni == 8) CAMX_EMB_SPLIT(8); else if (ni == 16) CAMX_EMB_SPLIT(16); else if (ni == 20) CAMX_EMB_SPLIT(20); else CAMX_EMB_SPLIT(4);
+#undef CAMX_EMB_SPLIT
+        CAMX_LAUNCH_RET();
+    }
+    const dim3 grid((a.n + 3) / 4);
 #define CAMX_EMB(NI, EX) (tail ? emb_rows<FMT, NI, true, EX><<<grid, block, 0, st>>>(a) : emb_rows<FMT, NI, false, EX><<<grid, block, 0, st>>>(a))
     if (ni == 8) CAMX_EMB(8, true); else if (ni == 16) CAMX_EMB(16, true); else if (ni == 20) CAMX_EMB(20, true); else if (ni == 4) CAMX_EMB(4, true);
     else if (ni <= 8) CAMX_EMB(8, false); else if (ni <= 16) CAMX_EMB(16, false); else if (ni <= 24) CAMX_EMB(24, false); else CAMX_EMB(32, false);

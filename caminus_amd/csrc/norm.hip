@@ -41,13 +41,17 @@ struct NormArgs {
 // wave (row r uses gamma row r % wr). The launcher gives these forms whole workgroups only.
 enum { NORM_H = 1, NORM_H16 = 2, NORM_HBF = 4, NORM_Q8 = 8, NORM_SCL = 16 };
 #define CAMX_ISSUE_GAP() do { if (OUT) { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_sleep(1); __builtin_amdgcn_sched_barrier(0); } } while (0)
-template <int NI_MAX, int ADD, bool EXACT, int OUT = 0, int GL = 0>
+// SPLIT (a batch too small to fill the chip, with a q8_1 copy): a workgroup per row. Every wave loads the row and walks the same
+// sum of squares (the same operations on the same values: the same bits in all four), but writes the residual and the copies of
+// the slabs j = wave (mod 4) only: the serial part behind the reduction, eight q8_1 slabs for a 2048-wide row, is a quarter as long.
+template <int NI_MAX, int ADD, bool EXACT, int OUT = 0, int GL = 0, bool SPLIT = false>
 __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
-    static_assert(OUT == 0 ? GL == 0 : EXACT, "the chunk form is straight-line code");
+    static_assert(OUT == 0 ? GL == 0 : (EXACT && !SPLIT), "the chunk form is straight-line code");
     extern __shared__ __attribute__((aligned(16))) float gsh[];
     const int lraw = threadIdx.x & 63, lane = slot_of(lraw), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int row = a.row0 + blockIdx.x * 4 + wave;
+    const int row = a.row0 + (SPLIT ? blockIdx.x : blockIdx.x * 4 + wave);
     if (!OUT && row >= a.rows) return;
+    auto mine = [&](int j) { return !SPLIT || (j & 3) == wave; };
     const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
     if (GL == 1) {
 #pragma unroll
@@ -141,13 +145,14 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     if (!GL) {
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
+            if (j < ni && mine(j)) g[j] = *(const f32x4 *)(gw + 256 * j + 4 * lane);
     }
+    if (SPLIT) __syncthreads();                   // every wave of the row has its loads back before any of them writes (x in place; h may be x)
     if (ADD == ADD_HC || (ADD == ADD_F32_SLOTS && a.S > 0) || ((ADD == ADD_F32_DIRECT || ADD == ADD_BF16) && a.d)) {
         // the updated residual goes back to the lines it was read from
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
+            if (j < ni && mine(j)) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
     }
     // sum of squares: logical thread 4 lane + k chains its elements in j order
     f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -159,7 +164,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         }
     const float tot = wave_groups_in_order(group32_sum(ss));
     const float scale = rsqrt_exact(tot / (float)N + a.eps);
-    if ((OUT ? (OUT & NORM_SCL) != 0 : a.scl != nullptr) && lane == 0) a.scl[row] = scale;
+    if ((OUT ? (OUT & NORM_SCL) != 0 : a.scl != nullptr) && lane == 0 && (!SPLIT || wave == 0)) a.scl[row] = scale;
     if (GL) {
         __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0): this wave's gamma pieces have landed in LDS (they were first in the queue)
         if (GL == 1) __syncthreads();
@@ -171,7 +176,7 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
         bool nan = false;
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) {
+            if (j < ni && mine(j)) {
                 const f32x4 gj = GL ? *(const f32x4 *)(gl + 256 * j + 4 * lane) : g[GL ? 0 : j];
                 f32x4 t, v;
                 t.x = xv[j].x * scale; t.y = xv[j].y * scale; t.z = xv[j].z * scale; t.w = xv[j].w * scale;
@@ -306,7 +311,18 @@ static int launch_norm(const NormArgs & a0, hipStream_t st) {
             a.row0 = done;                        // the last rows % 4 rows
         }
     }
-    const dim3 grid((a.rows - a.row0 + 3) / 4), block(256);
+    const dim3 block(256);
+    // a workgroup per row: up to 1024 rows when a q8_1 copy follows the reduction, else up to 256 (5120-wide rows: 7.3 us against 8.7 for
+    // 256 cold rows, equal from 512 rows on; 2048-wide rows: within 4 % either way)
+    if (vec && a.rows <= (a.q8 ? 1024 : 256)) {
+        const dim3 grid(a.rows);
+        switch (ni) {
+#define CAMX_NORM_SPLIT(NI) case NI: add_rms_rows<NI, ADD, true, 0, 0, true><<<grid, block, 0, st>>>(a); CAMX_LAUNCH_RET();
+            CAMX_NORM_SPLIT(4) CAMX_NORM_SPLIT(8) CAMX_NORM_SPLIT(10) CAMX_NORM_SPLIT(16) CAMX_NORM_SPLIT(20)
+#undef CAMX_NORM_SPLIT
+        }
+    }
+    const dim3 grid((a.rows - a.row0 + 3) / 4);
     if (!vec) add_rms_rows_any<ADD><<<grid, block, 0, st>>>(a);
     else switch (ni) {
 #define CAMX_NORM_EXACT(NI) case NI: add_rms_rows<NI, ADD, true><<<grid, block, 0, st>>>(a); break;

@@ -54,8 +54,10 @@ template <int S> CAMX_DEV float half_lane_bcast(float v) {   // every lane of a 
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x00 | (S << 5)));
 }
 
-template <bool YARN, bool Q8, bool BF16IN, int TPW>
-__global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
+// NW waves per workgroup and QR_STEPS wave steps per pass: 4 x 5 (a pass of 40 heads, ten per wave), or 10 x 2 for batches too small to
+// fill the chip, where a token's heads spread over more waves and each wave's chain of steps is two long instead of five.
+template <bool YARN, bool Q8, bool BF16IN, int TPW, int NW = 4, int QR_STEPS = 5>
+__global__ void __launch_bounds__(NW * 64) qk_rope_tokens(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[TPW][64];
     __shared__ __attribute__((aligned(16))) float rs[TPW][64];
     const int t0 = blockIdx.x * TPW, tid = threadIdx.x, lraw = tid & 63, lane = slot_of(lraw), l = lane & 31, wave = tid >> 6;
@@ -63,9 +65,9 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
     // heads (one per half-wave); the loads of up to QR_STEPS steps (one pass) are issued together, and before the cos / sin
     // rows are computed, so a decode token pays one memory round trip, not one per head.
     const int items = a.nh + 2 * a.nkv;
-    constexpr int QR_STEPS = 5;
-    const int npass = (items + 8 * QR_STEPS - 1) / (8 * QR_STEPS);
-    const int it_w = wave * 2 + (lane >> 5);                            // this half-wave's head inside a step of 8 heads
+    constexpr int HS = 2 * NW;                                          // heads per wave step of the workgroup
+    const int npass = (items + HS * QR_STEPS - 1) / (HS * QR_STEPS);
+    const int it_w = wave * 2 + (lane >> 5);                            // this half-wave's head inside a step of HS heads
     f32x4 xin[QR_STEPS], xnext[QR_STEPS];
     auto load = [&](f32x4 (&buf)[QR_STEPS], int tok, int base) {
         const int tk = tok < a.n ? tok : 0;
@@ -73,7 +75,7 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         const uint16_t * rowb = (const uint16_t *)a.qkv + (size_t)tk * a.ldq;
 #pragma unroll
         for (int s = 0; s < QR_STEPS; s++) {
-            const int it = base + 8 * s + it_w;
+            const int it = base + HS * s + it_w;
             const int hy = it < items ? it : 0;
             buf[s] = BF16IN ? unpack_bf16x4(*(const u32x2 *)(rowb + (size_t)hy * 128 + 4 * l)) : *(const f32x4 *)(row + (size_t)hy * 128 + 4 * l);
         }
@@ -81,7 +83,7 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
     load(xin, t0, 0);
     const f32x4 wq = *(const f32x4 *)(a.par + 4 * l), wk = *(const f32x4 *)(a.par + 128 + 4 * l);
     const float eps = a.par[257];
-    for (int tr = wave; tr < TPW; tr += 4) {                               // the tokens whose cos / sin rows this wave computes
+    for (int tr = wave; tr < TPW; tr += NW) {                               // the tokens whose cos / sin rows this wave computes
         if (t0 + tr < a.n) {
             const int pos = a.pos ? a.pos[t0 + tr] : a.pos0 + t0 + tr;
             float c, s;
@@ -95,9 +97,9 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
     const size_t rb = Q8 ? 2 * (M / 32) * 34 : 4 * M;
     const bool lo = l < 16;
     for (int it_tp = 0; it_tp < TPW * npass; it_tp++) {
-        const int ti = it_tp / npass, base = (it_tp - ti * npass) * 8 * QR_STEPS, t = t0 + ti;
+        const int ti = it_tp / npass, base = (it_tp - ti * npass) * HS * QR_STEPS, t = t0 + ti;
         if (t >= a.n) break;
-        if (it_tp + 1 < TPW * npass) { const int tn = (it_tp + 1) / npass; load(xnext, t0 + tn, ((it_tp + 1) - tn * npass) * 8 * QR_STEPS); }
+        if (it_tp + 1 < TPW * npass) { const int tn = (it_tp + 1) / npass; load(xnext, t0 + tn, ((it_tp + 1) - tn * npass) * HS * QR_STEPS); }
         const int pos = a.pos ? a.pos[t] : a.pos0 + t;
         uint8_t * cw = nullptr;
         // a position outside the sequence's table row (paged) or outside the cache (unpaged): bit 1, that sequence's row is not written
@@ -123,13 +125,16 @@ __global__ void __launch_bounds__(256) qk_rope_tokens(RopeArgs a) {
         for (int st = 1; st < QR_STEPS; st++) tv = (lraw & 31) == st ? tot[st] : tv;
         const float sc = rsqrt_exact(tv / 128 + eps);
         float scl[QR_STEPS];
-        scl[0] = half_lane_bcast<0>(sc); scl[1] = half_lane_bcast<1>(sc); scl[2] = half_lane_bcast<2>(sc); scl[3] = half_lane_bcast<3>(sc);
-        scl[4] = half_lane_bcast<4>(sc);
-        static_assert(QR_STEPS == 5, "the broadcasts above are written out for five steps");
+        static_assert(QR_STEPS <= 5, "the broadcasts below are written out for at most five steps");
+        scl[0] = half_lane_bcast<0>(sc);
+        if (QR_STEPS > 1) scl[1 % QR_STEPS] = half_lane_bcast<1>(sc);
+        if (QR_STEPS > 2) scl[2 % QR_STEPS] = half_lane_bcast<2>(sc);
+        if (QR_STEPS > 3) scl[3 % QR_STEPS] = half_lane_bcast<3>(sc);
+        if (QR_STEPS > 4) scl[4 % QR_STEPS] = half_lane_bcast<4>(sc);
 #pragma unroll
         for (int st = 0; st < QR_STEPS; st++) {
-            if (base + 8 * st + wave * 2 >= items) break;               // wave-uniform: neither half-wave has a head
-            const int it = base + 8 * st + it_w;
+            if (base + HS * st + wave * 2 >= items) break;               // wave-uniform: neither half-wave has a head
+            const int it = base + HS * st + it_w;
             const bool active = it < items;
             const int hy = active ? it : 0;
             const f32x4 x = xin[st];
@@ -941,6 +946,12 @@ static int rope_check(const RopeArgs & a, bool q8, bool bf16in) {
 }
 template <bool BF16IN, int TPW>
 static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st) {
+    if (TPW == 1 && a.n <= 1024) {                 // a batch that does not fill the chip: ten waves per token
+        const dim3 grid(a.n), block(640);
+        if (q8) { if (yarn) qk_rope_tokens<true, true, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); }
+        else { if (yarn) qk_rope_tokens<true, false, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); }
+        return;
+    }
     const dim3 grid((a.n + TPW - 1) / TPW), block(256);
     if (q8) { if (yarn) qk_rope_tokens<true, true, BF16IN, TPW><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true, BF16IN, TPW><<<grid, block, 0, st>>>(a); }
     else { if (yarn) qk_rope_tokens<true, false, BF16IN, TPW><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false, BF16IN, TPW><<<grid, block, 0, st>>>(a); }
