@@ -193,7 +193,9 @@ static int launch_emb(const EmbArgs & a0, hipStream_t st) {
     const dim3 block(256);
     const int ni = a.N >> 8;
     const bool tail = a.nw != nullptr;
-    if (a.n <= 1024 && (ni == 4 || ni == 8 || ni == 16 || ni == 20)) {          // a workgroup per row
+    // a workgroup per row while the chip is not full: 256 rows x 4 waves are one wave per SIMD; from 512 rows on the four-fold decode costs
+    // more than the shorter tail saves (2048-wide Q4_K rows with the fused tail: 6.6 us at 256 rows, 12.0 at 512 against 8 before)
+    if (a.n <= 256 && (ni == 4 || ni == 8 || ni == 16 || ni == 20)) {
         const dim3 grid(a.n);
 #define CAMX_EMB_SPLIT(NI) (tail ? emb_rows<FMT, NI, true, true, true><<<grid, block, 0, st>>>(a) : emb_rows<FMT, NI, false, true, true><<<grid, block, 0, st>>>(a))
         if (ni == 8) CAMX_EMB_SPLIT(8); else if (ni == 16) CAMX_EMB_SPLIT(16); else if (ni == 20) CAMX_EMB_SPLIT(20); else CAMX_EMB_SPLIT(4);

@@ -946,7 +946,7 @@ static int rope_check(const RopeArgs & a, bool q8, bool bf16in) {
 }
 template <bool BF16IN, int TPW>
 static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st) {
-    if (TPW == 1 && a.n <= 1024) {                 // a batch that does not fill the chip: ten waves per token
+    if (TPW == 1 && a.n <= 256) {                  // a batch that does not fill the chip: ten waves per token (256 tokens: 4.9 us against 6.0)
         const dim3 grid(a.n), block(640);
         if (q8) { if (yarn) qk_rope_tokens<true, true, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, true, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); }
         else { if (yarn) qk_rope_tokens<true, false, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); else qk_rope_tokens<false, false, BF16IN, 1, 10, 2><<<grid, block, 0, st>>>(a); }

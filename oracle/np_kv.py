@@ -1,6 +1,7 @@
-"""TEST INFRASTRUCTURE ONLY (like everything under oracle/): numpy statement of the Q8 KV row bytes and of the 128-point
-Hadamard rotation, written independently of oracle/camx_oracle.c so that the two can be compared bit for bit. Same functions, argument meanings and refusals as the reference's python/caminus/ref_kv.py:44-144
-(Q8KVLayout, hadamard128, encode_q8_kv, decode_q8_kv).
+"""TEST INFRASTRUCTURE ONLY (like everything under oracle/): numpy restatement of the Q8 KV row bytes and of the 128-point
+Hadamard rotation that follows the reference's python/caminus/ref_kv.py:44-144 function by function (Q8KVLayout, hadamard128,
+encode_q8_kv, decode_q8_kv: the same arguments, refusals and messages). It shares no code with oracle/camx_oracle.c, so the tests
+compare the two bit for bit; as a pin it adds only that cross-check to the literal vectors.
 
 A row is K then V, each the head-major vector cut into 32-value blocks of a little-endian fp16 scale and 32 signed bytes.
 Encode: fp32 amax / 127, its fp32 reciprocal, fp32 product, round half away from zero; only the STORED scale is rounded to
