@@ -34,6 +34,37 @@ __global__ void __launch_bounds__(256) kv_q8_append_rows(const float * __restric
     }
 }
 
+// The same rows for a chunk of tokens with at most 32 blocks per row (M <= 512, 16-byte aligned): a wave per row, its (up to) four
+// loads per lane issued together, four rows per workgroup. A workgroup per row is 4 KB of work; at chunk sizes the launch of 16384 such
+// workgroups, not the memory, sets the time.
+__global__ void __launch_bounds__(256) kv_q8_append_wave_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
+                                                              uint8_t * __restrict__ cache, int pos0, int rows, int T, int * __restrict__ err) {
+    const int tt = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tt >= T) return;
+    const long pos = (long)pos0 + (long)tt;
+    const int lane = slot_of(threadIdx.x & 63), sub = lane & 7;
+    if (pos < 0 || pos >= rows) {
+        if ((threadIdx.x & 63) == 0) atomicOr(err, 1);
+        return;
+    }
+    const int nb = M / 32;
+    uint8_t * dst = cache + (size_t)pos * ((size_t)2 * nb * 34);
+    f32x4 xv[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int b = it * 8 + (lane >> 3);
+        const int bb = b < 2 * nb ? b : 0;
+        const float * x = (bb < nb ? k + (size_t)tt * ldk : v + (size_t)tt * ldv) + (size_t)(bb % nb) * 32 + 4 * sub;
+        xv[it] = __builtin_nontemporal_load((const f32x4 *)x);
+    }
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int b = it * 8 + (lane >> 3);
+        const bool active = b < 2 * nb;
+        kv_q8_emit(xv[it], dst + (size_t)(active ? b : 0) * 34, sub, err, active);
+    }
+}
+
 // pf_kv_append (q8_0 rows): no refusal rules; d stored as half, codes roundf(x * (1 / d)); err bit 1 for a row outside
 __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
                                                          uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
@@ -94,6 +125,49 @@ __global__ void __launch_bounds__(256) kv_q8_read_rows(const uint8_t * __restric
     }
 }
 
+// The same reader for a chunk of rows with at most 32 blocks per row (M <= 512; row bytes a multiple of 16, 16-byte aligned cache): a
+// wave per row, four rows per workgroup; the row comes in as 16-byte pieces straight to the wave's LDS (two requests per wave instead
+// of three 2-byte loads per lane and block) and is decoded from there.
+template <bool F16>
+__global__ void __launch_bounds__(256) kv_q8_read_wave_rows(const uint8_t * __restrict__ cache, const int32_t * __restrict__ row_ids, int pos0, int rows, int M,
+                                                            void * __restrict__ k, int ldk, void * __restrict__ v, int ldv, int T, int * __restrict__ err) {
+    __shared__ __attribute__((aligned(16))) uint8_t stage_all[4][2 * 16 * 34];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, sub = lane & 7;
+    const int tt = blockIdx.x * 4 + wave;
+    if (tt >= T) return;
+    const long pos = row_ids ? (long)row_ids[tt] : (long)pos0 + (long)tt;
+    if (pos < 0 || pos >= rows) {
+        if (lane == 0) atomicOr(err, 1);
+        return;
+    }
+    const int nb = M / 32, rb = 2 * nb * 34, n16 = rb / 16;
+    const uint8_t * src = cache + (size_t)pos * rb;
+    uint8_t * stage = stage_all[wave];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int p = 64 * i + lane;
+        const uint8_t * q = src + 16 * (size_t)p;
+        if (p < n16)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)q, (__attribute__((address_space(3))) void *)(stage + 1024 * i), 16, 0, 2);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);                                    // vmcnt(0): the wave's own row has landed
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int b = it * 8 + (lane >> 3);
+        if (b >= 2 * nb) continue;
+        const uint8_t * blk = stage + (size_t)b * 34;
+        const float d = h2f_bits(*(const uint16_t *)blk);
+        const uint16_t * c = (const uint16_t *)(blk + 2 + 4 * sub);
+        const uint32_t w = (uint32_t)c[0] | ((uint32_t)c[1] << 16);
+        f32x4 y;
+        y.x = (float)(int8_t)(w & 0xff) * d; y.y = (float)(int8_t)((w >> 8) & 0xff) * d;
+        y.z = (float)(int8_t)((w >> 16) & 0xff) * d; y.w = (float)(int8_t)(w >> 24) * d;
+        const size_t o = (b < nb ? (size_t)tt * ldk : (size_t)tt * ldv) + (size_t)(b % nb) * 32 + 4 * sub;
+        if (F16) __builtin_nontemporal_store(pack_f16x4(y), (u32x2 *)((uint16_t *)(b < nb ? k : v) + o));
+        else __builtin_nontemporal_store(y, (f32x4 *)((float *)(b < nb ? k : v) + o));
+    }
+}
+
 // in-place orthonormal WHT of C chunks of n values, n in {64, 128, 256}: n / 4 lanes per chunk
 template <int N>
 __global__ void __launch_bounds__(256) hadamard_chunks(float * __restrict__ x, long C) {
@@ -140,7 +214,10 @@ int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, in
                           int T, hipStream_t st) {
     if (!k || !v || !cache || !err || T < 0 || ((uintptr_t)k & 3) || ((uintptr_t)v & 3) || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
-    kv_q8_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
+    const bool chunk = T >= 1024 && M >= 32 && M % 32 == 0 && M <= 512 && ldk >= M && ldv >= M && rows >= 1 &&
+                       ((ldk | ldv) & 3) == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
+    if (chunk) kv_q8_append_wave_rows<<<dim3((T + 3) / 4), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, T, err);
+    else kv_q8_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
     CAMX_LAUNCH_RET();
 }
 
@@ -152,7 +229,13 @@ int camx_own_kv_q8_read(const uint8_t * cache, const int32_t * row_ids, int pos0
     if (!cache || !k || !v || !err || T < 0 || ((uintptr_t)cache & 1) || ((uintptr_t)k & (f16 ? 7 : 3)) || ((uintptr_t)v & (f16 ? 7 : 3)) ||
         (f16 && ((ldk | ldv) & 3))) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
-    if (f16) kv_q8_read_rows<true><<<dim3(T), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, err);
+    const bool chunk = T >= 1024 && M >= 32 && M % 32 == 0 && M <= 512 && (2 * (M / 32) * 34) % 16 == 0 && ldk >= M && ldv >= M && rows >= 1 &&
+                       ((uintptr_t)cache & 15) == 0 && (f16 || ((((uintptr_t)k | (uintptr_t)v) & 15) == 0 && ((ldk | ldv) & 3) == 0));
+    if (chunk) {
+        if (f16) kv_q8_read_wave_rows<true><<<dim3((T + 3) / 4), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, T, err);
+        else kv_q8_read_wave_rows<false><<<dim3((T + 3) / 4), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, T, err);
+    }
+    else if (f16) kv_q8_read_rows<true><<<dim3(T), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, err);
     else kv_q8_read_rows<false><<<dim3(T), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, err);
     CAMX_LAUNCH_RET();
 }

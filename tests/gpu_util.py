@@ -63,15 +63,22 @@ def _row_scale(r):
     return np.maximum(r.max(axis=-1, keepdims=True) if r.ndim else r, 1e-30)
 
 
-def close_fp32(a, ref, rel=1e-5):
-    """per element: |a - ref| <= rel * |ref| + rel / 10 * (max |ref| of the element's row). The second term covers outputs that are a
+# Outputs behind the 128-point Hadamard transform of fp16-rounded values (the Q8 line's q16 and K rows): a one-ulp difference in one
+# rotary output before the rounding moves that input by 2^-10 of its size at most, and every output of the head by 1 / sqrt(128) of
+# that; by Parseval the largest output of a head is at least (largest input) / sqrt(128), so one such flip stays under 2^-10 of the
+# head's largest output. Twice that as the floor.
+HADAMARD_FLOOR = 2.0 ** -9
+
+
+def close_fp32(a, ref, rel=1e-5, floor=None):
+    """per element: |a - ref| <= rel * |ref| + floor * (max |ref| of the element's row), floor = rel / 10 unless given. The second term covers outputs that are a
     difference of products (a rotary pair, a gated sum), whose error scales with the operands and not with the result; it is tied to the
     element's own row, so a small value next to a large one in another row gets no slack from it."""
     a = np.asarray(a, np.float64); ref = np.asarray(ref, np.float64)
-    return bool((np.abs(a - ref) <= rel * np.abs(ref) + 0.1 * rel * _row_scale(ref)).all())
+    return bool((np.abs(a - ref) <= rel * np.abs(ref) + (0.1 * rel if floor is None else floor) * _row_scale(ref)).all())
 
 
-def close_16(bits, ref_bits, kind, rel=1e-5):
+def close_16(bits, ref_bits, kind, rel=1e-5, floor=None):
     """16-bit outputs within one unit in the last place of the reference value, plus the fp32 bound above; kind 'f16' | 'bf16'"""
     bits = np.asarray(bits, np.uint16); ref_bits = np.asarray(ref_bits, np.uint16)
     if kind == 'f16':
@@ -80,4 +87,4 @@ def close_16(bits, ref_bits, kind, rel=1e-5):
     else:
         a = (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64); r = (ref_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
         ulp = np.abs(r) * 2.0 ** -7 + 2.0 ** -133
-    return bool((np.abs(a - r) <= ulp + rel * np.abs(r) + 0.1 * rel * _row_scale(r)).all())
+    return bool((np.abs(a - r) <= ulp + rel * np.abs(r) + (0.1 * rel if floor is None else floor) * _row_scale(r)).all())

@@ -36,6 +36,29 @@ def test_kv_q8_append_bytes(heads, dim):
     assert bits_equal(host(bd2), got)
 
 
+@pytest.mark.parametrize('M,T,pad', [(512, 1100, 4), (1024, 1030, 0), (2048, 1024, 8), (256, 1200, 0), (96, 1100, 0)])
+def test_kv_q8_append_chunk(M, T, pad):
+    """a chunk of tokens (1024 rows and more take the kernel that assembles a row in LDS): random rows with zero blocks, valid blocks of
+    the reference's generator, and rows that hold a refused block, whose bytes must stay as they were while the rest of the row lands"""
+    rng = np.random.default_rng(M + T)
+    nb = M // 32
+    k = (rng.standard_normal((T, M)) * np.exp2(rng.integers(-10, 10, (T, 1)))).astype(np.float32); v = rng.standard_normal((T, M)).astype(np.float32)
+    k[3, 32:64] = 0.0; v[5] = 0.0
+    good = kv_valid_blocks(); bad = kv_invalid_blocks()
+    for i in range(min(len(good), T - 20)): k[10 + i, :32] = good[i]
+    for i, b in enumerate(bad): (k if i % 2 else v)[20 + 7 * i, 32 * (i % nb):32 * (i % nb) + 32] = b
+    ldk, ldv = M + pad, M + 2 * pad
+    kin = np.full((T, ldk), 999.0, np.float32); vin = np.full((T, ldv), -999.0, np.float32)
+    kin[:, :M] = k; vin[:, :M] = v
+    rb = 2 * nb * 34
+    cache0 = np.full((T + 3) * rb, 0xa5, np.uint8)
+    want, werr = O.kv_q8_append(kin, ldk, vin, ldv, M, cache0, 2, T)
+    cd = dev(cache0); err = dev(np.zeros(1, np.int32))
+    call('camx_own_kv_q8_append', ptr(dev(kin)), I(ldk), ptr(dev(vin)), I(ldv), I(M), ptr(cd), I(2), I(T + 3), ptr(err), I(T))
+    assert int(host(err)[0]) == werr == 2
+    assert bits_equal(host(cd), want)
+
+
 def test_kv_q8_refusals_and_error_bits():
     bad = kv_invalid_blocks(); good = kv_valid_blocks()[:len(bad)]
     M = 64
@@ -91,7 +114,8 @@ def test_hadamard128():
     assert bits_equal(host(y), O.hadamard128(xs))
 
 
-@pytest.mark.parametrize('M,T,f16', [(512, 300, False), (512, 300, True), (64, 5, False), (1024, 17, True)])
+@pytest.mark.parametrize('M,T,f16', [(512, 300, False), (512, 300, True), (64, 5, False), (1024, 17, True),
+                                     (512, 1100, False), (512, 1100, True), (1024, 1030, True), (2048, 1024, False), (256, 1500, True)])
 def test_kv_q8_read_round_trip(M, T, f16):
     """the reader: bit-exact against the oracle and the independent numpy decoder; encode -> decode stays within half a
     quantization step of the input (any size); rows addressed by id; a row outside the cache raises bit 1 and is left alone"""

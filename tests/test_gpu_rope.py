@@ -8,7 +8,7 @@ import pytest
 
 import oracle as O
 from caminus_amd import rope
-from gpu_util import F, I, NULL, bits_equal, call, close_16, close_fp32, dev, host, outliers, ptr
+from gpu_util import HADAMARD_FLOOR, F, I, NULL, bits_equal, call, close_16, close_fp32, dev, host, outliers, ptr
 from vectors import qk_par
 
 pytestmark = pytest.mark.gpu
@@ -104,7 +104,8 @@ def test_qk_rope_paged_decode_batch():
     assert bits_equal(host(q16, np.uint16), host(q16f, np.uint16))
     # the oracle on the same inputs: q16 within tolerance, and the same error word
     rq, _, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos, q8=True, rows=n_pages * page, page_table=table, page=page, n_pages=n_pages)
-    assert oerr == 8 and close_16(host(q16, np.uint16), rq, 'f16')
+    # (positions up to 131072: the device's and the host's cosf / sinf differ in the last place there, and q16 lies behind the transform)
+    assert oerr == 8 and close_16(host(q16, np.uint16), rq, 'f16', floor=HADAMARD_FLOOR)
 
 
 def test_qk_rope_paged_refuses_positions_outside_the_table_and_the_cache():
