@@ -87,6 +87,17 @@ class Bench:
         if self.flush_buf is None: self.flush_buf = torch.empty(512 << 20, dtype=torch.uint8, device=self.dev)
         self.flush_buf.fill_(1)
 
+    def ramp(self, seconds=0.25):
+        """keep the GPU busy (device copies of 256 MiB) until it has left its idle clocks"""
+        torch = self.torch
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=self.dev); dst = torch.empty_like(src)
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20): dst.copy_(src)
+            torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     def time_launch(self, fn, reps=50, warm=10, flush=False):
         """median and mean duration (us) of one launch of fn, HIP events on the launch stream"""
         torch = self.torch
@@ -532,6 +543,7 @@ def main():
         sys.exit(2)
     B = Bench()
     torch = B.torch
+    if a.only in ('sweep', 'ladder'): B.ramp()
     if a.only == 'sweep':
         print(json.dumps({'metric': 'fused-op HBM GB/s per entry point at prefill-scale sizes, 1 GPU', 'unit': 'GB/s', 'n_gpus': 1, 'data': 'synthetic',
                           'peak_GBps': HBM_PEAK_GBPS, 'tokens': a.sweep_tokens, 'sweep': prefill_scale_sweep(B, a.sweep_tokens, a.sweep_filter)}))

@@ -2,8 +2,9 @@
 // behind SwiGLU, and scattered to expert columns. Replaces gg_quantize_q8_1 / OP_GG_Q8_1 (kernels/k3_gguf.hip:29-36,
 // kernels/k3_gguf_ops.h:55-77,146-162) and quantize_mmq_q8_1<layout, scatter> (kernels/ggml_mmq/quantize_mmq.cuh:41-140).
 //
-// Layout: 8 lanes x 4 consecutive floats = one 32-value quantization group; a wave covers 256 values per step with one
-// 128-bit load per lane and writes each group's 32 codes as 8 dwords.
+// Layout of the general q8_1 kernel: 8 lanes x 4 consecutive floats = one 32-value quantization group; a wave covers 256 values
+// per step with one 128-bit load per lane. Batches that stream from HBM take a one-lane-per-block kernel (q8_1_blocks) and the
+// one-shot MMQ kernel (swiglu_mmq_oneshot), described where they stand.
 #include "common.cuh"
 #include <mutex>
 
@@ -242,8 +243,9 @@ static int launch_mmq(const MmqArgs & a, int layout, hipStream_t st) {
 //
 // A wave's work item is 8 tokens x one 128-value block column: lane l takes the 8 consecutive values 8 (l & 15) .. + 7 of
 // tokens (l >> 4) and (l >> 4) + 4 (load i = token half i), so that one 128-bit load instruction of g (and of u) fetches
-// four 256-byte row pieces, and the 16 waves of a workgroup, on neighbouring columns of the same 8 tokens, 4 KiB of each
-// row. A 32-value quantization group is the 4 lanes of a quad (for each i), a 128-value block 16 lanes. The reference's
+// four 256-byte row pieces. Items are numbered with the token group running fastest inside a band of four block columns,
+// so the waves that run together read different rows (1 KiB of each) and write four long runs of blocks. A 32-value
+// quantization group is the 4 lanes of a quad (for each i), a 128-value block 16 lanes. The reference's
 // 8 threads of a group are (lane & 3, half): thread 2 (lane & 3) + h holds values 4h .. 4h + 3 of the lane, so its
 // xor 4 / 2 / 1 butterfly is lane ^ 2, lane ^ 1 (quad permutes) and the lane's two halves. Lane (l & 3) == i does
 // group i's two IEEE divisions (127 / amax, 1 / d_inv); the quad reads d_inv back through a DPP broadcast.

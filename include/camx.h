@@ -99,9 +99,9 @@ int camx_quantize_mmq_q8_1_scatter(const float * x, const int32_t * ids, void * 
                                    long ne0, int ne1, int ne2, int n_expert_used, int layout, int ntok, camx_stream_t stream);
 /* Fused SwiGLU -> MMQ q8_1: gu bf16 [T][ld] = [g (F) | u (F)]; act = bf16(bf16(silu g) * u) (silu_mul_bf16,
  * kernels/core.hip:48-55) quantized as quantize_mmq_q8_1 of the fp32-widened act. act (optional, bf16 [T][F]) receives
- * the activation. Fills a per-device lookup table on its first call (synchronizes `stream` once). Finite inputs give
- * camx_silu_mul_bf16's bits; a NaN in the activation (a NaN or infinite input) is stored with the sign and payload of the
- * hardware conversion, not as the canonical 0x7fc0 that camx_silu_mul_bf16 writes (canonicalizing costs this kernel 2.5 %). */
+ * the activation. Fills the per-device lookup tables on its first call (synchronizes `stream` once). Every input gives
+ * camx_silu_mul_bf16's bits: a NaN in the activation (a NaN or infinite input) is stored as the canonical 0x7fc0 that f2bf
+ * (kernels/core.hip:14-21) writes, and the block sums are taken from that value. */
 int camx_swiglu_mmq_q8_1(const uint16_t * gu, long ld, long F, void * vy, uint16_t * act, int T, int layout, camx_stream_t stream);
 
 /* ---- SwiGLU, gates ------------------------------------------------------------------------------------------------------------ */
