@@ -140,6 +140,30 @@ __global__ void __launch_bounds__(256) gdn_conv_k(const void * __restrict__ x, c
     const float r = BF16 ? silu_fast(sumf) : silu_f(sumf);           // bf16 rows: the streaming kernel's form, so a token's bits do not depend on the chunk it came in
     if (BF16) ((uint16_t *)y)[(size_t)t * ldy + c] = to_bf16(r); else ((float *)y)[(size_t)t * ldy + c] = r;
 }
+// OP_GDN_CONV (kernels/k3_q35_ops.h:148-177): the decode / verify form with a lazy commit. Per channel: the state [3] first takes in
+// the mprev tokens of the previous pass that were accepted (its inputs, kept in xprev), and is stored; then the T tokens of this
+// pass are convolved from that state without committing them, and become the next pass's xprev. One thread per channel, the
+// window in registers; the same fma chain and silu as the kernel above.
+__global__ void __launch_bounds__(256) op_gdn_conv_k(const float * __restrict__ w, float * __restrict__ st, const float * __restrict__ x,
+                                                     const int32_t * __restrict__ params, float * __restrict__ y, float * __restrict__ xprev, int C, int T) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    int mprev = params[1];
+    mprev = mprev < 0 ? 0 : (mprev > T ? T : mprev);                 // (the host refuses a commit outside [0, T]; never read past xprev's rows)
+    float s0 = st[(size_t)c * 3], s1 = st[(size_t)c * 3 + 1], s2 = st[(size_t)c * 3 + 2];
+    const f32x4 w4 = *(const f32x4 *)(w + (size_t)c * 4);
+    for (int j = 0; j < mprev; j++) { s0 = s1; s1 = s2; s2 = xprev[(size_t)j * C + c]; }
+    st[(size_t)c * 3] = s0; st[(size_t)c * 3 + 1] = s1; st[(size_t)c * 3 + 2] = s2;
+    for (int t = 0; t < T; t++) {
+        const float xv = x[(size_t)t * C + c];
+        float sumf = 0.0f;
+        sumf = __builtin_fmaf(s0, w4.x, sumf); sumf = __builtin_fmaf(s1, w4.y, sumf);
+        sumf = __builtin_fmaf(s2, w4.z, sumf); sumf = __builtin_fmaf(xv, w4.w, sumf);
+        y[(size_t)t * C + c] = silu_f(sumf);
+        s0 = s1; s1 = s2; s2 = xv;
+        xprev[(size_t)t * C + c] = xv;
+    }
+}
 // Prefill chunks: a lane owns VW consecutive channels and walks TR consecutive tokens, with the rows of the next eight tokens
 // always in flight (a ring of eight 128-bit loads that is refilled as it is consumed) and the four-tap window in registers;
 // one wave per workgroup, so the grid's (channel groups x token ranges) waves spread evenly over the chip.
@@ -506,6 +530,14 @@ int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void 
     const dim3 grid((unsigned)(((long)T * C + 255) / 256)), block(256);
     if (bf16) gdn_conv_k<true><<<grid, block, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
     else gdn_conv_k<false><<<grid, block, 0, st>>>(x, w, state, y, C, T, ldx, ldy);
+    CAMX_LAUNCH_RET();
+}
+// OP_GDN_CONV with its Seg fields (python/caminus/engine/k3.py:993-1000): W = w [C][4], gs = state [C][3] (updated by the commit only),
+// a = x [T][C], asum = the pass parameters (int32, [1] = accepted tokens of the previous pass), y = out [T][C], aux = xprev [T][C],
+// N = C; T = the tape's tokens per pass
+int camx_op_gdn_conv(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, int C, int T, hipStream_t st) {
+    if (!w || !state || !x || !params || !y || !xprev || C < 1 || T < 1 || ((uintptr_t)w & 15)) return CAMX_EINVAL;
+    op_gdn_conv_k<<<dim3((C + 255) / 256), dim3(256), 0, st>>>(w, state, x, params, y, xprev, C, T);
     CAMX_LAUNCH_RET();
 }
 int camx_pf_conv_state(const void * x, float * state, int C, int T, int ldx, int bf16, hipStream_t st) {

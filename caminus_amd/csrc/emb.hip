@@ -106,6 +106,7 @@ struct EmbArgs {
     float * h; uint16_t * h16; uint8_t * q8;
     int * err;               // optional: bit ERR_TOKEN is set when an id lies outside [0, vocab) (the id is clamped either way)
     int stream;              // set by the launcher for large batches: the gathered rows leave as non-temporal stores
+    int key;                 // one token, given as the low half's complement of a 64-bit argmax key word at toks (OP_OWN_EMB's chained draft step)
 };
 
 // EXACT: the row has exactly NI_MAX slabs (straight-line loops: the loads are issued as one batch)
@@ -118,7 +119,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     const int t = SPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
     if (t >= a.n) return;
     auto mine = [&](int j) { return !SPLIT || (j & 3) == wave; };
-    int tok = a.toks[t];
+    int tok = a.key ? (int)~(uint32_t)((const unsigned long long *)a.toks)[0] : a.toks[t];
     if (a.err && (tok < 0 || tok >= a.vocab) && lane == 0) atomicOr(a.err, ERR_TOKEN);
     tok = tok < 0 ? 0 : tok; tok = tok > a.vocab - 1 ? a.vocab - 1 : tok;
     const uint8_t * row = a.W + (size_t)tok * a.rb;
@@ -257,6 +258,16 @@ int camx_q3p_emb(const uint8_t * W, int rb, int vocab, const int32_t * toks, flo
     return launch_emb<FMT_Q4_K>(a, st);
 }
 
+// OP_OWN_EMB with its Seg fields (python/caminus/engine/k3.py:904-921, kernels/k3_own_ops.h:273-304): W = the table, a = tok, y = x
+// [tokens][N], N = D, K = row bytes, work = the format's GG number (4 Q4_K, 7 IQ2_S; 3 Q8_0 as well), pad1 = 1: tok is the 64-bit key
+// word of the greedy pick and the token the complement of its low half (one token), pad2 = vocab, ntask = tokens
+int camx_op_own_emb(const uint8_t * W, const void * tok, float * x, int N, int K, int work, int pad1, int pad2, int tokens, hipStream_t st) {
+    const int fmt = work == 4 ? FMT_Q4_K : work == 7 ? FMT_IQ2_S : work == 3 ? FMT_Q8_0 : -1;
+    if (fmt < 0 || !x || (pad1 != 0 && pad1 != 1) || (pad1 && (tokens != 1 || ((uintptr_t)tok & 7)))) return CAMX_EINVAL;
+    EmbArgs a = {W, K, pad2, (const int32_t *)tok, x, nullptr, N, tokens, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr, nullptr, 0, pad1};
+    const int rc = emb_check(a, fmt);
+    return rc ? rc : launch_emb_fmt(a, fmt, st);
+}
 // gather + dequant with fp32 and / or bf16 outputs; fmt 0 = Q4_K, 1 = Q8_0, 2 = IQ4_XS, 3 = IQ2_S
 int camx_emb_gather(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int N, int n, int fmt, hipStream_t st) {
     EmbArgs a = {W, rb, vocab, toks, x, xbf, N, n, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr, nullptr};

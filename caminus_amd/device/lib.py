@@ -15,6 +15,10 @@ def load():
         p = os.path.join(d, _kernels.LIBNAME)
         if not os.path.isfile(p):
             raise FileNotFoundError(_kernels.missing_message('camx', d, where))
+        # one HIP runtime per process: PyTorch ships its own libamdhip64.so, and the library must resolve to the copy that owns the
+        # caller's device pointers. With torch loaded first the dynamic loader hands the library that copy; the other way round the
+        # library binds to the system's runtime and refuses torch's pointers (hipErrorInvalidValue).
+        import torch  # noqa: F401
         _lib = ctypes.CDLL(p)
         _lib.camx_error_string.restype = ctypes.c_char_p
         _lib.camx_error_string.argtypes = [ctypes.c_int]

@@ -67,6 +67,20 @@ int camx_op_own_add_rms16(float * x, const float * d, const float * w, int S, co
 /* OP_GG_Q8_1 (kernels/k3_gguf_ops.h:55-77) with the tape's Seg fields in their order (python/caminus/engine/k3.py:649-659):
  * a = x, y, N = n, work = 0 plain / 1 silu(x * rs) / 2 silu(x) * gs[i], rs, gs. The same blocks as camx_gg_quantize_q8_1. */
 int camx_op_gg_q8_1(const float * x, void * y, int n, int work, float rs, const float * gs, camx_stream_t stream);
+/* OP_OWN_EMB (kernels/k3_own_ops.h:273-304) with the tape's Seg fields (python/caminus/engine/k3.py:904-921): W = the raw GGUF
+ * table, a = tok, y = x fp32 [tokens][N], N = the row length D, K = row bytes, work = the format's GG number (4 Q4_K, 7 IQ2_S of
+ * kernels/k3_q35t_ops.h:147-175; 3 Q8_0 is taken too), pad1 = 1: tok is the 64-bit key word of OP_OWN_ARGMAX and the token the
+ * complement of its low half (tokens must be 1), pad2 = vocab (ids are clamped to [0, vocab)), ntask = tokens. The same rows as
+ * camx_q3p_emb / camx_emb_gather. */
+int camx_op_own_emb(const uint8_t * W, const void * tok, float * x, int N, int K, int work, int pad1, int pad2, int tokens,
+                    camx_stream_t stream);
+/* OP_GDN_CONV (kernels/k3_q35_ops.h:148-177) with the tape's Seg fields (python/caminus/engine/k3.py:993-1000): the decode / verify
+ * form of the GDN short convolution with a lazy commit. W = w fp32 [C][4], gs = state fp32 [C][3], a = x fp32 [T][C], asum = the
+ * pass parameters (int32; [1] = mprev, the previous pass's accepted tokens, clamped to [0, T]), y = out fp32 [T][C], aux = xprev
+ * fp32 [T][C], N = C; T = the tape's tokens per pass. Per channel: the state first shifts in xprev[0 .. mprev) and is stored; then
+ * out[t] = silu(state . w[0..2] + x[t] w[3]) along the T tokens without storing the state again, and xprev[t] = x[t]. */
+int camx_op_gdn_conv(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, int C, int T,
+                     camx_stream_t stream);
 /* OP_RMS_MUL (kernels/k3_gguf_ops.h:1233-1268; Seg fields: a = x, W = w, y, asum = q8, N = R, K, pad1 = wr, rs = eps). */
 int camx_op_rms_mul(const float * x, const float * w, float * y, void * q8, int R, int wr, int K, float eps, camx_stream_t stream);
 /* pf_hc_post_rms (kernels/prefill_glue.hip:130-170): row q = t * HC + h of N values: res[q] = fma(b[t], 2 sigmoid(inj[q] * rs),

@@ -263,6 +263,15 @@ def gdn_conv(x, w, st, ldx=None, ldy=None):
     return y, st
 
 
+def op_gdn_conv(w, st, x, mprev, xprev):
+    """OP_GDN_CONV -> (y [T, C], state after the commit [C, 3], xprev for the next pass [T, C])"""
+    x = _c(x, np.float32); w = _c(w, np.float32); st = _c(st, np.float32).copy(); xprev = _c(xprev, np.float32).copy()
+    T, C_ = x.shape
+    params = np.array([0, mprev, 0, 0], np.int32); y = np.zeros((T, C_), np.float32)
+    lib().orc_op_gdn_conv(_p(w), _p(st), _p(x), _p(params), _p(y), _p(xprev), I(C_), I(T))
+    return y, st, xprev
+
+
 def gdn_l2(x, T, heads, K, eps, ldx=None):
     x = _c(x, np.float32); ldx = heads * K if ldx is None else ldx
     y = np.empty((T * heads, K), np.float32)

@@ -451,6 +451,27 @@ ORC_API void orc_gdn_conv(const float * x, const float * w, const float * st, fl
             y[(size_t)t * ldy + c] = silu_f(sumf);
         }
 }
+/* OP_GDN_CONV (kernels/k3_q35_ops.h:148-177): commit mprev tokens of xprev into the state, store it, convolve this pass's T tokens
+ * from it without committing them, keep them as the next pass's xprev. (The sum of products is left to the compiler's contraction
+ * in the reference: tolerance class; stated here as the fma chain of orc_gdn_conv.) */
+ORC_API void orc_op_gdn_conv(const float * w, float * st, const float * x, const int32_t * params, float * y, float * xprev, int C, int T) {
+    int mprev = params[1];
+    mprev = mprev < 0 ? 0 : (mprev > T ? T : mprev);
+    for (int c = 0; c < C; c++) {
+        float s0 = st[(size_t)c * 3], s1 = st[(size_t)c * 3 + 1], s2 = st[(size_t)c * 3 + 2];
+        for (int j = 0; j < mprev; j++) { s0 = s1; s1 = s2; s2 = xprev[(size_t)j * C + c]; }
+        st[(size_t)c * 3] = s0; st[(size_t)c * 3 + 1] = s1; st[(size_t)c * 3 + 2] = s2;
+        for (int t = 0; t < T; t++) {
+            const float xv = x[(size_t)t * C + c];
+            float sumf = 0.0f;
+            sumf = fmaf(s0, w[(size_t)c * 4], sumf); sumf = fmaf(s1, w[(size_t)c * 4 + 1], sumf);
+            sumf = fmaf(s2, w[(size_t)c * 4 + 2], sumf); sumf = fmaf(xv, w[(size_t)c * 4 + 3], sumf);
+            y[(size_t)t * C + c] = silu_f(sumf);
+            s0 = s1; s1 = s2; s2 = xv;
+            xprev[(size_t)t * C + c] = xv;
+        }
+    }
+}
 ORC_API void orc_conv_state(const float * x, float * st, int C, int T, int ldx) {
     for (int c = 0; c < C; c++) {
         float s[3];

@@ -152,3 +152,26 @@ def test_cast_bf16_every_upper_half_with_edge_lower_halves():
     c1 = dev(np.zeros(x.size - 1, np.uint16))                             # the element-wise form
     call('camx_cast_bf16', ptr(dev(x)), ptr(c1), L64(x.size - 1))
     assert bits_equal(host(c1, np.uint16), O.f2bf(x)[:-1])
+
+
+@pytest.mark.parametrize('C,T', [(10240, 16), (96, 5), (300, 1)])
+def test_op_gdn_conv_lazy_commit(C, T):
+    """OP_GDN_CONV: two passes with every commit count; the state after the commit and the next pass's xprev bit for bit, the outputs
+    within the FP class (silu) and equal to the chunk kernel's on the same state"""
+    from gpu_util import close_fp32
+    rng = np.random.default_rng(C + T)
+    w = rng.standard_normal((C, 4)).astype(np.float32); st0 = rng.standard_normal((C, 3)).astype(np.float32)
+    x1 = outliers(rng, (T, C)); x2 = outliers(rng, (T, C)); junk = rng.standard_normal((T, C)).astype(np.float32)
+    wd = dev(w)
+    for m in sorted({0, 1, T // 2, T}):
+        std = dev(st0); xp = dev(junk); y = dev(np.zeros((T, C), np.float32))
+        call('camx_op_gdn_conv', ptr(wd), ptr(std), ptr(dev(x1)), ptr(dev(np.array([0, 0, 0, 0], np.int32))), ptr(y), ptr(xp), I(C), I(T))
+        ry1, rst1, rxp1 = O.op_gdn_conv(w, st0, x1, 0, junk)
+        assert bits_equal(host(std), rst1) and bits_equal(host(xp), rxp1) and close_fp32(host(y), ry1)
+        y2 = dev(np.zeros((T, C), np.float32))
+        call('camx_op_gdn_conv', ptr(wd), ptr(std), ptr(dev(x2)), ptr(dev(np.array([7, m, 0, 0], np.int32))), ptr(y2), ptr(xp), I(C), I(T))
+        ry2, rst2, rxp2 = O.op_gdn_conv(w, rst1, x2, m, rxp1)
+        assert bits_equal(host(std), rst2) and bits_equal(host(xp), rxp2) and close_fp32(host(y2), ry2)
+        yc = dev(np.zeros((T, C), np.float32))                      # the chunk kernel from the committed state: the same bits
+        call('camx_pf_gdn_conv', ptr(dev(x2)), ptr(wd), ptr(std), ptr(yc), I(C), I(T), I(C), I(C), I(0))
+        assert bits_equal(host(yc), host(y2))

@@ -115,3 +115,31 @@ def test_ple_rows_iq4nl(nuniq, nrows, bpr):
     assert e1 == 1 and int(host(err)[0]) == 1 and bits_equal(host(out), want)
     with pytest.raises(ValueError):
         mod.ple_rows_iq4nl((1,), (256,), rawd, invd, ctypes.c_int(nuniq), ctypes.c_int(nrows + 300), ctypes.c_int(bpr), out, err)
+
+
+def test_op_own_emb_tape_fields():
+    """OP_OWN_EMB with the Seg's fields: the same rows as the prefill entry points; the drafter's key form (the token is the complement
+    of the low half of a 64-bit argmax key); a format the op does not have is refused"""
+    rng = np.random.default_rng(77)
+    N, vocab, n = 2048, 500, 9
+    table = q4k_table(rng, vocab, N); rb = table.shape[1]
+    toks = rng.integers(0, vocab, n).astype(np.int32); toks[:2] = [-3, vocab + 1]
+    ref_x, _ = O.emb_q4k(table, vocab, toks, N)
+    Wd = dev(table); x = dev(np.zeros((n, N), np.float32))
+    call('camx_op_own_emb', ptr(Wd), ptr(dev(toks)), ptr(x), I(N), I(rb), I(4), I(0), I(vocab), I(n))
+    assert bits_equal(host(x), ref_x)
+    tok = 123
+    key = np.array([(0x3f80_0000 << 32) | (~tok & 0xffffffff)], np.uint64)
+    x1 = dev(np.zeros((1, N), np.float32))
+    call('camx_op_own_emb', ptr(Wd), ptr(dev(key.view(np.int64))), ptr(x1), I(N), I(rb), I(4), I(1), I(vocab), I(1))
+    assert bits_equal(host(x1), O.emb_q4k(table, vocab, np.array([tok], np.int32), N)[0])
+    import ctypes as C
+    from gpu_util import camx
+    dp = lambda t: C.c_void_p(t.data_ptr())
+    td, kd = dev(toks), dev(key.view(np.int64))
+    assert camx().camx_op_own_emb(dp(Wd), dp(td), dp(x), I(N), I(rb), I(9), I(0), I(vocab), I(n), NULL) == 1            # a format the op does not have
+    assert camx().camx_op_own_emb(dp(Wd), dp(kd), dp(x), I(N), I(rb), I(4), I(1), I(vocab), I(2), NULL) == 1            # the key form is one token
+    t80 = q80_table(rng, vocab, N)
+    x2 = dev(np.zeros((n, N), np.float32))
+    call('camx_op_own_emb', ptr(dev(t80)), ptr(dev(toks)), ptr(x2), I(N), I(t80.shape[1]), I(3), I(0), I(vocab), I(n))
+    assert bits_equal(host(x2), O.emb_q8_0(t80, vocab, toks, N)[0])

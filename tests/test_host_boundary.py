@@ -225,6 +225,7 @@ ENTRY_CASES = {
     'camx_add_rms_bf16': ([P, P, P, Cf(1e-6), P, P, Ci(5120), Ci(0)], [(0, NUL), (2, NUL), (6, Ci(0)), (7, Ci(-2))]),
     'camx_rmsnorm_f32': ([P, P, P, Ci(896), Cf(1e-6), Ci(0)], [(0, NUL), (2, NUL), (3, Ci(0)), (5, Ci(-1))]),
     'camx_gg_quantize_q8_1': ([P, P, Cl(0), Ci(0), Cf(0), NUL], [(0, NUL), (1, NUL), (3, Ci(3)), (3, Ci(2)), (1, ODD), (2, Cl(-1))]),
+    'camx_op_own_emb': ([P, P, P, Ci(2048), Ci(1152), Ci(4), Ci(0), Ci(1000), Ci(0)], [(0, NUL), (2, NUL), (5, Ci(9)), (6, Ci(2)), (3, Ci(100)), (4, Ci(100)), (7, Ci(0))]),
     'camx_q3p_swiglu': ([P, P, P, Ci(0)], [(0, NUL), (2, NUL), (3, Ci(-1))]),
     'camx_silu_mul_bf16': ([P, P, Ci(17408), Cl(0)], [(0, NUL), (2, Ci(0)), (3, Cl(5))]),
     'camx_q3p_qk_rope': ([P, Ci(5120), Ci(32), Ci(4), P, Ci(0), P, P, Ci(0), Ci(0)], [(0, NUL), (4, NUL), (1, Ci(100)), (8, Ci(-1))]),

@@ -794,3 +794,31 @@ def test_yarn_table_bits_against_the_reference_fixture():
         got = rope.yarn_table(n_rot, base, factor, ctx)
         assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32)), case
         assert rope.mscale(factor) == ms and tuple(rope.corr_dims(n_rot, ctx, base)) == tuple(corr)
+
+
+def test_op_gdn_conv_is_the_chunk_conv_with_a_lazy_commit():
+    """OP_GDN_CONV (kernels/k3_q35_ops.h:148-177) against what already is pinned and against float64: (a) with nothing to commit its
+    outputs are the prefill conv's on the same state and the state stays; (b) pass 2 with m tokens of pass 1 accepted equals the
+    prefill conv run on (state advanced over those m tokens); (c) xprev becomes this pass's inputs; (d) a float64 statement of the
+    window sum and silu, within the FP class"""
+    rng = np.random.default_rng(31)
+    C, T = 96, 5
+    w = rng.standard_normal((C, 4)).astype(np.float32); st0 = rng.standard_normal((C, 3)).astype(np.float32)
+    x1 = rng.standard_normal((T, C)).astype(np.float32); x2 = rng.standard_normal((T, C)).astype(np.float32)
+    junk = rng.standard_normal((T, C)).astype(np.float32)
+    y1, st1, xp1 = O.op_gdn_conv(w, st0, x1, 0, junk)
+    yref, _ = O.gdn_conv(x1, w, st0)
+    assert np.array_equal(y1.view(np.uint32), yref.view(np.uint32)) and np.array_equal(st1, st0) and np.array_equal(xp1, x1)
+    for m in (0, 1, 3, T):
+        y2, st2, xp2 = O.op_gdn_conv(w, st1, x2, m, xp1)
+        _, st_adv = O.gdn_conv(x1[:m], w, st0) if m else (None, st0)
+        yref2, _ = O.gdn_conv(x2, w, st_adv)
+        assert np.array_equal(st2, st_adv) and np.array_equal(y2.view(np.uint32), yref2.view(np.uint32)) and np.array_equal(xp2, x2)
+        win = np.concatenate([st_adv.T.astype(np.float64), x2.astype(np.float64)])          # [3 + T, C]
+        s = sum(win[j:j + T] * w[:, j].astype(np.float64) for j in range(4))
+        want = s / (1.0 + np.exp(-s))
+        assert np.abs(y2 - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+    # a commit count outside [0, T] is clamped (the host refuses it before the launch; the statement never reads past xprev)
+    y3, st3, _ = O.op_gdn_conv(w, st1, x2, T + 9, xp1)
+    y4, st4, _ = O.op_gdn_conv(w, st1, x2, T, xp1)
+    assert np.array_equal(y3, y4) and np.array_equal(st3, st4)
