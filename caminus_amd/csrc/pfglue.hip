@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(256) add_sum_k(const float * __restrict__ a, c
     const long q = (long)blockIdx.x * 256 + threadIdx.x;
     if (vec) {
         if (q * 4 >= n) return;
-        const f32x4 av = __builtin_nontemporal_load((const f32x4 *)a + q), bv = __builtin_nontemporal_load((const f32x4 *)b + q), yv = ((const f32x4 *)y)[q];
+        const f32x4 av = __builtin_nontemporal_load((const f32x4 *)a + q), bv = __builtin_nontemporal_load((const f32x4 *)b + q), yv = __builtin_nontemporal_load((const f32x4 *)y + q);
         f32x4 r; r.x = yv.x + (av.x + bv.x); r.y = yv.y + (av.y + bv.y); r.z = yv.z + (av.z + bv.z); r.w = yv.w + (av.w + bv.w);
         __builtin_nontemporal_store(r, (f32x4 *)y + q);
     } else {
@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(256) hc_avg_k(const float * __restrict__ r, fl
         f32x4 acc = __builtin_nontemporal_load((const f32x4 *)(r + (size_t)(tt * hc) * D + ii));
         for (int h = 1; h < hc; h++) acc = acc + __builtin_nontemporal_load((const f32x4 *)(r + (size_t)(tt * hc + h) * D + ii));
         acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
-        *(f32x4 *)(y + (size_t)tt * ldo + ii) = acc;
+        if (vec == 2) __builtin_nontemporal_store(acc, (f32x4 *)(y + (size_t)tt * ldo + ii)); else *(f32x4 *)(y + (size_t)tt * ldo + ii) = acc;     // (2: a batch that streams from HBM)
     } else {
         float acc = r[(size_t)(tt * hc) * D + ii];
         for (int h = 1; h < hc; h++) acc = acc + r[(size_t)(tt * hc + h) * D + ii];
@@ -335,7 +335,7 @@ int camx_pf_to_bf16(const float * x, int ldx, uint16_t * y, int T, int Tpad, int
 int camx_pf_hc_avg(const float * r, float * y, int T, int hc, int D, int ldo, hipStream_t st) {
     if (!r || !y || T < 0 || hc < 1 || D < 1 || ldo < D) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
-    const int vec = !((D | ldo) & 3) && !(((uintptr_t)r | (uintptr_t)y) & 15);
+    const int vec = !((D | ldo) & 3) && !(((uintptr_t)r | (uintptr_t)y) & 15) ? ((long)T * D >= (1L << 20) ? 2 : 1) : 0;
     const long n = (long)T * D / (vec ? 4 : 1);
     hc_avg_k<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(r, y, T, hc, D, ldo, vec);
     CAMX_LAUNCH_RET();
