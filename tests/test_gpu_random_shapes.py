@@ -21,7 +21,7 @@ def _generators(r):
     ri, ch = r.randint, r.choice
 
     def rows():
-        return ch([1, 2, 3, 5, 8, 17, 64, 255, 256, 257, 300, 515, 1030])
+        return ch([1, 2, 3, 5, 8, 17, 64, 255, 256, 257, 300, 515, 1023, 1024, 1025, 1026, 1030])
 
     def silu_actq():
         m, f = ri(2, 40), 128 * ri(1, 24)
@@ -61,7 +61,7 @@ def _generators(r):
         (Q.test_mmq_quantize, lambda: (4 * ri(1, 2500), ri(1, 700), ri(0, 1))),
         (Q.test_mmq_quantize_scatter, lambda: (4 * ri(1, 1000), ri(1, 40), ri(1, 8))),
         (Q.test_swiglu_mmq, lambda: (ri(1, 400), ch([4, 8]) * ri(1, 600), 8 * ri(0, 3), ri(0, 1))),
-        (RP.test_qk_rope_f16_and_q8, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 5, 33, 2048, 2051]), ri(0, 120000), ch([False, True]))),
+        (RP.test_qk_rope_f16_and_q8, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 5, 33, 256, 257, 2048, 2051]), ri(0, 120000), ch([False, True]))),
         (RP.test_pf_qk_nr, qk_nr),
         (RP.test_qk_rope_bf16, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 7, 2049]), ri(0, 120000), ch([False, True]), 8 * ri(0, 3))),
     ]
