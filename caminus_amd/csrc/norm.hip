@@ -107,13 +107,20 @@ __global__ void __launch_bounds__(256) add_rms_rows(NormArgs a) {
     }
     if (ADD == ADD_F32_DIRECT && a.d) {
         const float * dr = (const float *)a.d + (size_t)row * N;
-        f32x4 dv[NI_MAX];
+        // the chunk form of long rows takes the addend in two halves: 162 instead of 198 registers for a 5120-wide row, three waves per
+        // SIMD instead of two (4096 x 5120: 68.0 -> 66.6 us)
+        constexpr int HB = (OUT && NI_MAX > 12) ? (NI_MAX + 1) / 2 : NI_MAX;
 #pragma unroll
-        for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) { dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
+        for (int b0 = 0; b0 < NI_MAX; b0 += HB) {
+            f32x4 dv[HB];
 #pragma unroll
-        for (int j = 0; j < NI_MAX; j++)
-            if (j < ni) xv[j] = xv[j] + dv[j];
+            for (int j = 0; j < HB; j++)
+                if (b0 + j < ni && b0 + j < NI_MAX) { dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + 256 * (b0 + j) + 4 * lane)); CAMX_ISSUE_GAP(); }
+#pragma unroll
+            for (int j = 0; j < HB; j++)
+                if (b0 + j < ni && b0 + j < NI_MAX) xv[b0 + j] = xv[b0 + j] + dv[j];
+            if (HB < NI_MAX) __builtin_amdgcn_sched_barrier(0);
+        }
     }
     if (ADD == ADD_BF16 && a.d) {
         const uint16_t * dr = (const uint16_t *)a.d + (size_t)row * N;
@@ -357,16 +364,22 @@ __global__ void __launch_bounds__(256) add_rms_bf16_chunk(float * __restrict__ x
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(nw + 256 * j + 4 * lraw), (__attribute__((address_space(3))) void *)(gsh + 256 * j), 16, 0, 0);
     float * xr = x + row * N;
     const uint16_t * dr = d + row * N;
-    f32x4 xv[NI]; u32x2 dv[NI];
+    f32x4 xv[NI]; u32x2 dv[NI > 12 ? (NI + 1) / 2 : NI];
     // (the pause between requests: 4096 waves that each fire 40 requests at once measured 2 % slower than the same requests a few dozen cycles apart)
 #define CAMX_ISSUE_GAP() do { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_sleep(1); __builtin_amdgcn_sched_barrier(0); } while (0)
 #pragma unroll
     for (int j = 0; j < NI; j++) { xv[j] = __builtin_nontemporal_load((const f32x4 *)(xr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
+    // (long rows take the addend in two halves: fewer registers, one more wave per SIMD; 4096 x 5120: 44.1 -> 43.5 us, three parts: 44.6)
+    constexpr int HB = NI > 12 ? (NI + 1) / 2 : NI;
 #pragma unroll
-    for (int j = 0; j < NI; j++) { dv[j] = __builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
+    for (int b0 = 0; b0 < NI; b0 += HB) {
+#pragma unroll
+        for (int j = b0; j < b0 + HB && j < NI; j++) { dv[j - b0] = __builtin_nontemporal_load((const u32x2 *)(dr + 256 * j + 4 * lane)); CAMX_ISSUE_GAP(); }
+#pragma unroll
+        for (int j = b0; j < b0 + HB && j < NI; j++) xv[j] = xv[j] + unpack_bf16x4(dv[j - b0]);
+        if (HB < NI) __builtin_amdgcn_sched_barrier(0);
+    }
 #undef CAMX_ISSUE_GAP
-#pragma unroll
-    for (int j = 0; j < NI; j++) xv[j] = xv[j] + unpack_bf16x4(dv[j]);
 #pragma unroll
     for (int j = 0; j < NI; j++) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j + 4 * lane));
     f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
