@@ -132,16 +132,30 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
 #pragma unroll
         for (int j = 0; j < NI_MAX; j++)
             if (j < ni) {
-                if (mine(j)) gpre[j] = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
+                if (mine(j) && !(SPLIT && EXACT && NI_MAX % 4 == 0)) gpre[j] = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
                 if (a.d) dpre[j] = *(const f32x4 *)(a.d + (size_t)t * N + 256 * j + 4 * lane);
             }
     }
     // every table load first, then the stores: a load written after a store that might alias it cannot be hoisted above it,
     // and the row would cost one memory round trip per slab
     f32x4 xv[NI_MAX];
+    if (SPLIT && TAIL && FMT != FMT_Q8_0) {
+        // a workgroup per row with a tail: each wave decodes its own slabs and the four share them through LDS (with one wave per SIMD
+        // every instruction of a wave is latency: 270 fewer of them per wave than decoding a Q4_K row four times; Q8_0 decodes in two
+        // loads and four converts per lane, which the exchange does not beat)
+        __shared__ f32x4 xs[NI_MAX][64];
 #pragma unroll
-    for (int j = 0; j < NI_MAX; j++)
-        if (j < ni && (TAIL || mine(j))) xv[j] = emb_decode4<FMT>(row, j, lane);
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni && mine(j)) { xv[j] = emb_decode4<FMT>(row, j, lane); xs[j][lane] = xv[j]; }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni && !mine(j)) xv[j] = xs[j][lane];
+    } else {
+#pragma unroll
+        for (int j = 0; j < NI_MAX; j++)
+            if (j < ni && (TAIL || mine(j))) xv[j] = emb_decode4<FMT>(row, j, lane);
+    }
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni && mine(j)) {
@@ -173,6 +187,23 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
         }
     const float tot = wave_groups_in_order(group32_sum(ss));
     const float scale = rsqrt_exact(tot / (float)N + a.eps);
+    if (SPLIT && EXACT && NI_MAX % 4 == 0) {
+        // the wave's slabs wave, wave + 4, .. picked out of the register array by selects on the (uniform) wave number, so that their
+        // conversions and q8_1 blocks are one straight run of code and overlap each other's latencies
+#pragma unroll
+        for (int s = 0; s < NI_MAX / 4; s++) {
+            const int j = wave + 4 * s;
+            const f32x4 xa = wave == 0 ? xv[4 * s] : wave == 1 ? xv[4 * s + 1] : wave == 2 ? xv[4 * s + 2] : xv[4 * s + 3];
+            const f32x4 g = *(const f32x4 *)(a.nw + 256 * j + 4 * lane);
+            f32x4 v;
+            v.x = (xa.x * scale) * g.x; v.y = (xa.y * scale) * g.y; v.z = (xa.z * scale) * g.z; v.w = (xa.w * scale) * g.w;
+            const size_t o = (size_t)t * N + 256 * j + 4 * lane;
+            if (a.h) *(f32x4 *)(a.h + o) = v;
+            if (a.h16) *(u32x2 *)(a.h16 + o) = pack_f16x4(v);
+            if (a.q8) q8_1_emit(v, a.q8 + ((size_t)t * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < NI_MAX; j++)
         if (j < ni && mine(j)) {
