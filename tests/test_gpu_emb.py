@@ -28,10 +28,12 @@ def test_gather_q4k_q80(N, vocab, n):
 
 @pytest.mark.parametrize('fmt', [0, 1])
 @pytest.mark.parametrize('with_add', [False, True])
-def test_gather_add_rms_q8_1(fmt, with_add):
-    """config-2 op-set: gather + dequant -> fp32 + bf16, then (add +) RMSNorm + q8_1 from the same registers"""
-    rng = np.random.default_rng(1002 + fmt)
-    N, vocab, n = 2048, 4096, 256
+@pytest.mark.parametrize('N,n', [(2048, 256), (1024, 37), (4096, 130), (5120, 19), (2560, 40), (2048, 300)])
+def test_gather_add_rms_q8_1(fmt, with_add, N, n):
+    """config-2 op-set: gather + dequant -> fp32 + bf16, then (add +) RMSNorm + q8_1 from the same registers; every row width of the
+    workgroup-per-row form (up to 256 rows) and one batch beyond it"""
+    rng = np.random.default_rng(1002 + fmt + N)
+    vocab = 4096 if N == 2048 else 300
     table = (q4k_table if fmt == 0 else q80_table)(rng, vocab, N)
     toks = rng.integers(0, vocab, n).astype(np.int32)
     nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
