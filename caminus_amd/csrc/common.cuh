@@ -186,6 +186,59 @@ CAMX_DEV void q8_1_emit(f32x4 v, uint8_t * blk, int sub) {
     if (sub == 0) *(uint32_t *)blk = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
 }
 
+// ---- q8_1 block of 32 consecutive floats in LDS, all of it in one lane -------------------------------------------------------
+// in: the block's 32 values; out: its 9 dwords (LDS); rot: the lane's number (the pieces are read in the order rot, rot + 1, ..
+// mod 8, so that the lanes of a request fall on different banks). The sum keeps the 32-thread butterfly's tree (xor 16, 8, 4, 2, 1
+// over one value per thread): its first three levels add the 4-value pieces c and c + 4, then c and c + 2, then the last two, its
+// last two levels the four sums left; each level pairs pieces half a period apart, so the rotation changes no operand pair, and
+// max and the codes do not depend on order. Codes: v * (1 / d) rounded to nearest is roundf(v / d) whenever it is farther than
+// 2^-15 from a half-integer (|v / d| <= 127 and the refined reciprocal is within an ulp); a piece in which some lane's value is
+// closer, infinite or NaN is redone with the division (every lane of the wave must be here: the decision is a ballot).
+// MODE 1: the values are silu(v * rs) first (OP_GG_Q8_1's mode 1).
+CAMX_DEV float silu_div(float x) { return x / (1.0f + expf(-x)); }
+template <int MODE>
+CAMX_DEV void q8_1_block_lane(const float * in, uint32_t * out, int rot, float rs) {
+    f32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = *(const f32x4 *)(in + 4 * ((k + rot) & 7));
+    if (MODE == 1) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) { v[k].x = silu_div(v[k].x * rs); v[k].y = silu_div(v[k].y * rs); v[k].z = silu_div(v[k].z * rs); v[k].w = silu_div(v[k].w * rs); }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) amax = fmaxf(amax, absmax4(v[k]));
+    const f32x4 s0 = v[0] + v[4], s1 = v[1] + v[5], s2 = v[2] + v[6], s3 = v[3] + v[7];
+    const f32x4 u0 = s0 + s2, u1 = s1 + s3;
+    const f32x4 w = u0 + u1;
+    const float w0 = w.x + w.z, w1 = w.y + w.w;
+    const float sum = w0 + w1;
+    const float d = amax / 127.0f;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // (out may lie where other lanes' values were)
+    out[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
+    float r = __builtin_amdgcn_rcpf(d);
+    r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        float p[4] = {v[k].x * r, v[k].y * r, v[k].z * r, v[k].w * r};
+        int c[4];
+        bool safe = true;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float n = __builtin_rintf(p[e]);
+            safe &= fabsf(p[e] - n) <= 0.49996948f;                        // (false for NaN and for an infinite p)
+            c[e] = (int)n;
+        }
+        if (__builtin_amdgcn_ballot_w64(!safe && amax != 0.0f) != 0) {
+            p[0] = v[k].x / d; p[1] = v[k].y / d; p[2] = v[k].z / d; p[3] = v[k].w / d;
+#pragma unroll
+            for (int e = 0; e < 4; e++) c[e] = (int)(p[e] + __builtin_copysignf(0.49999997f, p[e]));
+        }
+        const uint32_t codes = ((uint32_t)c[0] & 0xffu) | (((uint32_t)c[1] & 0xffu) << 8) | (((uint32_t)c[2] & 0xffu) << 16) | ((uint32_t)c[3] << 24);
+        out[1 + ((k + rot) & 7)] = amax != 0.0f ? codes : 0u;
+    }
+}
+
 // ---- Q8 KV wire block (34 bytes) of 32 values held by 8 lanes x 4 registers ----------------------------------------------
 // amax / 127, its fp32 reciprocal, roundf(x * inv), only the stored scale rounded to half. A refused block (non-finite
 // input; nonzero block whose scale underflows, whose reciprocal overflows or whose half scale is not finite) keeps its

@@ -91,14 +91,8 @@ __global__ void __launch_bounds__(256) q8_1_flat(const float * __restrict__ x, u
 // The same blocks for a batch that streams from HBM (modes 0 and 1, whole steps of 2048 values, 16-byte aligned): one lane per
 // block. With four values per lane, as above, the eight lanes of a block each repeat the block's divide and walk two
 // butterflies, and the vector ALUs, not HBM, set the time. Here a wave's 2048 values go to its own LDS as they arrive (16 bytes
-// per lane, neighbouring lanes on neighbouring addresses, no registers held), lane l then reads block l whole, and everything
-// per block happens once. The sum keeps the 32-thread butterfly's tree (xor 16, 8, 4, 2, 1 over one value per thread): its
-// first three levels add the block's 4-value pieces c and c + 4, then c and c + 2, then the last two, its last two levels
-// the four sums left. A lane reads its pieces in the order l, l + 1, .. (mod 8), so that the lanes of a request fall on
-// different banks; each level pairs pieces half a period apart, so the rotation changes no operand pair, and max and the
-// codes do not depend on order. Codes: v * (1 / d) rounded to nearest is roundf(v / d) whenever it is farther than 2^-15
-// from a half-integer (|v / d| <= 127 and the refined reciprocal is within an ulp); a piece in which some lane's value
-// is closer, infinite or NaN (one in sixty) is redone with the division.
+// per lane, neighbouring lanes on neighbouring addresses, no registers held), lane l then quantizes block l whole
+// (q8_1_block_lane: everything per block happens once, same sum tree), and the blocks leave as 16-byte stores.
 template <int MODE>
 __global__ void __launch_bounds__(256) q8_1_blocks(const float * __restrict__ x, uint8_t * __restrict__ y, float rs) {
     __shared__ __attribute__((aligned(16))) float in_all[4][2048];
@@ -112,45 +106,7 @@ __global__ void __launch_bounds__(256) q8_1_blocks(const float * __restrict__ x,
     for (int i = 0; i < 8; i++)
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + 256 * i + 4 * l), (__attribute__((address_space(3))) void *)(in + 256 * i), 16, 0, 2);
     __builtin_amdgcn_s_waitcnt(0x0f70);                                    // vmcnt(0): the wave's own values have landed
-    f32x4 v[8];
-#pragma unroll
-    for (int k = 0; k < 8; k++) v[k] = *(const f32x4 *)(in + 32 * l + 4 * ((k + l) & 7));
-    if (MODE == 1) {
-#pragma unroll
-        for (int k = 0; k < 8; k++) { v[k].x = silu_f(v[k].x * rs); v[k].y = silu_f(v[k].y * rs); v[k].z = silu_f(v[k].z * rs); v[k].w = silu_f(v[k].w * rs); }
-    }
-    float amax = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 8; k++) amax = fmaxf(amax, absmax4(v[k]));
-    const f32x4 s0 = v[0] + v[4], s1 = v[1] + v[5], s2 = v[2] + v[6], s3 = v[3] + v[7];
-    const f32x4 u0 = s0 + s2, u1 = s1 + s3;
-    const f32x4 w = u0 + u1;
-    const float w0 = w.x + w.z, w1 = w.y + w.w;
-    const float sum = w0 + w1;
-    const float d = amax / 127.0f;
-    uint32_t * blk = stage + 9 * l;
-    blk[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
-    float r = __builtin_amdgcn_rcpf(d);
-    r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        float p[4] = {v[k].x * r, v[k].y * r, v[k].z * r, v[k].w * r};
-        int c[4];
-        bool safe = true;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const float n = __builtin_rintf(p[e]);
-            safe &= fabsf(p[e] - n) <= 0.49996948f;                        // (false for NaN and for an infinite p)
-            c[e] = (int)n;
-        }
-        if (__builtin_amdgcn_ballot_w64(!safe && amax != 0.0f) != 0) {
-            p[0] = v[k].x / d; p[1] = v[k].y / d; p[2] = v[k].z / d; p[3] = v[k].w / d;
-#pragma unroll
-            for (int e = 0; e < 4; e++) c[e] = (int)(p[e] + __builtin_copysignf(0.49999997f, p[e]));
-        }
-        const uint32_t codes = ((uint32_t)c[0] & 0xffu) | (((uint32_t)c[1] & 0xffu) << 8) | (((uint32_t)c[2] & 0xffu) << 16) | ((uint32_t)c[3] << 24);
-        blk[1 + ((k + l) & 7)] = amax != 0.0f ? codes : 0u;
-    }
+    q8_1_block_lane<MODE>(in + 32 * l, stage + 9 * l, l, rs);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // the wave's own LDS writes, in order
     u32x4 * dst = (u32x4 *)(y + step * 2304);
     __builtin_nontemporal_store(*(const u32x4 *)(stage + 4 * l), dst + l);
