@@ -13,6 +13,7 @@
 // Sums of the backward pass (dL/ds, the tie count, the RMSNorm dot) follow one fixed tree: a lane adds its terms in chunk
 // order with fmaf, the 32 lanes of a half-wave combine by xor 16, 8, 4, 2, 1, the eight half-wave sums are added in order.
 #include "common.cuh"
+#include <mutex>
 
 #define HSCALE 0.08837890625f      // bf16(1 / sqrt(128))
 
@@ -37,6 +38,7 @@ struct PlainF32 {
     static constexpr bool bf16_valued = false; static constexpr int NW = 2;
     const float * x; int K;
     CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); }
+    CAMX_DEV f32x4 operator()(int row, int k, u32x2 &) const { return (*this)(row, k); }
     CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { const u32x4 * p = (const u32x4 *)(x + (size_t)row * K + k); w[0] = p[0]; w[1] = p[1]; }
     CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b) const { a = __builtin_bit_cast(f32x4, w[0]); b = __builtin_bit_cast(f32x4, w[1]); }
 };
@@ -44,6 +46,7 @@ struct PlainBF16 {
     static constexpr bool bf16_valued = true; static constexpr int NW = 1;
     const uint16_t * x; int K;
     CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); }
+    CAMX_DEV f32x4 operator()(int row, int k, u32x2 &) const { return (*this)(row, k); }
     CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { w[0] = *(const u32x4 *)(x + (size_t)row * K + k); }
     CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b) const { unpack_bf16x8(w[0], a, b); }
 };
@@ -51,15 +54,16 @@ struct SiluMulSrc {
     static constexpr bool bf16_valued = true;      // the activation is rounded to bf16 as it is formed
     const uint16_t * gu; int ld, F;
     const uint16_t * lut;                          // bf16(silu g) for every bf16 g (the table silu_mul_bf16 uses: the same activation bits)
-    CAMX_DEV f32x4 operator()(int row, int k) const {
+    CAMX_DEV f32x4 operator()(int row, int k, u32x2 & keep) const {          // keep: the four bf16(silu g), for the backward's sink
         const uint16_t * r = gu + (size_t)row * ld;
         const u32x2 gw = *(const u32x2 *)(r + k);
         const f32x4 u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
-        f32x4 a;
-        a.x = rbf(bf2f(lut[gw.x & 0xffffu]) * u.x); a.y = rbf(bf2f(lut[gw.x >> 16]) * u.y);
-        a.z = rbf(bf2f(lut[gw.y & 0xffffu]) * u.z); a.w = rbf(bf2f(lut[gw.y >> 16]) * u.w);
-        return a;
+        keep.x = (uint32_t)lut[gw.x & 0xffffu] | ((uint32_t)lut[gw.x >> 16] << 16);
+        keep.y = (uint32_t)lut[gw.y & 0xffffu] | ((uint32_t)lut[gw.y >> 16] << 16);
+        const f32x4 sl = unpack_bf16x4(keep);
+        return rbf4_any((f32x4){sl.x * u.x, sl.y * u.y, sl.z * u.z, sl.w * u.w});      // (feeds the rotation: of a NaN only its NaN-ness survives)
     }
+    CAMX_DEV f32x4 operator()(int row, int k) const { u32x2 keep; return (*this)(row, k, keep); }
 };
 struct RmsSrc {
     static constexpr bool bf16_valued = false;
@@ -69,16 +73,19 @@ struct RmsSrc {
         f32x4 a; a.x = xv.x * rstd * wv.x; a.y = xv.y * rstd * wv.y; a.z = xv.z * rstd * wv.z; a.w = xv.w * rstd * wv.w;
         return a;
     }
+    CAMX_DEV f32x4 operator()(int row, int k, u32x2 &) const { return (*this)(row, k); }
 };
 
 // u = bf16(H128 . bf16(source)) for the NR rounds of this half-wave; returns the lane's max |u| over its active chunks
 template <int NR, typename Src>
-CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[NR]) {
+CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[NR], u32x2 * keep = nullptr) {
 #pragma unroll
     for (int c = 0; c < NR; c++) {
         const int ch = hw + 8 * c;
         f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (ch < nch) v = src(row, ch * 128 + 4 * l);
+        u32x2 kp = {0u, 0u};
+        if (ch < nch) v = src(row, ch * 128 + 4 * l, kp);
+        if (keep) keep[c] = kp;
         u[c] = v;
     }
     float amax = 0.0f;
@@ -276,21 +283,55 @@ CAMX_DEV void block8_sum2(float & a, float & b, float * lds16) {
     for (int w = 1; w < 8; w++) { a += lds16[w]; b += lds16[8 + w]; }
 }
 
-struct SinkF32 { float * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v) const { *(f32x4 *)(dx + (size_t)row * K + k) = v; } };
-struct SinkBF16 { uint16_t * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v) const { *(u32x2 *)(dx + (size_t)row * K + k) = pack_f2bf_x4(v); } };
-struct SinkLds { float * buf; CAMX_DEV void operator()(int, int k, f32x4 v) const { *(f32x4 *)(buf + k) = v; } };
+// u / s for a row's values, s the row's scale: the IEEE quotient by the compiler's own expansion (reciprocal, one Newton step,
+// the product and two corrections, each an fma) without its scaling and fix-up steps, which only act when an exponent is
+// extreme. Taken when s and max |u| / s lie in [2^-60, 2^60] and the lane's four quotients are at least 2^-60 in magnitude:
+// every intermediate is then a normal number and both forms run the same arithmetic (an exhaustive-neighbourhood check on a CPU
+// over 10^8 (u, s) pairs, with every reciprocal within an ulp, found no difference). Other lanes divide.
+struct RowDiv {
+    float s, r1; bool row_ok;
+    CAMX_DEV RowDiv(float s_, float amax) : s(s_) {
+        const float r0 = __builtin_amdgcn_rcpf(s_);
+        r1 = __builtin_fmaf(__builtin_fmaf(-s_, r0, 1.0f), r0, r0);
+        row_ok = s_ >= 0x1p-60f && s_ <= 0x1p60f && amax * r1 <= 0x1p60f;
+    }
+    CAMX_DEV f32x4 div4(f32x4 u) const {
+        f32x4 t, t0 = {u.x * r1, u.y * r1, u.z * r1, u.w * r1};
+#define T_(e) { const float rem = __builtin_fmaf(-s, t0.e, u.e), t1 = __builtin_fmaf(rem, r1, t0.e); t.e = __builtin_fmaf(__builtin_fmaf(-s, t1, u.e), r1, t1); }
+        CAMX_EACH4(T_)
+#undef T_
+        const float least = fminf(fminf(fabsf(t0.x), fabsf(t0.y)), fminf(fabsf(t0.z), fabsf(t0.w)));     // (a NaN quotient is a NaN either way)
+        if (!(row_ok && least >= 0x1p-60f)) { t.x = u.x / s; t.y = u.y / s; t.z = u.z / s; t.w = u.w / s; }
+        return t;
+    }
+};
+
+struct SinkF32 { float * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v, u32x2) const { *(f32x4 *)(dx + (size_t)row * K + k) = v; } };
+struct SinkBF16 { uint16_t * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v, u32x2) const { *(u32x2 *)(dx + (size_t)row * K + k) = pack_f2bf_x4(v); } };
+struct SinkLds { float * buf; CAMX_DEV void operator()(int, int k, f32x4 v, u32x2) const { *(f32x4 *)(buf + k) = v; } };
 // dact back through act = bf16(bf16(silu g) * u): each product rounded to bf16, then silu's derivative
-// ds * sig * fma(g, 1 - sig, 1), into dgu = [dg | du] rows of 2F
+// ds * sig * fma(g, 1 - sig, 1), into dgu = [dg | du] rows of 2F. g is a bf16 value, so sig = 1 / (1 + expf(-g))
+// is read from a table of all 65536 of them (filled on first use from the correctly rounded expf): one 4-byte load in place of an
+// exponential and a division per value. (A table that also holds the fma doubles the entry, and the values in use no longer
+// stay in the first-level cache: 15 % slower than no table at all.)
+__device__ __attribute__((aligned(16))) float g_dsilu_lut[65536];
+__global__ void __launch_bounds__(256) dsilu_lut_fill() {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    const float g = bf2f((uint16_t)i), ex = (float)exp(-(double)g), sig = 1.0f / (1.0f + ex);
+    g_dsilu_lut[i] = sig;
+}
 struct SinkSiluMul {
-    const uint16_t * gu; int ld, F; uint16_t * dgu; const uint16_t * lut;
-    CAMX_DEV void operator()(int row, int k, f32x4 dact) const {
+    const uint16_t * gu; int ld, F; uint16_t * dgu; const float * dlut;
+    CAMX_DEV void operator()(int row, int k, f32x4 dact, u32x2 keep) const {      // keep: the source's four bf16(silu g)
         const uint16_t * r = gu + (size_t)row * ld;
         const u32x2 gw = *(const u32x2 *)(r + k);
         const f32x4 g = unpack_bf16x4(gw), u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
-        const f32x4 sl4 = {bf2f(lut[gw.x & 0xffffu]), bf2f(lut[gw.x >> 16]), bf2f(lut[gw.y & 0xffffu]), bf2f(lut[gw.y >> 16])};
+        const uint32_t ix = gw.x & 0xffffu, iy = gw.x >> 16, iz = gw.y & 0xffffu, iw = gw.y >> 16;
+        const f32x4 sl4 = unpack_bf16x4(keep);
+        const f32x4 sig = {dlut[ix], dlut[iy], dlut[iz], dlut[iw]};
+        const f32x4 ds = rbf4_any((f32x4){dact.x * u.x, dact.y * u.y, dact.z * u.z, dact.w * u.w});       // (a NaN's bits are settled by the store's rounding)
         f32x4 dg, du;
-#define S_(e) { const float ex = expf(-g.e), sig = 1.0f / (1.0f + ex), ds = rbf(dact.e * u.e); \
-                du.e = dact.e * sl4.e; dg.e = ds * sig * __builtin_fmaf(g.e, 1.0f - sig, 1.0f); }
+#define S_(e) { du.e = dact.e * sl4.e; dg.e = ds.e * sig.e * __builtin_fmaf(g.e, 1.0f - sig.e, 1.0f); }
         CAMX_EACH4(S_)
 #undef S_
         uint16_t * o = dgu + (size_t)row * (2 * F);
@@ -311,23 +352,29 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
         if (ch < nch) raw = *(const u32x2 *)(g + (size_t)row * K + ch * 128 + 4 * l);
         gv[c] = unpack_bf16x4(raw);
     }
-    const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u), lds16);
+    u32x2 keep[NR];                                      // what the source hands to the sink (the fused SiLU form only)
+    const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u, keep), lds16);
     const float s_raw = amax * clip / (float)qmax, s = fmaxf(s_raw, 1e-8f);
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
     // dL/ds = sum g (q - m t) and the number of max-|u| elements; m: the rounded value lies strictly inside (lo, hi). The
     // straight-through part g m is formed here (g is not needed afterwards); the ties are counted from the compares' lane masks
     // on the scalar unit, one counter per half-wave (a count is exact in any order).
+    const RowDiv rd(s, amax);
     float dlds = 0.0f;
     int ties_lo = 0, ties_hi = 0;
+    uint32_t tied = 0;                                   // bit c: some lane of this wave holds a max-|u| element in round c
 #pragma unroll
     for (int c = 0; c < NR; c++) {
         if (hw + 8 * c < nch) {
-#define D_(e) { const float t = u[c].e / s, r = rintf(t), q = fminf(fmaxf(r, lo), hi); const bool m = r > lo && r < hi; \
+            const f32x4 t4 = rd.div4(u[c]);
+            uint64_t any = 0;
+#define D_(e) { const float t = t4.e, r = rintf(t), q = fminf(fmaxf(r, lo), hi); const bool m = r > lo && r < hi; \
                 dlds = __builtin_fmaf(gv[c].e, m ? q - t : q, dlds); gv[c].e = gv[c].e * (m ? 1.0f : 0.0f); \
-                const uint64_t tie = __builtin_amdgcn_ballot_w64(fabsf(u[c].e) == amax); \
+                const uint64_t tie = __builtin_amdgcn_ballot_w64(fabsf(u[c].e) == amax); any |= tie; \
                 ties_lo += __builtin_popcount((uint32_t)tie); ties_hi += __builtin_popcount((uint32_t)(tie >> 32)); }
             CAMX_EACH4(D_)
 #undef D_
+            if (any) tied |= 1u << c;
         }
     }
     float ties = (tid & 31) == 0 ? (float)((tid & 32) ? ties_hi : ties_lo) : 0.0f;
@@ -337,12 +384,13 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
     for (int c = 0; c < NR; c++) {
         const int ch = hw + 8 * c;
         if (ch < nch) {
-            f32x4 d;
-#define V_(e) { float v = gv[c].e; \
-                if (fabsf(u[c].e) == amax && u[c].e != 0.0f) v += u[c].e > 0.0f ? coef : -coef; d.e = v; }
-            CAMX_EACH4(V_)
+            f32x4 d = gv[c];
+            if (tied & (1u << c)) {                      // wave-uniform: a row has few such elements, most rounds skip this
+#define V_(e) if (fabsf(u[c].e) == amax && u[c].e != 0.0f) d.e += u[c].e > 0.0f ? coef : -coef;
+                CAMX_EACH4(V_)
 #undef V_
-            sink(row, ch * 128 + 4 * l, rbf4_canon(scaled4(hadamard128_l4(rbf4_any(d), l, false))));      // rbf4_any: the gradient of the bf16 tensor u
+            }
+            sink(row, ch * 128 + 4 * l, rbf4_canon(scaled4(hadamard128_l4(rbf4_any(d), l, false))), keep[c]);      // rbf4_any: the gradient of the bf16 tensor u
         }
     }
 }
@@ -444,6 +492,28 @@ __global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const 
 
 __attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut);       // quant.hip
 
+// the derivative table's device address, filled once per device in stream order before its first reader; callers on any host
+// thread go through one lock
+static std::mutex g_dlut_mu;
+static struct { bool ready; const float * lut; } g_dlut_dev[64];
+static int dsilu_lut_get(hipStream_t st, const float ** lut) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
+    std::lock_guard<std::mutex> lock(g_dlut_mu);
+    if (!g_dlut_dev[dev].ready) {
+        dsilu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+        void * sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_dsilu_lut)) != hipSuccess || !sym) return CAMX_EINVAL;
+        if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
+        g_dlut_dev[dev].lut = (const float *)sym;
+        g_dlut_dev[dev].ready = true;
+    }
+    *lut = g_dlut_dev[dev].lut;
+    return CAMX_OK;
+}
+
 // the wave-per-row forward kernel: rows of at most 2048 values, operands aligned for its 16-byte loads and 16- / 4-byte stores
 static bool actq_wave_ok(int K, const void * x, const void * y, const void * codes) { return K <= 2048 && !((uintptr_t)x & 15) && !((uintptr_t)y & 15) && !((uintptr_t)codes & 3); }
 
@@ -505,9 +575,11 @@ int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * 
     if (!gu || !g || !dgu || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)g & 7) || ((uintptr_t)dgu & 7)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
     const uint16_t * lut = nullptr;
-    const int rc = silu_lut_get(st, &lut);
+    const float * dlut = nullptr;
+    int rc = silu_lut_get(st, &lut);
+    if (!rc) rc = dsilu_lut_get(st, &dlut);
     if (rc) return rc;
-    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut}, g, SinkSiluMul{gu, ld, F, dgu, lut}, F, clip, qmax)))
+    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut}, g, SinkSiluMul{gu, ld, F, dgu, dlut}, F, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 // block_entry_bwd: dy bf16 [M][d], dab bf16 [M][nab] (needed when nab > 0), rstd [M] from the forward; dx fp32 [M][d]; d <= 1024

@@ -76,6 +76,32 @@ def test_actq_bwd(M, K, qmax):
         assert bits_equal(host(dx, np.uint16) if bf else host(dx), want)
 
 
+@pytest.mark.parametrize('K', [1024, 2048, 2560])
+def test_actq_bwd_quotients_at_the_exponent_limits(K):
+    """u / s where the quotient, the scale or their ratio leaves the range in which the kernel divides by a refined reciprocal:
+    rows scaled to 1e-30 and 1e30, a row of 1e-12 with one chunk at 1e20 (quotients near 1e-32), a row whose values span
+    1e-38 .. 1e38, inf and NaN entries, and a clip of 1e-20 (quotients near 1e21): the IEEE quotient in every case"""
+    rng = np.random.default_rng(500 + K)
+    M = 8
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    x[0] *= 1e-30; x[1] *= 1e30
+    x[2] *= 1e-12; x[2, 128:256] *= 1e32
+    x[3] *= (10.0 ** rng.uniform(-38, 38, K)).astype(np.float32)
+    x[4, 5] = np.inf; x[5, 130] = np.nan
+    x[6] *= 1e-12; x[6, :128] = 0; x[6, 300] = 1e25
+    x[7] = 0; x[7, 128:256] = 1e-30 * rng.standard_normal(128)
+    g = O.f2bf(rng.standard_normal((M, K)).astype(np.float32))
+    for bf in (False, True):
+        src = O.f2bf(x) if bf else x
+        for clip in (1.0, 1e-20):
+            want = O.actq_bwd(src, g, clip=clip, qmax=7, bf16=bf)
+            dx = dev(np.zeros((M, K), np.uint16 if bf else np.float32))
+            call('camx_actq_bwd', ptr(dev(src)), I(int(bf)), ptr(dev(g)), ptr(dx), I(K), F(clip), I(7), I(M))
+            got = host(dx, np.uint16) if bf else host(dx)
+            nan_w = np.isnan(O.bf2f(want)) if bf else np.isnan(want); nan_g = np.isnan(O.bf2f(got)) if bf else np.isnan(got)
+            assert np.array_equal(nan_w, nan_g) and bits_equal(np.where(nan_w, 0, got), np.where(nan_w, 0, want))
+
+
 @pytest.mark.parametrize('M,d,nab', [(6, 896, 14), (5, 1024, 0), (9, 256, 2), (130, 896, 16)])
 def test_block_entry_bwd(M, d, nab):
     rng = np.random.default_rng(200 + d + nab)
