@@ -3,8 +3,9 @@
 // actq_fwd_codes_{f32,bf16}, actq_bwd_{f32,bf16}, silu_mul_actq_{fwd,bwd} and block_entry_{fwd,bwd} (kernels/actq.hip:40-53,
 // 96-218, 247-333).
 //
-// Forward of plain fp32 / bf16 rows of at most 2048 values: one wave per row (actq_fwd_wave_k below, 30 vector instructions per
-// value against 44). Everything else:
+// Rows of at most 2048 values with 16-byte aligned operands, forward and backward, plain and SiLU-fused: one wave per row
+// (actq_fwd_wave_k, actq_bwd_wave_k; 30 vector instructions per value against 44 forward, 63 against 78 backward), the fused
+// forms with the gates' tables in LDS. Everything else (longer rows, the RMSNorm-fused block entry, unaligned operands):
 // One 256-thread workgroup per row. A half-wave (32 lanes) transforms one 128-chunk: lane l holds elements 4l .. 4l + 3,
 // butterfly stages 1-2 in registers, 4 .. 64 across lanes; half-wave h takes chunks h, h + 8, ... (the reference's wave h of
 // 32), NR = ceil(K / 1024) rounds of them stay in registers across the row-wide reductions. Kernels are instantiated per
@@ -35,35 +36,66 @@ CAMX_DEV f32x4 scaled4(f32x4 v) { v.x *= HSCALE; v.y *= HSCALE; v.z *= HSCALE; v
 // loads (NW 128-bit words), value8() turns them into floats later, so that the next row's loads fly during this row's arithmetic.
 CAMX_DEV void unpack_bf16x8(u32x4 w, f32x4 & a, f32x4 & b) { a = unpack_bf16x4((u32x2){w.x, w.y}); b = unpack_bf16x4((u32x2){w.z, w.w}); }
 struct PlainF32 {
-    static constexpr bool bf16_valued = false; static constexpr int NW = 2;
+    static constexpr bool bf16_valued = false, lds_tables = false; static constexpr int NW = 2;
+    CAMX_DEV void set_small(const uint16_t *) {}
     const float * x; int K;
     CAMX_DEV f32x4 operator()(int row, int k) const { return *(const f32x4 *)(x + (size_t)row * K + k); }
     CAMX_DEV f32x4 operator()(int row, int k, u32x2 &) const { return (*this)(row, k); }
     CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { const u32x4 * p = (const u32x4 *)(x + (size_t)row * K + k); w[0] = p[0]; w[1] = p[1]; }
-    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b) const { a = __builtin_bit_cast(f32x4, w[0]); b = __builtin_bit_cast(f32x4, w[1]); }
+    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b, u32x4 &) const { a = __builtin_bit_cast(f32x4, w[0]); b = __builtin_bit_cast(f32x4, w[1]); }
 };
 struct PlainBF16 {
-    static constexpr bool bf16_valued = true; static constexpr int NW = 1;
+    static constexpr bool bf16_valued = true, lds_tables = false; static constexpr int NW = 1;
+    CAMX_DEV void set_small(const uint16_t *) {}
     const uint16_t * x; int K;
     CAMX_DEV f32x4 operator()(int row, int k) const { return unpack_bf16x4(*(const u32x2 *)(x + (size_t)row * K + k)); }
     CAMX_DEV f32x4 operator()(int row, int k, u32x2 &) const { return (*this)(row, k); }
     CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { w[0] = *(const u32x4 *)(x + (size_t)row * K + k); }
-    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b) const { unpack_bf16x8(w[0], a, b); }
+    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b, u32x4 &) const { unpack_bf16x8(w[0], a, b); }
 };
+// the bf16 words {t[g0], t[g1]} and {t[g2], t[g3]} of four packed bf16 gates: from the small table in LDS when there is one and it
+// holds all four, else from the full table in device memory
+CAMX_DEV u32x2 silu_lookup4(u32x2 gw, const uint16_t * small, const uint16_t * lut) {
+    u32x2 r;
+    bool outside = true;
+    if (small) {                                                           // (the index of a gate outside the table is a valid entry too)
+        outside = false;
+        const uint32_t i01 = small_index2(gw.x, outside), i23 = small_index2(gw.y, outside);
+        r.x = (uint32_t)small[i01 & 0xffffu] | ((uint32_t)small[i01 >> 16] << 16);
+        r.y = (uint32_t)small[i23 & 0xffffu] | ((uint32_t)small[i23 >> 16] << 16);
+    }
+    if (outside) {
+        r.x = (uint32_t)lut[gw.x & 0xffffu] | ((uint32_t)lut[gw.x >> 16] << 16);
+        r.y = (uint32_t)lut[gw.y & 0xffffu] | ((uint32_t)lut[gw.y >> 16] << 16);
+    }
+    return r;
+}
 struct SiluMulSrc {
     static constexpr bool bf16_valued = true;      // the activation is rounded to bf16 as it is formed
+    static constexpr bool lds_tables = true;       // the wave-per-row kernels hold the small tables in LDS
+    CAMX_DEV void set_small(const uint16_t * p) { small = p; }
     const uint16_t * gu; int ld, F;
     const uint16_t * lut;                          // bf16(silu g) for every bf16 g (the table silu_mul_bf16 uses: the same activation bits)
+    const uint16_t * small;                        // its small form in LDS, or null
     CAMX_DEV f32x4 operator()(int row, int k, u32x2 & keep) const {          // keep: the four bf16(silu g), for the backward's sink
         const uint16_t * r = gu + (size_t)row * ld;
         const u32x2 gw = *(const u32x2 *)(r + k);
         const f32x4 u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
-        keep.x = (uint32_t)lut[gw.x & 0xffffu] | ((uint32_t)lut[gw.x >> 16] << 16);
-        keep.y = (uint32_t)lut[gw.y & 0xffffu] | ((uint32_t)lut[gw.y >> 16] << 16);
+        keep = silu_lookup4(gw, small, lut);
         const f32x4 sl = unpack_bf16x4(keep);
         return rbf4_any((f32x4){sl.x * u.x, sl.y * u.y, sl.z * u.z, sl.w * u.w});      // (feeds the rotation: of a NaN only its NaN-ness survives)
     }
     CAMX_DEV f32x4 operator()(int row, int k) const { u32x2 keep; return (*this)(row, k, keep); }
+    static constexpr int NW = 2;                   // the wave-per-row form: eight gates, eight multipliers
+    CAMX_DEV void fetch(int row, int k, u32x4 (&w)[NW]) const { const uint16_t * r = gu + (size_t)row * ld + k; w[0] = *(const u32x4 *)r; w[1] = *(const u32x4 *)(r + F); }
+    CAMX_DEV void value8(const u32x4 (&w)[NW], f32x4 & a, f32x4 & b, u32x4 & keep) const {
+        const u32x2 k0 = silu_lookup4((u32x2){w[0].x, w[0].y}, small, lut), k1 = silu_lookup4((u32x2){w[0].z, w[0].w}, small, lut);
+        keep = (u32x4){k0.x, k0.y, k1.x, k1.y};
+        f32x4 sa, sb, ua, ub;
+        unpack_bf16x8(keep, sa, sb); unpack_bf16x8(w[1], ua, ub);
+        a = rbf4_any((f32x4){sa.x * ua.x, sa.y * ua.y, sa.z * ua.z, sa.w * ua.w});
+        b = rbf4_any((f32x4){sb.x * ub.x, sb.y * ub.y, sb.z * ub.z, sb.w * ub.w});
+    }
 };
 struct RmsSrc {
     static constexpr bool bf16_valued = false;
@@ -198,11 +230,11 @@ CAMX_DEV float wave_max64(float v) {
 }
 // u = bf16(H128 . bf16(source)) of the lane's 32 values from the fetched words; returns the row's max |u|
 template <typename Src>
-CAMX_DEV float actq_rotate_w(const Src & src, const u32x4 (&raw)[4][Src::NW], int q, float (&u)[4][8]) {
+CAMX_DEV float actq_rotate_w(const Src & src, const u32x4 (&raw)[4][Src::NW], int q, float (&u)[4][8], u32x4 (&keep)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         f32x4 a, b;
-        src.value8(raw[j], a, b);
+        src.value8(raw[j], a, b, keep[j]);
         if (!Src::bf16_valued) { a = rbf4_any(a); b = rbf4_any(b); }              // autocast's bf16 input
         u[j][0] = a.x; u[j][1] = a.y; u[j][2] = a.z; u[j][3] = a.w; u[j][4] = b.x; u[j][5] = b.y; u[j][6] = b.z; u[j][7] = b.w;
     }
@@ -228,21 +260,37 @@ CAMX_DEV void fetch_row_w(const Src & src, int row, int c, int q, bool on, u32x4
     }
 }
 
-// One row per wave, four rows per workgroup: with many more workgroups than the chip holds at once, the loads of the workgroups
-// that start overlap the arithmetic of those that run (walking several rows per wave with the next row's loads in flight
-// measured 15 % slower).
+// a table into LDS, 16 bytes per lane straight from device memory
+CAMX_DEV void lds_table_copy(const void * src, void * dst, int bytes) {          // bytes % 1024 == 0; all four waves
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int j = wave; j < bytes / 1024; j += 4)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((const uint8_t *)src + 1024 * j + 16 * lane),
+                                         (__attribute__((address_space(3))) void *)((uint8_t *)dst + 1024 * j), 16, 0, 0);
+}
+// One row per wave, four rows per workgroup. The kernel's time at 8192 rows is its arithmetic plus the launch's ramp, the first
+// loads and the last stores, whatever the number of waves in flight (3 to 8 per SIMD measured alike); a wave that walks several
+// rows with the next row's loads in flight measured 5 to 15 % slower.
 template <typename Src>
 __global__ void __launch_bounds__(256) actq_fwd_wave_k(Src src, uint16_t * __restrict__ y, float * __restrict__ s_out, uint16_t * __restrict__ codes,
-                                                       int K, float clip, int qmax, int M) {
+                                                       int K, float clip, int qmax, int M, const uint16_t * small_g = nullptr) {
     const int lane = threadIdx.x & 63, nch = K / 128, c = lane >> 2, q = lane & 3;
     const bool on = c < nch;
     const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (row >= M) return;
+    if (!Src::lds_tables && row >= M) return;
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
     u32x4 raw[4][Src::NW];
-    fetch_row_w(src, row, c, q, on, raw);
+    fetch_row_w(src, min(row, M - 1), c, q, on, raw);
+    if (Src::lds_tables) {                               // the gates' table, shared by the workgroup's four rows
+        __shared__ __attribute__((aligned(16))) uint16_t small[SWS_TAB];
+        lds_table_copy(small_g, small, 2 * SWS_TAB);
+        __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0): this wave's part of the table (and its row)
+        __syncthreads();
+        src.set_small(small);
+        if (row >= M) return;
+    }
     float u[4][8];
-    const float amax = actq_rotate_w(src, raw, q, u);
+    u32x4 keep[4];                                       // (only the backward uses it)
+    const float amax = actq_rotate_w(src, raw, q, u, keep);
     const float s = fmaxf(amax * clip / (float)qmax, 1e-8f), s_rcp = __builtin_amdgcn_rcpf(s);
     if (lane == 0 && s_out) s_out[row] = s;
     if (!on) return;
@@ -295,48 +343,91 @@ struct RowDiv {
         r1 = __builtin_fmaf(__builtin_fmaf(-s_, r0, 1.0f), r0, r0);
         row_ok = s_ >= 0x1p-60f && s_ <= 0x1p60f && amax * r1 <= 0x1p60f;
     }
-    CAMX_DEV f32x4 div4(f32x4 u) const {
+    CAMX_DEV f32x4 div4(f32x4 u, bool needed = true) const {       // needed: false in a lane whose values are padding
         f32x4 t, t0 = {u.x * r1, u.y * r1, u.z * r1, u.w * r1};
 #define T_(e) { const float rem = __builtin_fmaf(-s, t0.e, u.e), t1 = __builtin_fmaf(rem, r1, t0.e); t.e = __builtin_fmaf(__builtin_fmaf(-s, t1, u.e), r1, t1); }
         CAMX_EACH4(T_)
 #undef T_
         const float least = fminf(fminf(fabsf(t0.x), fabsf(t0.y)), fminf(fabsf(t0.z), fabsf(t0.w)));     // (a NaN quotient is a NaN either way)
-        if (!(row_ok && least >= 0x1p-60f)) { t.x = u.x / s; t.y = u.y / s; t.z = u.z / s; t.w = u.w / s; }
+        if (needed && !(row_ok && least >= 0x1p-60f)) { t.x = u.x / s; t.y = u.y / s; t.z = u.z / s; t.w = u.w / s; }
         return t;
     }
 };
 
-struct SinkF32 { float * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v, u32x2) const { *(f32x4 *)(dx + (size_t)row * K + k) = v; } };
-struct SinkBF16 { uint16_t * dx; int K; CAMX_DEV void operator()(int row, int k, f32x4 v, u32x2) const { *(u32x2 *)(dx + (size_t)row * K + k) = pack_f2bf_x4(v); } };
+struct SinkF32 {
+    float * dx; int K;
+    CAMX_DEV void operator()(int row, int k, f32x4 v, u32x2) const { *(f32x4 *)(dx + (size_t)row * K + k) = v; }
+    CAMX_DEV void st8(int row, int k, f32x4 a, f32x4 b, u32x4) const { f32x4 * p = (f32x4 *)(dx + (size_t)row * K + k); p[0] = a; p[1] = b; }
+    CAMX_DEV void set_small(const float *) {}
+};
+struct SinkBF16 {
+    uint16_t * dx; int K;
+    CAMX_DEV void operator()(int row, int k, f32x4 v, u32x2) const { *(u32x2 *)(dx + (size_t)row * K + k) = pack_f2bf_x4(v); }
+    CAMX_DEV void st8(int row, int k, f32x4 a, f32x4 b, u32x4) const {
+        const u32x2 pa = pack_f2bf_x4(a), pb = pack_f2bf_x4(b);
+        *(u32x4 *)(dx + (size_t)row * K + k) = (u32x4){pa.x, pa.y, pb.x, pb.y};
+    }
+    CAMX_DEV void set_small(const float *) {}
+};
 struct SinkLds { float * buf; CAMX_DEV void operator()(int, int k, f32x4 v, u32x2) const { *(f32x4 *)(buf + k) = v; } };
 // dact back through act = bf16(bf16(silu g) * u): each product rounded to bf16, then silu's derivative
 // ds * sig * fma(g, 1 - sig, 1), into dgu = [dg | du] rows of 2F. g is a bf16 value, so sig = 1 / (1 + expf(-g))
 // is read from a table of all 65536 of them (filled on first use from the correctly rounded expf): one 4-byte load in place of an
-// exponential and a division per value. (A table that also holds the fma doubles the entry, and the values in use no longer
-// stay in the first-level cache: 15 % slower than no table at all.)
+// exponential and a division per value; the wave-per-row kernel holds the table's small form in LDS. (A table in device memory
+// that also holds the fma doubles the entry, and the values in use no longer stay in the first-level cache: 15 % slower than
+// no table at all.)
 __device__ __attribute__((aligned(16))) float g_dsilu_lut[65536];
+__device__ __attribute__((aligned(16))) float g_dsilu_small[SWS_TAB];            // the small form, for LDS
 __global__ void __launch_bounds__(256) dsilu_lut_fill() {
     const uint32_t i = blockIdx.x * 256 + threadIdx.x;
     const float g = bf2f((uint16_t)i), ex = (float)exp(-(double)g), sig = 1.0f / (1.0f + ex);
     g_dsilu_lut[i] = sig;
 }
+__global__ void __launch_bounds__(256) dsilu_small_fill() {              // after dsilu_lut_fill, on the same stream
+    const uint32_t e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= SWS_TAB) return;
+    const uint32_t sign = e >> 12, i = e & SWS_SPAN;
+    g_dsilu_small[e] = g_dsilu_lut[i == SWS_SPAN ? sign << 15 : (sign << 15) | (SWS_A0 + i)];
+}
 struct SinkSiluMul {
     const uint16_t * gu; int ld, F; uint16_t * dgu; const float * dlut;
+    const float * dsmall;                          // the small sigmoid table in LDS, or null
+    CAMX_DEV void set_small(const float * p) { dsmall = p; }
     CAMX_DEV void operator()(int row, int k, f32x4 dact, u32x2 keep) const {      // keep: the source's four bf16(silu g)
         const uint16_t * r = gu + (size_t)row * ld;
-        const u32x2 gw = *(const u32x2 *)(r + k);
-        const f32x4 g = unpack_bf16x4(gw), u = unpack_bf16x4(*(const u32x2 *)(r + F + k));
-        const uint32_t ix = gw.x & 0xffffu, iy = gw.x >> 16, iz = gw.y & 0xffffu, iw = gw.y >> 16;
-        const f32x4 sl4 = unpack_bf16x4(keep);
-        const f32x4 sig = {dlut[ix], dlut[iy], dlut[iz], dlut[iw]};
+        u32x2 dgp, dup;
+        grads4(*(const u32x2 *)(r + k), *(const u32x2 *)(r + F + k), keep, dact, dgp, dup);
+        uint16_t * o = dgu + (size_t)row * (2 * F);
+        *(u32x2 *)(o + k) = dgp;
+        *(u32x2 *)(o + F + k) = dup;
+    }
+    // four values' dg and du from their gates, multipliers, bf16(silu g) and dact
+    CAMX_DEV void grads4(u32x2 gw, u32x2 uw, u32x2 keep, f32x4 dact, u32x2 & dgp, u32x2 & dup) const {
+        const f32x4 g = unpack_bf16x4(gw), u = unpack_bf16x4(uw), sl4 = unpack_bf16x4(keep);
+        bool outside = true;
+        f32x4 sig;
+        if (dsmall) {
+            outside = false;
+            const uint32_t i01 = small_index2(gw.x, outside), i23 = small_index2(gw.y, outside);
+            sig = (f32x4){dsmall[i01 & 0xffffu], dsmall[i01 >> 16], dsmall[i23 & 0xffffu], dsmall[i23 >> 16]};
+        }
+        if (outside) sig = (f32x4){dlut[gw.x & 0xffffu], dlut[gw.x >> 16], dlut[gw.y & 0xffffu], dlut[gw.y >> 16]};
         const f32x4 ds = rbf4_any((f32x4){dact.x * u.x, dact.y * u.y, dact.z * u.z, dact.w * u.w});       // (a NaN's bits are settled by the store's rounding)
         f32x4 dg, du;
 #define S_(e) { du.e = dact.e * sl4.e; dg.e = ds.e * sig.e * __builtin_fmaf(g.e, 1.0f - sig.e, 1.0f); }
         CAMX_EACH4(S_)
 #undef S_
-        uint16_t * o = dgu + (size_t)row * (2 * F);
-        *(u32x2 *)(o + k) = pack_f2bf_x4(dg);
-        *(u32x2 *)(o + F + k) = pack_f2bf_x4(du);
+        dgp = pack_f2bf_x4(dg); dup = pack_f2bf_x4(du);
+    }
+    CAMX_DEV void st8(int row, int k, f32x4 a, f32x4 b, u32x4 keep) const {
+        const uint16_t * r = gu + (size_t)row * ld + k;
+        const u32x4 gw = *(const u32x4 *)r, uw = *(const u32x4 *)(r + F);
+        u32x2 dg0, du0, dg1, du1;
+        grads4((u32x2){gw.x, gw.y}, (u32x2){uw.x, uw.y}, (u32x2){keep.x, keep.y}, a, dg0, du0);
+        grads4((u32x2){gw.z, gw.w}, (u32x2){uw.z, uw.w}, (u32x2){keep.z, keep.w}, b, dg1, du1);
+        uint16_t * o = dgu + (size_t)row * (2 * F) + k;
+        *(u32x4 *)o = (u32x4){dg0.x, dg0.y, dg1.x, dg1.y};
+        *(u32x4 *)(o + F) = (u32x4){du0.x, du0.y, du1.x, du1.y};
     }
 };
 
@@ -399,6 +490,118 @@ template <int NR, typename Src, typename Sink>
 __global__ void __launch_bounds__(256) actq_bwd_k(Src src, const uint16_t * g, Sink sink, int K, float clip, int qmax) {
     __shared__ float lds[16];
     actq_bwd_row<NR>(src, blockIdx.x, g, sink, K, clip, qmax, lds);
+}
+
+// ---- backward of rows of at most 2048 values: one wave per row, in the layout of actq_fwd_wave_k ------------------------------------
+// The sum of dL/ds keeps the tree of the workgroup form. There, the lane of half-wave h with index l adds the terms of elements
+// 4 l .. 4 l + 3 of chunk h, then of chunk h + 8, in order; here those eight terms sit in two lanes (c = h and c = h + 8, 32 lanes
+// apart) as registers 4 kk .. 4 kk + 3 of group j, with l = 8 j + 2 q + kk. Every lane runs the four-term chain from zero, the upper
+// 32 lanes fetch the lower lanes' results and run theirs again from there. The 32 sums of a half-wave then combine by
+// l ^ 16, 8 (registers j), 4, 2 (lanes q), 1 (registers kk), and the eight half-wave sums, held by lanes 32 + 4 h, are added in order.
+CAMX_DEV float from_other_half(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * (lane ^ 32), __builtin_bit_cast(int, v)));
+}
+template <typename Src, typename Sink>
+__global__ void __launch_bounds__(256) actq_bwd_wave_k(Src src, const uint16_t * __restrict__ g, Sink sink, int K, float clip, int qmax, int M,
+                                                       const uint16_t * small_g = nullptr, const float * dsmall_g = nullptr) {
+    const int lane = threadIdx.x & 63, nch = K / 128, c = lane >> 2, q = lane & 3;
+    const bool on = c < nch, upper = lane >= 32;
+    const int row_raw = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (!Src::lds_tables && row_raw >= M) return;
+    const int row = min(row_raw, M - 1);
+    u32x4 raw[4][Src::NW], graw[4];
+    fetch_row_w(src, row, c, q, on, raw);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        graw[j] = (u32x4){0u, 0u, 0u, 0u};
+        if (on) graw[j] = *(const u32x4 *)(g + (size_t)row * K + c * 128 + 32 * j + 8 * q);
+    }
+    if (Src::lds_tables) {                               // the gates' tables, shared by the workgroup's four rows
+        __shared__ __attribute__((aligned(16))) uint16_t small[SWS_TAB];
+        __shared__ __attribute__((aligned(16))) float dsmall[SWS_TAB];
+        lds_table_copy(small_g, small, 2 * SWS_TAB);
+        lds_table_copy(dsmall_g, dsmall, 4 * SWS_TAB);
+        __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0): this wave's part of the tables (and its row)
+        __syncthreads();
+        src.set_small(small); sink.set_small(dsmall);
+        if (row_raw >= M) return;
+    }
+    float u[4][8];
+    u32x4 keep[4];
+    const float amax = actq_rotate_w(src, raw, q, u, keep);
+    const float s_raw = amax * clip / (float)qmax, s = fmaxf(s_raw, 1e-8f);
+    const float lo = (float)(-qmax - 1), hi = (float)qmax;
+    const RowDiv rd(s, amax);
+    const uint64_t on_mask = __builtin_amdgcn_ballot_w64(on);
+    float gm[4][8], part[4][2];                          // g m; the reference lanes' sums of dL/ds terms
+    int ties_n = 0;
+    uint32_t tied = 0;                                   // bit j: group j holds a max-|u| element in some lane
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        f32x4 ga, gb;
+        unpack_bf16x8(graw[j], ga, gb);
+        const float g8[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+        const f32x4 ta = rd.div4((f32x4){u[j][0], u[j][1], u[j][2], u[j][3]}, on), tb = rd.div4((f32x4){u[j][4], u[j][5], u[j][6], u[j][7]}, on);
+        const float t8[8] = {ta.x, ta.y, ta.z, ta.w, tb.x, tb.y, tb.z, tb.w};
+        float x8[8];
+        uint64_t any = 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float t = t8[k], r = rintf(t), qv = fminf(fmaxf(r, lo), hi);
+            const bool m = r > lo && r < hi;
+            x8[k] = m ? qv - t : qv;
+            gm[j][k] = g8[k] * (m ? 1.0f : 0.0f);
+            const uint64_t tie = __builtin_amdgcn_ballot_w64(fabsf(u[j][k]) == amax) & on_mask;
+            any |= tie;
+            ties_n += __builtin_popcountll(tie);
+        }
+        if (any) tied |= 1u << j;
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            float a = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) a = __builtin_fmaf(g8[4 * kk + e], x8[4 * kk + e], a);
+            const float below = from_other_half(a, lane);
+            float b = below;
+#pragma unroll
+            for (int e = 0; e < 4; e++) b = __builtin_fmaf(g8[4 * kk + e], x8[4 * kk + e], b);
+            part[j][kk] = upper ? (on ? b : below) : a;
+        }
+    }
+    float dlds;
+    {
+        const float b00 = part[0][0] + part[2][0], b01 = part[0][1] + part[2][1], b10 = part[1][0] + part[3][0], b11 = part[1][1] + part[3][1];   // l ^ 16
+        float c0 = b00 + b10, c1 = b01 + b11;                                                                                                      // l ^ 8
+        c0 += lane_xor2(c0); c1 += lane_xor2(c1);                                                                                                  // l ^ 4
+        c0 += lane_xor1(c0); c1 += lane_xor1(c1);                                                                                                  // l ^ 2
+        const float d = c0 + c1;                                                                                                                   // l ^ 1
+        dlds = lane_read(d, 32);
+#pragma unroll
+        for (int h = 1; h < 8; h++) dlds += lane_read(d, 32 + 4 * h);
+    }
+    const float coef = s_raw >= 1e-8f ? dlds * clip / (float)qmax / (float)ties_n : 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if (tied & (1u << j)) {                          // wave-uniform: a row has few such elements
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if (on && fabsf(u[j][k]) == amax && u[j][k] != 0.0f) gm[j][k] += u[j][k] > 0.0f ? coef : -coef;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int k = 0; k < 8; k += 4) {
+            const f32x4 v = rbf4_any((f32x4){gm[j][k], gm[j][k + 1], gm[j][k + 2], gm[j][k + 3]});      // the gradient of the bf16 tensor u
+            gm[j][k] = v.x; gm[j][k + 1] = v.y; gm[j][k + 2] = v.z; gm[j][k + 3] = v.w;
+        }
+    hadamard128_w32(gm, q);
+    if (!on) return;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const f32x4 a = rbf4_canon(scaled4((f32x4){gm[j][0], gm[j][1], gm[j][2], gm[j][3]})), b = rbf4_canon(scaled4((f32x4){gm[j][4], gm[j][5], gm[j][6], gm[j][7]}));
+        sink.st8(row, c * 128 + 32 * j + 8 * q, a, b, keep[j]);
+    }
 }
 
 // ---- block entry: h = RMSNorm(x) never materialized ------------------------------------------------------------------------
@@ -490,27 +693,31 @@ __global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const 
     }
 }
 
-__attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut);       // quant.hip
+__attribute__((visibility("hidden"))) int silu_luts_get(hipStream_t st, const uint16_t ** lut, const uint16_t ** small);       // quant.hip
 
 // the derivative table's device address, filled once per device in stream order before its first reader; callers on any host
 // thread go through one lock
 static std::mutex g_dlut_mu;
-static struct { bool ready; const float * lut; } g_dlut_dev[64];
-static int dsilu_lut_get(hipStream_t st, const float ** lut) {
+static struct { bool ready; const float * lut; const float * small; } g_dlut_dev[64];
+static int dsilu_luts_get(hipStream_t st, const float ** lut, const float ** small) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
     std::lock_guard<std::mutex> lock(g_dlut_mu);
     if (!g_dlut_dev[dev].ready) {
         dsilu_lut_fill<<<dim3(256), dim3(256), 0, st>>>();
+        dsilu_small_fill<<<dim3((SWS_TAB + 255) / 256), dim3(256), 0, st>>>();
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
-        void * sym = nullptr;
+        void * sym = nullptr, * sym_small = nullptr;
         if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_dsilu_lut)) != hipSuccess || !sym) return CAMX_EINVAL;
+        if (hipGetSymbolAddress(&sym_small, HIP_SYMBOL(g_dsilu_small)) != hipSuccess || !sym_small) return CAMX_EINVAL;
         if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
         g_dlut_dev[dev].lut = (const float *)sym;
+        g_dlut_dev[dev].small = (const float *)sym_small;
         g_dlut_dev[dev].ready = true;
     }
     *lut = g_dlut_dev[dev].lut;
+    *small = g_dlut_dev[dev].small;
     return CAMX_OK;
 }
 
@@ -547,10 +754,14 @@ int camx_actq_fwd(const void * x, int is_bf16, uint16_t * y, float * s, uint16_t
 int camx_silu_mul_actq_fwd(const uint16_t * gu, int ld, int F, uint16_t * y, float * s, uint16_t * codes, float clip, int qmax, int M, hipStream_t st) {
     if (!gu || (!y && !codes) || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    const uint16_t * lut = nullptr;
-    const int rc = silu_lut_get(st, &lut);
+    const uint16_t * lut = nullptr, * small = nullptr;
+    const int rc = silu_luts_get(st, &lut, &small);
     if (rc) return rc;
-    ACTQ_ROUNDS(F, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut}, y, s, codes, F, clip, qmax)))
+    if (F <= 2048 && !(ld & 7) && !((uintptr_t)gu & 15) && actq_wave_ok(F, gu, y, codes)) {       // one wave per row
+        actq_fwd_wave_k<<<dim3((M + 3) / 4), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut, nullptr}, y, s, codes, F, clip, qmax, M, small);
+        CAMX_LAUNCH_RET();
+    }
+    ACTQ_ROUNDS(F, (actq_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut, nullptr}, y, s, codes, F, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y, float * s, uint16_t * codes,
@@ -566,6 +777,11 @@ int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab
 int camx_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, int K, float clip, int qmax, int M, hipStream_t st) {
     if (!x || !g || !dx || actq_check(K, qmax, M) || ((uintptr_t)x & (is_bf16 ? 7 : 15)) || ((uintptr_t)dx & (is_bf16 ? 7 : 15)) || ((uintptr_t)g & 7)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
+    if (K <= 2048 && !(((uintptr_t)x | (uintptr_t)g | (uintptr_t)dx) & 15)) {                  // one wave per row
+        if (is_bf16) actq_bwd_wave_k<<<dim3((M + 3) / 4), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, g, SinkBF16{(uint16_t *)dx, K}, K, clip, qmax, M);
+        else actq_bwd_wave_k<<<dim3((M + 3) / 4), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, g, SinkF32{(float *)dx, K}, K, clip, qmax, M);
+        CAMX_LAUNCH_RET();
+    }
     if (is_bf16) { ACTQ_ROUNDS(K, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainBF16{(const uint16_t *)x, K}, g, SinkBF16{(uint16_t *)dx, K}, K, clip, qmax))) }
     else { ACTQ_ROUNDS(K, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(PlainF32{(const float *)x, K}, g, SinkF32{(float *)dx, K}, K, clip, qmax))) }
     CAMX_LAUNCH_RET();
@@ -574,12 +790,16 @@ int camx_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, in
 int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, float clip, int qmax, int M, hipStream_t st) {
     if (!gu || !g || !dgu || actq_check(F, qmax, M) || ld < 2 * F || (ld & 3) || ((uintptr_t)gu & 7) || ((uintptr_t)g & 7) || ((uintptr_t)dgu & 7)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    const uint16_t * lut = nullptr;
-    const float * dlut = nullptr;
-    int rc = silu_lut_get(st, &lut);
-    if (!rc) rc = dsilu_lut_get(st, &dlut);
+    const uint16_t * lut = nullptr, * small = nullptr;
+    const float * dlut = nullptr, * dsmall = nullptr;
+    int rc = silu_luts_get(st, &lut, &small);
+    if (!rc) rc = dsilu_luts_get(st, &dlut, &dsmall);
     if (rc) return rc;
-    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut}, g, SinkSiluMul{gu, ld, F, dgu, dlut}, F, clip, qmax)))
+    if (F <= 2048 && !(ld & 7) && !(((uintptr_t)gu | (uintptr_t)g | (uintptr_t)dgu) & 15)) {      // one wave per row
+        actq_bwd_wave_k<<<dim3((M + 3) / 4), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut, nullptr}, g, SinkSiluMul{gu, ld, F, dgu, dlut, nullptr}, F, clip, qmax, M, small, dsmall);
+        CAMX_LAUNCH_RET();
+    }
+    ACTQ_ROUNDS(F, (actq_bwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(SiluMulSrc{gu, ld, F, lut, nullptr}, g, SinkSiluMul{gu, ld, F, dgu, dlut, nullptr}, F, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 // block_entry_bwd: dy bf16 [M][d], dab bf16 [M][nab] (needed when nab > 0), rstd [M] from the forward; dx fp32 [M][d]; d <= 1024

@@ -295,6 +295,22 @@ CAMX_DEV f32x4 hadamard128_l4(f32x4 v, int lane, bool scale) {
     return v;
 }
 
+// ---- the small tables of a bf16 gate ---------------------------------------------------------------------------------------------
+// 8192 entries cover +-0 and 2^-24 <= |g| < 2^8 (less two values): positive gates first, then negative ones; a kernel that looks
+// gates up from LDS holds these and goes to the full 65536-entry table in device memory for a gate outside them.
+#define SWS_A0 0x3380u                 // bf16 bits of 2^-24: the first magnitude
+#define SWS_SPAN 0x0fffu               // magnitudes per sign; index SWS_SPAN is the entry of +-0 (and the stand-in of every gate outside the table)
+#define SWS_TAB (2 * (SWS_SPAN + 1))
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+// the entries of two packed gates (16 bits each); outside: set when one of them is not in the table
+CAMX_DEV uint32_t small_index2(uint32_t w, bool & outside) {
+    const u16x2 a2 = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+    const u16x2 i2 = __builtin_elementwise_min(a2 - (u16x2){SWS_A0, SWS_A0}, (u16x2){SWS_SPAN, SWS_SPAN});      // below the table: wraps, clamps
+    const u16x2 lo = a2 - (u16x2){1, 1};                                                                       // (a zero wraps to 0xffff: inside)
+    outside |= (lo.x < SWS_A0 - 1) | (lo.y < SWS_A0 - 1) | (a2.x >= SWS_A0 + SWS_SPAN) | (a2.y >= SWS_A0 + SWS_SPAN);
+    return ((w >> 3) & 0x10001000u) | __builtin_bit_cast(uint32_t, i2);                                        // the sign in bit 12
+}
+
 // ---- host-side helpers -------------------------------------------------------------------------------------------------------
 #define CAMX_OK 0
 #define CAMX_EINVAL 1     // hipErrorInvalidValue

@@ -273,9 +273,6 @@ CAMX_DEV void swm_load(SwmItem & it, const void * __restrict__ src, const int32_
 // rare redo of the one-shot kernel). LUT_SMALL: the 8192-entry table of the one-shot kernel, which holds the gates a model produces
 // (+-0 and 2^-24 <= |g| < 2^8 less two values); bit 1 of the result reports a gate outside it, and the caller redoes the item with the full table.
 enum { LUT_FULL = 0, LUT_SMALL = 1 };
-#define SWS_A0 0x3380u                 // bf16 bits of 2^-24: the small table's first magnitude
-#define SWS_SPAN 0x0fffu               // magnitudes per sign; index SWS_SPAN is the entry of +-0 (and the stand-in of every gate outside the table)
-typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 template <int LAYOUT, int SRC, bool CANON = false, int LUTMODE = LUT_FULL>
 CAMX_DEV int swm_compute(const SwmItem & it, const uint16_t * lut, uint8_t * stage, long F, uint16_t * __restrict__ act, int T, long tg, long unit,
                          int lane) {
@@ -409,7 +406,6 @@ __global__ void __launch_bounds__(1024) swiglu_mmq_lut(const void * __restrict__
 // magnitude's offset from 2^-24 clamped to the last entry, which holds +-0. A wave that meets a gate outside the table (2 in the
 // flags) redoes its item with the full table in device memory; one that meets a NaN redoes it with the canonical NaN.
 #define SWS_WAVES 4
-#define SWS_TAB (2 * (SWS_SPAN + 1))                                       // entries: positive gates, then negative ones
 __device__ __attribute__((aligned(16))) uint16_t g_silu_small[SWS_TAB];
 
 __global__ void __launch_bounds__(256) silu_small_fill() {             // after silu_lut_fill, on the same stream
@@ -542,8 +538,8 @@ __global__ void __launch_bounds__(1024) silu_mul_lut(const uint16_t * __restrict
 // The table is filled once per device, in stream order before its first reader, and the kernels that hold it in LDS get their
 // dynamic LDS limit raised; callers on any host thread go through one lock. *ncu: the device's CU count.
 static std::mutex g_lut_mu;
-static struct { bool ready; int ncu; const uint16_t * lut; } g_lut_dev[64];
-static int silu_lut_ready(hipStream_t st, int * ncu, const uint16_t ** lut = nullptr) {
+static struct { bool ready; int ncu; const uint16_t * lut; const uint16_t * small; } g_lut_dev[64];
+static int silu_lut_ready(hipStream_t st, int * ncu, const uint16_t ** lut = nullptr, const uint16_t ** small = nullptr) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CAMX_EINVAL;
     std::lock_guard<std::mutex> lock(g_lut_mu);
@@ -557,21 +553,28 @@ static int silu_lut_ready(hipStream_t st, int * ncu, const uint16_t ** lut = nul
         if (hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_DS4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void *)swiglu_mmq_lut<MMQ_D4, SRC_SWIGLU_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, SWM_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void *)silu_mul_lut, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return CAMX_EINVAL;
-        void * sym = nullptr;
+        void * sym = nullptr, * sym_small = nullptr;
         if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_silu_lut)) != hipSuccess || !sym) return CAMX_EINVAL;
+        if (hipGetSymbolAddress(&sym_small, HIP_SYMBOL(g_silu_small)) != hipSuccess || !sym_small) return CAMX_EINVAL;
         if (hipStreamSynchronize(st) != hipSuccess) return CAMX_EINVAL;     // later calls may come on other streams
         g_lut_dev[dev].lut = (const uint16_t *)sym;
+        g_lut_dev[dev].small = (const uint16_t *)sym_small;
         g_lut_dev[dev].ncu = n;
         g_lut_dev[dev].ready = true;
     }
     *ncu = g_lut_dev[dev].ncu;
     if (lut) *lut = g_lut_dev[dev].lut;
+    if (small) *small = g_lut_dev[dev].small;
     return CAMX_OK;
 }
-// the table's device address for kernels of other files (filled and synchronized on first use)
+// the tables' device addresses for kernels of other files (filled and synchronized on first use)
 __attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut) {
     int ncu = 0;
     return silu_lut_ready(st, &ncu, lut);
+}
+__attribute__((visibility("hidden"))) int silu_luts_get(hipStream_t st, const uint16_t ** lut, const uint16_t ** small) {
+    int ncu = 0;
+    return silu_lut_ready(st, &ncu, lut, small);
 }
 
 // the wide form of silu_mul_bf16 (rows of H = 8 k values, 16-byte aligned, at least 2^22 values); CAMX_EINVAL: not applicable

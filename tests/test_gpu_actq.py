@@ -42,10 +42,11 @@ def test_block_entry_fwd():
     assert bits_equal(host(ab, np.uint16), rab)
 
 
-@pytest.mark.parametrize('M,Fh', [(5, 768), (2100, 1024), (2050, 1920), (2049, 2176), (4099, 128)])
+@pytest.mark.parametrize('M,Fh', [(5, 768), (2100, 1024), (2050, 1920), (2049, 2176), (4099, 128), (5, 2304), (303, 2048)])
 def test_silu_mul_actq_fwd(M, Fh):
     rng = np.random.default_rng(12 + M)
     gu = O.f2bf(outliers(rng, (M, 2 * Fh)))
+    gu[M - 1, :10] = O.f2bf(np.array([256., -256., 255., -255., 2.0 ** -24, -2.0 ** -24, 2.0 ** -25, -2.0 ** -25, 1e4, -1e-30], np.float32))      # the edges of the small table
     y = dev(np.zeros((M, Fh), np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros((M, Fh // 2), np.uint8))
     gud = dev(gu)
     call('camx_silu_mul_actq_fwd', ptr(gud), I(2 * Fh), I(Fh), ptr(y), ptr(s), ptr(c), F(1.0), I(7), I(M))
@@ -116,12 +117,16 @@ def test_block_entry_bwd(M, d, nab):
     assert bits_equal(host(dx), want)
 
 
-@pytest.mark.parametrize('M,Fh,ld', [(24, 768, 1536), (12, 2048, 4608), (9, 256, 512)])
+@pytest.mark.parametrize('M,Fh,ld', [(24, 768, 1536), (12, 2048, 4608), (9, 256, 512), (1100, 256, 520), (2300, 1024, 2048), (4099, 128, 256),
+                                      (24, 768, 1540), (1030, 2304, 4608), (7, 2304, 4612), (1500, 640, 1284)])
 def test_silu_mul_actq_bwd(M, Fh, ld):
-    """the recomputed activation is the table's (the oracle's bits); silu's derivative uses the device's expf: one bf16 step"""
+    """the recomputed activation is the table's (the oracle's bits); the sigmoid of silu's derivative comes from a table of the correctly
+    rounded expf, the oracle's from the C library's (within an ulp of it): one bf16 step at most. Row widths and strides that take
+    the wave-per-row form (tables in LDS, gates at their edges in the last row) and the workgroup-per-row form (longer or unaligned rows)"""
     rng = np.random.default_rng(300 + Fh)
     base = O.f2bf((rng.standard_normal((M, ld)) * 2).astype(np.float32))
     base[0, :8] = O.f2bf(np.array([30., -30., 0., -0.0, 1e-3, -88., 88., 3.], np.float32))
+    base[M - 1, :10] = O.f2bf(np.array([256., -256., 255., -255., 2.0 ** -24, -2.0 ** -24, 2.0 ** -25, -2.0 ** -25, 1e4, -1e-30], np.float32))    # the edges of the small tables
     g = O.f2bf(rng.standard_normal((M, Fh)).astype(np.float32))
     bd = dev(base)
     dgu = dev(np.zeros((M, 2 * Fh), np.uint16))
