@@ -25,7 +25,7 @@ def _generators(r):
 
     def silu_actq():
         m, f = ri(2, 40), 128 * ri(1, 24)
-        return m, f, 2 * f + 8 * ri(0, 4)
+        return m, f, 2 * f + 4 * ri(0, 8)                      # strides for the wave-per-row form (16-byte rows) and the workgroup form
 
     def rms_mul():
         wr = ch([1, 1, 2, 4])
@@ -40,6 +40,7 @@ def _generators(r):
         (A.test_actq_bwd, lambda: (ri(1, 300), 128 * ri(1, 64), ch([1, 3, 7, 7, 15, 127]))),
         (A.test_block_entry_bwd, lambda: (ri(1, 200), 128 * ri(1, 8), 2 * ri(0, 8))),
         (A.test_silu_mul_actq_bwd, silu_actq),
+        (A.test_silu_mul_actq_fwd, lambda: (ri(2, 300), 128 * ri(1, 24))),
         (E.test_swiglu, lambda: (ri(1, 70000),)),
         (E.test_silu_mul_bf16, lambda: (ri(1, 300), ri(6, 3000))),
         (E.test_gdn_conv, lambda: (ri(1, 600), ch([6, 64, 100, 256, 512, 1000, 4096, 8200, 10240]))),
