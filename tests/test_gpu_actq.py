@@ -141,6 +141,33 @@ def test_silu_mul_actq_bwd(M, Fh, ld):
     assert (got == want).mean() > 0.99
 
 
+@pytest.mark.parametrize('M,Fh', [(6, 1024), (1200, 256), (5, 2304)])
+def test_silu_mul_actq_gates_of_every_magnitude(M, Fh):
+    """gates and multipliers over the whole bf16 exponent range (most gates outside the small tables the wave-per-row kernels hold in
+    LDS), +-inf gates, a NaN gate and a NaN multiplier: the forward bit for bit, the backward within a bf16 step, NaN for NaN"""
+    from test_gpu_value_sweeps import values
+    rng = np.random.default_rng(900 + M)
+    with np.errstate(all='ignore'):
+        gu = O.f2bf(values(rng, (M, 2 * Fh), emin=-130.0, emax=120.0))
+        gu[1, :Fh] = O.f2bf(values(rng, Fh, emin=-30.0, emax=12.0))
+        gu[2, 5] = 0x7f80; gu[2, 6] = 0xff80; gu[3, 9] = 0x7fc1; gu[4, Fh + 3] = 0xffc0
+        g = O.f2bf(rng.standard_normal((M, Fh)).astype(np.float32))
+        fy, fs, fc = O.silu_mul_actq_fwd(gu)
+        want = O.silu_mul_actq_bwd(gu, g)
+    gud = dev(gu)
+    y = dev(np.zeros((M, Fh), np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros((M, Fh // 2), np.uint8))
+    call('camx_silu_mul_actq_fwd', ptr(gud), I(2 * Fh), I(Fh), ptr(y), ptr(s), ptr(c), F(1.0), I(7), I(M))
+    nan_s = np.isnan(fs)
+    assert np.array_equal(np.isnan(host(s)), nan_s) and bits_equal(host(s)[~nan_s], fs[~nan_s])
+    assert bits_equal(host(y, np.uint16)[~nan_s], fy[~nan_s]) and bits_equal(host(c)[~nan_s], fc[~nan_s])
+    dgu = dev(np.zeros((M, 2 * Fh), np.uint16))
+    call('camx_silu_mul_actq_bwd', ptr(gud), I(2 * Fh), I(Fh), ptr(dev(g)), ptr(dgu), F(1.0), I(7), I(M))
+    got = host(dgu, np.uint16)
+    nan_w = np.isnan(O.bf2f(want)); nan_g = np.isnan(O.bf2f(got))
+    assert np.array_equal(nan_w, nan_g)
+    assert close_16(np.where(nan_w, 0, got).astype(np.uint16), np.where(nan_w, 0, want).astype(np.uint16), 'bf16')
+
+
 def test_actq_autograd_wrappers():
     """caminus_amd.train.actq end to end: values, codes, scales and every gradient equal the C entry points' results"""
     import torch
