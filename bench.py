@@ -370,6 +370,18 @@ def prefill_scale_sweep(B, T=4096, only=None):
         gu = B.acts((Mr, 2 * Kq), torch.bfloat16, i); g = B.acts((Mr, Kq), torch.bfloat16, i + 1); d = torch.empty((Mr, 2 * Kq), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_silu_mul_actq_bwd', _p(gu), I(2 * Kq), I(Kq), _p(g), _p(d), F(1.0), I(7), I(Mr))
     timeit('silu_mul_actq_bwd 8192x2048', Mr * Kq * 10, mk)
+    De = 1024; nab = 16
+    nwe = torch.rand(De, device=dev) + 0.5; wab = (torch.randn(nab, De, device=dev) / 30).to(torch.bfloat16)
+    def mk(i):
+        x = B.acts((Mr, De), torch.float32, i); y = torch.empty((Mr, De), dtype=torch.bfloat16, device=dev); s = torch.empty(Mr, device=dev)
+        c = torch.empty((Mr, De // 2), dtype=torch.uint8, device=dev); ab = torch.empty((Mr, nab), dtype=torch.bfloat16, device=dev); rstd = torch.empty(Mr, device=dev)
+        return lambda: B.call('camx_block_entry_fwd', _p(x), _p(nwe), _p(wab), I(nab), F(1e-6), _p(y), _p(s), _p(c), _p(ab), _p(rstd), I(De), F(1.0), I(7), I(Mr))
+    timeit('block_entry_fwd 8192x1024, 16 projections', Mr * (De * 6.5 + nab * 2 + 8), mk)
+    def mk(i):
+        x = B.acts((Mr, De), torch.float32, i); dy = B.acts((Mr, De), torch.bfloat16, i + 1); dab = B.acts((Mr, nab), torch.bfloat16, i + 2)
+        rstd = torch.rand(Mr, device=dev) + 0.5; dx = torch.empty((Mr, De), device=dev)
+        return lambda: B.call('camx_block_entry_bwd', _p(x), _p(nwe), _p(rstd), _p(wab), I(nab), _p(dy), _p(dab), _p(dx), I(De), F(1.0), I(7), I(Mr))
+    timeit('block_entry_bwd 8192x1024, 16 projections', Mr * (De * 10 + nab * 2 + 4), mk)
     def mk(i):
         x = B.acts((Mr * Kq,), torch.float32, i); m = B.acts((Mr * Kq,), torch.bfloat16, i + 1); y = B.acts((Mr * Kq,), torch.bfloat16, i + 2); o = torch.empty(Mr * Kq, device=dev)
         return lambda: B.call('camx_residual3', _p(x), _p(m), _p(y), _p(o), L64(Mr * Kq))

@@ -109,11 +109,12 @@ struct RmsSrc {
 };
 
 // u = bf16(H128 . bf16(source)) for the NR rounds of this half-wave; returns the lane's max |u| over its active chunks
-template <int NR, typename Src>
+// NHW: the half-waves that share a row (8: a 256-thread workgroup; 2: one wave); half-wave hw takes chunks hw, hw + NHW, ...
+template <int NR, typename Src, int NHW = 8>
 CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[NR], u32x2 * keep = nullptr) {
 #pragma unroll
     for (int c = 0; c < NR; c++) {
-        const int ch = hw + 8 * c;
+        const int ch = hw + NHW * c;
         f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
         u32x2 kp = {0u, 0u};
         if (ch < nch) v = src(row, ch * 128 + 4 * l, kp);
@@ -126,7 +127,7 @@ CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[
         const f32x4 in = Src::bf16_valued ? u[c] : rbf4_any(u[c]);                // autocast's bf16 input
         const f32x4 v = rbf4_any(scaled4(hadamard128_l4(in, l, false)));
         u[c] = v;
-        if (hw + 8 * c < nch) amax = fmaxf(amax, absmax4(v));
+        if (hw + NHW * c < nch) amax = fmaxf(amax, absmax4(v));
     }
     return amax;
 }
@@ -146,28 +147,30 @@ CAMX_DEV f32x4 rint_div4(f32x4 u, float s, float s_rcp) {
 }
 
 // row-wide max (order-free); lds: 4 floats
+template <int NHW = 8>
 CAMX_DEV float row_max(float amax, float * lds) {
     const int tid = threadIdx.x;
 #pragma unroll
     for (int m = 32; m > 0; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    if (NHW == 2) return amax;                           // the row is this wave's
     __syncthreads();
     if ((tid & 63) == 0) lds[tid >> 6] = amax;
     __syncthreads();
     return fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
 }
 
-template <int NR, typename Src>
+template <int NR, typename Src, int NHW = 8>
 CAMX_DEV void actq_fwd_row(Src src, int row, uint16_t * __restrict__ y, float * __restrict__ s_out, int K, float clip, int qmax,
                            uint16_t * __restrict__ codes, float * lds) {
     const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
     f32x4 u[NR];
-    const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u), lds);
+    const float amax = row_max<NHW>(actq_rotate<NR, Src, NHW>(src, row, l, hw, nch, u), lds);
     const float s = fmaxf(amax * clip / (float)qmax, 1e-8f), s_rcp = __builtin_amdgcn_rcpf(s);
     if (tid == 0 && s_out) s_out[row] = s;
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
 #pragma unroll
     for (int c = 0; c < NR; c++) {
-        const int ch = hw + 8 * c;
+        const int ch = hw + NHW * c;
         if (ch < nch) {
             f32x4 q;
             f32x4 r = rint_div4(u[c], s, s_rcp);
@@ -635,9 +638,15 @@ struct AbTerm {
     CAMX_DEV f32x4 other(int k) const { return unpack_bf16x4(*(const u32x2 *)(wab + k)); }
 };
 
-template <int NR>
-__global__ void __launch_bounds__(256) block_entry_fwd_k(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y,
-                                                         float * s, uint16_t * codes, uint16_t * ab, float * rstd_out, int d, float clip, int qmax) {
+// NHW = 8: a 256-thread workgroup per row (NR rounds of 1024 values); NHW = 2: one wave per row for rows of at most 1024 values (NR
+// rounds of 256): a lane then holds 16 values instead of 4, and what every lane computes once per row (the square root, the
+// divisions, the reductions' tails, 900 instructions in all) is spread over four times as many values.
+// The projections: wave w takes rows w, w + W, ... of wab (W waves per row), four of them at a time so that their loads fly together,
+// each under the 256-thread tree (a lane holds the logical threads 4 lane .. 4 lane + 3, which add their elements 256 apart in
+// order); rows of at most 2048 values keep bf16(h) in registers.
+template <int NR, int NHW>
+__global__ void __launch_bounds__(32 * NHW) block_entry_fwd_k(const float * x, const float * nw, const uint16_t * wab, int nab, float eps, uint16_t * y,
+                                                              float * s, uint16_t * codes, uint16_t * ab, float * rstd_out, int d, float clip, int qmax) {
     __shared__ float lds[4];
     __shared__ float slot;
     const int row = blockIdx.x;
@@ -645,10 +654,46 @@ __global__ void __launch_bounds__(256) block_entry_fwd_k(const float * x, const 
     const float ss = row_tree_sum(SqTerm{xr}, d, &slot);
     const float rstd = rsqrt_exact(ss / (float)d + eps);
     if (threadIdx.x == 0 && rstd_out) rstd_out[row] = rstd;
-    actq_fwd_row<NR>(RmsSrc{x, nw, rstd, d}, row, y, s, d, clip, qmax, codes, lds);
-    for (int j = 0; j < nab; j++) {
-        const float v = row_tree_sum(AbTerm{xr, nw, rstd, wab + (size_t)j * d}, d, &slot);
-        if (threadIdx.x == 0) ab[(size_t)row * nab + j] = f2bf(v);
+    actq_fwd_row<NR, RmsSrc, NHW>(RmsSrc{x, nw, rstd, d}, row, y, s, d, clip, qmax, codes, lds);
+    if (nab == 0) return;
+    constexpr int NW = NHW / 2, NA = NR * NHW / 2;       // waves per row; 256-element steps of a row
+    constexpr bool KEEP = NA <= 8;
+    const int lane = slot_of(threadIdx.x & 63), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const AbTerm term{xr, nw, rstd, wab};
+    f32x4 hk[KEEP ? NA : 1];
+    if (KEEP) {
+#pragma unroll
+        for (int i = 0; i < NA; i++) { const int k = 256 * i + 4 * lane; hk[KEEP ? i : 0] = k < d ? term(k) : (f32x4){0.0f, 0.0f, 0.0f, 0.0f}; }
+    }
+    for (int j0 = wave; j0 < nab; j0 += 4 * NW) {
+        u32x2 wv[4][NA];
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const int j = j0 + NW * jj;
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                const int k = 256 * i + 4 * lane;
+                wv[jj][i] = (u32x2){0u, 0u};
+                if (j < nab && k < d) wv[jj][i] = *(const u32x2 *)(wab + (size_t)j * d + k);
+            }
+        }
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const int j = j0 + NW * jj;
+            if (j >= nab) break;                         // (wave-uniform)
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                const int k = 256 * i + 4 * lane;
+                if (k < d) {
+                    const f32x4 a = KEEP ? hk[KEEP ? i : 0] : term(k), b = unpack_bf16x4(wv[jj][i]);
+                    acc.x = __builtin_fmaf(a.x, b.x, acc.x); acc.y = __builtin_fmaf(a.y, b.y, acc.y);
+                    acc.z = __builtin_fmaf(a.z, b.z, acc.z); acc.w = __builtin_fmaf(a.w, b.w, acc.w);
+                }
+            }
+            const float tot = wave_groups_in_order(group32_sum(acc));
+            if ((threadIdx.x & 63) == 0) ab[(size_t)row * nab + j] = f2bf(tot);
+        }
     }
 }
 
@@ -666,20 +711,36 @@ __global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const 
     actq_bwd_row<1>(RmsSrc{x, nw, rstd, d}, row, dy, SinkLds{dh}, d, clip, qmax, lds);
     if (tid < nab) dabs[tid] = bf2f(dab[(size_t)row * nab + tid]);
     __syncthreads();
-    const int half = nab / 2;
+    if (nab) {                                           // the projections' part of dh, four neighbouring elements per thread (8-byte loads of wab)
+        const int k4 = 4 * tid, half = nab / 2;
+        if (k4 < d) {
+            u32x2 wv[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) { wv[j] = (u32x2){0u, 0u}; if (j < nab) wv[j] = *(const u32x2 *)(wab + (size_t)j * d + k4); }
+            f32x4 pa = {0.0f, 0.0f, 0.0f, 0.0f}, pb = pa;
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                if (j < nab) {                               // (uniform) rows [0, half) add into pa, [half, nab) into pb, each in order
+                    const f32x4 w = unpack_bf16x4(wv[j]);
+                    const float c = dabs[j];
+                    if (j < half) { pa.x = __builtin_fmaf(c, w.x, pa.x); pa.y = __builtin_fmaf(c, w.y, pa.y); pa.z = __builtin_fmaf(c, w.z, pa.z); pa.w = __builtin_fmaf(c, w.w, pa.w); }
+                    else { pb.x = __builtin_fmaf(c, w.x, pb.x); pb.y = __builtin_fmaf(c, w.y, pb.y); pb.z = __builtin_fmaf(c, w.z, pb.z); pb.w = __builtin_fmaf(c, w.w, pb.w); }
+                }
+            }
+            f32x4 g = *(const f32x4 *)(dh + k4);
+            const f32x4 ra = rbf4_canon(pa), rb = rbf4_canon(pb);
+            g.x = (g.x + ra.x) + rb.x; g.y = (g.y + ra.y) + rb.y; g.z = (g.z + ra.z) + rb.z; g.w = (g.w + ra.w) + rb.w;
+            *(f32x4 *)(dh + k4) = g;
+        }
+        __syncthreads();
+    }
     float dot = 0.0f, none = 0.0f, gk[4], xh[4], wk[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int k = t + 256 * i;
         gk[i] = xh[i] = wk[i] = 0.0f;
         if (k < d) {
-            float g = dh[k];
-            if (nab) {
-                float pa = 0.0f, pb = 0.0f;
-                for (int j = 0; j < half; j++) pa = __builtin_fmaf(dabs[j], bf2f(wab[(size_t)j * d + k]), pa);
-                for (int j = half; j < nab; j++) pb = __builtin_fmaf(dabs[j], bf2f(wab[(size_t)j * d + k]), pb);
-                g = (g + rbf(pa)) + rbf(pb);
-            }
+            const float g = dh[k];
             gk[i] = g; wk[i] = nw[k]; xh[i] = xr[k] * rstd;
             dot = __builtin_fmaf(g * wk[i], xh[i], dot);
         }
@@ -769,7 +830,16 @@ int camx_block_entry_fwd(const float * x, const float * nw, const uint16_t * wab
     if (!x || !nw || (!y && !codes) || actq_check(d, qmax, M) || nab < 0 || nab > 16 || (nab && (!wab || !ab)) || ((uintptr_t)x & 15) ||
         ((uintptr_t)nw & 15) || ((uintptr_t)wab & 7) || ((uintptr_t)y & 7) || ((uintptr_t)codes & 1)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    ACTQ_ROUNDS(d, (block_entry_fwd_k<NR><<<dim3(M), dim3(256), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax)))
+    if (d <= 1024) {                                     // one wave per row, rounds of 256 values
+        switch ((d + 255) / 256) {
+            case 1: block_entry_fwd_k<1, 2><<<dim3(M), dim3(64), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax); break;
+            case 2: block_entry_fwd_k<2, 2><<<dim3(M), dim3(64), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax); break;
+            case 3: block_entry_fwd_k<3, 2><<<dim3(M), dim3(64), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax); break;
+            default: block_entry_fwd_k<4, 2><<<dim3(M), dim3(64), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax); break;
+        }
+        CAMX_LAUNCH_RET();
+    }
+    ACTQ_ROUNDS(d, (block_entry_fwd_k<NR, 8><<<dim3(M), dim3(256), 0, st>>>(x, nw, wab, nab, eps, y, s, codes, ab, rstd_out, d, clip, qmax)))
     CAMX_LAUNCH_RET();
 }
 

@@ -29,17 +29,20 @@ def test_actq_fwd(M, K, qmax):
             if qmax <= 7: assert bits_equal(host(c)[2 * shift:2 * shift + M * K // 2].reshape(M, K // 2), rc)
 
 
-def test_block_entry_fwd():
-    rng = np.random.default_rng(11)
-    M, d, nab = 6, 896, 8
+@pytest.mark.parametrize('M,d,nab', [(6, 896, 8), (5, 1024, 16), (3, 2048, 5), (2, 4096, 2), (130, 1024, 14), (4, 128, 1), (3, 8192, 3), (7, 768, 0),
+                                     (9, 512, 6), (5, 256, 16), (300, 640, 3), (4, 1152, 9)])
+def test_block_entry_fwd(M, d, nab):
+    """rows of at most 1024 values: one wave per row, every round count; longer rows: a workgroup per row. The projections run one
+    per wave (rows w, w + W, ... of wab): counts that are not multiples of four, rows that keep bf16(h) in registers and longer ones"""
+    rng = np.random.default_rng(11 + d + nab)
     x = outliers(rng, (M, d)); nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32); wab = O.f2bf(rng.standard_normal((nab, d)) * 0.05)
-    ry, rs, rc, rab, rstd = O.block_entry_fwd(x, nw, wab, 1e-6)
+    ry, rs, rc, rab, rstd = O.block_entry_fwd(x, nw, wab if nab else None, 1e-6)
     y = dev(np.zeros((M, d), np.uint16)); s = dev(np.zeros(M, np.float32)); c = dev(np.zeros((M, d // 2), np.uint8))
-    ab = dev(np.zeros((M, nab), np.uint16)); rstd_d = dev(np.zeros(M, np.float32))
-    call('camx_block_entry_fwd', ptr(dev(x)), ptr(dev(nw)), ptr(dev(wab)), I(nab), F(1e-6), ptr(y), ptr(s), ptr(c), ptr(ab), ptr(rstd_d),
-         I(d), F(1.0), I(7), I(M))
+    ab = dev(np.zeros((M, max(nab, 1)), np.uint16)); rstd_d = dev(np.zeros(M, np.float32))
+    call('camx_block_entry_fwd', ptr(dev(x)), ptr(dev(nw)), ptr(dev(wab)) if nab else NULL, I(nab), F(1e-6), ptr(y), ptr(s), ptr(c),
+         ptr(ab) if nab else NULL, ptr(rstd_d), I(d), F(1.0), I(7), I(M))
     assert bits_equal(host(rstd_d), rstd) and bits_equal(host(s), rs) and bits_equal(host(c), rc) and bits_equal(host(y, np.uint16), ry)
-    assert bits_equal(host(ab, np.uint16), rab)
+    if nab: assert bits_equal(host(ab, np.uint16), rab)
 
 
 @pytest.mark.parametrize('M,Fh', [(5, 768), (2100, 1024), (2050, 1920), (2049, 2176), (4099, 128), (5, 2304), (303, 2048)])
@@ -103,7 +106,7 @@ def test_actq_bwd_quotients_at_the_exponent_limits(K):
             assert np.array_equal(nan_w, nan_g) and bits_equal(np.where(nan_w, 0, got), np.where(nan_w, 0, want))
 
 
-@pytest.mark.parametrize('M,d,nab', [(6, 896, 14), (5, 1024, 0), (9, 256, 2), (130, 896, 16)])
+@pytest.mark.parametrize('M,d,nab', [(6, 896, 14), (5, 1024, 0), (9, 256, 2), (130, 896, 16), (7, 1024, 16), (3, 128, 4)])
 def test_block_entry_bwd(M, d, nab):
     rng = np.random.default_rng(200 + d + nab)
     x = outliers(rng, (M, d)); nw = (0.5 + rng.random(d)).astype(np.float32)
