@@ -435,31 +435,34 @@ struct SinkSiluMul {
 };
 
 // lds16: 16 floats. sink receives bf16-valued floats: the gradient of the bf16 source, before any widening store.
-template <int NR, typename Src, typename Sink>
-CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Sink sink, int K, float clip, int qmax, float * lds16) {
+// NHW = 8: a 256-thread workgroup per row. NHW = 2: one wave per row of at most 1024 values (each half-wave sum of the tree is
+// then one chunk's: round c holds chunks 2 c and 2 c + 1); out, when given, receives round c's result in place of the sink.
+template <int NR, typename Src, typename Sink, int NHW = 8>
+CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Sink sink, int K, float clip, int qmax, float * lds16, f32x4 * out = nullptr) {
     const int tid = threadIdx.x, l = slot_of(tid) & 31, hw = tid >> 5, nch = K / 128;
     f32x4 u[NR], gv[NR];
 #pragma unroll
     for (int c = 0; c < NR; c++) {
-        const int ch = hw + 8 * c;
+        const int ch = hw + NHW * c;
         u32x2 raw = {0u, 0u};
         if (ch < nch) raw = *(const u32x2 *)(g + (size_t)row * K + ch * 128 + 4 * l);
         gv[c] = unpack_bf16x4(raw);
     }
     u32x2 keep[NR];                                      // what the source hands to the sink (the fused SiLU form only)
-    const float amax = row_max(actq_rotate<NR>(src, row, l, hw, nch, u, keep), lds16);
+    const float amax = row_max<NHW>(actq_rotate<NR, Src, NHW>(src, row, l, hw, nch, u, keep), lds16);
     const float s_raw = amax * clip / (float)qmax, s = fmaxf(s_raw, 1e-8f);
     const float lo = (float)(-qmax - 1), hi = (float)qmax;
     // dL/ds = sum g (q - m t) and the number of max-|u| elements; m: the rounded value lies strictly inside (lo, hi). The
     // straight-through part g m is formed here (g is not needed afterwards); the ties are counted from the compares' lane masks
     // on the scalar unit, one counter per half-wave (a count is exact in any order).
     const RowDiv rd(s, amax);
-    float dlds = 0.0f;
+    float dlds = 0.0f, part[NHW == 2 ? NR : 1];           // NHW == 2: a sum per round (a reference lane's terms are one chunk's)
     int ties_lo = 0, ties_hi = 0;
     uint32_t tied = 0;                                   // bit c: some lane of this wave holds a max-|u| element in round c
 #pragma unroll
     for (int c = 0; c < NR; c++) {
-        if (hw + 8 * c < nch) {
+        if (NHW == 2) dlds = 0.0f;
+        if (hw + NHW * c < nch) {
             const f32x4 t4 = rd.div4(u[c]);
             uint64_t any = 0;
 #define D_(e) { const float t = t4.e, r = rintf(t), q = fminf(fmaxf(r, lo), hi); const bool m = r > lo && r < hi; \
@@ -470,13 +473,28 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
 #undef D_
             if (any) tied |= 1u << c;
         }
+        if (NHW == 2) part[NHW == 2 ? c : 0] = dlds;
     }
-    float ties = (tid & 31) == 0 ? (float)((tid & 32) ? ties_hi : ties_lo) : 0.0f;
-    block8_sum2(dlds, ties, lds16);
+    float ties;
+    if (NHW == 2) {                                      // the eight chunk sums in order (absent chunks add +0, as idle half-waves do)
+        ties = (float)(ties_lo + ties_hi);
+#pragma unroll
+        for (int c = 0; c < NR; c++) {
+            const float hs = half32_sum(part[NHW == 2 ? c : 0]);
+            const float even = lane_read(hs, 0), odd = lane_read(hs, 32);
+            dlds = c == 0 ? even : dlds + even;
+            dlds += odd;
+        }
+        if (2 * NR < 8) dlds += 0.0f;
+    } else {
+        ties = (tid & 31) == 0 ? (float)((tid & 32) ? ties_hi : ties_lo) : 0.0f;
+        block8_sum2(dlds, ties, lds16);
+    }
     const float coef = s_raw >= 1e-8f ? dlds * clip / (float)qmax / ties : 0.0f;
 #pragma unroll
     for (int c = 0; c < NR; c++) {
-        const int ch = hw + 8 * c;
+        const int ch = hw + NHW * c;
+        if (out) out[c] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
         if (ch < nch) {
             f32x4 d = gv[c];
             if (tied & (1u << c)) {                      // wave-uniform: a row has few such elements, most rounds skip this
@@ -484,7 +502,8 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
                 CAMX_EACH4(V_)
 #undef V_
             }
-            sink(row, ch * 128 + 4 * l, rbf4_canon(scaled4(hadamard128_l4(rbf4_any(d), l, false))), keep[c]);      // rbf4_any: the gradient of the bf16 tensor u
+            const f32x4 r = rbf4_canon(scaled4(hadamard128_l4(rbf4_any(d), l, false)));      // rbf4_any: the gradient of the bf16 tensor u
+            if (out) out[c] = r; else sink(row, ch * 128 + 4 * l, r, keep[c]);
         }
     }
 }
@@ -641,7 +660,7 @@ struct AbTerm {
 // NHW = 8: a 256-thread workgroup per row (NR rounds of 1024 values); NHW = 2: one wave per row for rows of at most 1024 values (NR
 // rounds of 256): a lane then holds 16 values instead of 4, and what every lane computes once per row (the square root, the
 // divisions, the reductions' tails, 900 instructions in all) is spread over four times as many values.
-// The projections: wave w takes rows w, w + W, ... of wab (W waves per row), four of them at a time so that their loads fly together,
+// The projections: wave w takes rows w, w + W, ... of wab (W waves per row), up to four of them at a time so that their loads fly together,
 // each under the 256-thread tree (a lane holds the logical threads 4 lane .. 4 lane + 3, which add their elements 256 apart in
 // order); rows of at most 2048 values keep bf16(h) in registers.
 template <int NR, int NHW>
@@ -665,10 +684,11 @@ __global__ void __launch_bounds__(32 * NHW) block_entry_fwd_k(const float * x, c
 #pragma unroll
         for (int i = 0; i < NA; i++) { const int k = 256 * i + 4 * lane; hk[KEEP ? i : 0] = k < d ? term(k) : (f32x4){0.0f, 0.0f, 0.0f, 0.0f}; }
     }
-    for (int j0 = wave; j0 < nab; j0 += 4 * NW) {
-        u32x2 wv[4][NA];
+    constexpr int JB = NA <= 4 ? 4 : NA <= 8 ? 2 : 1;   // rows of wab whose loads fly together
+    for (int j0 = wave; j0 < nab; j0 += JB * NW) {
+        u32x2 wv[JB][NA];
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++) {
+        for (int jj = 0; jj < JB; jj++) {
             const int j = j0 + NW * jj;
 #pragma unroll
             for (int i = 0; i < NA; i++) {
@@ -678,7 +698,7 @@ __global__ void __launch_bounds__(32 * NHW) block_entry_fwd_k(const float * x, c
             }
         }
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++) {
+        for (int jj = 0; jj < JB; jj++) {
             const int j = j0 + NW * jj;
             if (j >= nab) break;                         // (wave-uniform)
             f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -699,58 +719,82 @@ __global__ void __launch_bounds__(32 * NHW) block_entry_fwd_k(const float * x, c
 
 // dh = actq backward of dy, plus the two projection groups' input gradients (wab rows [0, nab / 2) and [nab / 2, nab), each
 // group's sum rounded to bf16); then the RMSNorm backward dx = rstd (dh w - xhat mean(dh w xhat)), xhat = x rstd. d <= 1024.
-// Thread t (slot space) owns elements t, t + 256, ...
-__global__ void __launch_bounds__(256) block_entry_bwd_k(const float * x, const float * nw, const float * rstd_in, const uint16_t * wab, int nab,
-                                                         const uint16_t * dy, const uint16_t * dab, float * dx, int d, float clip, int qmax) {
-    __shared__ __attribute__((aligned(16))) float dh[1024];
-    __shared__ float lds[16];
-    __shared__ float dabs[16];
-    const int row = blockIdx.x, tid = threadIdx.x, t = slot_of(tid);
+// One wave per row, NR = ceil(d / 256) rounds: lane (slot la) holds elements 256 c + 4 la .. + 3 of round c through all three steps,
+// i.e. the logical threads 4 la .. 4 la + 3 of the 256-thread tree of the dot product (thread t owns elements t, t + 256, ...).
+struct SinkNone { CAMX_DEV void operator()(int, int, f32x4, u32x2) const {} };
+template <int NR>
+__global__ void __launch_bounds__(64) block_entry_bwd_k(const float * x, const float * nw, const float * rstd_in, const uint16_t * wab, int nab,
+                                                        const uint16_t * dy, const uint16_t * dab, float * dx, int d, float clip, int qmax) {
+    const int row = blockIdx.x, la = slot_of(threadIdx.x);
     const float rstd = rstd_in[row];
     const float * xr = x + (size_t)row * d;
-    actq_bwd_row<1>(RmsSrc{x, nw, rstd, d}, row, dy, SinkLds{dh}, d, clip, qmax, lds);
-    if (tid < nab) dabs[tid] = bf2f(dab[(size_t)row * nab + tid]);
-    __syncthreads();
-    if (nab) {                                           // the projections' part of dh, four neighbouring elements per thread (8-byte loads of wab)
-        const int k4 = 4 * tid, half = nab / 2;
-        if (k4 < d) {
-            u32x2 wv[16];
+    f32x4 dh[NR];
+    actq_bwd_row<NR, RmsSrc, SinkNone, 2>(RmsSrc{x, nw, rstd, d}, row, dy, SinkNone{}, d, clip, qmax, nullptr, dh);
+    if (nab) {                                           // the projections' part of dh
+        const int half = nab / 2;
+        float dabs[2][8];                                // the row's dab by group, the same in every lane: scalar registers
 #pragma unroll
-            for (int j = 0; j < 16; j++) { wv[j] = (u32x2){0u, 0u}; if (j < nab) wv[j] = *(const u32x2 *)(wab + (size_t)j * d + k4); }
-            f32x4 pa = {0.0f, 0.0f, 0.0f, 0.0f}, pb = pa;
+        for (int h = 0; h < 2; h++)
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-                if (j < nab) {                               // (uniform) rows [0, half) add into pa, [half, nab) into pb, each in order
-                    const f32x4 w = unpack_bf16x4(wv[j]);
-                    const float c = dabs[j];
-                    if (j < half) { pa.x = __builtin_fmaf(c, w.x, pa.x); pa.y = __builtin_fmaf(c, w.y, pa.y); pa.z = __builtin_fmaf(c, w.z, pa.z); pa.w = __builtin_fmaf(c, w.w, pa.w); }
-                    else { pb.x = __builtin_fmaf(c, w.x, pb.x); pb.y = __builtin_fmaf(c, w.y, pb.y); pb.z = __builtin_fmaf(c, w.z, pb.z); pb.w = __builtin_fmaf(c, w.w, pb.w); }
-                }
+            for (int j = 0; j < 8; j++) {
+                const uint32_t w = j < half ? (uint32_t)__builtin_amdgcn_readfirstlane((int)dab[(size_t)row * nab + h * half + j]) : 0u;
+                dabs[h][j] = __builtin_bit_cast(float, w << 16);
             }
-            f32x4 g = *(const f32x4 *)(dh + k4);
-            const f32x4 ra = rbf4_canon(pa), rb = rbf4_canon(pb);
-            g.x = (g.x + ra.x) + rb.x; g.y = (g.y + ra.y) + rb.y; g.z = (g.z + ra.z) + rb.z; g.w = (g.w + ra.w) + rb.w;
-            *(f32x4 *)(dh + k4) = g;
-        }
-        __syncthreads();
-    }
-    float dot = 0.0f, none = 0.0f, gk[4], xh[4], wk[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int k = t + 256 * i;
-        gk[i] = xh[i] = wk[i] = 0.0f;
-        if (k < d) {
-            const float g = dh[k];
-            gk[i] = g; wk[i] = nw[k]; xh[i] = xr[k] * rstd;
-            dot = __builtin_fmaf(g * wk[i], xh[i], dot);
+        for (int c = 0; c < NR; c++) {
+            const int k = 256 * c + 4 * la;
+            if (k < d) {
+                f32x4 p[2];                              // rows [0, half) of wab add into p[0], [half, nab) into p[1], each in order
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    u32x2 wv[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) { wv[j] = (u32x2){0u, 0u}; if (j < half) wv[j] = *(const u32x2 *)(wab + (size_t)(h * half + j) * d + k); }
+                    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        if (j < half) {                  // (uniform)
+                            const f32x4 w = unpack_bf16x4(wv[j]);
+                            const float cj = dabs[h][j];
+                            acc.x = __builtin_fmaf(cj, w.x, acc.x); acc.y = __builtin_fmaf(cj, w.y, acc.y); acc.z = __builtin_fmaf(cj, w.z, acc.z); acc.w = __builtin_fmaf(cj, w.w, acc.w);
+                        }
+                    }
+                    p[h] = acc;
+                }
+                const f32x4 ra = rbf4_canon(p[0]), rb = rbf4_canon(p[1]);
+                f32x4 g = dh[c];
+                g.x = (g.x + ra.x) + rb.x; g.y = (g.y + ra.y) + rb.y; g.z = (g.z + ra.z) + rb.z; g.w = (g.w + ra.w) + rb.w;
+                dh[c] = g;
+            }
         }
     }
-    block8_sum2(dot, none, lds);
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, gw[NR], xh[NR];
+#pragma unroll
+    for (int c = 0; c < NR; c++) {
+        const int k = 256 * c + 4 * la;
+        gw[c] = xh[c] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        if (k < d) {
+            const f32x4 w = *(const f32x4 *)(nw + k), xv = *(const f32x4 *)(xr + k);
+            gw[c] = (f32x4){dh[c].x * w.x, dh[c].y * w.y, dh[c].z * w.z, dh[c].w * w.w};
+            xh[c] = (f32x4){xv.x * rstd, xv.y * rstd, xv.z * rstd, xv.w * rstd};
+            acc.x = __builtin_fmaf(gw[c].x, xh[c].x, acc.x); acc.y = __builtin_fmaf(gw[c].y, xh[c].y, acc.y);
+            acc.z = __builtin_fmaf(gw[c].z, xh[c].z, acc.z); acc.w = __builtin_fmaf(gw[c].w, xh[c].w, acc.w);
+        }
+    }
+    const float gs = group32_sum(acc);                   // the 32 logical threads of a group, then the eight groups in order
+    float dot = lane_read(gs, 0);
+#pragma unroll
+    for (int q = 1; q < 8; q++) dot += lane_read(gs, 8 * q);
     dot = dot / (float)d;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int k = t + 256 * i;
-        if (k < d) dx[(size_t)row * d + k] = rstd * (gk[i] * wk[i] - xh[i] * dot);
+    for (int c = 0; c < NR; c++) {
+        const int k = 256 * c + 4 * la;
+        if (k < d) {
+            f32x4 r;
+            r.x = rstd * (gw[c].x - xh[c].x * dot); r.y = rstd * (gw[c].y - xh[c].y * dot);
+            r.z = rstd * (gw[c].z - xh[c].z * dot); r.w = rstd * (gw[c].w - xh[c].w * dot);
+            *(f32x4 *)(dx + (size_t)row * d + k) = r;
+        }
     }
 }
 
@@ -876,9 +920,14 @@ int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * 
 int camx_block_entry_bwd(const float * x, const float * nw, const float * rstd, const uint16_t * wab, int nab, const uint16_t * dy,
                          const uint16_t * dab, float * dx, int d, float clip, int qmax, int M, hipStream_t st) {
     if (!x || !nw || !rstd || !dy || !dx || actq_check(d, qmax, M) || d > 1024 || nab < 0 || nab > 16 || (nab & 1) || (nab && (!wab || !dab)) ||
-        ((uintptr_t)x & 15) || ((uintptr_t)nw & 15) || ((uintptr_t)dy & 7)) return CAMX_EINVAL;
+        ((uintptr_t)x & 15) || ((uintptr_t)nw & 15) || ((uintptr_t)dy & 7) || ((uintptr_t)dx & 15) || ((uintptr_t)wab & 7)) return CAMX_EINVAL;
     if (M == 0) return CAMX_OK;
-    block_entry_bwd_k<<<dim3(M), dim3(256), 0, st>>>(x, nw, rstd, wab, nab, dy, dab, dx, d, clip, qmax);
+    switch ((d + 255) / 256) {
+        case 1: block_entry_bwd_k<1><<<dim3(M), dim3(64), 0, st>>>(x, nw, rstd, wab, nab, dy, dab, dx, d, clip, qmax); break;
+        case 2: block_entry_bwd_k<2><<<dim3(M), dim3(64), 0, st>>>(x, nw, rstd, wab, nab, dy, dab, dx, d, clip, qmax); break;
+        case 3: block_entry_bwd_k<3><<<dim3(M), dim3(64), 0, st>>>(x, nw, rstd, wab, nab, dy, dab, dx, d, clip, qmax); break;
+        default: block_entry_bwd_k<4><<<dim3(M), dim3(64), 0, st>>>(x, nw, rstd, wab, nab, dy, dab, dx, d, clip, qmax); break;
+    }
     CAMX_LAUNCH_RET();
 }
 

@@ -288,7 +288,8 @@ int camx_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void * dx, in
 int camx_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, float clip, int qmax, int M,
                            camx_stream_t stream);
 /* block_entry_bwd (kernels/actq.hip:275-304): rstd [M] as the forward wrote it; dy bf16 [M][d]; dab bf16 [M][nab] (nab even; rows
- * [0, nab / 2) and [nab / 2, nab) of wab are two projections); dx fp32 [M][d]; d <= 1024. */
+ * [0, nab / 2) and [nab / 2, nab) of wab are two projections); dx fp32 [M][d]; d <= 1024. x, nw and dx 16-byte aligned, dy and wab
+ * 8-byte aligned. */
 int camx_block_entry_bwd(const float * x, const float * nw, const float * rstd, const uint16_t * wab, int nab, const uint16_t * dy,
                          const uint16_t * dab, float * dx, int d, float clip, int qmax, int M, camx_stream_t stream);
 
