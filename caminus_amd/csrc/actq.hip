@@ -477,7 +477,7 @@ CAMX_DEV void actq_bwd_row(Src src, int row, const uint16_t * __restrict__ g, Si
     }
     float ties;
     if (NHW == 2) {                                      // the eight chunk sums in order (absent chunks add +0, as idle half-waves do)
-        ties = (float)(ties_lo + ties_hi);
+        ties = lane_read((float)(ties_lo + ties_hi), 0);          // lane 0's count: its half-wave is in every round that any lane is in (the counters of a lane that sits out a round miss that round)
 #pragma unroll
         for (int c = 0; c < NR; c++) {
             const float hs = half32_sum(part[NHW == 2 ? c : 0]);

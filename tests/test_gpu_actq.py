@@ -106,10 +106,15 @@ def test_actq_bwd_quotients_at_the_exponent_limits(K):
             assert np.array_equal(nan_w, nan_g) and bits_equal(np.where(nan_w, 0, got), np.where(nan_w, 0, want))
 
 
-@pytest.mark.parametrize('M,d,nab', [(6, 896, 14), (5, 1024, 0), (9, 256, 2), (130, 896, 16), (7, 1024, 16), (3, 128, 4)])
+@pytest.mark.parametrize('M,d,nab', [(6, 896, 14), (5, 1024, 0), (9, 256, 2), (130, 896, 16), (7, 1024, 16), (3, 128, 4), (171, 896, 8), (12, 640, 6), (9, 384, 0)])
 def test_block_entry_bwd(M, d, nab):
+    """every round count of the wave-per-row kernel; row 1 has one value in the row's last chunk and one in chunk 1 with the same
+    |h|: their chunks rotate to constants, so 256 elements tie for the row's maximum across rounds that not all lanes take part in"""
     rng = np.random.default_rng(200 + d + nab)
     x = outliers(rng, (M, d)); nw = (0.5 + rng.random(d)).astype(np.float32)
+    if d >= 384:
+        last = d - 128 + 5
+        nw[last] = nw[128 + 7]; x[1] = 0; x[1, 128 + 7] = 3.0; x[1, last] = -3.0
     wab = O.f2bf((rng.standard_normal((max(nab, 2), d)) / 30).astype(np.float32))[:nab]
     dy = O.f2bf(rng.standard_normal((M, d)).astype(np.float32)); dab = O.f2bf(rng.standard_normal((M, max(nab, 1))).astype(np.float32))[:, :nab]
     rstd = O.block_entry_fwd(x, nw, wab if nab else None, 1e-6)[4]
