@@ -197,31 +197,35 @@ __global__ void __launch_bounds__(256) hc_avg_k(const float * __restrict__ r, fl
 // One workgroup per token; the dot product is the 256-thread tree with a product and a sum per element; HC <= 8.
 __global__ void __launch_bounds__(256) ple_gate_k(const float * kn, const float * q, const float * qscl, const float * qw, const float * val, int ldv,
                                                   float * gated, float * gate_out, int HC, int D) {
-    __shared__ float part[8];
+    __shared__ float part[8][8];                         // [stream][half-wave]
     __shared__ float gate[8];
     const int tid = threadIdx.x, t = slot_of(tid), tt = blockIdx.x;
     const float * k_ = kn + (size_t)tt * HC * D, * q_ = q + (size_t)tt * HC * D, * v_ = val + (size_t)tt * ldv;
-    for (int st = 0; st < HC; st++) {
-        float acc = 0.0f;
-        for (int i = t; i < D; i += 256) {
-            const float qv = qscl ? (q_[(size_t)st * D + i] * qscl[tt * HC + st]) * qw[(size_t)st * D + i] : q_[(size_t)st * D + i];
-            acc = acc + k_[(size_t)st * D + i] * qv;
+    // the streams' dot products side by side (each under its own 256-thread tree), one pair of barriers for all of them, and the
+    // gates of the HC streams on HC threads
+#pragma unroll
+    for (int st = 0; st < 8; st++) {
+        if (st < HC) {
+            float acc = 0.0f;
+            for (int i = t; i < D; i += 256) {
+                const float qv = qscl ? (q_[(size_t)st * D + i] * qscl[tt * HC + st]) * qw[(size_t)st * D + i] : q_[(size_t)st * D + i];
+                acc = acc + k_[(size_t)st * D + i] * qv;
+            }
+            acc += lane_xor16(acc); acc += lane_xor8(acc); acc += lane_xor4(acc); acc += lane_xor2(acc); acc += lane_xor1(acc);
+            if ((tid & 31) == 0) part[st][tid >> 5] = acc;
         }
-        acc += lane_xor16(acc); acc += lane_xor8(acc); acc += lane_xor4(acc); acc += lane_xor2(acc); acc += lane_xor1(acc);
-        __syncthreads();
-        if ((tid & 31) == 0) part[tid >> 5] = acc;
-        __syncthreads();
-        if (tid == 0) {
-            float sum = 0.0f;
-            for (int w = 0; w < 8; w++) sum += part[w];
-            const float s = sum * (1.0f / sqrtf((float)D));
-            const float mag = sqrtf(fmaxf(fabsf(s), 1e-6f));
-            const float sgn = s > 0.0f ? 1.0f : (s < 0.0f ? -1.0f : 0.0f);
-            const float gv = 1.0f / (1.0f + expf(-(sgn * mag)));
-            gate[st] = gv; gate_out[tt * HC + st] = gv;
-        }
-        __syncthreads();
     }
+    __syncthreads();
+    if (tid < HC) {
+        float sum = 0.0f;
+        for (int w = 0; w < 8; w++) sum += part[tid][w];
+        const float s = sum * (1.0f / sqrtf((float)D));
+        const float mag = sqrtf(fmaxf(fabsf(s), 1e-6f));
+        const float sgn = s > 0.0f ? 1.0f : (s < 0.0f ? -1.0f : 0.0f);
+        const float gv = 1.0f / (1.0f + expf(-(sgn * mag)));
+        gate[tid] = gv; gate_out[tt * HC + tid] = gv;
+    }
+    __syncthreads();
     // (gated may alias kn: every read of this token's kn rows is behind the barriers above)
     for (int c = tid; c < HC * D; c += 256) gated[(size_t)tt * HC * D + c] = v_[c % D] * gate[c / D];
 }
