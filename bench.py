@@ -386,6 +386,38 @@ def prefill_scale_sweep(B, T=4096, only=None):
         x = B.acts((Mr * Kq,), torch.float32, i); m = B.acts((Mr * Kq,), torch.bfloat16, i + 1); y = B.acts((Mr * Kq,), torch.bfloat16, i + 2); o = torch.empty(Mr * Kq, device=dev)
         return lambda: B.call('camx_residual3', _p(x), _p(m), _p(y), _p(o), L64(Mr * Kq))
     timeit('residual3 16M', Mr * Kq * 12, mk)
+    nys = 1024
+    ys = B.acts((nys, Kq), torch.bfloat16, 77); pos = torch.full((Mr,), -1, dtype=torch.int32, device=dev); pos[::Mr // nys] = torch.arange(nys, dtype=torch.int32, device=dev)
+    def mk(i):
+        x = B.acts((Mr, Kq), torch.float32, i); m = B.acts((Mr, Kq), torch.bfloat16, i + 1); mlp = B.acts((Mr, Kq), torch.bfloat16, i + 2); o = torch.empty((Mr, Kq), device=dev)
+        return lambda: B.call('camx_residual_slices_fwd', _p(x), _p(m), _p(mlp), _p(ys), _p(pos), _p(o), I(Kq), L64(Mr * Kq // 4))
+    timeit('residual_slices_fwd 8192x2048, 1024 slices', Mr * Kq * 12 + nys * Kq * 2, mk)
+    def mk(i):
+        do = B.acts((Mr, Kq), torch.float32, i); dm = torch.empty((Mr, Kq), dtype=torch.bfloat16, device=dev); dmlp = torch.empty_like(dm); dys = torch.empty((nys, Kq), dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_residual_slices_bwd', _p(do), _p(pos), _p(dm), _p(dmlp), _p(dys), I(Kq), L64(Mr * Kq // 4))
+    timeit('residual_slices_bwd 8192x2048, 1024 slices', Mr * Kq * 8 + nys * Kq * 2, mk)
+    wn = B.gamma(Kq, 9)
+    def mk(i):
+        x = B.acts((Mr, Kq), torch.float32, i); o = torch.empty((Mr, Kq), device=dev)
+        return lambda: B.call('camx_rmsnorm_f32', _p(x), _p(wn), _p(o), I(Kq), F(1e-6), I(Mr))
+    timeit('rmsnorm_f32 8192x2048', Mr * Kq * 8, mk)
+    def mk(i):
+        x = B.acts((Mr * Kq,), torch.float32, i); o = torch.empty(Mr * Kq, dtype=torch.bfloat16, device=dev)
+        return lambda: B.call('camx_cast_bf16', _p(x), _p(o), L64(Mr * Kq))
+    timeit('cast_bf16 16M', Mr * Kq * 6, mk)
+    ntk, Ks, neu = T, 2048, 8
+    def mk(i):
+        x = B.acts((ntk, Ks), torch.float32, i); ids = torch.randperm(ntk * neu, device=dev).to(torch.int32); vy = torch.empty((Ks // 128) * ntk * neu * 144, dtype=torch.uint8, device=dev)
+        return lambda: B.call('camx_quantize_mmq_q8_1_scatter', _p(x), _p(ids), _p(vy), L64(Ks), L64(0), L64(Ks), L64(0), L64(Ks), I(ntk * neu), I(1), I(neu), I(1), I(ntk))
+    timeit(f'quantize_mmq_q8_1_scatter {T}x2048 to 8 columns each', ntk * Ks * 4 + (Ks // 128) * ntk * neu * 144, mk)
+    def mk(i):
+        k = B.acts((T, 512), torch.float32, i); v = B.acts((T, 512), torch.float32, i + 2); cache = torch.empty(T * 1088, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_pf_kv_append', _p(k), I(512), _p(v), I(512), I(512), _p(cache), I(0), I(T), _p(err), I(T))
+    timeit(f'pf_kv_append {T}x512', T * (512 * 8 + 1088), mk)
+    def mk(i):
+        x = B.acts((T * 36, 128), torch.float32, i)
+        return lambda: B.call('camx_pf_hadamard', _p(x), I(T * 36), I(128), I(4))
+    timeit(f'pf_hadamard {T}x36 chunks of 128', T * 36 * 128 * 8, mk)
     rows_g, Kg = T * 48, 128
     def mk(i):
         o = B.acts((rows_g, Kg), torch.float32, i); z = B.acts((rows_g, Kg), torch.float32, i + 1, frac=0); wg = B.gamma(Kg, 5); y16 = torch.empty((rows_g, Kg), dtype=torch.float16, device=dev)

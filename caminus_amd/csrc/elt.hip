@@ -467,6 +467,34 @@ __global__ void __launch_bounds__(256) residual_slices_fwd_k(const float * __res
     *(f32x4 *)(out + e) = o;
 }
 
+// the same with the row in blockIdx.y (no division of a 64-bit element index per thread) and every streamed operand non-temporal
+// (8192 x 2048: 38.9 -> 34.5 us forward, 29.1 -> 26.2 us backward; 16-byte accesses of eight values per thread measured no better)
+__global__ void __launch_bounds__(256) residual_slices_fwd_rows(const float * __restrict__ x, const uint16_t * __restrict__ m, const uint16_t * __restrict__ mlp,
+                                                                const uint16_t * __restrict__ ys, const int * __restrict__ pos, float * __restrict__ out, int d) {
+    const int r = blockIdx.y, c = 4 * (blockIdx.x * 256 + threadIdx.x);
+    if (c >= d) return;
+    const size_t e = (size_t)r * d + c;
+    const f32x4 xv = __builtin_nontemporal_load((const f32x4 *)(x + e));
+    const f32x4 mv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)(m + e))), lv = unpack_bf16x4(__builtin_nontemporal_load((const u32x2 *)(mlp + e)));
+    const int p = pos ? pos[r] : -1;
+    f32x4 sv = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (p >= 0) sv = unpack_bf16x4(*(const u32x2 *)(ys + (size_t)p * d + c));
+    f32x4 o;
+    o.x = ((xv.x + mv.x) + lv.x) + sv.x; o.y = ((xv.y + mv.y) + lv.y) + sv.y;
+    o.z = ((xv.z + mv.z) + lv.z) + sv.z; o.w = ((xv.w + mv.w) + lv.w) + sv.w;
+    __builtin_nontemporal_store(o, (f32x4 *)(out + e));
+}
+__global__ void __launch_bounds__(256) residual_slices_bwd_rows(const float * __restrict__ dout, const int * __restrict__ pos, uint16_t * __restrict__ dm,
+                                                                uint16_t * __restrict__ dmlp, uint16_t * __restrict__ dys, int d) {
+    const int r = blockIdx.y, c = 4 * (blockIdx.x * 256 + threadIdx.x);
+    if (c >= d) return;
+    const size_t e = (size_t)r * d + c;
+    const u32x2 b = pack_f2bf_x4(__builtin_nontemporal_load((const f32x4 *)(dout + e)));
+    __builtin_nontemporal_store(b, (u32x2 *)(dm + e)); __builtin_nontemporal_store(b, (u32x2 *)(dmlp + e));
+    const int p = pos ? pos[r] : -1;
+    if (p >= 0) *(u32x2 *)(dys + (size_t)p * d + c) = b;
+}
+
 __attribute__((visibility("hidden"))) int silu_mul_bf16_wide(const uint16_t * gu, uint16_t * act, int H, long n, hipStream_t st);   // quant.hip
 __attribute__((visibility("hidden"))) int silu_lut_get(hipStream_t st, const uint16_t ** lut);                                        // quant.hip
 
@@ -628,7 +656,9 @@ __global__ void __launch_bounds__(256) residual_slices_bwd_k(const float * __res
 int camx_residual_slices_bwd(const float * dout, const int * pos, uint16_t * dm, uint16_t * dmlp, uint16_t * dys, int d, long n4, hipStream_t st) {
     if (!dout || !dm || !dmlp || d < 4 || d % 4 || n4 < 0 || (pos && !dys) || (((uintptr_t)dout) & 15) || (((uintptr_t)dm | (uintptr_t)dmlp | (uintptr_t)dys) & 7)) return CAMX_EINVAL;
     if (n4 == 0) return CAMX_OK;
-    residual_slices_bwd_k<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st>>>(dout, pos, dm, dmlp, dys, d, n4);
+    if ((n4 * 4) % d == 0 && n4 * 4 / d <= 65535)                       // whole rows: the row in blockIdx.y
+        residual_slices_bwd_rows<<<dim3((unsigned)((d / 4 + 255) / 256), (unsigned)(n4 * 4 / d)), dim3(256), 0, st>>>(dout, pos, dm, dmlp, dys, d);
+    else residual_slices_bwd_k<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st>>>(dout, pos, dm, dmlp, dys, d, n4);
     CAMX_LAUNCH_RET();
 }
 int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t * mlp, const uint16_t * ys, const int * pos, float * out,
@@ -636,7 +666,9 @@ int camx_residual_slices_fwd(const float * x, const uint16_t * m, const uint16_t
     if (!x || !m || !mlp || !out || d < 4 || d % 4 || n4 < 0 || ((uintptr_t)x & 15) || ((uintptr_t)out & 15) || ((uintptr_t)m & 7) ||
         ((uintptr_t)mlp & 7) || ((uintptr_t)ys & 7)) return CAMX_EINVAL;
     if (n4 == 0) return CAMX_OK;
-    residual_slices_fwd_k<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st>>>(x, m, mlp, ys, pos, out, d, n4);
+    if ((n4 * 4) % d == 0 && n4 * 4 / d <= 65535)                       // whole rows: the row in blockIdx.y
+        residual_slices_fwd_rows<<<dim3((unsigned)((d / 4 + 255) / 256), (unsigned)(n4 * 4 / d)), dim3(256), 0, st>>>(x, m, mlp, ys, pos, out, d);
+    else residual_slices_fwd_k<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st>>>(x, m, mlp, ys, pos, out, d, n4);
     CAMX_LAUNCH_RET();
 }
 

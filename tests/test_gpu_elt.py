@@ -114,6 +114,32 @@ def test_core_and_fuse():
         assert bits_equal(host(o2), O.residual_slices_fwd(x2, m, y, ys if has else None, pos if has else None))
 
 
+@pytest.mark.parametrize('T,D', [(9, 896), (300, 2048), (7, 892), (33, 100), (5, 8)])
+def test_residual_slices_widths(T, D):
+    """several row widths and counts, forward and backward, with and without slices, non-finite and subnormal values"""
+    rng = np.random.default_rng(60 + D)
+    nys = 4
+    x = outliers(rng, (T, D)); m = O.f2bf(outliers(rng, (T, D))); mlp = O.f2bf(outliers(rng, (T, D))); ys = O.f2bf(outliers(rng, (nys, D)))
+    pos = rng.integers(-1, nys, T).astype(np.int32); pos[rng.random(T) < 0.5] = -1
+    taken = pos[pos >= 0]; pos[pos >= 0] = np.where(np.arange(len(taken)) < nys, rng.permutation(nys)[np.arange(len(taken)) % nys], -1)   # each slice at most once
+    seen = set()
+    for r in range(T):
+        if pos[r] >= 0 and int(pos[r]) in seen: pos[r] = -1
+        elif pos[r] >= 0: seen.add(int(pos[r]))
+    x[0, :4] = [np.nan, np.inf, -0.0, 1e-40]
+    for has in (True, False):
+        o = dev(np.zeros((T, D), np.float32))
+        call('camx_residual_slices_fwd', ptr(dev(x)), ptr(dev(m)), ptr(dev(mlp)), ptr(dev(ys)) if has else NULL, ptr(dev(pos)) if has else NULL, ptr(o), I(D), L64(T * D // 4))
+        want = O.residual_slices_fwd(x, m, mlp, ys if has else None, pos if has else None)
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(host(o)), nan) and bits_equal(np.where(nan, 0, host(o)), np.where(nan, 0, want))
+    rdm, rdmlp, rdys = O.residual_slices_bwd(x, pos, nys)
+    dm = dev(np.zeros((T, D), np.uint16)); dmlp = dev(np.zeros((T, D), np.uint16)); dys = dev(np.zeros((nys, D), np.uint16))
+    call('camx_residual_slices_bwd', ptr(dev(x)), ptr(dev(pos)), ptr(dm), ptr(dmlp), ptr(dys), I(D), L64(T * D // 4))
+    used = sorted(seen)
+    assert bits_equal(host(dm, np.uint16), rdm) and bits_equal(host(dmlp, np.uint16), rdmlp) and bits_equal(host(dys, np.uint16)[used], rdys[used])
+
+
 def test_residual_slices_bwd_and_autograd():
     """the backward kernel against the oracle, and the autograd wrapper end to end against torch's own graph of the same sum"""
     import torch

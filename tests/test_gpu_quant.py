@@ -56,15 +56,17 @@ def test_mmq_quantize(K, ncols, layout):
         assert bits_equal(host(y), ref)
 
 
-@pytest.mark.parametrize('K,ntok,k', [(768, 9, 8), (2048, 4, 2)])
-def test_mmq_quantize_scatter(K, ntok, k):
+@pytest.mark.parametrize('K,ntok,k,pad', [(768, 9, 8, 0), (2048, 4, 2, 0), (264, 2051, 3, 8), (1024, 2048, 8, 0), (392, 4100, 1, 4)])
+def test_mmq_quantize_scatter(K, ntok, k, pad):
+    """small batches and prefill chunks: token counts that end inside a group of 8, widths that end inside a block, padded source rows"""
     rng = np.random.default_rng(K)
-    x = outliers(rng, (ntok, K))
+    rows = outliers(rng, (ntok, K + pad))
+    x = np.ascontiguousarray(rows[:, :K])
     ids_inv = rng.permutation(ntok * k).astype(np.int32)
     for layout in (0, 1):
         ref = O.mmq_q8_1_scatter(x, K, ntok, ids_inv, k, layout)
-        y = dev(np.zeros(ref.shape, np.uint8))
-        call('camx_quantize_mmq_q8_1_scatter', ptr(dev(x)), ptr(dev(ids_inv)), ptr(y), L64(K), L64(0), L64(K), L64(0), L64(O.k_pad(K)),
+        y = dev(np.full(ref.shape, 0xA5, np.uint8))
+        call('camx_quantize_mmq_q8_1_scatter', ptr(dev(rows)), ptr(dev(ids_inv)), ptr(y), L64(K), L64(0), L64(K + pad), L64(0), L64(O.k_pad(K)),
              I(ntok * k), I(1), I(k), I(layout), I(ntok))
         assert bits_equal(host(y), ref)
 
