@@ -341,7 +341,7 @@ __global__ void __launch_bounds__(256) hc_post_k(const float * __restrict__ b, c
     if (i >= (long)T * D) return;
     const int tt = (int)(i / D), ii = (int)(i - (long)tt * D);
     float bv[VW];
-    if (VEC) { const f32x4 v = *(const f32x4 *)(b + i); bv[0] = v.x; if (VW > 1) { bv[1] = v.y; bv[2] = v.z; bv[3] = v.w; } }
+    if (VEC) { const f32x4 v = __builtin_nontemporal_load((const f32x4 *)(b + i)); bv[0] = v.x; if (VW > 1) { bv[1] = v.y; bv[2] = v.z; bv[3] = v.w; } }
     else bv[0] = b[i];
     for (int h = 0; h < HC; h++) {
         const float v = inj[tt * HC + h] * rs;
@@ -349,7 +349,7 @@ __global__ void __launch_bounds__(256) hc_post_k(const float * __restrict__ b, c
         const float ph = sgm * 2.0f;
         const size_t o = (size_t)(tt * HC + h) * D + ii;
         if (VEC) {
-            f32x4 r = *(const f32x4 *)(res + o);
+            f32x4 r = __builtin_nontemporal_load((const f32x4 *)(res + o));
             r.x = __builtin_fmaf(bv[0], ph, r.x); r.y = __builtin_fmaf(bv[1 % VW], ph, r.y); r.z = __builtin_fmaf(bv[2 % VW], ph, r.z); r.w = __builtin_fmaf(bv[3 % VW], ph, r.w);
             __builtin_nontemporal_store(r, (f32x4 *)(res + o));
         } else res[o] = __builtin_fmaf(bv[0], ph, res[o]);

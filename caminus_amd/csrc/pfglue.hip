@@ -254,6 +254,52 @@ __global__ void __launch_bounds__(256) ple_conv_k(const float * __restrict__ x, 
     if (y) y[i] = o;
     if (res) { const float ab = a[i] + o; res[i] = res[i] + ab; }
 }
+// the same for C % 4 == 0, D % 4 == 0 and 16-byte aligned operands: the token in blockIdx.y (no division of an element index), four
+// channels per thread (their sixteen fp16 weights in two 16-byte loads), streamed outputs non-temporal
+__global__ void __launch_bounds__(256) ple_conv_rows(const float * __restrict__ x, const float * __restrict__ xscl, const float * __restrict__ xw,
+                                                     const uint16_t * __restrict__ w, const float * __restrict__ hist, float * __restrict__ y,
+                                                     const float * __restrict__ a, float * __restrict__ res, int C, int D, int dil) {
+    const int t = blockIdx.y, c = 4 * (blockIdx.x * 256 + threadIdx.x), hl = 3 * dil;
+    if (c >= C) return;
+    const u32x4 w0 = *(const u32x4 *)(w + (size_t)c * 4), w1 = *(const u32x4 *)(w + (size_t)c * 4 + 8);
+    const uint32_t ww[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};      // channel j's taps: halves 4 j .. 4 j + 3
+    f32x4 xwv = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (xscl) xwv = *(const f32x4 *)(xw + c);
+    float conv[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int back = (3 - k) * dil;
+        float xv[4];
+        if (back <= t) {
+            const int tb = t - back;
+            const f32x4 v = *(const f32x4 *)(x + (size_t)tb * C + c);
+            xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+            if (xscl) {
+                const float sc = xscl[tb * (C / D) + c / D];
+                xv[0] = (xv[0] * sc) * xwv.x; xv[1] = (xv[1] * sc) * xwv.y; xv[2] = (xv[2] * sc) * xwv.z; xv[3] = (xv[3] * sc) * xwv.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) xv[j] = hist[(size_t)(c + j) * hl + hl - (back - t)];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t pair = ww[2 * j + (k >> 1)];
+            const float term = xv[j] * h2f_bits((uint16_t)((k & 1) ? pair >> 16 : pair & 0xffffu));
+            conv[j] = k == 0 ? term : conv[j] + term;
+        }
+    }
+    f32x4 o;
+    o.x = conv[0] / (1.0f + expf(-conv[0])); o.y = conv[1] / (1.0f + expf(-conv[1]));
+    o.z = conv[2] / (1.0f + expf(-conv[2])); o.w = conv[3] / (1.0f + expf(-conv[3]));
+    const size_t i = (size_t)t * C + c;
+    if (y) __builtin_nontemporal_store(o, (f32x4 *)(y + i));
+    if (res) {
+        const f32x4 av = __builtin_nontemporal_load((const f32x4 *)(a + i)), rv = __builtin_nontemporal_load((const f32x4 *)(res + i));
+        f32x4 r; r.x = rv.x + (av.x + o.x); r.y = rv.y + (av.y + o.y); r.z = rv.z + (av.z + o.z); r.w = rv.w + (av.w + o.w);
+        __builtin_nontemporal_store(r, (f32x4 *)(res + i));
+    }
+}
 // hist[c] = the last 3 dil inputs of [hist[c], x[0 .. T - 1][c]]; 3 dil <= 32
 __global__ void __launch_bounds__(256) ple_hist_k(const float * __restrict__ x, const float * __restrict__ xscl, const float * __restrict__ xw,
                                                   float * __restrict__ hist, int C, int T, int D, int dil) {
@@ -356,6 +402,10 @@ int camx_pf_ple_conv(const float * x, const float * xscl, const float * xw, cons
     if (!x || !w || !hist || (!y && !res) || (res && !a) || C < 1 || T < 0 || D < 1 || C % D || dil < 1 || ((xscl == nullptr) != (xw == nullptr))) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     if ((long)T * C >= 0x7fffffffL * 256) return CAMX_EINVAL;
+    if (C % 4 == 0 && D % 4 == 0 && T <= 65535 && !(((uintptr_t)x | (uintptr_t)xw | (uintptr_t)w | (uintptr_t)y | (uintptr_t)a | (uintptr_t)res) & 15)) {
+        ple_conv_rows<<<dim3((unsigned)((C / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st>>>(x, xscl, xw, w, hist, y, a, res, C, D, dil);
+        CAMX_LAUNCH_RET();
+    }
     ple_conv_k<<<dim3((unsigned)(((long)T * C + 255) / 256)), dim3(256), 0, st>>>(x, xscl, xw, w, hist, y, a, res, C, T, D, dil);
     CAMX_LAUNCH_RET();
 }

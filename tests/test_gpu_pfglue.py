@@ -75,7 +75,7 @@ def test_add_sum_bf16_copies_hc_avg():
         assert bits_equal(host(y), O.hc_avg(r, ldo=ldo))
 
 
-@pytest.mark.parametrize('T,HC,D,dil', [(50, 4, 256, 3), (9, 2, 96, 1), (300, 4, 640, 10)])
+@pytest.mark.parametrize('T,HC,D,dil', [(50, 4, 256, 3), (9, 2, 96, 1), (300, 4, 640, 10), (40, 3, 6, 2), (2, 1, 1030, 4)])        # (D % 4 != 0: the one-channel-per-thread conv)
 def test_ple_gate_conv_hist(T, HC, D, dil):
     rng = np.random.default_rng(T + D)
     kn = rng.standard_normal((T, HC, D)).astype(f32); q = rng.standard_normal((T, HC, D)).astype(f32); val = rng.standard_normal((T, D + 4)).astype(f32)

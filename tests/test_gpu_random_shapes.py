@@ -60,7 +60,7 @@ def _generators(r):
         (P.test_ple_gate_conv_hist, lambda: (ri(2, 400), ri(1, 4), 32 * ri(1, 24), ri(1, 10))),
         (Q.test_q8_1_plain, lambda: (ri(1, 600000),)),
         (Q.test_mmq_quantize, lambda: (4 * ri(1, 2500), ch([ri(1, 700), ri(1, 700), 2048 + ri(0, 2000)]), ri(0, 1))),
-        (Q.test_mmq_quantize_scatter, lambda: (4 * ri(1, 1000), ri(1, 40), ri(1, 8))),
+        (Q.test_mmq_quantize_scatter, lambda: (4 * ri(1, 1000), ri(1, 40), ri(1, 8), 4 * ri(0, 3))),
         (Q.test_swiglu_mmq, lambda: (ch([ri(1, 400), ri(1, 400), 2048 + ri(0, 3000)]), ch([4, 8]) * ri(1, 600), 8 * ri(0, 3), ri(0, 1))),
         (RP.test_qk_rope_f16_and_q8, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 5, 33, 256, 257, 2048, 2051]), ri(0, 120000), ch([False, True]))),
         (RP.test_pf_qk_nr, qk_nr),
