@@ -418,6 +418,35 @@ def prefill_scale_sweep(B, T=4096, only=None):
         x = B.acts((T * 36, 128), torch.float32, i)
         return lambda: B.call('camx_pf_hadamard', _p(x), I(T * 36), I(128), I(4))
     timeit(f'pf_hadamard {T}x36 chunks of 128', T * 36 * 128 * 8, mk)
+    rows_n = T * 32
+    wg128 = B.gamma(128, 6)
+    def mk(i):
+        o = B.acts((rows_n, 128), torch.float32, i); z = B.acts((rows_n, 128), torch.float32, i + 1, frac=0); y = torch.empty((rows_n, 128), device=dev)
+        return lambda: B.call('camx_pf_gdn_norm', _p(o), _p(wg128), _p(z), _p(y), I(128), F(1e-6), C.c_long(rows_n), I(1))
+    timeit(f'pf_gdn_norm {T}x32x128 silu', rows_n * 128 * 12, mk)
+    def mk(i):
+        k = B.acts((T, 1024), torch.float32, i); v = B.acts((T, 1024), torch.float32, i + 1); cache = torch.empty((T, 2048), dtype=torch.float16, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_q35p_kv_append16', _p(k), I(1024), _p(v), I(1024), _p(cache), I(1024), I(0), I(T), _p(err), I(T))
+    timeit(f'q35p_kv_append16 {T}x1024', T * 1024 * 12, mk)
+    def mk(i):
+        b = B.acts((2048, 2560), torch.float32, i); inj = B.acts((2048, 4), torch.float32, i + 1, frac=0); r = B.acts((2048, 4, 2560), torch.float32, i + 2)
+        return lambda: B.call('camx_pf_hc_post', _p(b), _p(inj), _p(r), I(2048), I(4), I(2560), F(1.0))
+    timeit('pf_hc_post 2048x4x2560', 2048 * 2560 * 36, mk)
+    def mk(i):
+        g = B.acts((Mr * Kq,), torch.float32, i, frac=0); u = B.acts((Mr * Kq,), torch.float32, i + 1); h = torch.empty(Mr * Kq, device=dev)
+        return lambda: B.call('camx_gg_silu_mul', _p(g), _p(u), _p(h), I(Mr * Kq))
+    timeit('gg_silu_mul 16M', Mr * Kq * 12, mk)
+    Cp, Dp = 1024, 256
+    wpc = (torch.randn(Cp, 4, device=dev) * 0.5).to(torch.float16); hist = torch.randn(Cp, 6, device=dev)
+    def mk(i):
+        x = B.acts((T, Cp), torch.float32, i, frac=0); y = torch.empty((T, Cp), device=dev)
+        return lambda: B.call('camx_pf_ple_conv', _p(x), NULL, NULL, _p(wpc), _p(hist), _p(y), NULL, NULL, I(Cp), I(T), I(Dp), I(2))
+    timeit(f'pf_ple_conv {T}x1024, dilation 2', T * Cp * 8, mk)
+    def mk(i):
+        kn = B.acts((T, 4, Dp), torch.float32, i, frac=0); q = B.acts((T, 4, Dp), torch.float32, i + 1, frac=0); val = B.acts((T, Dp), torch.float32, i + 2, frac=0)
+        gated = torch.empty((T, 4, Dp), device=dev); gate = torch.empty((T, 4), device=dev)
+        return lambda: B.call('camx_pf_ple_gate', _p(kn), _p(q), NULL, NULL, _p(val), I(Dp), _p(gated), _p(gate), I(4), I(Dp), I(T))
+    timeit(f'pf_ple_gate {T}x4x256', T * 4 * Dp * 12 + T * Dp * 4, mk)
     rows_g, Kg = T * 48, 128
     def mk(i):
         o = B.acts((rows_g, Kg), torch.float32, i); z = B.acts((rows_g, Kg), torch.float32, i + 1, frac=0); wg = B.gamma(Kg, 5); y16 = torch.empty((rows_g, Kg), dtype=torch.float16, device=dev)
