@@ -66,6 +66,16 @@ __global__ void __launch_bounds__(256) kv_q8_append_wave_rows(const float * __re
 }
 
 // pf_kv_append (q8_0 rows): no refusal rules; d stored as half, codes roundf(x * (1 / d)); err bit 1 for a row outside
+CAMX_DEV void pf_q8_0_emit(f32x4 xv, uint8_t * blk, int sub, bool active) {        // 8 lanes x 4 values: one block
+    const float amax = group8_max(absmax4(xv));
+    const float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
+    if (!active) return;
+    f32x4 t; t.x = xv.x * id; t.y = xv.y * id; t.z = xv.z * id; t.w = xv.w * id;
+    const uint32_t q = pack_round_i8x4(t);
+    uint16_t * o = (uint16_t *)(blk + 2 + 4 * sub);
+    o[0] = (uint16_t)q; o[1] = (uint16_t)(q >> 16);
+    if (sub == 0) *(uint16_t *)blk = f2h_bits(d);
+}
 __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
                                                          uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
     const int tt = blockIdx.x, pos = pos0 + tt;
@@ -77,16 +87,32 @@ __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restric
         const bool active = b < 2 * nb;
         const int bb = active ? b : 0;
         const float * x = (bb < nb ? k + (size_t)tt * ldk : v + (size_t)tt * ldv) + (size_t)(bb % nb) * 32 + 4 * sub;
-        const f32x4 xv = *(const f32x4_a4 *)x;
-        const float amax = group8_max(absmax4(xv));
-        const float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
-        if (!active) continue;
-        f32x4 t; t.x = xv.x * id; t.y = xv.y * id; t.z = xv.z * id; t.w = xv.w * id;
-        const uint32_t q = pack_round_i8x4(t);
-        uint8_t * blk = base + (size_t)bb * 34;
-        uint16_t * o = (uint16_t *)(blk + 2 + 4 * sub);
-        o[0] = (uint16_t)q; o[1] = (uint16_t)(q >> 16);
-        if (sub == 0) *(uint16_t *)blk = f2h_bits(d);
+        pf_q8_0_emit(*(const f32x4_a4 *)x, base + (size_t)bb * 34, sub, active);
+    }
+}
+// a chunk of rows of at most 32 blocks (M <= 512, 16-byte aligned): a wave per row, as kv_q8_append_wave_rows
+__global__ void __launch_bounds__(256) pf_kv_append_wave_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
+                                                              uint8_t * __restrict__ cache, int pos0, int rows, int T, int * __restrict__ err) {
+    const int tt = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tt >= T) return;
+    const int pos = pos0 + tt;
+    const int lane = slot_of(threadIdx.x & 63), sub = lane & 7;
+    if (pos < 0 || pos >= rows) { if ((threadIdx.x & 63) == 0) atomicOr(err, 1); return; }
+    const int nb = M / 32;
+    uint8_t * dst = cache + (size_t)pos * ((size_t)2 * nb * 34);
+    f32x4 xv[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int b = it * 8 + (lane >> 3);
+        const int bb = b < 2 * nb ? b : 0;
+        const float * x = (bb < nb ? k + (size_t)tt * ldk : v + (size_t)tt * ldv) + (size_t)(bb % nb) * 32 + 4 * sub;
+        xv[it] = __builtin_nontemporal_load((const f32x4 *)x);
+    }
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int b = it * 8 + (lane >> 3);
+        const bool active = b < 2 * nb;
+        pf_q8_0_emit(xv[it], dst + (size_t)(active ? b : 0) * 34, sub, active);
     }
 }
 
@@ -243,7 +269,9 @@ int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M,
                       int T, hipStream_t st) {
     if (!k || !v || !cache || !err || T < 0 || M < 32 || M % 32 || ldk < M || ldv < M || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
-    pf_kv_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
+    if (T >= 1024 && M <= 512 && !(((uintptr_t)k | (uintptr_t)v) & 15) && !((ldk | ldv) & 3))
+        pf_kv_append_wave_rows<<<dim3((T + 3) / 4), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, T, err);
+    else pf_kv_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
     CAMX_LAUNCH_RET();
 }
 

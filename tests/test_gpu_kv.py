@@ -83,7 +83,7 @@ def test_kv_q8_refusals_and_error_bits():
         if bit == 4: assert (host(cd) == 0xa5).all()
 
 
-@pytest.mark.parametrize('M,T', [(512, 9), (64, 3)])
+@pytest.mark.parametrize('M,T', [(512, 9), (64, 3), (512, 1027), (96, 1500), (1024, 1100)])        # chunks: a wave per row up to 32 blocks per row
 def test_pf_kv_append(M, T):
     rng = np.random.default_rng(M)
     k = rng.standard_normal((T, M)).astype(np.float32); v = rng.standard_normal((T, M)).astype(np.float32); k[0, :32] = 0
