@@ -62,7 +62,7 @@ def test_gdn_conv(T, C):
     assert close_fp32(host(y), ref_y) and bits_equal(host(sd), ref_st)
 
 
-@pytest.mark.parametrize('T,heads,K', [(16, 32, 128), (16, 48, 128), (3, 5, 256), (2, 3, 96), (1030, 32, 128), (683, 48, 128)])
+@pytest.mark.parametrize('T,heads,K', [(16, 32, 128), (16, 48, 128), (3, 5, 256), (2, 3, 96), (1030, 32, 128), (683, 48, 128), (2049, 32, 128), (1401, 48, 128)])
 def test_gdn_l2(T, heads, K):
     rng = np.random.default_rng(K + heads)
     ldx = heads * K + 64
