@@ -112,7 +112,7 @@ __global__ void __launch_bounds__(256) kv_append16_k(const float * __restrict__ 
     if (vec) {
         for (int i = 4 * threadIdx.x; i < M; i += 1024) {
             const f32x4 kv = __builtin_nontemporal_load((const f32x4 *)(k + (size_t)tt * ldk + i)), vv = __builtin_nontemporal_load((const f32x4 *)(v + (size_t)tt * ldv + i));
-            *(u32x2 *)(c + i) = pack_f16x4(kv); *(u32x2 *)(c + M + i) = pack_f16x4(vv);
+            __builtin_nontemporal_store(pack_f16x4(kv), (u32x2 *)(c + i)); __builtin_nontemporal_store(pack_f16x4(vv), (u32x2 *)(c + M + i));
         }
     } else {
         for (int i = threadIdx.x; i < M; i += 256) { c[i] = f2h_bits(k[(size_t)tt * ldk + i]); c[M + i] = f2h_bits(v[(size_t)tt * ldv + i]); }
