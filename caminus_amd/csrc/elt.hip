@@ -110,11 +110,11 @@ __global__ void __launch_bounds__(256) gate_mul_vec(const void * __restrict__ a,
         }
 #pragma unroll
         for (int k = 0; k < VW; k++) { const float sgm = IO == 0 ? 1.0f / (1.0f + expf(-gv[k])) : sigmoid_fast(gv[k]); v[k] = av[k] * sgm; }
-        if (IO == 0) *(f32x4 *)((float *)y + ai) = (f32x4){v[0], v[1], v[2], v[3]};
-        else if (IO == 1) *(u32x2 *)((uint16_t *)y + ai) = pack_f16x4((f32x4){v[0], v[1], v[2], v[3]});
+        if (IO == 0) __builtin_nontemporal_store((f32x4){v[0], v[1], v[2], v[3]}, (f32x4 *)((float *)y + ai));
+        else if (IO == 1) __builtin_nontemporal_store(pack_f16x4((f32x4){v[0], v[1], v[2], v[3]}), (u32x2 *)((uint16_t *)y + ai));
         else {
             const u32x2 lo = pack_bf16x4_rne((f32x4){v[0], v[1], v[2], v[3]}), hi = pack_bf16x4_rne((f32x4){v[4 % VW], v[5 % VW], v[6 % VW], v[7 % VW]});
-            *(u32x4 *)((uint16_t *)y + ai) = (u32x4){lo.x, lo.y, hi.x, hi.y};
+            __builtin_nontemporal_store((u32x4){lo.x, lo.y, hi.x, hi.y}, (u32x4 *)((uint16_t *)y + ai));
         }
     }
 }
@@ -451,7 +451,7 @@ __global__ void __launch_bounds__(256) hc_mean_k(const float * __restrict__ x, c
             }
         }
     }
-    if (VEC) *(f32x4 *)(out + i) = (f32x4){rs * sum[0], rs * sum[1 % VW], rs * sum[2 % VW], rs * sum[3 % VW]};
+    if (VEC) __builtin_nontemporal_store((f32x4){rs * sum[0], rs * sum[1 % VW], rs * sum[2 % VW], rs * sum[3 % VW]}, (f32x4 *)(out + i));
     else out[i] = rs * sum[0];
 }
 
