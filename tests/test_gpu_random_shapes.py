@@ -39,16 +39,18 @@ def _generators(r):
         (A.test_actq_fwd, lambda: (ri(1, 400), 128 * ri(1, 64), ch([1, 3, 7, 7, 7, 15, 127]))),
         (A.test_actq_bwd, lambda: (ri(1, 300), 128 * ri(1, 64), ch([1, 3, 7, 7, 15, 127]))),
         (A.test_block_entry_bwd, lambda: (ri(1, 200), 128 * ri(1, 8), 2 * ri(0, 8))),
+        (A.test_block_entry_fwd, lambda: (ri(1, 200), 128 * ch([ri(1, 8), ri(1, 8), ri(9, 64)]), ri(0, 16))),
         (A.test_silu_mul_actq_bwd, silu_actq),
         (A.test_silu_mul_actq_fwd, lambda: (ri(2, 300), 128 * ri(1, 24))),
         (E.test_swiglu, lambda: (ri(1, 70000),)),
         (E.test_silu_mul_bf16, lambda: (ri(1, 300), ri(6, 3000))),
         (E.test_gdn_conv, lambda: (ri(1, 600), ch([6, 64, 100, 256, 512, 1000, 4096, 8200, 10240]))),
-        (E.test_gdn_l2, lambda: (ri(1, 1100), ri(1, 48), ch([32, 64, 96, 128, 128, 256]))),
+        (E.test_gdn_l2, lambda: ch([(ri(1, 1100), ri(1, 48), ch([32, 64, 96, 128, 128, 256])), (ri(1400, 2300), ch([32, 48]), 128)])),
+        (E.test_residual_slices_widths, lambda: (ri(1, 400), 4 * ri(1, 700))),
         (M.test_gather_q4k_q80, lambda: (256 * ri(1, 32), ri(4, 2000), ri(3, 600))),
         (M.test_gather_iq4xs_iq2s, lambda: (256 * ri(1, 32), ri(4, 300), ri(3, 300))),
         (M.test_ple_rows_iq4nl, lambda: (ri(1, 100), ri(7, 5000), ri(1, 12))),
-        (KV.test_pf_kv_append, lambda: (32 * ri(1, 40), ri(1, 40))),
+        (KV.test_pf_kv_append, lambda: (32 * ri(1, 40), ch([ri(1, 40), ri(1, 40), ri(1024, 1300)]))),
         (KV.test_kv_q8_read_round_trip, lambda: (32 * ri(1, 40), ri(2, 400), ch([False, True]))),
         (N.test_q3p_add_rms16, lambda: (rows(), 256 * ri(1, 8), ri(0, 8), ch([False, True]))),
         (N.test_q35p_add_rms16, lambda: (rows(), 256 * ri(1, 40))),
