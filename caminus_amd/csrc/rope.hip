@@ -432,24 +432,34 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
 // Rows of exactly 16 STEPS heads (STEPS <= 5) with nh and nkv multiples of 4, so a wave step of four heads is wholly q, k or v and
 // no lane is ever predicated; positions pos0 + t. TPW tokens per workgroup, all their loads issued before anything else (one
 // burst of reads per wave, then its arithmetic, then one burst of writes), the norm weights and the tokens' cos / sin rows in LDS.
-// The operations and their order are qk_rope_wide_tokens': same bits.
-template <bool YARN, int STEPS, int TPW>
+// The operations and their order are qk_rope_wide_tokens': same bits. F32IN: fp32 rows (two 128-bit loads per lane and step) of up to 48
+// heads, the last step possibly short (16384 tokens x 40 heads: 92 -> 86.5 us against the pipelined kernel).
+template <bool YARN, int STEPS, int TPW, bool F32IN = false>
 __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[TPW][64];
     __shared__ __attribute__((aligned(16))) float rs[TPW][64];
     __shared__ __attribute__((aligned(16))) float nrm[256];                  // q_norm | k_norm
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, hq = lane >> 4;
     const int t0 = blockIdx.x * TPW;
-    const int nqk = a.nh + a.nkv;
+    const int nqk = a.nh + a.nkv, items = a.nh + 2 * a.nkv;             // (F32IN: the last step may hold fewer than 16 heads; a wave's four are all there or not)
     const size_t M = (size_t)a.nkv * 128;
     const int lo = 128 * hq + 8 * l16;                                      // this lane's element offset inside a wave step
-    u32x4 xin[TPW][STEPS];
+    constexpr int NW = F32IN ? 2 : 1;
+    u32x4 xin[TPW][STEPS][NW];
 #pragma unroll
     for (int ti = 0; ti < TPW; ti++) {
         const int tk = t0 + ti < a.n ? t0 + ti : a.n - 1;
-        const uint16_t * p = (const uint16_t *)a.qkv + (size_t)tk * a.ldq + 512 * wave + lo;      // heads 16 s + 4 wave .. + 3
+        const size_t e = (size_t)tk * a.ldq + 512 * wave + lo;               // heads 16 s + 4 wave .. + 3
 #pragma unroll
-        for (int s = 0; s < STEPS; s++) xin[ti][s] = __builtin_nontemporal_load((const u32x4 *)(p + 2048 * s));
+        for (int s = 0; s < STEPS; s++) {
+            if (F32IN) {
+                xin[ti][s][0] = xin[ti][s][NW - 1] = (u32x4){0u, 0u, 0u, 0u};
+                if (16 * s + 4 * wave < items) {
+                    const float * p = (const float *)a.qkv + e + 2048 * s;
+                    xin[ti][s][0] = __builtin_nontemporal_load((const u32x4 *)p); xin[ti][s][NW - 1] = __builtin_nontemporal_load((const u32x4 *)(p + 4));
+                }
+            } else xin[ti][s][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)a.qkv + e + 2048 * s));
+        }
     }
     nrm[tid] = a.par[tid];
     if (wave < TPW) {                                                       // wave w: the cos / sin row of token t0 + w
@@ -482,9 +492,15 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
             float sq[8];
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                const uint32_t b = xin[ti][s][p];
-                const float x0 = __builtin_bit_cast(float, b << 16), x1 = __builtin_bit_cast(float, b & 0xffff0000u);
-                sq[2 * p] = x0 * x0; sq[2 * p + 1] = x1 * x1;
+                if (F32IN) {
+                    const uint32_t b0 = xin[ti][s][0][p], b1 = xin[ti][s][NW - 1][p];
+                    const float x0 = __builtin_bit_cast(float, b0), x1 = __builtin_bit_cast(float, b1);
+                    sq[p] = x0 * x0; sq[4 + p] = x1 * x1;
+                } else {
+                    const uint32_t b = xin[ti][s][0][p];
+                    const float x0 = __builtin_bit_cast(float, b << 16), x1 = __builtin_bit_cast(float, b & 0xffff0000u);
+                    sq[2 * p] = x0 * x0; sq[2 * p + 1] = x1 * x1;
+                }
             }
 #pragma unroll
             for (int k = 0; k < 8; k++) sq[k] = add_xor2(sq[k]);
@@ -511,9 +527,13 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
             const int h0 = 16 * s + 4 * wave;                               // wave-uniform
+            if (F32IN && h0 >= items) break;
             float x[8];
 #pragma unroll
-            for (int p = 0; p < 4; p++) { const uint32_t b = xin[ti][s][p]; x[2 * p] = __builtin_bit_cast(float, b << 16); x[2 * p + 1] = __builtin_bit_cast(float, b & 0xffff0000u); }
+            for (int p = 0; p < 4; p++) {
+                if (F32IN) { const uint32_t b0 = xin[ti][s][0][p], b1 = xin[ti][s][NW - 1][p]; x[p] = __builtin_bit_cast(float, b0); x[4 + p] = __builtin_bit_cast(float, b1); }
+                else { const uint32_t b = xin[ti][s][0][p]; x[2 * p] = __builtin_bit_cast(float, b << 16); x[2 * p + 1] = __builtin_bit_cast(float, b & 0xffff0000u); }
+            }
             u32x4 out;
             if (h0 >= nqk) {                                                // V heads: fp16 copy
 #pragma unroll
@@ -535,6 +555,19 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
             RSTORE((u32x4 *)((isq ? qw + (size_t)h0 * 128 : cw + (size_t)(h0 - a.nh) * 128) + lo), out);
         }
     }
+}
+// fp32 rows: any number of heads up to 48 with nh and nkv multiples of 4
+template <bool YARN, int TPW>
+static bool rope_chunk_launch_f32(const RopeArgs & a, hipStream_t st) {
+    const int items = a.nh + 2 * a.nkv;
+    if (a.pos || a.page_table || items > 48 || (a.nh & 3) || (a.nkv & 3)) return false;
+    const dim3 grid((a.n + TPW - 1) / TPW), block(256);
+    switch ((items + 15) >> 4) {
+    case 1: qk_rope_chunk<YARN, 1, TPW, true><<<grid, block, 0, st>>>(a); break;
+    case 2: qk_rope_chunk<YARN, 2, TPW, true><<<grid, block, 0, st>>>(a); break;
+    default: qk_rope_chunk<YARN, 3, TPW, true><<<grid, block, 0, st>>>(a); break;
+    }
+    return true;
 }
 template <bool YARN, int TPW>
 static bool rope_chunk_launch(const RopeArgs & a, hipStream_t st) {
@@ -968,6 +1001,7 @@ static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bo
         if (yarn) qk_rope_wide_tokens<true, 2, false, 5, false><<<g2, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 2, false, 5, false><<<g2, dim3(256), 0, st>>>(a);
     }
     else if (wide && bf16in) { if (yarn) qk_rope_wide_tokens<true, 1, false, 5, false><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 1, false, 5, false><<<dim3(a.n), dim3(256), 0, st>>>(a); }
+    else if (wide && !q8 && a.n >= 2048 && (yarn ? rope_chunk_launch_f32<true, 1>(a, st) : rope_chunk_launch_f32<false, 1>(a, st))) {}
     else if (wide && a.n >= 2048) {               // fp32 rows of a prefill chunk: the same kernel, three wave steps (48 heads) per pass
         const dim3 g4((a.n + 3) / 4);
         if (q8) { if (yarn) qk_rope_wide_tokens<true, 4, true, 3, true><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, true, 3, true><<<g4, dim3(256), 0, st>>>(a); }

@@ -55,7 +55,8 @@ def _run_pair(nh, nkv, n, pos0, yarn, rng, rows):
 
 
 @pytest.mark.parametrize('nh,nkv,n,pos0,yarn', [(32, 4, 1, 1234, False), (32, 4, 5, 0, False), (64, 8, 9, 4090, True), (16, 2, 3, 131000, True),
-                                                (5, 3, 4, 77, False), (8, 2, 2050, 11, False), (45, 4, 2049, 0, True), (96, 8, 2048, 5, False), (32, 4, 2048, 100, True)])
+                                                (5, 3, 4, 77, False), (8, 2, 2050, 11, False), (45, 4, 2049, 0, True), (96, 8, 2048, 5, False), (32, 4, 2048, 100, True),
+                                                (32, 4, 2051, 7, False), (16, 4, 2048, 3, False), (36, 4, 2049, 120000, True), (40, 4, 2050, 9, False), (8, 4, 2048, 0, True)])   # (fp32 chunks: 1 to 3 wave steps, the last one partial)
 def test_qk_rope_f16_and_q8(nh, nkv, n, pos0, yarn):
     _run_pair(nh, nkv, n, pos0, yarn, np.random.default_rng(1001 + nh + n), rows=pos0 + n + 2)
 
