@@ -65,6 +65,7 @@ def _generators(r):
         (Q.test_mmq_quantize_scatter, lambda: (4 * ri(1, 1000), ri(1, 40), ri(1, 8), 4 * ri(0, 3))),
         (Q.test_swiglu_mmq, lambda: (ch([ri(1, 400), ri(1, 400), 2048 + ri(0, 3000)]), ch([4, 8]) * ri(1, 600), 8 * ri(0, 3), ri(0, 1))),
         (RP.test_qk_rope_f16_and_q8, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 5, 33, 256, 257, 2048, 2051]), ri(0, 120000), ch([False, True]))),
+        (RP.test_qk_rope_f16_and_q8, lambda: (4 * ri(1, 10), 4, ch([2048, 2049, 2300]), ri(0, 120000), ch([False, True]))),      # fp32 chunks: whole groups of four heads
         (RP.test_pf_qk_nr, qk_nr),
         (RP.test_qk_rope_bf16, lambda: (ri(1, 96), ri(1, 8), ch([1, 2, 7, 2049]), ri(0, 120000), ch([False, True]), 8 * ri(0, 3))),
     ]
