@@ -434,7 +434,7 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
 // burst of reads per wave, then its arithmetic, then one burst of writes), the norm weights and the tokens' cos / sin rows in LDS.
 // The operations and their order are qk_rope_wide_tokens': same bits. F32IN: fp32 rows (two 128-bit loads per lane and step) of up to 48
 // heads, the last step possibly short (16384 tokens x 40 heads: 92 -> 86.5 us against the pipelined kernel).
-template <bool YARN, int STEPS, int TPW, bool F32IN = false>
+template <bool YARN, int STEPS, int TPW, bool F32IN = false, bool Q8 = false>
 __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[TPW][64];
     __shared__ __attribute__((aligned(16))) float rs[TPW][64];
@@ -535,6 +535,34 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
                 else { const uint32_t b = xin[ti][s][0][p]; x[2 * p] = __builtin_bit_cast(float, b << 16); x[2 * p + 1] = __builtin_bit_cast(float, b & 0xffff0000u); }
             }
             u32x4 out;
+            if constexpr (Q8) {                                             // the Q8 rows, as in qk_rope_wide_tokens (a wave's four heads are of one kind)
+                const bool q_heads = h0 < a.nh, v_heads = h0 >= nqk;
+                const int h = h0 + hq;
+                uint8_t * cwb = (uint8_t *)a.cache + (size_t)pos * (2 * (M / 32) * 34);
+                float v8[8];
+                if (v_heads) {
+#pragma unroll
+                    for (int k = 0; k < 8; k++) v8[k] = f16r(x[k]);
+                } else {
+                    const float * wp = nrm + (q_heads ? 0 : 128) + 8 * l16;
+                    const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        const float y1 = (scale[s] * x[k]) * (k < 4 ? w0[k] : w1[k - 4]);
+                        v8[k] = f16r(__builtin_fmaf(y1, k < 4 ? c4[0][k] : c4[1][k - 4], mul_ror8(y1, k < 4 ? s4[0][k] : s4[1][k - 4])));
+                    }
+                    hadamard128_w8(v8, l16);
+                }
+                if (q_heads) {
+#pragma unroll
+                    for (int p = 0; p < 4; p++) out[p] = pack_f16x2(v8[2 * p], v8[2 * p + 1]);
+                    RSTORE((u32x4 *)(qw + (size_t)h * 128 + 8 * l16), out);
+                } else {
+                    const size_t b = v_heads ? M / 32 + (size_t)(h - nqk) * 4 + (l16 >> 2) : (size_t)(h - a.nh) * 4 + (l16 >> 2);
+                    kv_q8_emit_w8(v8, cwb + b * 34, l16 & 3, a.err, true);
+                }
+                continue;
+            }
             if (h0 >= nqk) {                                                // V heads: fp16 copy
 #pragma unroll
                 for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[2 * p], x[2 * p + 1]);
@@ -557,15 +585,15 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     }
 }
 // fp32 rows: any number of heads up to 48 with nh and nkv multiples of 4
-template <bool YARN, int TPW>
+template <bool YARN, int TPW, bool Q8>
 static bool rope_chunk_launch_f32(const RopeArgs & a, hipStream_t st) {
     const int items = a.nh + 2 * a.nkv;
-    if (a.pos || a.page_table || items > 48 || (a.nh & 3) || (a.nkv & 3)) return false;
+    if (a.pos || a.page_table || items > 48 || (a.nh & 3) || (a.nkv & 3) || (Q8 && (a.pos0 < 0 || a.rows != 0))) return false;
     const dim3 grid((a.n + TPW - 1) / TPW), block(256);
     switch ((items + 15) >> 4) {
-    case 1: qk_rope_chunk<YARN, 1, TPW, true><<<grid, block, 0, st>>>(a); break;
-    case 2: qk_rope_chunk<YARN, 2, TPW, true><<<grid, block, 0, st>>>(a); break;
-    default: qk_rope_chunk<YARN, 3, TPW, true><<<grid, block, 0, st>>>(a); break;
+    case 1: qk_rope_chunk<YARN, 1, TPW, true, Q8><<<grid, block, 0, st>>>(a); break;
+    case 2: qk_rope_chunk<YARN, 2, TPW, true, Q8><<<grid, block, 0, st>>>(a); break;
+    default: qk_rope_chunk<YARN, 3, TPW, true, Q8><<<grid, block, 0, st>>>(a); break;
     }
     return true;
 }
@@ -1001,7 +1029,8 @@ static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bo
         if (yarn) qk_rope_wide_tokens<true, 2, false, 5, false><<<g2, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 2, false, 5, false><<<g2, dim3(256), 0, st>>>(a);
     }
     else if (wide && bf16in) { if (yarn) qk_rope_wide_tokens<true, 1, false, 5, false><<<dim3(a.n), dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 1, false, 5, false><<<dim3(a.n), dim3(256), 0, st>>>(a); }
-    else if (wide && !q8 && a.n >= 2048 && (yarn ? rope_chunk_launch_f32<true, 1>(a, st) : rope_chunk_launch_f32<false, 1>(a, st))) {}
+    else if (wide && !q8 && a.n >= 2048 && (yarn ? rope_chunk_launch_f32<true, 1, false>(a, st) : rope_chunk_launch_f32<false, 1, false>(a, st))) {}
+    else if (wide && q8 && a.n >= 2048 && (yarn ? rope_chunk_launch_f32<true, 1, true>(a, st) : rope_chunk_launch_f32<false, 1, true>(a, st))) {}
     else if (wide && a.n >= 2048) {               // fp32 rows of a prefill chunk: the same kernel, three wave steps (48 heads) per pass
         const dim3 g4((a.n + 3) / 4);
         if (q8) { if (yarn) qk_rope_wide_tokens<true, 4, true, 3, true><<<g4, dim3(256), 0, st>>>(a); else qk_rope_wide_tokens<false, 4, true, 3, true><<<g4, dim3(256), 0, st>>>(a); }
