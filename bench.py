@@ -488,7 +488,7 @@ def prefill_scale_sweep(B, T=4096, only=None):
     return res
 
 
-def batch_ladder(B):
+def batch_ladder(B, tokens=(16, 64, 256, 512, 1024, 2048, 4096), only=None):
     """the op-sets of the configs from a verify batch to a prefill chunk (bench.py --only ladder): us per launch and GB/s at 16 .. 4096
     tokens, 30 launches back to back over copies in rotation (footprint >= 1.2 GB or 16 copies: the small batches stay cache-resident, as
     they are in a decode loop). The launchers switch kernels with the batch size; this shows the switches as a curve."""
@@ -531,8 +531,9 @@ def batch_ladder(B):
                 'q3p_qk_rope f32 40 heads': (T * ldq * 6, rope_f32), 'q3p_qk_rope_q8 40 heads': (T * (ldq * 4 + nh * 256 + rbq), rope_q8),
                 'add_rms_bf16 x5120': (T * 5120 * 12, add_rms_bf16), 'qk_rope_bf16 80 heads': (T * 80 * 128 * 4, rope_bf16), 'swiglu_mmq_q8_1 x17408': (T * 17408 * 5.125, swiglu_mmq)}
 
-    for T in (16, 64, 256, 512, 1024, 2048, 4096):
+    for T in tokens:
         for name, (by, mk) in ops(T).items():
+            if only and not any(f in name for f in only.split(',')): continue
             ncopy = max(3, min(16, -(-1_200_000_000 // int(by))))
             fns = [mk(i) for i in range(ncopy)]
             for f in fns: f()
@@ -604,7 +605,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--copies', type=int, default=8, help='copies of the batch taken in rotation (8: no launch finds its lines in the Infinity Cache)')
     ap.add_argument('--sweep-tokens', type=int, default=4096, help='rows of the --only sweep shapes')
-    ap.add_argument('--sweep-filter', default=None, help='--only sweep: entries whose name contains one of these comma-separated texts')
+    ap.add_argument('--sweep-filter', default=None, help='--only sweep / ladder: entries whose name contains one of these comma-separated texts')
+    ap.add_argument('--ladder-tokens', default='16,64,256,512,1024,2048,4096', help='--only ladder: the batch sizes')
     ap.add_argument('--no-ramp', action='store_true', help='skip the untimed clock ramp-up after the warm-up steps')
     ap.add_argument('--no-cpu', action='store_true')
     ap.add_argument('--no-extra', action='store_true')
@@ -622,7 +624,7 @@ def main():
                           'peak_GBps': HBM_PEAK_GBPS, 'tokens': a.sweep_tokens, 'sweep': prefill_scale_sweep(B, a.sweep_tokens, a.sweep_filter)}))
         return
     if a.only == 'ladder':
-        print(json.dumps({'metric': 'us per launch and GB/s of the configs\' op-sets from 16 to 4096 tokens, 1 GPU', 'n_gpus': 1, 'data': 'synthetic', 'ladder': batch_ladder(B)}))
+        print(json.dumps({'metric': 'us per launch and GB/s of the configs\' op-sets from 16 to 4096 tokens, 1 GPU', 'n_gpus': 1, 'data': 'synthetic', 'ladder': batch_ladder(B, tuple(int(t) for t in a.ladder_tokens.split(',')), a.sweep_filter)}))
         return
     if a.only == 'copy_ref':
         # a plain device copy of known size (256 MiB read + 256 MiB written per launch): the yardstick that FETCH_SIZE / WRITE_SIZE

@@ -826,6 +826,11 @@ static int dsilu_luts_get(hipStream_t st, const float ** lut, const float ** sma
     return CAMX_OK;
 }
 
+__attribute__((visibility("hidden"))) int dsilu_luts_init(hipStream_t st) {       // camx_init's half of this file
+    const float * lut = nullptr, * small = nullptr;
+    return dsilu_luts_get(st, &lut, &small);
+}
+
 // the wave-per-row forward kernel: rows of at most 2048 values, operands aligned for its 16-byte loads and 16- / 4-byte stores
 static bool actq_wave_ok(int K, const void * x, const void * y, const void * codes) { return K <= 2048 && !((uintptr_t)x & 15) && !((uintptr_t)y & 15) && !((uintptr_t)codes & 3); }
 

@@ -167,11 +167,18 @@ __global__ void __launch_bounds__(256) op_gdn_conv_k(const float * __restrict__ 
 // Prefill chunks: a lane owns VW consecutive channels and walks TR consecutive tokens, with the rows of the next eight tokens
 // always in flight (a ring of eight 128-bit loads that is refilled as it is consumed) and the four-tap window in registers;
 // one wave per workgroup, so the grid's (channel groups x token ranges) waves spread evenly over the chip.
-template <bool BF16>
+// L2: the L2 norm of the q / k heads (the first heads * 128 channels) in the same pass, from the values as they are stored: qk
+// [T][heads][128]. A head is 16 lanes x 8 channels (bf16 rows) or 32 lanes x 4 (fp32 rows, the lanes in slot order), whole heads per
+// wave (C % 128 == 0), so every lane of a head is present.
+CAMX_DEV void l2_head_w8(const float (&v)[8], float (&o)[8], float rs);
+CAMX_DEV f32x4 l2_head_l4(f32x4 v, int lane, float rs);
+template <bool BF16, bool L2 = false>
 __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
-                                                      void * __restrict__ y, int C, int T, int ldx, int ldy, int TR) {
+                                                      void * __restrict__ y, int C, int T, int ldx, int ldy, int TR,
+                                                      void * __restrict__ qk = nullptr, int heads = 0, float rs = 0.0f) {
     constexpr int VW = BF16 ? 8 : 4, P = 8;
-    const int cv = blockIdx.x * 64 + threadIdx.x;
+    const int lane_l2 = slot_of(threadIdx.x);
+    const int cv = blockIdx.x * 64 + (L2 && !BF16 ? lane_l2 : (int)threadIdx.x);
     if (cv * VW >= C) return;
     const int c0 = cv * VW, t0 = blockIdx.y * TR, t1 = T < t0 + TR ? T : t0 + TR;
     auto row = [&](int t) {                                            // (a row index past the range is clamped: the load is harmless and never used)
@@ -215,8 +222,24 @@ __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ 
         const size_t o = (size_t)tt * ldy + c0;
         if (BF16) {
             const u32x2 lo = pack_bf16x4_rne((f32x4){r[0], r[1], r[2], r[3]}), hi = pack_bf16x4_rne((f32x4){r[4 % VW], r[5 % VW], r[6 % VW], r[7 % VW]});
-            __builtin_nontemporal_store((u32x4){lo.x, lo.y, hi.x, hi.y}, (u32x4 *)((uint16_t *)y + o));     // (on cold lines: 38.5 us against 42.2 with plain stores, 4096 x 10240)
-        } else __builtin_nontemporal_store((f32x4){r[0], r[1], r[2], r[3]}, (f32x4 *)((float *)y + o));
+            if (!L2 || y) __builtin_nontemporal_store((u32x4){lo.x, lo.y, hi.x, hi.y}, (u32x4 *)((uint16_t *)y + o));     // (on cold lines: 38.5 us against 42.2 with plain stores, 4096 x 10240)
+            if constexpr (L2) {
+                const f32x4 a = unpack_bf16x4(lo), b = unpack_bf16x4(hi);
+                const float v8[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                float o8[8];
+                l2_head_w8(v8, o8, rs);
+                if (c0 < heads * 128) {
+                    const u32x2 pa = pack_bf16x4_rne((f32x4){o8[0], o8[1], o8[2], o8[3]}), pb = pack_bf16x4_rne((f32x4){o8[4], o8[5], o8[6], o8[7]});
+                    __builtin_nontemporal_store((u32x4){pa.x, pa.y, pb.x, pb.y}, (u32x4 *)((uint16_t *)qk + (size_t)tt * heads * 128 + c0));
+                }
+            }
+        } else {
+            if (!L2 || y) __builtin_nontemporal_store((f32x4){r[0], r[1], r[2], r[3]}, (f32x4 *)((float *)y + o));
+            if constexpr (L2) {
+                const f32x4 q4 = l2_head_l4((f32x4){r[0], r[1], r[2], r[3]}, lane_l2, rs);
+                if (c0 < heads * 128) __builtin_nontemporal_store(q4, (f32x4 *)((float *)qk + (size_t)tt * heads * 128 + c0));
+            }
+        }
     };
     int t = t0;
     for (; t + P <= t1; t += P) {                                      // whole groups of eight tokens: no guards
@@ -381,6 +404,128 @@ __global__ void __launch_bounds__(256) gdn_l2_128_w8(const void * __restrict__ x
         if (t < total) {
             if (BF16) { const u32x2 pa = pack_bf16x4_rne(oa), pb = pack_bf16x4_rne(ob); __builtin_nontemporal_store((u32x4){pa.x, pa.y, pb.x, pb.y}, (u32x4 *)((uint16_t *)y + yo)); }
             else { __builtin_nontemporal_store(oa, (f32x4 *)((float *)y + yo)); __builtin_nontemporal_store(ob, (f32x4 *)((float *)y + yo + 4)); }
+        }
+    }
+}
+
+// ---- conv4 + SiLU with the L2 norm of the q / k heads in the same pass ---------------------------------------------------------------
+// The reference appends OP_GDN_CONV and OP_GDN_L2 back to back (python/caminus/engine/q35_dense.py:399-400; kernels/k3_q35_ops.h:152-194):
+// the L2 norm reads the first heads * 128 channels of the convolution's output. Here the lane that produced four (eight) of a head's
+// channels keeps them and the head's 32 (16) lanes form the sum of squares in gdn_l2_128's (gdn_l2_128_w8's) tree, from the values as
+// the convolution stores them (rounded to bf16 first when the rows are bf16), so y and qk carry the bits of the two separate kernels.
+CAMX_DEV f32x4 l2_head_l4(f32x4 v, int lane, float rs) {           // a head of 128 values in 32 lanes x 4 (lane: its slot), as gdn_l2_128
+    f32x4 ss;
+    ss.x = __builtin_fmaf(v.x, v.x, 0.0f); ss.y = __builtin_fmaf(v.y, v.y, 0.0f); ss.z = __builtin_fmaf(v.z, v.z, 0.0f); ss.w = __builtin_fmaf(v.w, v.w, 0.0f);
+    const float tot = half_groups_in_order<4>(group32_sum(ss), lane & 32);
+    const float scale = rsqrt_exact(tot / 128.0f + rs), s2 = 1.0f / sqrtf(128.0f);
+    f32x4 o;
+    o.x = (scale * v.x) * s2; o.y = (scale * v.y) * s2; o.z = (scale * v.z) * s2; o.w = (scale * v.w) * s2;
+    return o;
+}
+CAMX_DEV void l2_head_w8(const float (&v)[8], float (&o)[8], float rs) {   // a head of 128 values in 16 lanes x 8, as gdn_l2_128_w8
+    float s[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) s[k] = __builtin_fmaf(v[k], v[k], 0.0f);
+#pragma unroll
+    for (int k = 0; k < 8; k++) s[k] += lane_xor2(s[k]);
+#pragma unroll
+    for (int k = 0; k < 8; k++) s[k] += lane_xor1(s[k]);
+    const float a0 = s[0] + s[4], a1 = s[1] + s[5], a2 = s[2] + s[6], a3 = s[3] + s[7];
+    const float b0 = a0 + a2, b1 = a1 + a3;
+    const float g = b0 + b1;
+    float tot = 0.0f;
+    tot += row16_bcast<0>(g); tot += row16_bcast<4>(g); tot += row16_bcast<8>(g); tot += row16_bcast<12>(g);
+    const float scale = rsqrt_exact(tot / 128.0f + rs), s2 = 1.0f / sqrtf(128.0f);
+#pragma unroll
+    for (int k = 0; k < 8; k++) o[k] = (scale * v[k]) * s2;
+}
+// Decode / verify batches: a half-wave per (token, 128 channels), lane l (its slot) at channels 4 l .. 4 l + 3 of the group. y optional.
+template <bool BF16>
+__global__ void __launch_bounds__(256) gdn_conv_l2_k(const void * __restrict__ x, const float * __restrict__ w, const float * __restrict__ st,
+                                                     void * __restrict__ y, void * __restrict__ qk, int C, int T, int ldx, int ldy, int heads, float rs) {
+    const int lane = slot_of(threadIdx.x & 63), l = lane & 31;
+    const int G = C >> 7;
+    const long u = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+    const bool on = u < (long)T * G;
+    const int t = on ? (int)(u / G) : 0, cg = on ? (int)(u - (long)t * G) : 0;
+    const int c0 = 128 * cg + 4 * l;
+    f32x4 in[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int tj = t - 3 + j;
+        if (tj >= 0) in[j] = BF16 ? unpack_bf16x4(*(const u32x2 *)((const uint16_t *)x + (size_t)tj * ldx + c0)) : *(const f32x4 *)((const float *)x + (size_t)tj * ldx + c0);
+        else {
+#pragma unroll
+            for (int k = 0; k < 4; k++) in[j][k] = st[(size_t)(c0 + k) * 3 + 3 + tj];
+        }
+    }
+    f32x4 v;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const f32x4 w4 = *(const f32x4 *)(w + (size_t)(c0 + k) * 4);
+        float sumf = 0.0f;
+        sumf = __builtin_fmaf(in[0][k], w4.x, sumf); sumf = __builtin_fmaf(in[1][k], w4.y, sumf);
+        sumf = __builtin_fmaf(in[2][k], w4.z, sumf); sumf = __builtin_fmaf(in[3][k], w4.w, sumf);
+        v[k] = BF16 ? silu_fast(sumf) : silu_f(sumf);
+    }
+    if (BF16) {
+        const u32x2 pk = pack_bf16x4_rne(v);
+        if (on && y) *(u32x2 *)((uint16_t *)y + (size_t)t * ldy + c0) = pk;
+        v = unpack_bf16x4(pk);
+    } else if (on && y) *(f32x4 *)((float *)y + (size_t)t * ldy + c0) = v;
+    const f32x4 o = l2_head_l4(v, lane, rs);
+    if (on && cg < heads) {
+        const size_t qo = ((size_t)t * heads + cg) * 128 + 4 * l;
+        if (BF16) *(u32x2 *)((uint16_t *)qk + qo) = pack_bf16x4_rne(o); else *(f32x4 *)((float *)qk + qo) = o;
+    }
+}
+// OP_GDN_CONV followed by OP_GDN_L2 on the tape (decode / verify pass of T tokens, fp32, lazy commit as in op_gdn_conv_k): a half-wave per
+// 128 channels walks the pass's tokens; the state, the weights and the window stay in registers.
+__global__ void __launch_bounds__(256) op_gdn_conv_l2_k(const float * __restrict__ w, float * __restrict__ st, const float * __restrict__ x,
+                                                        const int32_t * __restrict__ params, float * __restrict__ y, float * __restrict__ xprev,
+                                                        float * __restrict__ qk, int C, int T, int heads, float rs) {
+    const int lane = slot_of(threadIdx.x & 63), l = lane & 31;
+    const int G = C >> 7;
+    const int cgr = ((int)blockIdx.x * 4 + (int)(threadIdx.x >> 6)) * 2 + (lane >> 5);
+    const bool on = cgr < G;
+    const int cg = on ? cgr : 0, c0 = 128 * cg + 4 * l;
+    int mprev = params[1];
+    mprev = mprev < 0 ? 0 : (mprev > T ? T : mprev);
+    float s[3][4];
+    f32x4 w4[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        w4[k] = *(const f32x4 *)(w + (size_t)(c0 + k) * 4);
+#pragma unroll
+        for (int j = 0; j < 3; j++) s[j][k] = st[(size_t)(c0 + k) * 3 + j];
+    }
+    for (int j = 0; j < mprev; j++) {
+        const f32x4 xp = *(const f32x4 *)(xprev + (size_t)j * C + c0);
+#pragma unroll
+        for (int k = 0; k < 4; k++) { s[0][k] = s[1][k]; s[1][k] = s[2][k]; s[2][k] = xp[k]; }
+    }
+    if (on) {
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int j = 0; j < 3; j++) st[(size_t)(c0 + k) * 3 + j] = s[j][k];
+    }
+    for (int t = 0; t < T; t++) {
+        const f32x4 xv = *(const f32x4 *)(x + (size_t)t * C + c0);
+        f32x4 v;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float sumf = 0.0f;
+            sumf = __builtin_fmaf(s[0][k], w4[k].x, sumf); sumf = __builtin_fmaf(s[1][k], w4[k].y, sumf);
+            sumf = __builtin_fmaf(s[2][k], w4[k].z, sumf); sumf = __builtin_fmaf(xv[k], w4[k].w, sumf);
+            v[k] = silu_f(sumf);
+            s[0][k] = s[1][k]; s[1][k] = s[2][k]; s[2][k] = xv[k];
+        }
+        const f32x4 o = l2_head_l4(v, lane, rs);
+        if (on) {
+            *(f32x4 *)(y + (size_t)t * C + c0) = v;
+            *(f32x4 *)(xprev + (size_t)t * C + c0) = xv;
+            if (cg < heads) *(f32x4 *)(qk + ((size_t)t * heads + cg) * 128 + 4 * l) = o;
         }
     }
 }
@@ -652,6 +797,45 @@ int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs
     else { if (vec) gdn_l2_k<false, true><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); else gdn_l2_k<false, false><<<grid, block, 0, st>>>(x, y, heads, K, ldx, rs, total); }
     CAMX_LAUNCH_RET();
 }
+// conv4 + SiLU and the L2 norm of the first `heads` heads of 128 channels in one launch: y (optional) = camx_pf_gdn_conv's rows, qk
+// [T][heads][128] = camx_pf_gdn_l2(y, heads, 128, ldy, rs) bit for bit. C % 128 == 0, 16-byte aligned operands.
+int camx_gdn_conv_l2(const void * x, const float * w, const float * state, void * y, void * qk, int C, int T, int ldx, int ldy, int heads, float rs,
+                     int bf16, hipStream_t st) {
+    const int vw = bf16 ? 8 : 4;
+    if (!x || !w || !state || !qk || C < 128 || (C & 127) || T < 1 || ldx < C || (y && ldy < C) || heads < 1 || heads > C / 128 || (ldx % vw) || (y && ldy % vw) ||
+        ((uintptr_t)w & 15) || (((uintptr_t)x | (uintptr_t)y | (uintptr_t)qk) & 15)) return CAMX_EINVAL;
+    if ((long)T * C >= (1L << 20)) {
+        const int tr = 32;
+        const dim3 gs((unsigned)((C / vw + 63) / 64), (unsigned)((T + tr - 1) / tr)), bs(64);
+        if (bf16) gdn_conv_stream<true, true><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr, qk, heads, rs);
+        else gdn_conv_stream<false, true><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr, qk, heads, rs);
+        CAMX_LAUNCH_RET();
+    }
+    const dim3 grid((unsigned)(((long)T * (C >> 7) + 7) / 8)), block(256);
+    if (bf16) gdn_conv_l2_k<true><<<grid, block, 0, st>>>(x, w, state, y, qk, C, T, ldx, ldy, heads, rs);
+    else gdn_conv_l2_k<false><<<grid, block, 0, st>>>(x, w, state, y, qk, C, T, ldx, ldy, heads, rs);
+    CAMX_LAUNCH_RET();
+}
+// OP_GDN_CONV then OP_GDN_L2 of the decode tape in one launch (python/caminus/engine/q35_dense.py:399-400): camx_op_gdn_conv's arguments,
+// then qk = the L2 norm (rs = eps / 128) of the first `heads` heads of 128 channels of y, as camx_op_gdn_l2(y, qk, heads, 128, rs, C, T)
+int camx_op_gdn_conv_l2(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, float * qk, int C, int T,
+                        int heads, float rs, hipStream_t st) {
+    if (!w || !state || !x || !params || !y || !xprev || !qk || C < 128 || (C & 127) || T < 1 || heads < 1 || heads > C / 128 ||
+        (((uintptr_t)w | (uintptr_t)x | (uintptr_t)y | (uintptr_t)xprev | (uintptr_t)qk) & 15)) return CAMX_EINVAL;
+    op_gdn_conv_l2_k<<<dim3((unsigned)(((C >> 7) + 7) / 8)), dim3(256), 0, st>>>(w, state, x, params, y, xprev, qk, C, T, heads, rs);
+    CAMX_LAUNCH_RET();
+}
+// the remaining elementwise ops of the decode tape by their Seg fields
+// OP_GDN_L2 (python/caminus/engine/k3.py:1002-1008): a = x, y = out, rs = eps / dim, N = T * heads, K = dim, pad1 = x_stride (0: heads * dim)
+int camx_op_gdn_l2(const float * x, float * out, int heads, int dim, float rs, int x_stride, int T, hipStream_t st) {
+    return camx_pf_gdn_l2(x, out, heads, dim, x_stride ? x_stride : heads * dim, rs, T, 0, st);
+}
+// OP_GATE_MUL16 (python/caminus/engine/k3.py:1209-1219): a, W = gate, y = out16, N = n, K = dim, pad1 = head_stride, pad2 = offset
+int camx_op_gate_mul16(const float * a, const float * gate, int head_stride, int offset, uint16_t * out16, int n, int dim, hipStream_t st) {
+    return camx_gate_mul(a, gate, out16, (long)n, dim, head_stride, offset, 1, st);
+}
+// OP_OWN_SWIGLU16 (python/caminus/engine/k3.py:854-860): a = g, W = u, y = y16, N = n
+int camx_op_own_swiglu16(const float * g, const float * u, uint16_t * y16, int n, hipStream_t st) { return camx_q3p_swiglu(g, u, y16, n, st); }
 int camx_pf_hc_post(const float * b, const float * inj, float * res, int T, int HC, int D, float rs, hipStream_t st) {
     if (!b || !inj || !res || T < 0 || HC < 1 || D < 1) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;

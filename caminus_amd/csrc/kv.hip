@@ -11,11 +11,13 @@ typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 // Error bits: 1 position span, 2 numerical domain, 4 layout.
 __global__ void __launch_bounds__(256) kv_q8_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
-                                                         uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
+                                                         uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err,
+                                                         const int32_t * __restrict__ posb = nullptr) {
     if (M < 32 || M % 32 || ldk < M || ldv < M || rows < 1) {
         if (threadIdx.x == 0) atomicOr(err, 4);
         return;
     }
+    if (posb) pos0 = posb[0];                            // the tape's device-resident position
     const long pos = (long)pos0 + (long)blockIdx.x;      // widened before the sum: a bad position cannot wrap into a valid row
     if (pos < 0 || pos >= rows) {
         if (threadIdx.x == 0) atomicOr(err, 1);
@@ -38,9 +40,11 @@ __global__ void __launch_bounds__(256) kv_q8_append_rows(const float * __restric
 // loads per lane issued together, four rows per workgroup. A workgroup per row is 4 KB of work; at chunk sizes the launch of 16384 such
 // workgroups, not the memory, sets the time.
 __global__ void __launch_bounds__(256) kv_q8_append_wave_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
-                                                              uint8_t * __restrict__ cache, int pos0, int rows, int T, int * __restrict__ err) {
+                                                              uint8_t * __restrict__ cache, int pos0, int rows, int T, int * __restrict__ err,
+                                                              const int32_t * __restrict__ posb = nullptr) {
     const int tt = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (tt >= T) return;
+    if (posb) pos0 = posb[0];
     const long pos = (long)pos0 + (long)tt;
     const int lane = slot_of(threadIdx.x & 63), sub = lane & 7;
     if (pos < 0 || pos >= rows) {
@@ -77,8 +81,10 @@ CAMX_DEV void pf_q8_0_emit(f32x4 xv, uint8_t * blk, int sub, bool active) {     
     if (sub == 0) *(uint16_t *)blk = f2h_bits(d);
 }
 __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
-                                                         uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err) {
-    const int tt = blockIdx.x, pos = pos0 + tt;
+                                                         uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err,
+                                                         const int32_t * __restrict__ posb = nullptr) {
+    if (posb) pos0 = posb[0];
+    const int tt = blockIdx.x; const long pos = (long)pos0 + tt;
     if (pos < 0 || pos >= rows) { if (threadIdx.x == 0) atomicOr(err, 1); return; }
     const int nb = M / 32, lane = slot_of(threadIdx.x & 63), sub = lane & 7;
     uint8_t * base = cache + (size_t)pos * ((size_t)2 * nb * 34);
@@ -92,10 +98,12 @@ __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restric
 }
 // a chunk of rows of at most 32 blocks (M <= 512, 16-byte aligned): a wave per row, as kv_q8_append_wave_rows
 __global__ void __launch_bounds__(256) pf_kv_append_wave_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
-                                                              uint8_t * __restrict__ cache, int pos0, int rows, int T, int * __restrict__ err) {
+                                                              uint8_t * __restrict__ cache, int pos0, int rows, int T, int * __restrict__ err,
+                                                              const int32_t * __restrict__ posb = nullptr) {
     const int tt = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (tt >= T) return;
-    const int pos = pos0 + tt;
+    if (posb) pos0 = posb[0];
+    const long pos = (long)pos0 + tt;
     const int lane = slot_of(threadIdx.x & 63), sub = lane & 7;
     if (pos < 0 || pos >= rows) { if ((threadIdx.x & 63) == 0) atomicOr(err, 1); return; }
     const int nb = M / 32;
@@ -247,15 +255,19 @@ __global__ void __launch_bounds__(256) hadamard128_heads(const float * __restric
 
 extern "C" {
 
-int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
-                          int T, hipStream_t st) {
+static int own_kv_q8_append_launch(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, const int32_t * posb, int rows,
+                                   int * err, int T, hipStream_t st) {
     if (!k || !v || !cache || !err || T < 0 || ((uintptr_t)k & 3) || ((uintptr_t)v & 3) || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     const bool chunk = T >= 1024 && M >= 32 && M % 32 == 0 && M <= 512 && ldk >= M && ldv >= M && rows >= 1 &&
                        ((ldk | ldv) & 3) == 0 && (((uintptr_t)k | (uintptr_t)v) & 15) == 0;
-    if (chunk) kv_q8_append_wave_rows<<<dim3((T + 3) / 4), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, T, err);
-    else kv_q8_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
+    if (chunk) kv_q8_append_wave_rows<<<dim3((T + 3) / 4), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, T, err, posb);
+    else kv_q8_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err, posb);
     CAMX_LAUNCH_RET();
+}
+int camx_own_kv_q8_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
+                          int T, hipStream_t st) {
+    return own_kv_q8_append_launch(k, ldk, v, ldv, M, cache, pos0, nullptr, rows, err, T, st);
 }
 
 // The Q8 KV reader (no kernel of its own in the reference: the decode is inlined in its attention kernels). Row t = row_ids ?
@@ -276,15 +288,34 @@ int camx_own_kv_q8_read(const uint8_t * cache, const int32_t * row_ids, int pos0
     else kv_q8_read_rows<false><<<dim3(T), dim3(256), 0, st>>>(cache, row_ids, pos0, rows, M, k, ldk, v, ldv, err);
     CAMX_LAUNCH_RET();
 }
-int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
-                      int T, hipStream_t st) {
+static int pf_kv_append_launch(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, const int32_t * posb, int rows, int * err,
+                               int T, hipStream_t st) {
     if (!k || !v || !cache || !err || T < 0 || M < 32 || M % 32 || ldk < M || ldv < M || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     if (T >= 1024 && M <= 512 && !(((uintptr_t)k | (uintptr_t)v) & 15) && !((ldk | ldv) & 3))
-        pf_kv_append_wave_rows<<<dim3((T + 3) / 4), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, T, err);
-    else pf_kv_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err);
+        pf_kv_append_wave_rows<<<dim3((T + 3) / 4), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, T, err, posb);
+    else pf_kv_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err, posb);
     CAMX_LAUNCH_RET();
 }
+int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
+                      int T, hipStream_t st) {
+    return pf_kv_append_launch(k, ldk, v, ldv, M, cache, pos0, nullptr, rows, err, T, st);
+}
+// OP_KV_APPEND by its Seg fields (python/caminus/engine/k3.py:1065-1089; kernels/k3_gguf_ops.h:1520-1553, kernels/k3_q35_kvq8_ops.h:16-27): a = k,
+// W = v (fp32 [T][M]), y = cache, asum = pos (int32 [1] on the device: token t goes to row pos[0] + t), N = M, gs = err. work 0: fp16 rows
+// [K | V]; 1: ggml q8_0 rows (no refusal rules); 2: the dense Q8 line's blocks with the codec's refusal rules (the reference selects it by its
+// K3_Q35_KV_Q8 build, with work = 1 and the error word in gs). rows = the cache's rows, checked on the device as the reference's launch guard
+// does (err bit 1, the row is not written); err bit 2 a refused block, 4 layout (work 2).
+int camx_i_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, const int32_t * posb, int rows, int * err, int T, hipStream_t st);
+int camx_op_kv_append(const float * k, const float * v, void * cache, const int32_t * pos, int M, int work, int * err, int rows, int T, hipStream_t st) {
+    if (!pos || work < 0 || work > 2) return CAMX_EINVAL;
+    if (work == 0) return camx_i_kv_append16(k, M, v, M, (uint16_t *)cache, M, 0, pos, rows, err, T, st);
+    if (work == 1) return pf_kv_append_launch(k, M, v, M, M, (uint8_t *)cache, 0, pos, rows, err, T, st);
+    return own_kv_q8_append_launch(k, M, v, M, M, (uint8_t *)cache, 0, pos, rows, err, T, st);
+}
+// OP_HADAMARD by its Seg fields (python/caminus/engine/k3.py:1244-1257): y = x (in place), N = C chunks, K = n, rows_per_task = chunks per task
+int camx_pf_hadamard(float * x, int C, int n, int rpb, hipStream_t st);
+int camx_op_hadamard(float * x, int C, int n, int rows_per_task, hipStream_t st) { return camx_pf_hadamard(x, C, n, rows_per_task, st); }
 
 int camx_pf_hadamard(float * x, int C, int n, int rpb, hipStream_t st) {
     (void)rpb;

@@ -104,7 +104,9 @@ __global__ void __launch_bounds__(256) gdn_gates_k(const float * __restrict__ al
 
 // ---- fp16 KV append: cache[pos0 + t] = fp16(k[t]) | fp16(v[t]) -----------------------------------------------------------------
 __global__ void __launch_bounds__(256) kv_append16_k(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv,
-                                                     uint16_t * __restrict__ cache, int M, int pos0, int rows, int * __restrict__ err, int vec) {
+                                                     uint16_t * __restrict__ cache, int M, int pos0, int rows, int * __restrict__ err, int vec,
+                                                     const int32_t * __restrict__ posb) {
+    if (posb) pos0 = posb[0];                             // the tape's device-resident position
     const int tt = blockIdx.x;
     const long pos = (long)pos0 + tt;
     if (pos < 0 || pos >= rows) { if (threadIdx.x == 0) atomicOr(err, 1); return; }
@@ -351,12 +353,16 @@ int camx_pf_gdn_gates(const float * al, int lda, const float * be, int ldb, cons
     gdn_gates_k<<<dim3((unsigned)(((long)T * H + 255) / 256)), dim3(256), 0, st>>>(al, lda, be, ldb, dt, A, y, H, T);
     CAMX_LAUNCH_RET();
 }
-int camx_q35p_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, int rows, int * err, int T, hipStream_t st) {
+// (internal: also the fp16 form of camx_op_kv_append, whose position is a device word)
+int camx_i_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, const int32_t * posb, int rows, int * err, int T, hipStream_t st) {
     if (!k || !v || !cache || !err || M < 1 || ldk < M || ldv < M || T < 0 || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     const int vec = !((M | ldk | ldv) & 3) && !(((uintptr_t)k | (uintptr_t)v) & 15) && !((uintptr_t)cache & 7);
-    kv_append16_k<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, cache, M, pos0, rows, err, vec);
+    kv_append16_k<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, cache, M, pos0, rows, err, vec, posb);
     CAMX_LAUNCH_RET();
+}
+int camx_q35p_kv_append16(const float * k, int ldk, const float * v, int ldv, uint16_t * cache, int M, int pos0, int rows, int * err, int T, hipStream_t st) {
+    return camx_i_kv_append16(k, ldk, v, ldv, cache, M, pos0, nullptr, rows, err, T, st);
 }
 int camx_pf_add_sum(const float * a, const float * b, float * y, long n, hipStream_t st) {
     if (!a || !b || !y || n < 0) return CAMX_EINVAL;

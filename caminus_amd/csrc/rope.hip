@@ -45,7 +45,9 @@ struct RopeArgs {
     const int32_t * page_table; int pt_stride, page, n_pages;   // paged addressing (null: row = position)
     int n;
     int rows;                        // unpaged: rows of the cache when positions come from the caller's array (0: not checked here)
+    const int32_t * posb;            // the tape's device-resident position: token t is at posb[0] + t (pos and pos0 unused)
 };
+CAMX_DEV int rope_pos(const RopeArgs & a, int t) { return a.pos ? a.pos[t] : (a.posb ? a.posb[0] : a.pos0) + t; }
 
 // TPW tokens per workgroup: 1 for decode-sized batches (wave 0 computes the token's cos / sin row); 4 for prefill chunks, where
 // wave w computes token w's row, one barrier publishes all four, and each wave then walks the tokens with the next token's
@@ -85,7 +87,7 @@ __global__ void __launch_bounds__(NW * 64) qk_rope_tokens(RopeArgs a) {
     const float eps = a.par[257];
     for (int tr = wave; tr < TPW; tr += NW) {                               // the tokens whose cos / sin rows this wave computes
         if (t0 + tr < a.n) {
-            const int pos = a.pos ? a.pos[t0 + tr] : a.pos0 + t0 + tr;
+            const int pos = rope_pos(a, t0 + tr);
             float c, s;
             if (YARN) { const float theta = (float)pos * a.par[258 + lraw], ms = a.par[322]; c = cosf(theta) * ms; s = sinf(theta) * ms; }
             else { const float theta = (float)pos * rope_freq(a.par[256], lraw); c = cosf(theta); s = sinf(theta); }
@@ -100,7 +102,7 @@ __global__ void __launch_bounds__(NW * 64) qk_rope_tokens(RopeArgs a) {
         const int ti = it_tp / npass, base = (it_tp - ti * npass) * HS * QR_STEPS, t = t0 + ti;
         if (t >= a.n) break;
         if (it_tp + 1 < TPW * npass) { const int tn = (it_tp + 1) / npass; load(xnext, t0 + tn, ((it_tp + 1) - tn * npass) * HS * QR_STEPS); }
-        const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+        const int pos = rope_pos(a, t);
         uint8_t * cw = nullptr;
         // a position outside the sequence's table row (paged) or outside the cache (unpaged): bit 1, that sequence's row is not written
         const bool span = pos >= 0 && (a.page_table ? pos / a.page < a.pt_stride : (a.rows == 0 || pos < a.rows));
@@ -293,7 +295,7 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
     nrm[tid] = a.par[tid];
     for (int tr = wave; tr < TPW; tr += 4) {                               // the tokens whose cos / sin rows this wave computes
         if (t0 + tr < a.n) {
-            const int pos = a.pos ? a.pos[t0 + tr] : a.pos0 + t0 + tr;
+            const int pos = rope_pos(a, t0 + tr);
             float c, sn;
             if (YARN) { const float theta = (float)pos * a.par[258 + lane], ms = a.par[322]; c = cosf(theta) * ms; sn = sinf(theta) * ms; }
             else { const float theta = (float)pos * rope_freq(a.par[256], lane); c = cosf(theta); sn = sinf(theta); }
@@ -306,7 +308,7 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
         const int ti = it / nchunk, base = (it - ti * nchunk) * 16 * STEPS, t = t0 + ti;
         if (t >= a.n) break;
         if (it + 1 < TPW * nchunk) { const int tn = (it + 1) / nchunk; load(xnext, t0 + tn, ((it + 1) - tn * nchunk) * 16 * STEPS); }
-        const int pos = a.pos ? a.pos[t] : a.pos0 + t;
+        const int pos = rope_pos(a, t);
         const bool span = pos >= 0 && (a.rows == 0 || pos < a.rows);          // (wave-uniform) outside the cache: bit 1, no row written
         if (!span && a.err && tid == 0 && base == 0) atomicOr(a.err, 1);
         uint16_t * cw = (uint16_t *)a.cache + (size_t)(span ? pos : 0) * 2 * M;
@@ -588,7 +590,7 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
 template <bool YARN, int TPW, bool Q8>
 static bool rope_chunk_launch_f32(const RopeArgs & a, hipStream_t st) {
     const int items = a.nh + 2 * a.nkv;
-    if (a.pos || a.page_table || items > 48 || (a.nh & 3) || (a.nkv & 3) || (Q8 && (a.pos0 < 0 || a.rows != 0))) return false;
+    if (a.pos || a.posb || a.page_table || items > 48 || (a.nh & 3) || (a.nkv & 3) || (Q8 && (a.pos0 < 0 || a.rows != 0))) return false;
     const dim3 grid((a.n + TPW - 1) / TPW), block(256);
     switch ((items + 15) >> 4) {
     case 1: qk_rope_chunk<YARN, 1, TPW, true, Q8><<<grid, block, 0, st>>>(a); break;
@@ -600,7 +602,7 @@ static bool rope_chunk_launch_f32(const RopeArgs & a, hipStream_t st) {
 template <bool YARN, int TPW>
 static bool rope_chunk_launch(const RopeArgs & a, hipStream_t st) {
     const int items = a.nh + 2 * a.nkv;
-    if (a.pos || a.page_table || (items & 15) || items > 80 || (a.nh & 3) || (a.nkv & 3)) return false;
+    if (a.pos || a.posb || a.page_table || (items & 15) || items > 80 || (a.nh & 3) || (a.nkv & 3)) return false;
     const dim3 grid((a.n + TPW - 1) / TPW), block(256);
     switch (items >> 4) {
     case 1: qk_rope_chunk<YARN, 1, TPW><<<grid, block, 0, st>>>(a); break;
@@ -615,7 +617,10 @@ static bool rope_chunk_launch(const RopeArgs & a, hipStream_t st) {
 // ---- pf_qk_nr: any head dim D <= 512, rotary on the first n_rot dims, input heads at head_stride ------------------------------
 struct NrArgs {
     const void * x; int head_stride, heads; const float * w; int D, nrot; float theta_scale, eps; int pos0; const int32_t * pos; void * out; int T;
+    const int32_t * posb;            // the tape's device-resident position: row r sits at posb[0] + r (pos and pos0 unused)
+    const void * x2; int head_stride2, heads2; const float * w2; void * out2;   // a second group of heads per token (k beside q); qk_nr_heads only
 };
+CAMX_DEV float nr_pos(const NrArgs & a, int tok) { return (float)(a.pos ? a.pos[tok] : (a.posb ? a.posb[0] : a.pos0) + tok); }
 // One wave per (token, head), four per workgroup, nothing shared between them: each wave issues its head's loads, computes
 // the token's cos / sin for the rotated pairs into its own LDS rows while they are in flight, normalizes, parks the normed
 // head in LDS for the partner reads of the rotation, and stores. No barrier; a verify batch of 16 tokens x 28 heads is 448
@@ -626,9 +631,13 @@ __global__ void __launch_bounds__(256) qk_nr_heads(NrArgs a) {
     __shared__ __attribute__((aligned(16))) float nrm[4][512];
     const int tid = threadIdx.x, lraw = tid & 63, lane = slot_of(lraw), wave = tid >> 6, half = a.nrot / 2;
     const long gw = (long)blockIdx.x * 4 + wave;
-    if (gw >= (long)a.T * a.heads) return;
-    const int tok = (int)(gw / a.heads);
-    const size_t xo = (size_t)gw * a.head_stride, yo = (size_t)gw * a.D;
+    const int hpt = a.heads + a.heads2;                          // heads per token over both groups
+    if (gw >= (long)a.T * hpt) return;
+    const int tok = (int)(gw / hpt), hh = (int)(gw - (long)tok * hpt);
+    const bool g2 = hh >= a.heads;                               // (wave-uniform) this head belongs to the second group
+    if (g2) { a.x = a.x2; a.w = a.w2; a.out = a.out2; a.head_stride = a.head_stride2; }
+    const size_t hi = g2 ? (size_t)tok * a.heads2 + (hh - a.heads) : (size_t)tok * a.heads + hh;
+    const size_t xo = hi * a.head_stride, yo = hi * a.D;
     float xv[2][4];
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -651,7 +660,7 @@ __global__ void __launch_bounds__(256) qk_nr_heads(NrArgs a) {
     for (int j = 0; j < 2; j++)
 #pragma unroll
         for (int k = 0; k < 4; k++) { const int i = 256 * j + 4 * lane + k; wv[j][k] = i < a.D ? a.w[i] : 0.0f; }
-    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    const float pos = nr_pos(a, tok);
     for (int j = lraw; j < half; j += 64) {
         const float theta = pos * rope_freq(a.theta_scale, j);
         rc[wave][j] = cosf(theta); rs[wave][j] = sinf(theta);
@@ -726,7 +735,7 @@ __global__ void __launch_bounds__(256) qk_nr_tokens_vec(NrArgs a) {
     for (int j = 0; j < 2; j++)
 #pragma unroll
         for (int k = 0; k < 4; k++) { const int i = 256 * j + 4 * lane + k; wv[j][k] = i < a.D ? a.w[i] : 0.0f; }
-    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    const float pos = nr_pos(a, tok);
     for (int j = tid; j < half; j += 256) {
         const float theta = pos * rope_freq(a.theta_scale, j);
         rc[j] = cosf(theta); rs[j] = sinf(theta);
@@ -812,7 +821,7 @@ __global__ void __launch_bounds__(256) qk_nr_tokens_fast(NrArgs a) {
     Raw r0 = load(wave), r1 = load(wave + 4);
     f32x4 wv = {0.0f, 0.0f, 0.0f, 0.0f};
     if (on) wv = *(const f32x4 *)(a.w + i0);
-    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    const float pos = nr_pos(a, tok);
     if (tid < half) {
         const float theta = pos * rope_freq(a.theta_scale, tid);
         rc[tid] = cosf(theta); rs[tid] = sinf(theta);
@@ -894,7 +903,7 @@ __global__ void __launch_bounds__(256) qk_nr_tokens_w8(NrArgs a) {
     };
     load(0);
     const f32x4 w0 = *(const f32x4 *)(a.w + i0), w1 = *(const f32x4 *)(a.w + i0 + 4);
-    const float pos = (float)(a.pos ? a.pos[tok] : a.pos0 + tok);
+    const float pos = nr_pos(a, tok);
     if (tid < half) {
         const float theta = pos * rope_freq(a.theta_scale, tid);
         rc[tid] = cosf(theta); rs[tid] = sinf(theta);
@@ -993,6 +1002,112 @@ static void launch_nr(const NrArgs & a, int io, hipStream_t st) {
     else { if (vec) qk_nr_heads<false, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<false, false><<<grid, block, 0, st>>>(a); }
 }
 
+// ---- the dense Q8 line's per-token chain in one launch ------------------------------------------------------------------------------
+// The reference appends, per full-attention layer, OP_QK_NR (k) -> OP_HADAMARD 256 (k) -> OP_HADAMARD 64 (v) -> OP_KV_APPEND (Q8 blocks with
+// the codec's refusal rules) and OP_QK_NR (q) -> OP_HADAMARD 256 (q) (python/caminus/engine/q35_dense.py:409-418; kernels/k3_q35_ops.h:341-364,
+// kernels/k3_q35_kvq8_ops.h:16-50, kernels/own_kv_codec.h:57-72): six tape segments through fp32 buffers. Here a half-wave owns one item of
+// 256 values (a q head, a k head, or 256 values of the token's v row = four 64-point chunks), lane l at values 8 l .. 8 l + 7: norm and
+// rotary as qk_nr_tokens_w8 forms them, the Walsh-Hadamard stages in the reference's order (h = 1, 2, 4 in registers, then lanes l ^ 1,
+// 2, 4, 8, 16; 8 lanes per 64-point chunk), the scale 1 / sqrtf(n) (a power of two), and the K / V blocks of 32 values from 4 lanes x 8.
+// Sums and differences are the same operations on the same operands as in the separate kernels, so every byte is theirs.
+template <int LOGL> CAMX_DEV void hadamard_w8_lanes(float (&e)[8], int l, float scale) {     // 8 << LOGL points: 1 << LOGL lanes x 8 registers
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if (!(k & h)) { const float a = e[k], b = e[k + h]; e[k] = a + b; e[k + h] = a - b; }
+#define W8L_STAGE(BIT, PARTNER)                                                                                  \
+    {                                                                                                              \
+        const uint32_t m = (l & BIT) ? 0x80000000u : 0u;                                                           \
+        _Pragma("unroll") for (int k = 0; k < 8; k++) {                                                            \
+            const float own = e[k];                                                                                \
+            e[k] = PARTNER(own) + __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, own) ^ m);                \
+        }                                                                                                          \
+    }
+#define W8L_XOR4(x) __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x101F))
+#define W8L_XOR16(x) __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F))
+    if (LOGL > 0) W8L_STAGE(1, dpp_full<0xB1>)
+    if (LOGL > 1) W8L_STAGE(2, dpp_full<0x4E>)
+    if (LOGL > 2) W8L_STAGE(4, W8L_XOR4)
+    if (LOGL > 3) W8L_STAGE(8, dpp_full<0x128>)
+    if (LOGL > 4) W8L_STAGE(16, W8L_XOR16)
+#undef W8L_XOR16
+#undef W8L_XOR4
+#undef W8L_STAGE
+#pragma unroll
+    for (int k = 0; k < 8; k++) e[k] *= scale;
+}
+struct NrQ8Args {
+    const float * q; int q_stride, nh; const float * k; int ldk; const float * v; int ldv; int nkv;
+    const float * qn, * kn; float theta_scale, eps; int pos0; const int32_t * posb, * pos;
+    float * qo; uint8_t * cache; int rows; int * err; int T;
+};
+template <int XL>
+__global__ void __launch_bounds__(256) qk_nr_q8_k(NrQ8Args a) {
+    __shared__ __attribute__((aligned(16))) float rc[128], rs[128];
+    constexpr int nrot = 16 * XL, half = nrot / 2;
+    const int tid = threadIdx.x, l32 = tid & 31, hw = tid >> 5, i0 = 8 * l32;
+    const int items = a.nh + 2 * a.nkv, G = (items + 7) >> 3;
+    const int tok = blockIdx.x / G, item = (blockIdx.x - tok * G) * 8 + hw;
+    const bool on = item < items;
+    const int kind = !on ? 3 : item < a.nh ? 0 : item < a.nh + a.nkv ? 1 : 2;                 // q head, k head, 256 values of v
+    const float * src = kind == 1 ? a.k + (size_t)tok * a.ldk + (size_t)(item - a.nh) * 256
+                      : kind == 2 ? a.v + (size_t)tok * a.ldv + (size_t)(item - a.nh - a.nkv) * 256
+                      : a.q + ((size_t)tok * a.nh + (on ? item : 0)) * a.q_stride;
+    const f32x4 r0 = *(const f32x4 *)(src + i0), r1 = *(const f32x4 *)(src + i0 + 4);
+    const long pos = (long)(a.pos ? a.pos[tok] : (a.posb ? a.posb[0] : a.pos0)) + (a.pos ? 0 : tok);
+    if (tid < half) {
+        const float theta = (float)(int)pos * rope_freq(a.theta_scale, tid);
+        rc[tid] = cosf(theta); rs[tid] = sinf(theta);
+    }
+    __syncthreads();
+    if (!on) return;
+    float e[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+    if (kind < 2) {
+        const float * wp = (kind == 0 ? a.qn : a.kn) + i0;
+        const f32x4 w0 = *(const f32x4 *)wp, w1 = *(const f32x4 *)(wp + 4);
+        float sq[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) sq[k] = e[k] * e[k];
+#pragma unroll
+        for (int k = 0; k < 8; k++) sq[k] = add_xor2(sq[k]);
+#pragma unroll
+        for (int k = 0; k < 8; k++) sq[k] = add_xor1(sq[k]);
+        const float b0 = sq[0] + sq[4], b1 = sq[1] + sq[5], b2 = sq[2] + sq[6], b3 = sq[3] + sq[7];
+        const float e0 = b0 + b2, e1 = b1 + b3;
+        const float g = e0 + e1;
+        const float tot = ((((((swz_group32<0>(g) + swz_group32<1>(g)) + swz_group32<2>(g)) + swz_group32<3>(g)) + swz_group32<4>(g)) + swz_group32<5>(g)) +
+                           swz_group32<6>(g)) + swz_group32<7>(g);
+        const float scale = rsqrt_exact(tot / 256.0f + a.eps);
+        const bool rot = i0 < nrot;
+        f32x4 c4[2] = {{1.0f, 1.0f, 1.0f, 1.0f}, {1.0f, 1.0f, 1.0f, 1.0f}}, s4[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+        if (rot) {
+            const int jj = i0 & (half - 1);
+            c4[0] = *(const f32x4 *)(rc + jj); c4[1] = *(const f32x4 *)(rc + jj + 4);
+            s4[0] = *(const f32x4 *)(rs + jj); s4[1] = *(const f32x4 *)(rs + jj + 4);
+            if (i0 < half) { s4[0] = -s4[0]; s4[1] = -s4[1]; }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float xn = (scale * e[k]) * (k < 4 ? w0[k] : w1[k - 4]);
+            const float pr = nr8_partner<XL>(xn);
+            e[k] = rot ? xn * (k < 4 ? c4[0][k] : c4[1][k - 4]) + pr * (k < 4 ? s4[0][k] : s4[1][k - 4]) : xn;
+        }
+        hadamard_w8_lanes<5>(e, l32, 0.0625f);
+    } else hadamard_w8_lanes<3>(e, l32, 0.125f);
+    if (kind == 0) {
+        float * o = a.qo + ((size_t)tok * a.nh + item) * 256 + i0;
+        *(f32x4 *)o = (f32x4){e[0], e[1], e[2], e[3]}; *(f32x4 *)(o + 4) = (f32x4){e[4], e[5], e[6], e[7]};
+        return;
+    }
+    const bool span = pos >= 0 && pos < a.rows;
+    if (!span && l32 == 0) atomicOr(a.err, 1);
+    const size_t nb = (size_t)a.nkv * 8;                                                     // blocks of K (and of V) per row
+    const size_t b = (kind == 1 ? (size_t)(item - a.nh) * 8 : nb + (size_t)(item - a.nh - a.nkv) * 8) + (l32 >> 2);
+    uint8_t * row = a.cache + (size_t)(span ? pos : 0) * (2 * nb * 34);
+    kv_q8_emit_w8(e, row + b * 34, l32 & 3, a.err, span);
+}
+
 __global__ void rope_freqs_k(float theta_scale, int n, float * out) {
     const int j = blockIdx.x * blockDim.x + threadIdx.x;
     if (j < n) out[j] = rope_freq(theta_scale, j);
@@ -1003,6 +1118,8 @@ static int rope_check(const RopeArgs & a, bool q8, bool bf16in) {
     if (((uintptr_t)a.qkv & (bf16in ? 7 : 15)) || ((uintptr_t)a.par & 15) || ((uintptr_t)a.q16 & 7) || ((uintptr_t)a.cache & (q8 ? 1 : 7))) return CAMX_EINVAL;
     if (q8 && !a.err) return CAMX_EINVAL;
     if (a.page_table && (a.page < 1 || a.n_pages < 1 || a.pt_stride < 1 || !a.err)) return CAMX_EINVAL;
+    if (!a.pos && !a.posb && (a.pos0 < 0 || a.pos0 > 0x7fffffff - a.n)) return CAMX_EINVAL;     // the reference's host span check (python/caminus/engine/k3.py:413-433)
+    if (a.posb && (!a.err || a.rows < 1)) return CAMX_EINVAL;
     return CAMX_OK;
 }
 template <bool BF16IN, int TPW>
@@ -1090,6 +1207,63 @@ int camx_qk_nr_pos(const void * xin, int head_stride, int heads, const float * w
     NrArgs a = {xin, head_stride, heads, w, D, nrot, theta_scale, eps, 0, pos, out, T};
     launch_nr(a, io, st);
     CAMX_LAUNCH_RET();
+}
+// OP_QK_NR by its Seg fields (python/caminus/engine/k3.py:1057-1063): a = x, pad1 = head_stride, W = w, asum = pos (int32 [1] on the device:
+// row r sits at pos[0] + r / heads), y = out, out_f32 = n_rot, rs = theta_scale, pad2 = the bit pattern of eps, N = T * heads, K = dim; fp32
+int camx_op_qk_nr(const float * x, int head_stride, int heads, int dim, const float * w, const int32_t * pos, float * out, int n_rot, float theta_scale,
+                  int eps_bits, int T, hipStream_t st) {
+    if (!x || !w || !out || !pos || T < 0 || heads < 1 || dim < 1 || dim > 512 || head_stride < dim || n_rot < 0 || n_rot > dim || (n_rot & 1)) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    NrArgs a = {x, head_stride, heads, w, dim, n_rot, theta_scale, __builtin_bit_cast(float, eps_bits), 0, nullptr, out, T, pos};
+    launch_nr(a, 0, st);
+    CAMX_LAUNCH_RET();
+}
+// q and k heads of a token in one launch (two OP_QK_NR segments of the tape, python/caminus/engine/q35_dense.py:408-415): group 1 = nh heads at
+// xq + (t * nh + h) * q_stride with weight wq -> outq [T][nh][D]; group 2 = nkv heads at xk + (t * nkv + h) * k_stride with wk -> outk. Row t at
+// pos ? pos[t] : (pos_dev ? pos_dev[0] : pos0) + t. A wave per head (the decode / verify form of camx_pf_qk_nr at every size).
+int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const void * xk, int k_stride, int nkv, const float * wk, int D, int nrot,
+                  float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, void * outq, void * outk, int T, int io, hipStream_t st) {
+    if (!xq || !xk || !wq || !wk || !outq || !outk || T < 0 || nh < 1 || nkv < 1 || D < 1 || D > 512 || q_stride < D || k_stride < D || nrot < 0 || nrot > D ||
+        (nrot & 1) || io < 0 || io > 1 || (!pos && !pos_dev && pos0 < 0)) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    NrArgs a = {xq, q_stride, nh, wq, D, nrot, theta_scale, eps, pos0, pos, outq, T, pos_dev, xk, k_stride, nkv, wk, outk};
+    const int es = io ? 2 : 4;
+    const bool vec = (D & 3) == 0 && ((q_stride | k_stride) & 3) == 0 && (((uintptr_t)xq | (uintptr_t)xk | (uintptr_t)outq | (uintptr_t)outk) & (4 * es - 1)) == 0;
+    const dim3 grid((unsigned)(((long)T * (nh + nkv) + 3) / 4)), block(256);
+    if (io) { if (vec) qk_nr_heads<true, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<true, false><<<grid, block, 0, st>>>(a); }
+    else { if (vec) qk_nr_heads<false, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<false, false><<<grid, block, 0, st>>>(a); }
+    CAMX_LAUNCH_RET();
+}
+// The dense Q8 line's six segments in one launch (see qk_nr_q8_k): heads of 256 dims. q [T][nh] heads at q_stride floats (the q | gate
+// interleave), k and v [T][nkv * 256] at ldk / ldv; qo fp32 [T][nh][256] = H256(rotary(norm(q) * qn)); cache row pos + t = Q8 blocks of
+// H256(rotary(norm(k) * kn)) per head | Q8 blocks of H64(v) per 64 values. err bits: 1 a row outside [0, rows) (not written; qo is),
+// 2 a refused block (bytes untouched). nrot in {16, 32, 64, 128, 256}.
+int camx_qk_nr_q8(const float * q, int q_stride, int nh, const float * k, int ldk, const float * v, int ldv, int nkv, const float * qn, const float * kn,
+                  int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, float * qo, uint8_t * cache, int rows,
+                  int * err, int T, hipStream_t st) {
+    if (!q || !k || !v || !qn || !kn || !qo || !cache || !err || T < 0 || nh < 1 || nkv < 1 || q_stride < 256 || (q_stride & 3) || ldk < nkv * 256 || ldv < nkv * 256 ||
+        ((ldk | ldv) & 3) || rows < 1 || (!pos && !pos_dev && pos0 < 0) ||
+        (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)qn | (uintptr_t)kn | (uintptr_t)qo) & 15) || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
+    if (nrot != 16 && nrot != 32 && nrot != 64 && nrot != 128 && nrot != 256) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    NrQ8Args a = {q, q_stride, nh, k, ldk, v, ldv, nkv, qn, kn, theta_scale, eps, pos0, pos_dev, pos, qo, cache, rows, err, T};
+    const dim3 grid((unsigned)((long)T * ((nh + 2 * nkv + 7) / 8))), block(256);
+    switch (nrot) {
+    case 16: qk_nr_q8_k<1><<<grid, block, 0, st>>>(a); break;
+    case 32: qk_nr_q8_k<2><<<grid, block, 0, st>>>(a); break;
+    case 64: qk_nr_q8_k<4><<<grid, block, 0, st>>>(a); break;
+    case 128: qk_nr_q8_k<8><<<grid, block, 0, st>>>(a); break;
+    default: qk_nr_q8_k<16><<<grid, block, 0, st>>>(a); break;
+    }
+    CAMX_LAUNCH_RET();
+}
+// The OP_OWN_ATTS prologue with the tape's device-resident position (kernels/k3_own_atts.h:183-274; Seg.asum = pos int32 [1]): token t at
+// pos[0] + t, checked on the device against the cache's `rows` (err bit 1, the row is not written; q16 is). q8 selects the row format.
+int camx_op_own_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16, void * cache, int rows,
+                        int * err, int n, int yarn, int q8, hipStream_t st) {
+    if (!pos) return CAMX_EINVAL;
+    RopeArgs a = {qkv, ldq, nh, nkv, par, 0, nullptr, q16, cache, err, nullptr, 0, 0, 0, n, rows, pos};
+    return rope_launch(a, yarn, q8 != 0, st);
 }
 // the per-pair frequencies the rotary kernels use: out[j] = (float)pow((double)theta_scale, j), j < n
 int camx_rope_freqs(float theta_scale, int n, float * out, hipStream_t st) {

@@ -160,6 +160,11 @@ def _glue(K):
             'pf_ple_gate': _rows('camx_pf_ple_gate'), 'pf_ple_conv': _plain('camx_pf_ple_conv'), 'pf_ple_hist': _plain('camx_pf_ple_hist')}
 
 
+def _pf_kv_append16(g, b, v):     # the PREFILL_KV_F16 build of pf_kv_append: (k, ldk, v, ldv, M, cache, pos0, rows, err); grid T
+    k, ldk, vv, ldv, M, cache, pos0, rows, err = v
+    return [k, ldk, vv, ldv, cache, M, pos0, rows, err, I(g[0])]
+
+
 _ATTN = {'pf_qk_nr': ('camx_pf_qk_nr', _pf_qk_nr), 'pf_hadamard': _plain('camx_pf_hadamard'), 'pf_kv_append': _rows('camx_pf_kv_append'),
          'pf_gate_mul': _gate(0), 'pf_hc_avg': _plain('camx_pf_hc_avg')}
 def _gdn_norm(silu):
@@ -176,7 +181,8 @@ SYMBOLS = {
     'q3m_prefill': _q3m(False, False), 'q3m_prefill_kvq8': _q3m(False, True), 'q3m_prefill_yarn': _q3m(True, False),
     'q3m_prefill_kvq8_yarn': _q3m(True, True), 'q35_prefill': _Q35,
     'prefill_glue': _glue(2560), 'prefill_glue_q35': _glue(2048), 'prefill_glue_q35d': _glue(5120),
-    'prefill_attn': _ATTN, 'prefill_attn_q35': _ATTN, 'prefill_attn_q35d': _ATTN, 'prefill_gdn': _GDN, 'prefill_gdn_q35': _GDN_SILU,
+    'prefill_attn': _ATTN, 'prefill_attn_q35': _ATTN, 'prefill_attn_q35d': _ATTN,
+    'prefill_attn_f16': dict(_ATTN, pf_kv_append=('camx_q35p_kv_append16', _pf_kv_append16)),      # fp16 cache rows (python/caminus/prefill/attn.py:150-155) 'prefill_gdn': _GDN, 'prefill_gdn_q35': _GDN_SILU,
     'prefill_mmq_glue': {},      # its quantizers are template instances in the reference: caminus_amd.prefill.mmq binds them
     'camx': {},                  # direct access to every C entry point by its own name (Module('camx').camx_...)
 }

@@ -39,3 +39,120 @@ def kv_rows(cache, M, q8):
     if nb % pb or not 0 < nb // pb < 2 ** 31:
         raise ValueError(f'k3 KV cache: {nb} bytes is not a whole number of {pb}-byte positions')
     return nb // pb
+
+
+# ---- the hot-path ops of the tape as immediate launches -------------------------------------------------------------------------------
+# The reference's K3 object appends a Seg per op and runs the whole tape in one persistent launch (python/caminus/engine/k3.py:393-399).
+# The tape walker is not part of this library; TapeOps offers the same methods with the same arguments for the row ops this library
+# covers, each launched at once through the C ABI's camx_op_* entry points (dep / team / rows_per_task describe the tape's scheduling
+# and are accepted and ignored). The position is the tape's own: an int32 word on the device, so a captured graph of these launches
+# advances when the caller increments that word.
+OWN_BLOCK = {'Q4_K': 144, 'IQ2_S': 82}
+OWN_FMT = {'Q4_K': 4, 'IQ2_S': 7}
+
+
+class TapeOps:
+    def __init__(self, T=1, kv_q8_dense=False, kv_error=None):
+        """T: tokens per pass; kv_q8_dense: kv_append(q8=True) writes the dense Q8 line's blocks with the codec's refusal rules (the
+        reference's K3_Q35_KV_Q8 modules) and needs kv_error, the sticky int32 word"""
+        import ctypes
+        import torch
+        from ..device import lib as _lib
+        self.T, self.kv_q8_dense, self.kv_error = int(T), bool(kv_q8_dense), kv_error
+        if self.kv_q8_dense and kv_error is None: raise ValueError('TapeOps: the dense Q8 KV line needs its error word (kv_error)')
+        self._C, self._torch, self._L, self._check = ctypes, torch, _lib.load(), _lib.check
+        self.params = None              # the pass parameters of gdn_conv (int32 [4] on the device; [1] = tokens of the previous pass to commit)
+        self.n = 0
+
+    def _p(self, t):
+        return self._C.c_void_p(None if t is None else t.data_ptr())
+
+    def _go(self, name, *args):
+        st = self._C.c_void_p(self._torch.cuda.current_stream().cuda_stream)
+        self._check(getattr(self._L, name)(*args, st))
+        self.n += 1
+        return self.n - 1
+
+    def gg_q8_1(self, x, yq, dep=-1, team=-1, silu_scale=None, mul=None):
+        I, F = self._C.c_int, self._C.c_float
+        n = x.numel(); assert mul is None or (silu_scale is None and mul.numel() == n)
+        work = 2 if mul is not None else 0 if silu_scale is None else 1
+        return self._go('camx_op_gg_q8_1', self._p(x), self._p(yq), I(n), I(work), F(0.0 if silu_scale is None else silu_scale), self._p(mul))
+
+    def rms_mul(self, x, w, out, eps, dep=-1, team=-1, q8=None):
+        I, F = self._C.c_int, self._C.c_float
+        K = x.shape[-1]; R = x.numel() // K; wr = w.numel() // K; assert R % wr == 0 and (q8 is None or K % 32 == 0)
+        return self._go('camx_op_rms_mul', self._p(x), self._p(w), self._p(out), self._p(q8), I(R), I(wr), I(K), F(eps))
+
+    def own_add_rms16(self, x, nw, h, h16, eps, d=None, slots=0, w=None, dep=-1, team=-1, tokens=1, h16_stride=None):
+        I, F = self._C.c_int, self._C.c_float
+        n = x.numel() // tokens; hs = n if h16_stride is None else int(h16_stride)
+        if n % 256 or not 256 <= n <= 2048: raise ValueError(f'own_add_rms16: n {n} (a multiple of 256, at most 2048)')
+        assert 0 <= slots <= 8 and (slots == 0 or d.numel() >= tokens * slots * n) and (w is None or w.numel() >= tokens * slots)
+        return self._go('camx_op_own_add_rms16', self._p(x), self._p(d), self._p(w), I(slots), self._p(nw), F(eps), self._p(h), self._p(h16), I(n), I(hs), I(tokens))
+
+    def own_emb(self, w, fmt, vocab, D, tok, x, dep=-1, team=-1, tokens=1, key=False):
+        I = self._C.c_int
+        if fmt not in OWN_FMT: raise ValueError(f'own_emb: {fmt} (Q4_K, IQ2_S)')
+        rb = D // 256 * OWN_BLOCK[fmt]; assert D % 256 == 0 and w.numel() * w.element_size() >= vocab * rb and x.numel() >= tokens * D
+        return self._go('camx_op_own_emb', self._p(w), self._p(tok), self._p(x), I(D), I(rb), I(OWN_FMT[fmt]), I(1 if key else 0), I(vocab), I(tokens))
+
+    def own_swiglu16(self, g, u, y16, rows_per_task=1024, dep=-1, team=-1):
+        n = g.numel(); assert u.numel() == n and y16.dtype == self._torch.float16 and y16.numel() >= n
+        return self._go('camx_op_own_swiglu16', self._p(g), self._p(u), self._p(y16), self._C.c_int(n))
+
+    def qk_nr(self, x, head_stride, heads, dim, w, pos, out, n_rot, theta_scale, eps, dep=-1, team=-1):
+        I, F = self._C.c_int, self._C.c_float
+        eb = int(np.array([eps], dtype=np.float32).view(np.int32)[0])
+        return self._go('camx_op_qk_nr', self._p(x), I(head_stride), I(heads), I(dim), self._p(w), self._p(pos), self._p(out), I(n_rot), F(theta_scale), I(eb), I(self.T))
+
+    def kv_append(self, k, v, cache, pos, q8=False, dep=-1, team=-1):
+        I = self._C.c_int
+        if k.numel() % self.T: raise ValueError('kv_append: K must contain a whole row per pass token')
+        M = k.numel() // self.T
+        rows = kv_rows(cache, M, q8)
+        if rows < self.T: raise ValueError('kv_append: fewer physical cache rows than pass tokens')
+        work = (2 if self.kv_q8_dense else 1) if q8 else 0
+        err = self.kv_error
+        if err is None: raise ValueError('kv_append: an int32 error word (kv_error) receives the span / codec bits')
+        return self._go('camx_op_kv_append', self._p(k), self._p(v), self._p(cache), self._p(pos), I(M), I(work), self._p(err), I(rows), I(self.T))
+
+    def hadamard(self, x, n, rows_per_task=1, dep=-1, team=-1):
+        assert n in (64, 128, 256) and x.numel() % n == 0
+        if (isinstance(rows_per_task, (bool, np.bool_)) or not isinstance(rows_per_task, (int, np.integer))
+                or not 1 <= rows_per_task < 2 ** 31 or not 0 < x.numel() // n < 2 ** 31):
+            raise ValueError('k3 Q8 Hadamard: positive int32 chunk/task counts required')
+        I = self._C.c_int
+        return self._go('camx_op_hadamard', self._p(x), I(x.numel() // n), I(n), I(int(rows_per_task)))
+
+    def gate_mul16(self, a, gate, head_stride, offset, out16, dim, rows_per_task=256, dep=-1, team=-1):
+        I = self._C.c_int
+        n = a.numel(); assert n % dim == 0 and gate.numel() >= (n // dim - 1) * head_stride + offset + dim
+        assert out16.dtype == self._torch.float16 and out16.numel() >= n
+        return self._go('camx_op_gate_mul16', self._p(a), self._p(gate), I(head_stride), I(offset), self._p(out16), I(n), I(dim))
+
+    def gdn_l2(self, x, out, heads, dim, eps, x_stride=0, dep=-1, team=-1):
+        I, F = self._C.c_int, self._C.c_float
+        return self._go('camx_op_gdn_l2', self._p(x), self._p(out), I(heads), I(dim), F(np.float32(eps / dim)), I(x_stride), I(self.T))
+
+    def gdn_conv(self, x, w, state, out, xprev, rows_per_task=256, dep=-1, team=-1):
+        I = self._C.c_int
+        C_ = x.numel() // self.T; assert xprev.numel() >= x.numel()
+        if self.params is None: raise ValueError('gdn_conv: set TapeOps.params (int32 [4] on the device; [1] = tokens to commit)')
+        return self._go('camx_op_gdn_conv', self._p(w), self._p(state), self._p(x), self._p(self.params), self._p(out), self._p(xprev), I(C_), I(self.T))
+
+    # the two chains the reference's dense engine appends back to back (python/caminus/engine/q35_dense.py:399-400, 409-418), one launch each
+    def gdn_conv_l2(self, x, w, state, out, xprev, qk, heads, dim, eps, dep=-1, team=-1):
+        I, F = self._C.c_int, self._C.c_float
+        C_ = x.numel() // self.T
+        if dim != 128: raise ValueError('gdn_conv_l2: key heads of 128 values')
+        if self.params is None: raise ValueError('gdn_conv_l2: set TapeOps.params (int32 [4] on the device; [1] = tokens to commit)')
+        return self._go('camx_op_gdn_conv_l2', self._p(w), self._p(state), self._p(x), self._p(self.params), self._p(out), self._p(xprev), self._p(qk), I(C_), I(self.T),
+                        I(heads), F(np.float32(eps / dim)))
+
+    def qk_nr_q8(self, q, q_head_stride, heads, k, v, kv_heads, qn, kn, pos, qo, cache, n_rot, theta_scale, eps, dep=-1, team=-1):
+        I, F = self._C.c_int, self._C.c_float
+        M = kv_heads * 256
+        rows = kv_rows(cache, M, True)
+        return self._go('camx_qk_nr_q8', self._p(q), I(q_head_stride), I(heads), self._p(k), I(M), self._p(v), I(M), I(kv_heads), self._p(qn), self._p(kn), I(n_rot),
+                        F(theta_scale), F(eps), I(0), self._p(pos), self._p(None), self._p(qo), self._p(cache), I(rows), self._p(self.kv_error), I(self.T))

@@ -7,8 +7,8 @@
  *     launched). camx_error_string() names the value.
  *   - The library allocates nothing per call and keeps no state between calls, except a 128 KiB lookup table of
  *     bf16(silu(g)) for every bf16 g that camx_swiglu_mmq_q8_1, camx_silu_mul_bf16 and camx_silu_mul_actq_fwd / _bwd share and
- *     the first of them to be called fills once per device (that call waits for its stream once: make it before any graph
- *     capture). All four therefore produce the same activation bits for a row, whatever the batch size.
+ *     that camx_init(), or else the first of them to be called, fills once per device (that call waits for its stream once: call
+ *     camx_init() before any graph capture). All four therefore produce the same activation bits for a row, whatever the batch size.
  *   - bf16 / fp16 values travel as uint16_t bit patterns. "rows" / "n" / "T" arguments that the reference kernels took
  *     from their launch grid are explicit trailing arguments here.
  *   - Device-side errors are sticky int32 words OR-ed by the kernels and never cleared by them; bit meanings are given at
@@ -36,6 +36,11 @@ typedef struct ihipStream_t * camx_stream_t;      /* = hipStream_t */
 int camx_version(void);
 const char * camx_arch(void);                     /* "gfx950" */
 const char * camx_error_string(int err);          /* hipGetErrorString; replaces device/hip.py:35-37's lookup */
+/* Fills the current device's lookup tables (bf16(silu g), the fused backward's sigmoid, their LDS extracts) on `stream` and waits for it
+ * once; afterwards no entry point synchronizes on this device, so every later call may sit inside a stream capture (the reference loads
+ * its code objects before it captures: python/caminus/prefill/attn.py:150-155). Idempotent and thread-safe. Without it the first call of
+ * an entry point that needs a table does the same work. */
+int camx_init(camx_stream_t stream);
 
 /* ---- residual add + RMSNorm -------------------------------------------------------------------------------------------- */
 /* q3p_add_rms16 (kernels/q3m_prefill.hip:385-415) = OP_OWN_ADD_RMS16 (kernels/k3_own_ops.h:326-383).
@@ -83,6 +88,35 @@ int camx_op_gdn_conv(const float * w, float * state, const float * x, const int3
                      camx_stream_t stream);
 /* OP_RMS_MUL (kernels/k3_gguf_ops.h:1233-1268; Seg fields: a = x, W = w, y, asum = q8, N = R, K, pad1 = wr, rs = eps). */
 int camx_op_rms_mul(const float * x, const float * w, float * y, void * q8, int R, int wr, int K, float eps, camx_stream_t stream);
+/* The remaining hot-path ops of the decode tape by their Seg fields (python/caminus/engine/k3.py:393-399). The tape keeps its position in an
+ * int32 word ON THE DEVICE (Seg.asum), so a captured graph advances by a device-side increment; these forms read it there.
+ * OP_QK_NR (k3.py:1057-1063; kernels/k3_gguf_ops.h:1495-1518): a = x, pad1 = head_stride, W = w, asum = pos (row r at pos[0] + r / heads),
+ * y = out, out_f32 = n_rot, rs = theta_scale, pad2 = eps_bits (the bit pattern of eps), N = T * heads, K = dim; fp32. */
+int camx_op_qk_nr(const float * x, int head_stride, int heads, int dim, const float * w, const int32_t * pos, float * out, int n_rot,
+                  float theta_scale, int eps_bits, int T, camx_stream_t stream);
+/* OP_KV_APPEND (k3.py:1065-1089; kernels/k3_gguf_ops.h:1520-1553, kernels/k3_q35_kvq8_ops.h:16-27): a = k, W = v (fp32 [T][M]), y = cache,
+ * asum = pos (token t to row pos[0] + t), N = M, gs = err. work 0: fp16 rows [K | V]; 1: ggml q8_0 rows; 2: the dense Q8 line's blocks with
+ * the codec's refusal rules (the reference selects that form by its K3_Q35_KV_Q8 build, with work = 1 and its sticky word in gs). rows =
+ * the cache's rows, checked on the device as the reference's launch guard does: err bit 1, the row is not written; bit 2 a refused block
+ * (bytes untouched), bit 4 layout (work 2). */
+int camx_op_kv_append(const float * k, const float * v, void * cache, const int32_t * pos, int M, int work, int * err, int rows, int T,
+                      camx_stream_t stream);
+/* OP_HADAMARD (k3.py:1244-1257): y = x in place, N = C chunks, K = n in {64, 128, 256}; rows_per_task is the tape's task size (ignored). */
+int camx_op_hadamard(float * x, int C, int n, int rows_per_task, camx_stream_t stream);
+/* OP_GATE_MUL16 (k3.py:1209-1219; kernels/k3_q35_ops.h:381-391): a, W = gate, y = out16 fp16, N = n, K = dim, pad1 = head_stride, pad2 = offset. */
+int camx_op_gate_mul16(const float * a, const float * gate, int head_stride, int offset, uint16_t * out16, int n, int dim, camx_stream_t stream);
+/* OP_GDN_L2 (k3.py:1002-1008; kernels/k3_q35_ops.h:181-194): a = x, y = out, rs = eps / dim, N = T * heads, K = dim, pad1 = x_stride (0: heads * dim). */
+int camx_op_gdn_l2(const float * x, float * out, int heads, int dim, float rs, int x_stride, int T, camx_stream_t stream);
+/* OP_OWN_SWIGLU16 (k3.py:854-860; kernels/k3_own_ops.h:258-262): a = g, W = u, y = y16, N = n. */
+int camx_op_own_swiglu16(const float * g, const float * u, uint16_t * y16, int n, camx_stream_t stream);
+/* The prologue of OP_OWN_ATTS (k3.py:1151-1199, Seg.asum = pos; kernels/k3_own_atts.h:183-274): camx_q3p_qk_rope / _q8 with token t at
+ * pos[0] + t read on the device, checked there against the cache's `rows` (err bit 1: the row is not written, q16 is). err is required. */
+int camx_op_own_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16, void * cache,
+                        int rows, int * err, int n, int yarn, int q8, camx_stream_t stream);
+/* OP_GDN_CONV followed by OP_GDN_L2, the pair the tape appends back to back (python/caminus/engine/q35_dense.py:399-400), in one launch:
+ * camx_op_gdn_conv's arguments, then qk [T][heads][128] = camx_op_gdn_l2(y, qk, heads, 128, rs, C, T). Same bits as the two. C % 128 == 0. */
+int camx_op_gdn_conv_l2(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, float * qk, int C,
+                        int T, int heads, float rs, camx_stream_t stream);
 /* pf_hc_post_rms (kernels/prefill_glue.hip:130-170): row q = t * HC + h of N values: res[q] = fma(b[t], 2 sigmoid(inj[q] * rs),
  * res[q]) in place, then the norm of the updated row with w[h]: xn fp32, xnbf bf16, scl the row scale [T * HC], each optional.
  * The reference kernel is built for N = 2560; N is an argument here. */
@@ -134,7 +168,8 @@ int camx_gate_mul(const void * a, const void * gate, void * y, long N, int D, in
 /* q3p_qk_rope (kernels/q3m_prefill.hip:534-591, F16 form; yarn = the Q3P_YARN build): n tokens at positions pos0 + t;
  * qkv fp32 [n][ldq] = q (nh heads of 128) | k (nkv) | v (nkv); par = q_norm[128] | k_norm[128] | theta_scale | eps
  * (| freq[64] | mscale when yarn); q16 fp16 [n][nh][128]; cache = fp16 rows [K | V] indexed by position. The caller has
- * checked the positions against the cache's rows (prefill/q3m_ops.py:103-117). */
+ * checked the positions against the cache's rows (prefill/q3m_ops.py:103-117); pos0 < 0 (or pos0 + n past INT_MAX) is refused here (1), for
+ * this and the next two entry points. */
 int camx_q3p_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, int pos0, uint16_t * q16, uint16_t * cache,
                      int n, int yarn, camx_stream_t stream);
 /* q3p_qk_rope_q8 (same source under Q3P_KV_Q8; rotation kernels/own_kv_rot128.h:21-33, block encode
@@ -161,6 +196,22 @@ int camx_pf_qk_nr(const void * xin, int head_stride, int heads, const float * w,
 /* The same with one position per row (a speculative-verify batch). */
 int camx_qk_nr_pos(const void * xin, int head_stride, int heads, const float * w, int D, int nrot, float theta_scale, float eps,
                    const int32_t * pos, void * out, int T, int io, camx_stream_t stream);
+/* The q heads and the k heads of a token in one launch (the two OP_QK_NR segments of a full-attention layer,
+ * python/caminus/engine/q35_dense.py:408-415): nh heads at xq + (t * nh + h) * q_stride with weight wq -> outq [T][nh][D], nkv heads at
+ * xk + (t * nkv + h) * k_stride with wk -> outk [T][nkv][D]. Row t sits at pos[t] (pos given), else pos_dev[0] + t (pos_dev given: a
+ * device word), else pos0 + t. The same bits as two camx_pf_qk_nr / camx_qk_nr_pos calls. */
+int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const void * xk, int k_stride, int nkv, const float * wk, int D,
+                  int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, void * outq, void * outk,
+                  int T, int io, camx_stream_t stream);
+/* The dense Q8 line's per-token chain in one launch (python/caminus/engine/q35_dense.py:409-418: OP_QK_NR k -> OP_HADAMARD 256 ->
+ * OP_HADAMARD 64 on v -> OP_KV_APPEND with kernels/k3_q35_kvq8_ops.h:16-27's Q8 writer, and OP_QK_NR q -> OP_HADAMARD 256): heads of 256
+ * dims, fp32. q [T][nh] heads at q_stride floats (the q | gate interleave), k and v [T][nkv * 256] at ldk / ldv; qo [T][nh][256] = the
+ * transformed q; cache row (position) = Q8 blocks of the transformed k heads | Q8 blocks of H64(v). Positions as in camx_qk_nr_qk. err bits:
+ * 1 a position outside [0, rows) (row not written; qo is), 2 a refused block (its bytes stay). nrot in {16, 32, 64, 128, 256}. Every byte
+ * equals camx_pf_qk_nr + camx_pf_hadamard + camx_own_kv_q8_append on the same inputs. */
+int camx_qk_nr_q8(const float * q, int q_stride, int nh, const float * k, int ldk, const float * v, int ldv, int nkv, const float * qn,
+                  const float * kn, int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, float * qo,
+                  uint8_t * cache, int rows, int * err, int T, camx_stream_t stream);
 /* out[j] = the frequency of rotary pair j as the kernels above compute it: the correctly rounded theta_scale ** j. */
 int camx_rope_freqs(float theta_scale, int n, float * out, camx_stream_t stream);
 
@@ -221,6 +272,12 @@ int camx_pf_conv_state(const void * x, float * state, int C, int T, int ldx, int
 /* pf_gdn_l2 (kernels/prefill_gdn.hip:66-78) = OP_GDN_L2 (kernels/k3_q35_ops.h:181-194): per head of K <= 512 values
  * y = (scale * x) * (1 / sqrt(K)), scale = 1 / sqrt(sum x^2 / K + rs); head h of token t at x + t * ldx + h * K. */
 int camx_pf_gdn_l2(const void * x, void * y, int heads, int K, int ldx, float rs, int T, int bf16, camx_stream_t stream);
+/* pf_gdn_conv and pf_gdn_l2 in one launch (the reference runs them back to back: python/caminus/engine/q35_dense.py:399-400,
+ * kernels/k3_q35_ops.h:152-194): y (optional) = camx_pf_gdn_conv's rows; qk [T][heads][128] = camx_pf_gdn_l2(y, heads, 128, ldy, rs), the
+ * norm of the first heads * 128 channels, taken from the values as y stores them. Same bits as the two calls. C % 128 == 0, operands
+ * 16-byte aligned, ldx / ldy multiples of 4 (fp32) or 8 (bf16). The state is read only (camx_pf_conv_state advances it). */
+int camx_gdn_conv_l2(const void * x, const float * w, const float * state, void * y, void * qk, int C, int T, int ldx, int ldy, int heads,
+                     float rs, int bf16, camx_stream_t stream);
 
 /* ---- S1 core and fused residual (kernels/core.hip, kernels/fuse.hip) ------------------------------------------------------------- */
 int camx_embedding_f32(const int * tok, const float * emb, float * out, int D, int T, camx_stream_t stream);          /* core.hip:23-28 */

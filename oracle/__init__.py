@@ -278,6 +278,31 @@ def gdn_l2(x, T, heads, K, eps, ldx=None):
     lib().orc_gdn_l2(_p(x), _p(y), I(T), I(heads), I(K), I(ldx), F(np.float32(eps / K))); return y
 
 
+def gdn_conv_l2(x, w, st, heads, eps, bf16=False):
+    """OP_GDN_CONV then OP_GDN_L2 as the reference's dense engine appends them (python/caminus/engine/q35_dense.py:399-400): the L2 norm reads
+    the first heads * 128 channels of the convolution's stored output (bf16: rounded first). -> (y [T, C], qk [T * heads, 128])"""
+    y, _ = gdn_conv(x, w, st)
+    if bf16: y = bf2f(f2bf(y))
+    T, C_ = y.shape
+    return y, gdn_l2(y, T, heads, 128, eps, ldx=C_)
+
+
+def qk_nr_q8(q, q_stride, nh, k, v, nkv, qn, kn, n_rot, theta_scale, eps, pos, cache, rows):
+    """the dense Q8 line's chain (python/caminus/engine/q35_dense.py:409-418): qo = H256(qk_nr(q)); cache row pos[t] = Q8 blocks of
+    H256(qk_nr(k)) | Q8 blocks of H64(v) with the codec's refusals (kernels/k3_q35_kvq8_ops.h:16-50). pos: one position per token.
+    -> (qo [T * nh, 256], cache bytes, err)"""
+    T = len(pos); M = nkv * 256; err = 0
+    k = _c(k, np.float32).reshape(T, M); v = _c(v, np.float32).reshape(T, M)
+    qo = np.concatenate([hadamard_n(qk_nr(_c(q, np.float32)[t * nh:(t + 1) * nh], q_stride, nh, qn, 256, n_rot, theta_scale, eps, int(pos[t]), 1), 256) for t in range(T)])
+    cache = _c(cache, np.uint8).copy()
+    for t in range(T):
+        ko = hadamard_n(qk_nr(k[t].reshape(nkv, 256), 256, nkv, kn, 256, n_rot, theta_scale, eps, int(pos[t]), 1), 256).reshape(1, M)
+        vo = hadamard_n(v[t], 64).reshape(1, M)
+        cache, e = kv_q8_append(ko, M, vo, M, M, cache, int(pos[t]), 1, rows=rows)
+        err |= e
+    return qo, cache, err
+
+
 # ---- rotary ---------------------------------------------------------------------------------------------------------------
 
 

@@ -1,0 +1,362 @@
+"""GPU parity of the fused chains (conv4 + SiLU + L2 norm; QK-norm + partial rotary + Hadamard + Q8 blocks), of the tape-shaped entry
+points that read their position from a device word, and of camx_init. A fused launch must leave the bytes of the separate launches it
+replaces (that is its contract); the separate launches are held to the oracle by their own tests, and the fused outputs are checked
+against the oracle's composition as well."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import F, HADAMARD_FLOOR, I, L64, NULL, bits_equal, call, camx, close_16, close_fp32, dev, host, outliers, ptr, stream
+from vectors import qk_par
+
+pytestmark = pytest.mark.gpu
+RS = np.float32(1e-6 / 128)
+
+
+def _theta(base, n_rot):
+    return float(np.float32(np.float32(base) ** np.float32(-2.0 / n_rot)))
+
+
+# ---- conv4 + SiLU + L2 ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('T,C,heads', [(16, 10240, 32), (16, 10240, 48), (1, 128, 1), (5, 1024, 3), (3, 384, 3), (300, 4096, 16), (4096, 10240, 32), (1100, 1024, 8)])
+@pytest.mark.parametrize('bf16', [0, 1])
+def test_gdn_conv_l2_equals_the_two_launches(T, C, heads, bf16):
+    rng = np.random.default_rng(T + C + heads)
+    pad = 8
+    x = outliers(rng, (T, C + pad)); w = rng.standard_normal((C, 4)).astype(np.float32); st = rng.standard_normal((C, 3)).astype(np.float32)
+    xin = O.f2bf(x) if bf16 else x
+    dt = np.uint16 if bf16 else np.float32
+    xd, wd, sd = dev(xin), dev(w), dev(st)
+    y1 = dev(np.zeros((T, C), dt)); q1 = dev(np.zeros((T * heads, 128), dt))
+    call('camx_pf_gdn_conv', ptr(xd), ptr(wd), ptr(sd), ptr(y1), I(C), I(T), I(C + pad), I(C), I(bf16))
+    call('camx_pf_gdn_l2', ptr(y1), ptr(q1), I(heads), I(128), I(C), F(RS), I(T), I(bf16))
+    y2 = dev(np.full((T, C), 7, dt)); q2 = dev(np.full((T * heads, 128), 7, dt))
+    call('camx_gdn_conv_l2', ptr(xd), ptr(wd), ptr(sd), ptr(y2), ptr(q2), I(C), I(T), I(C + pad), I(C), I(heads), F(RS), I(bf16))
+    assert torch.equal(y1, y2) and torch.equal(q1, q2)
+    q3 = dev(np.full((T * heads, 128), 7, dt))                      # without the convolution's own output
+    call('camx_gdn_conv_l2', ptr(xd), ptr(wd), ptr(sd), NULL, ptr(q3), I(C), I(T), I(C + pad), I(C), I(heads), F(RS), I(bf16))
+    assert torch.equal(q1, q3)
+    if T * C <= 16 * 10240 or (T, C) == (300, 4096):                # against the oracle (the big shapes are covered by the equality above)
+        xs = O.bf2f(xin) if bf16 else x
+        ry, _ = O.gdn_conv(xs, w, st, ldx=C + pad)
+        if bf16:
+            assert close_16(host(y2, np.uint16), O.f2bf(ry), 'bf16')
+            assert bits_equal(host(q2, np.uint16), O.f2bf(O.gdn_l2(O.bf2f(host(y2, np.uint16)), T, heads, 128, 1e-6, ldx=C)))   # exact from the stored y on
+        else:
+            assert close_fp32(host(y2), ry)
+            assert bits_equal(host(q2), O.gdn_l2(host(y2), T, heads, 128, 1e-6, ldx=C))
+
+
+def test_gdn_conv_l2_refuses_shapes_it_does_not_cover():
+    L = camx(); z = dev(np.zeros(1024, np.float32))
+    p = lambda t: C.c_void_p(t.data_ptr())
+    assert L.camx_gdn_conv_l2(p(z), p(z), p(z), p(z), p(z), I(200), I(1), I(200), I(200), I(1), F(RS), I(0), stream()) == 1      # C % 128
+    assert L.camx_gdn_conv_l2(p(z), p(z), p(z), p(z), p(z), I(256), I(1), I(256), I(256), I(3), F(RS), I(0), stream()) == 1      # more heads than channels
+    assert L.camx_gdn_conv_l2(p(z), p(z), p(z), p(z), NULL, I(256), I(1), I(256), I(256), I(1), F(RS), I(0), stream()) == 1     # no qk
+
+
+@pytest.mark.parametrize('C_,T,heads', [(10240, 16, 32), (256, 4, 2), (128, 1, 1), (1024, 7, 5)])
+def test_op_gdn_conv_l2_equals_the_two_tape_ops(C_, T, heads):
+    rng = np.random.default_rng(C_ + T)
+    w = rng.standard_normal((C_, 4)).astype(np.float32); st0 = rng.standard_normal((C_, 3)).astype(np.float32)
+    junk = rng.standard_normal((T, C_)).astype(np.float32)
+    wd = dev(w)
+    s1, s2 = dev(st0), dev(st0); xp1, xp2 = dev(junk), dev(junk)
+    m = 0
+    for step in range(3):                                           # three passes; the second and third commit m tokens of the one before
+        x = outliers(rng, (T, C_)); xd = dev(x)
+        par = dev(np.array([7, m, 0, 0], np.int32))
+        ya = dev(np.zeros((T, C_), np.float32)); qa = dev(np.zeros((T * heads, 128), np.float32))
+        call('camx_op_gdn_conv', ptr(wd), ptr(s1), ptr(xd), ptr(par), ptr(ya), ptr(xp1), I(C_), I(T))
+        call('camx_op_gdn_l2', ptr(ya), ptr(qa), I(heads), I(128), F(RS), I(C_), I(T))
+        yb = dev(np.full((T, C_), 3, np.float32)); qb = dev(np.full((T * heads, 128), 3, np.float32))
+        call('camx_op_gdn_conv_l2', ptr(wd), ptr(s2), ptr(xd), ptr(par), ptr(yb), ptr(xp2), ptr(qb), I(C_), I(T), I(heads), F(RS))
+        assert torch.equal(ya, yb) and torch.equal(qa, qb) and torch.equal(s1, s2) and torch.equal(xp1, xp2), f'pass {step}'
+        assert bits_equal(host(qb), O.gdn_l2(host(yb), T, heads, 128, 1e-6, ldx=C_))
+        m = int(rng.integers(0, T + 1))
+
+
+# ---- the dense Q8 line: QK-norm + partial rotary + Hadamard + Q8 blocks ---------------------------------------------------------------
+def _dense_q8_inputs(rng, T, nh, nkv):
+    q = outliers(rng, (T * nh, 512)); k = outliers(rng, (T, nkv * 256)); v = outliers(rng, (T, nkv * 256))
+    qn = (1 + 0.1 * rng.standard_normal(256)).astype(np.float32); kn = (1 + 0.1 * rng.standard_normal(256)).astype(np.float32)
+    return q, k, v, qn, kn
+
+
+def _dense_q8_separate(qd, kd, vd, qnd, knd, nh, nkv, nrot, ts, pos0, T, rows, fill=0xa5):
+    """the six launches of the reference's chain, through their own entry points"""
+    M = nkv * 256; rb = 2 * (M // 32) * 34
+    ko = dev(np.zeros((T * nkv, 256), np.float32)); qo = dev(np.zeros((T * nh, 256), np.float32)); vr = vd.clone()
+    cache = dev(np.full((rows, rb), fill, np.uint8)); err = dev(np.zeros(1, np.int32))
+    call('camx_pf_qk_nr', ptr(kd), I(256), I(nkv), ptr(knd), I(256), I(nrot), F(ts), F(1e-6), I(pos0), ptr(ko), I(T), I(0))
+    call('camx_pf_hadamard', ptr(ko), I(T * nkv), I(256), I(1))
+    call('camx_pf_hadamard', ptr(vr), I(T * M // 64), I(64), I(1))
+    call('camx_own_kv_q8_append', ptr(ko), I(M), ptr(vr), I(M), I(M), ptr(cache), I(pos0), I(rows), ptr(err), I(T))
+    call('camx_pf_qk_nr', ptr(qd), I(512), I(nh), ptr(qnd), I(256), I(nrot), F(ts), F(1e-6), I(pos0), ptr(qo), I(T), I(0))
+    call('camx_pf_hadamard', ptr(qo), I(T * nh), I(256), I(1))
+    return qo, cache, err
+
+
+@pytest.mark.parametrize('T,nh,nkv,nrot,pos0', [(16, 24, 4, 64, 40000), (1, 24, 4, 64, 65535), (3, 5, 3, 256, 7), (2, 1, 1, 16, 0), (4096, 24, 4, 64, 100), (700, 8, 2, 128, 60000)])
+def test_qk_nr_q8_equals_the_six_launches(T, nh, nkv, nrot, pos0):
+    rng = np.random.default_rng(1004 + T + nh)
+    q, k, v, qn, kn = _dense_q8_inputs(rng, T, nh, nkv)
+    ts = _theta(1e7, nrot); rows = pos0 + T + 3
+    qd, kd, vd, qnd, knd = (dev(a) for a in (q, k, v, qn, kn))
+    qo1, c1, e1 = _dense_q8_separate(qd, kd, vd, qnd, knd, nh, nkv, nrot, ts, pos0, T, rows)
+    M = nkv * 256; rb = 2 * (M // 32) * 34
+    for mode in ('host', 'device', 'array'):
+        qo2 = dev(np.full((T * nh, 256), 9, np.float32)); c2 = dev(np.full((rows, rb), 0xa5, np.uint8)); e2 = dev(np.zeros(1, np.int32))
+        pd = dev(np.array([pos0], np.int32)) if mode == 'device' else None
+        pa = dev((pos0 + np.arange(T)).astype(np.int32)) if mode == 'array' else None
+        call('camx_qk_nr_q8', ptr(qd), I(512), I(nh), ptr(kd), I(M), ptr(vd), I(M), I(nkv), ptr(qnd), ptr(knd), I(nrot), F(ts), F(1e-6),
+             I(pos0 if mode == 'host' else 0), ptr(pd), ptr(pa), ptr(qo2), ptr(c2), I(rows), ptr(e2), I(T))
+        assert torch.equal(qo1, qo2) and torch.equal(c1, c2) and int(host(e2)[0]) == int(host(e1)[0]) == 0, mode
+    assert torch.equal(vd, dev(v))                                  # the fused launch leaves v alone (the chain rotates it in place)
+    if T <= 16:                                                     # the oracle's composition: q within the rotary tolerance behind a Hadamard transform
+        rq, rc, rerr = O.qk_nr_q8(q, 512, nh, k, v, nkv, qn, kn, nrot, ts, 1e-6, pos0 + np.arange(T), np.full((rows, rb), 0xa5, np.uint8), rows)
+        assert rerr == 0 and close_fp32(host(qo2), rq, floor=HADAMARD_FLOOR)
+        got = host(c2).reshape(rows, rb)
+        assert bits_equal(got[:pos0], rc.reshape(rows, rb)[:pos0]) and bits_equal(got[pos0 + T:], rc.reshape(rows, rb)[pos0 + T:])    # rows outside the span untouched
+        assert bits_equal(got[:, M // 32 * 34:], rc.reshape(rows, rb)[:, M // 32 * 34:])          # V: no transcendental before the codec, exact
+        # K: exact from the fp32 rotary output on; take that from the separate kernel (held to the oracle by its own test)
+        ko = dev(np.zeros((T * nkv, 256), np.float32))
+        call('camx_pf_qk_nr', ptr(kd), I(256), I(nkv), ptr(knd), I(256), I(nrot), F(ts), F(1e-6), I(pos0), ptr(ko), I(T), I(0))
+        kb, ok = O.kv_q8_encode(O.hadamard_n(host(ko), 256).reshape(-1, 32))
+        assert ok.all() and bits_equal(got[pos0:pos0 + T, :M // 32 * 34], kb.reshape(T, -1))
+
+
+def test_qk_nr_q8_refusals():
+    rng = np.random.default_rng(5)
+    T, nh, nkv, nrot, rows = 6, 4, 2, 64, 10
+    q, k, v, qn, kn = _dense_q8_inputs(rng, T, nh, nkv)
+    v[1, 300] = np.inf                                              # one V block of token 1 is refused; its 34 bytes stay
+    k[2, 5] = np.nan                                                # a NaN in a k head poisons the whole head's 8 blocks (norm, then the transform)
+    ts = _theta(1e7, nrot); M = nkv * 256; rb = 2 * (M // 32) * 34
+    pos = np.array([3, 9, 0, 10, -1, 5], np.int32)                  # tokens 3 and 4 sit outside [0, 10)
+    qd, kd, vd, qnd, knd = (dev(a) for a in (q, k, v, qn, kn))
+    qo = dev(np.zeros((T * nh, 256), np.float32)); c = dev(np.full((rows, rb), 0xa5, np.uint8)); e = dev(np.zeros(1, np.int32))
+    call('camx_qk_nr_q8', ptr(qd), I(512), I(nh), ptr(kd), I(M), ptr(vd), I(M), I(nkv), ptr(qnd), ptr(knd), I(nrot), F(ts), F(1e-6), I(0), NULL, ptr(dev(pos)),
+         ptr(qo), ptr(c), I(rows), ptr(e), I(T))
+    rq, rc, rerr = O.qk_nr_q8(q, 512, nh, k, v, nkv, qn, kn, nrot, ts, 1e-6, pos, np.full((rows, rb), 0xa5, np.uint8), rows)
+    assert int(host(e)[0]) == rerr == 3
+    got = host(c).reshape(rows, rb); want = rc.reshape(rows, rb)
+    assert bits_equal(got[:, M // 32 * 34:], want[:, M // 32 * 34:])                                # V blocks, the refused one untouched
+    written = got[:, :M // 32 * 34] != 0xa5
+    assert not written[[1, 2, 4, 6, 7, 8]].any()                                                       # rows no token goes to
+    assert (got[0, :8 * 34] == 0xa5).all() and not (got[0, 8 * 34:M // 32 * 34] == 0xa5).all()       # token 2's first k head refused, its second written
+    assert close_fp32(host(qo), rq, floor=HADAMARD_FLOOR)                                              # every q row is written, also of the tokens outside
+
+
+@pytest.mark.parametrize('io', [0, 1])
+@pytest.mark.parametrize('T,nh,nkv,D,nrot', [(16, 24, 4, 256, 64), (1, 24, 4, 256, 64), (3, 5, 2, 128, 128), (2, 3, 1, 96, 32), (300, 8, 2, 256, 64)])
+def test_qk_nr_qk_equals_two_launches(T, nh, nkv, D, nrot, io):
+    rng = np.random.default_rng(T + nh + D)
+    qs, ks = 2 * D, D + (8 if D % 8 == 0 else 4)
+    xq = outliers(rng, (T * nh, qs)); xk = outliers(rng, (T * nkv, ks))
+    wq = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32); wk = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    ts = _theta(1e7, nrot); pos = rng.integers(0, 65536, T).astype(np.int32)
+    dt = np.uint16 if io else np.float32
+    xqd, xkd = dev(O.f2bf(xq) if io else xq), dev(O.f2bf(xk) if io else xk)
+    wqd, wkd, posd = dev(wq), dev(wk), dev(pos)
+    oq1 = dev(np.zeros((T * nh, D), dt)); ok1 = dev(np.zeros((T * nkv, D), dt))
+    call('camx_qk_nr_pos', ptr(xqd), I(qs), I(nh), ptr(wqd), I(D), I(nrot), F(ts), F(1e-6), ptr(posd), ptr(oq1), I(T), I(io))
+    call('camx_qk_nr_pos', ptr(xkd), I(ks), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6), ptr(posd), ptr(ok1), I(T), I(io))
+    oq2 = dev(np.full((T * nh, D), 5, dt)); ok2 = dev(np.full((T * nkv, D), 5, dt))
+    call('camx_qk_nr_qk', ptr(xqd), I(qs), I(nh), ptr(wqd), ptr(xkd), I(ks), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6), I(0), NULL, ptr(posd),
+         ptr(oq2), ptr(ok2), I(T), I(io))
+    assert torch.equal(oq1, oq2) and torch.equal(ok1, ok2)
+    # contiguous positions from a device word and from the host
+    p0 = 1234
+    call('camx_pf_qk_nr', ptr(xqd), I(qs), I(nh), ptr(wqd), I(D), I(nrot), F(ts), F(1e-6), I(p0), ptr(oq1), I(T), I(io))
+    call('camx_pf_qk_nr', ptr(xkd), I(ks), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6), I(p0), ptr(ok1), I(T), I(io))
+    for pd, ph in ((dev(np.array([p0], np.int32)), 0), (None, p0)):
+        call('camx_qk_nr_qk', ptr(xqd), I(qs), I(nh), ptr(wqd), ptr(xkd), I(ks), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6), I(ph), ptr(pd), NULL,
+             ptr(oq2), ptr(ok2), I(T), I(io))
+        assert torch.equal(oq1, oq2) and torch.equal(ok1, ok2)
+
+
+# ---- tape-shaped entry points: the position is a device word --------------------------------------------------------------------------
+@pytest.mark.parametrize('T,heads,D,nrot,stride', [(1, 24, 256, 64, 512), (16, 4, 256, 64, 256), (3, 5, 128, 128, 128), (2, 3, 96, 32, 100), (600, 8, 256, 64, 256)])
+def test_op_qk_nr_reads_its_position_on_the_device(T, heads, D, nrot, stride):
+    rng = np.random.default_rng(D + T)
+    x = outliers(rng, (T * heads, stride)); w = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32); ts = _theta(1e7, nrot)
+    xd, wd = dev(x), dev(w)
+    pd = dev(np.array([0], np.int32))
+    eb = int(np.array([1e-6], np.float32).view(np.int32)[0])
+    for p0 in (0, 777, 65000):
+        a = dev(np.zeros((T * heads, D), np.float32)); b = dev(np.ones((T * heads, D), np.float32))
+        call('camx_pf_qk_nr', ptr(xd), I(stride), I(heads), ptr(wd), I(D), I(nrot), F(ts), F(1e-6), I(p0), ptr(a), I(T), I(0))
+        pd.fill_(p0)
+        call('camx_op_qk_nr', ptr(xd), I(stride), I(heads), I(D), ptr(wd), ptr(pd), ptr(b), I(nrot), F(ts), I(eb), I(T))
+        assert torch.equal(a, b)
+    assert close_fp32(host(b), O.qk_nr(x, stride, heads, w, D, nrot, ts, 1e-6, 65000, T))
+
+
+@pytest.mark.parametrize('M,T', [(1024, 1), (512, 16), (64, 3), (512, 1100)])
+def test_op_kv_append_three_row_formats(M, T):
+    rng = np.random.default_rng(M + T)
+    k = outliers(rng, (T, M)); v = outliers(rng, (T, M)); kd, vd = dev(k), dev(v)
+    rows = T + 9; p0 = 5
+    pd = dev(np.array([p0], np.int32))
+    for work, entry, rbytes in ((0, 'camx_q35p_kv_append16', 4 * M), (1, 'camx_pf_kv_append', 2 * (M // 32) * 34), (2, 'camx_own_kv_q8_append', 2 * (M // 32) * 34)):
+        c1 = dev(np.full((rows, rbytes), 0x5a, np.uint8)); c2 = dev(np.full((rows, rbytes), 0x5a, np.uint8)); e1 = dev(np.zeros(1, np.int32)); e2 = dev(np.zeros(1, np.int32))
+        if work == 0: call(entry, ptr(kd), I(M), ptr(vd), I(M), ptr(c1), I(M), I(p0), I(rows), ptr(e1), I(T))
+        else: call(entry, ptr(kd), I(M), ptr(vd), I(M), I(M), ptr(c1), I(p0), I(rows), ptr(e1), I(T))
+        call('camx_op_kv_append', ptr(kd), ptr(vd), ptr(c2), ptr(pd), I(M), I(work), ptr(e2), I(rows), I(T))
+        assert torch.equal(c1, c2) and int(host(e1)[0]) == int(host(e2)[0]) == 0, work
+        assert (host(c2)[:p0] == 0x5a).all() and (host(c2)[p0 + T:] == 0x5a).all()
+        # a position word that runs the pass over the end of the cache: bit 1, the rows inside are written, nothing else
+        pd2 = dev(np.array([rows - 1], np.int32)); c3 = dev(np.full((rows, rbytes), 0x5a, np.uint8)); e3 = dev(np.zeros(1, np.int32))
+        call('camx_op_kv_append', ptr(kd), ptr(vd), ptr(c3), ptr(pd2), I(M), I(work), ptr(e3), I(rows), I(T))
+        assert int(host(e3)[0]) == (1 if T > 1 else 0) and (host(c3)[:rows - 1] == 0x5a).all() and bits_equal(host(c3)[rows - 1], host(c1)[p0])
+    # against the oracle's writers
+    c = dev(np.zeros((rows, 2 * (M // 32) * 34), np.uint8)); e = dev(np.zeros(1, np.int32))
+    call('camx_op_kv_append', ptr(kd), ptr(vd), ptr(c), ptr(pd), I(M), I(2), ptr(e), I(rows), I(T))
+    rc, rerr = O.kv_q8_append(k, M, v, M, M, np.zeros((rows, 2 * (M // 32) * 34), np.uint8), p0, T, rows=rows)
+    assert rerr == 0 and bits_equal(host(c).reshape(-1), rc.reshape(-1))
+
+
+def test_thin_tape_ops_equal_their_prefill_namesakes():
+    rng = np.random.default_rng(31)
+    x = outliers(rng, (64, 256)); xa, xb = dev(x), dev(x)
+    call('camx_pf_hadamard', ptr(xa), I(64), I(256), I(1)); call('camx_op_hadamard', ptr(xb), I(64), I(256), I(4))
+    assert torch.equal(xa, xb)
+    T, nh, D = 3, 24, 256
+    a = outliers(rng, (T * nh, D)); qg = outliers(rng, (T * nh, 2 * D)); ad, qgd = dev(a), dev(qg)
+    y1 = dev(np.zeros((T * nh, D), np.uint16)); y2 = dev(np.ones((T * nh, D), np.uint16))
+    call('camx_gate_mul', ptr(ad), ptr(qgd), ptr(y1), L64(a.size), I(D), I(2 * D), I(D), I(1))
+    call('camx_op_gate_mul16', ptr(ad), ptr(qgd), I(2 * D), I(D), ptr(y2), I(a.size), I(D))
+    assert torch.equal(y1, y2) and close_16(host(y2, np.uint16), O.gate_mul(a, qg, D, 2 * D, D, f16=True), 'f16')
+    g = outliers(rng, (6144,)); u = outliers(rng, (6144,)); gd, ud = dev(g), dev(u)
+    s1 = dev(np.zeros(6144, np.uint16)); s2 = dev(np.ones(6144, np.uint16))
+    call('camx_q3p_swiglu', ptr(gd), ptr(ud), ptr(s1), I(6144)); call('camx_op_own_swiglu16', ptr(gd), ptr(ud), ptr(s2), I(6144))
+    assert torch.equal(s1, s2)
+    xl = outliers(rng, (T, 10240)); l1 = dev(np.zeros((T * 32, 128), np.float32)); l2 = dev(np.ones((T * 32, 128), np.float32))
+    call('camx_pf_gdn_l2', ptr(dev(xl)), ptr(l1), I(32), I(128), I(10240), F(RS), I(T), I(0))
+    call('camx_op_gdn_l2', ptr(dev(xl)), ptr(l2), I(32), I(128), F(RS), I(10240), I(T))
+    assert torch.equal(l1, l2) and bits_equal(host(l2), O.gdn_l2(xl, T, 32, 128, 1e-6, ldx=10240))
+    xc = outliers(rng, (T, 32 * 128)); l3 = dev(np.ones((T * 32, 128), np.float32))
+    call('camx_op_gdn_l2', ptr(dev(xc)), ptr(l3), I(32), I(128), F(RS), I(0), I(T))            # x_stride 0: heads * dim
+    assert bits_equal(host(l3), O.gdn_l2(xc, T, 32, 128, 1e-6))
+
+
+@pytest.mark.parametrize('n,q8,yarn', [(1, 1, 0), (1, 0, 0), (7, 1, 1), (16, 0, 1), (2100, 1, 0), (2100, 0, 0)])
+def test_op_own_qk_rope_reads_its_position_on_the_device(n, q8, yarn):
+    rng = np.random.default_rng(n + q8)
+    nh, nkv = 32, 4; ldq = (nh + 2 * nkv) * 128; M = nkv * 128
+    from caminus_amd import rope as _rope
+    qkv = outliers(rng, (n, ldq)); par = qk_par(rng, yarn_table=_rope.yarn_table(128, 1e6, 4.0, 32768) if yarn else None)
+    rows = n + 40; p0 = 33
+    rbytes = 2 * (M // 32) * 34 if q8 else 4 * M
+    qd, pd = dev(qkv), dev(par)
+    q1 = dev(np.zeros((n, nh, 128), np.uint16)); c1 = dev(np.full((rows, rbytes), 0x11, np.uint8)); e1 = dev(np.zeros(1, np.int32))
+    if q8: call('camx_q3p_qk_rope_q8', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), I(p0), ptr(q1), ptr(c1), ptr(e1), I(n), I(yarn))
+    else: call('camx_q3p_qk_rope', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), I(p0), ptr(q1), ptr(c1), I(n), I(yarn))
+    pw = dev(np.array([p0], np.int32))
+    q2 = dev(np.ones((n, nh, 128), np.uint16)); c2 = dev(np.full((rows, rbytes), 0x11, np.uint8)); e2 = dev(np.zeros(1, np.int32))
+    call('camx_op_own_qk_rope', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), ptr(pw), ptr(q2), ptr(c2), I(rows), ptr(e2), I(n), I(yarn), I(q8))
+    assert torch.equal(q1, q2) and torch.equal(c1, c2) and int(host(e2)[0]) == 0
+    pw.fill_(rows - 1)                                              # the pass runs over the end of the cache: bit 1, q16 still written
+    c3 = dev(np.full((rows, rbytes), 0x11, np.uint8)); e3 = dev(np.zeros(1, np.int32)); q3 = dev(np.ones((n, nh, 128), np.uint16))
+    call('camx_op_own_qk_rope', ptr(qd), I(ldq), I(nh), I(nkv), ptr(pd), ptr(pw), ptr(q3), ptr(c3), I(rows), ptr(e3), I(n), I(yarn), I(q8))
+    assert int(host(e3)[0]) == (1 if n > 1 else 0) and (host(c3)[:rows - 1] == 0x11).all() and not (host(c3)[rows - 1] == 0x11).all()
+    assert not (host(q3) == 1).all(axis=-1).any()
+
+
+def test_pos0_forms_refuse_a_negative_position():
+    L = camx(); z = dev(np.zeros(4096 * 6, np.float32)); par = dev(qk_par(np.random.default_rng(1)))
+    p = lambda t: C.c_void_p(t.data_ptr())
+    for n in (1, 2048):
+        assert L.camx_q3p_qk_rope(p(z), I(768), I(4), I(1), p(par), I(-1), p(z), p(z), I(n), I(0), stream()) == 1
+        assert L.camx_q3p_qk_rope_q8(p(z), I(768), I(4), I(1), p(par), I(-1), p(z), p(z), p(z), I(n), I(0), stream()) == 1
+        assert L.camx_qk_rope_bf16(p(z), I(768), I(4), I(1), p(par), I(-5), p(z), p(z), I(n), I(0), stream()) == 1
+        assert L.camx_q3p_qk_rope(p(z), I(768), I(4), I(1), p(par), I(2 ** 31 - 3), p(z), p(z), I(n + 8), I(0), stream()) == 1
+    torch.cuda.synchronize()
+
+
+# ---- camx_init and a captured decode step whose position lives on the device ----------------------------------------------------------
+def test_init_then_graph_replays_at_three_positions():
+    from caminus_amd.device import lib as _lib
+    L = camx()
+    _lib.check(L.camx_init(stream())); _lib.check(L.camx_init(stream()))              # idempotent
+    rng = np.random.default_rng(9)
+    nh, nkv, T, rows = 24, 4, 1, 64
+    q, k, v, qn, kn = _dense_q8_inputs(rng, T, nh, nkv)
+    M = nkv * 256; rb = 2 * (M // 32) * 34; ts = _theta(1e7, 64)
+    Cc, heads = 1024, 4
+    xc = outliers(rng, (T, Cc)); wc = rng.standard_normal((Cc, 4)).astype(np.float32); st0 = rng.standard_normal((Cc, 3)).astype(np.float32)
+    gu = O.f2bf(outliers(rng, (T, 2 * 512)))
+    qd, kd, vd, qnd, knd, xcd, wcd, gud = (dev(a) for a in (q, k, v, qn, kn, xc, wc, gu))
+    pos = dev(np.array([0], np.int32)); par = dev(np.array([0, 0, 0, 0], np.int32))
+    qo = dev(np.zeros((T * nh, 256), np.float32)); cache = dev(np.zeros((rows, rb), np.uint8)); err = dev(np.zeros(1, np.int32))
+    std = dev(st0); yc = dev(np.zeros((T, Cc), np.float32)); xp = dev(np.zeros((T, Cc), np.float32)); qk = dev(np.zeros((T * heads, 128), np.float32))
+    act = dev(np.zeros((T, 512), np.uint16)); mmq = dev(np.zeros(4 * T * 144, np.uint8))
+
+    def launch_all():
+        s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        p = lambda t: C.c_void_p(t.data_ptr())
+        _lib.check(L.camx_qk_nr_q8(p(qd), I(512), I(nh), p(kd), I(M), p(vd), I(M), I(nkv), p(qnd), p(knd), I(64), F(ts), F(1e-6), I(0), p(pos), NULL, p(qo), p(cache), I(rows), p(err), I(T), s))
+        _lib.check(L.camx_op_gdn_conv_l2(p(wcd), p(std), p(xcd), p(par), p(yc), p(xp), p(qk), I(Cc), I(T), I(heads), F(RS), s))
+        _lib.check(L.camx_swiglu_mmq_q8_1(p(gud), L64(1024), L64(512), p(mmq), p(act), I(T), I(1), s))     # a table reader: no fill, no wait after camx_init
+
+    def reset():
+        cache.zero_(); err.zero_(); std.copy_(dev(st0))
+        for t in (qo, yc, xp, qk, act, mmq): t.zero_()
+        torch.cuda.synchronize()
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return [host(t).copy() for t in (qo, cache, err, std, yc, xp, qk, act, mmq)]
+
+    eager = {}
+    for p0 in (5, 40, 63):
+        reset(); pos.fill_(p0); launch_all(); eager[p0] = snapshot()
+        assert eager[p0][1][p0].any() and not eager[p0][1][:p0].any()
+    reset(); pos.fill_(5)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch_all()
+    for p0 in (40, 5, 63, 40):                                      # one capture, replayed after the position word changed
+        reset(); pos.fill_(p0)
+        torch.zeros(1 << 20, device=qo.device).add_(1.0)
+        g.replay()
+        for a, b in zip(snapshot(), eager[p0]):
+            assert bits_equal(a, b), f'replay at {p0}'
+
+
+def test_tape_ops_object_and_f16_module():
+    """the host mirror: TapeOps' methods (the reference's K3 op methods, launched at once) and Module('prefill_attn_f16').pf_kv_append"""
+    from caminus_amd.device.hip import LOADED, Module
+    from caminus_amd.engine.k3 import TapeOps
+    rng = np.random.default_rng(12)
+    T, nh, nkv = 2, 4, 1
+    M = nkv * 256; rows = 16
+    q, k, v, qn, kn = _dense_q8_inputs(rng, T, nh, nkv)
+    qd, kd, vd, qnd, knd = (dev(a) for a in (q, k, v, qn, kn))
+    err = dev(np.zeros(1, np.int32)); pos = dev(np.array([3], np.int32))
+    ops = TapeOps(T=T, kv_q8_dense=True, kv_error=err)
+    ts = _theta(1e7, 64)
+    ko = dev(np.zeros((T * nkv, 256), np.float32)); vr = vd.clone(); qo = dev(np.zeros((T * nh, 256), np.float32))
+    cache = torch.full((rows * 2 * (M // 32) * 34,), 0x22, dtype=torch.uint8, device=qd.device)
+    i0 = ops.qk_nr(kd, 256, nkv, 256, knd, pos, ko, 64, ts, 1e-6)
+    ops.hadamard(ko, 256); ops.hadamard(vr, 64)
+    ops.kv_append(ko, vr, cache, pos, q8=True)
+    ops.qk_nr(qd, 512, nh, 256, qnd, pos, qo, 64, ts, 1e-6); i5 = ops.hadamard(qo, 256)
+    assert i5 == i0 + 5
+    qo2 = dev(np.zeros((T * nh, 256), np.float32)); cache2 = torch.full_like(cache, 0x22)
+    ops.qk_nr_q8(qd, 512, nh, kd, vd, nkv, qnd, knd, pos, qo2, cache2, 64, ts, 1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(qo, qo2) and torch.equal(cache, cache2) and int(host(err)[0]) == 0
+    with pytest.raises(ValueError): ops.hadamard(qo, 256, rows_per_task=0)
+    with pytest.raises(ValueError): TapeOps(T=1, kv_q8_dense=True)
+    # the fp16-cache build of the prefill attention module
+    m = Module('prefill_attn_f16'); assert 'prefill_attn_f16' in LOADED
+    c16 = torch.zeros((rows, 2 * M), dtype=torch.float16, device=qd.device); e16 = dev(np.zeros(1, np.int32))
+    m.pf_kv_append((T,), (256,), kd, I(M), vd, I(M), I(M), c16, I(3), I(rows), e16)
+    torch.cuda.synchronize()
+    want, werr = O.kv_append16(k, v, M, np.zeros((rows, 2 * M), np.uint16), 3)
+    assert werr == 0 and bits_equal(host(c16.view(torch.int16), np.uint16), want)
