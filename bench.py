@@ -211,6 +211,35 @@ def extra_opsets(B):
     l2o = torch.empty((T4 * 32, 128), dtype=torch.bfloat16, device=B.dev)
     out.append(('c4_l2norm_qk', T4 * 32 * 128 * 4,
                 lambda: B.call('camx_pf_gdn_l2', _p(yc), _p(l2o), I(32), I(128), I(Cc), F(1e-6 / 128), I(T4), I(1))))
+    # the same op-sets as the reference's engine chains them (python/caminus/engine/q35_dense.py:399-400, 408-418), one launch each
+    l2f = torch.empty((T4 * 32, 128), dtype=torch.bfloat16, device=B.dev); ycf = torch.empty((T4, Cc), dtype=torch.bfloat16, device=B.dev)
+    out.append(('c4_conv4_silu_l2_one_launch', T4 * Cc * 4 + Cc * 16 + Cc * 12 + T4 * 32 * 128 * 2,
+                lambda: B.call('camx_gdn_conv_l2', _p(xc), _p(wc), _p(st), _p(ycf), _p(l2f), I(Cc), I(T4), I(Cc), I(Cc), I(32), F(1e-6 / 128), I(1))))
+    kx = B.acts((T4 * 4, D4), torch.bfloat16, 47); wk4 = B.gamma(D4, 48); ok4 = torch.empty((T4 * 4, D4), dtype=torch.bfloat16, device=B.dev)
+    out.append(('c4_qk_nr_partial_rotary_k', T4 * 4 * D4 * 4 + D4 * 4,
+                lambda: B.call('camx_qk_nr_pos', _p(kx), I(D4), I(4), _p(wk4), I(D4), I(64), F(ts7), F(1e-6), _p(pos), _p(ok4), I(T4), I(1))))
+    out.append(('c4_qk_nr_partial_rotary_q_and_k_one_launch', T4 * 28 * D4 * 4 + 2 * D4 * 4,
+                lambda: B.call('camx_qk_nr_qk', _p(qg), I(2 * D4), I(24), _p(w4), _p(kx), I(D4), I(4), _p(wk4), I(D4), I(64), F(ts7), F(1e-6), I(0), NULL, _p(pos),
+                               _p(o4), _p(ok4), I(T4), I(1))))
+    # the dense Q8 line of the same layer shape (fp32, as the reference's decode tape runs it): six launches, and the one that replaces them
+    M4 = 4 * D4; rows4 = 65536 + T4; rb4 = 2 * (M4 // 32) * 34
+    q32 = B.acts((T4 * 24, 2 * D4), torch.float32, 71); k32 = B.acts((T4, M4), torch.float32, 72); v32 = B.acts((T4, M4), torch.float32, 73)
+    ko32 = torch.empty((T4 * 4, D4), device=B.dev); qo32 = torch.empty((T4 * 24, D4), device=B.dev); vr32 = v32.clone()
+    cache4 = torch.zeros(rows4 * rb4, dtype=torch.uint8, device=B.dev); err4 = torch.zeros(1, dtype=torch.int32, device=B.dev)
+    posw = torch.tensor([40000], dtype=torch.int32, device=B.dev)
+    def dense_q8_six():
+        B.call('camx_pf_qk_nr', _p(k32), I(D4), I(4), _p(wk4), I(D4), I(64), F(ts7), F(1e-6), I(40000), _p(ko32), I(T4), I(0))
+        B.call('camx_pf_hadamard', _p(ko32), I(T4 * 4), I(256), I(1))
+        B.call('camx_pf_hadamard', _p(vr32), I(T4 * M4 // 64), I(64), I(1))
+        B.call('camx_own_kv_q8_append', _p(ko32), I(M4), _p(vr32), I(M4), I(M4), _p(cache4), I(40000), I(rows4), _p(err4), I(T4))
+        B.call('camx_pf_qk_nr', _p(q32), I(2 * D4), I(24), _p(w4), I(D4), I(64), F(ts7), F(1e-6), I(40000), _p(qo32), I(T4), I(0))
+        B.call('camx_pf_hadamard', _p(qo32), I(T4 * 24), I(256), I(1))
+    by4 = T4 * (24 + 4 + 4) * D4 * 4 + T4 * 24 * D4 * 4 + T4 * rb4 + 2 * D4 * 4
+    out.append(('c4_dense_q8_qk_nr_hadamard_append_six_launches', by4, dense_q8_six))
+    out.append(('c4_dense_q8_qk_nr_hadamard_append_one_launch', by4,
+                lambda: B.call('camx_qk_nr_q8', _p(q32), I(2 * D4), I(24), _p(k32), I(M4), _p(v32), I(M4), I(4), _p(w4), _p(wk4), I(64), F(ts7), F(1e-6), I(0), _p(posw), NULL,
+                               _p(qo32), _p(cache4), I(rows4), _p(err4), I(T4))))
+    out.append(('_keep4', 0, [l2f, ycf, kx, wk4, ok4, q32, k32, v32, ko32, qo32, vr32, cache4, err4, posw]))
     # batched decode: 256 sequences, Q8 KV codec into a paged cache
     S5 = 256
     x5 = B.acts((S5, N), torch.float32, 51); d5 = B.acts((S5, 1, N), torch.float32, 52)
@@ -709,7 +738,7 @@ def main():
         ops = {}
         sets = extra_opsets(B)
         for name, by, fn in sets:
-            if name == '_keep': continue
+            if name.startswith('_keep'): continue
             med, mean = B.time_launch(fn, reps=50, warm=10, flush=True)
             med_hot, _ = B.time_launch(fn, reps=50, warm=10, flush=False)
             q0, q1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -721,12 +750,19 @@ def main():
         # the only per-op times the reference publishes for this path (another GPU: RX 7900 XTX, docs/specs/spec-prefill-cache.md:276)
         for k, ref_us in (('hc_post_rms_2048x4x2560_bf16_scale', 466.0), ('hc_mean_2048x4x2560_from_residual', 267.0)):
             if k in ops: ops[k]['reference_rx7900xtx_us'] = ref_us
+        # a fused launch beside the launches it replaces
+        for fused, parts in (('c4_conv4_silu_l2_one_launch', ('c4_conv4_silu', 'c4_l2norm_qk')),
+                             ('c4_qk_nr_partial_rotary_q_and_k_one_launch', ('c4_qk_nr_partial_rotary_q', 'c4_qk_nr_partial_rotary_k')),
+                             ('c4_dense_q8_qk_nr_hadamard_append_one_launch', ('c4_dense_q8_qk_nr_hadamard_append_six_launches',))):
+            if fused in ops:
+                for key in ('us', 'us_cache_hot', 'us_queued'):
+                    ops[fused][key + '_of_the_launches_it_replaces'] = round(sum(ops[p][key] for p in parts), 2)
         out['opsets'] = ops
         # the launch-bound op-sets as they would run in a decode loop: each shape's launches captured once into a HIP graph
         # and replayed (every entry point is stream-ordered, allocates nothing and keeps no host state per call)
         graphs = {}
         for prefix in ('c1_', 'c4_', 'c5_'):
-            fns = [fn for name, _, fn in sets if name.startswith(prefix)]
+            fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'six_launches' not in name and not name.endswith('_k')]
             for fn in fns: fn()
             torch.cuda.synchronize()
             gr = torch.cuda.CUDAGraph()

@@ -182,7 +182,8 @@ SYMBOLS = {
     'q3m_prefill_kvq8_yarn': _q3m(True, True), 'q35_prefill': _Q35,
     'prefill_glue': _glue(2560), 'prefill_glue_q35': _glue(2048), 'prefill_glue_q35d': _glue(5120),
     'prefill_attn': _ATTN, 'prefill_attn_q35': _ATTN, 'prefill_attn_q35d': _ATTN,
-    'prefill_attn_f16': dict(_ATTN, pf_kv_append=('camx_q35p_kv_append16', _pf_kv_append16)),      # fp16 cache rows (python/caminus/prefill/attn.py:150-155) 'prefill_gdn': _GDN, 'prefill_gdn_q35': _GDN_SILU,
+    'prefill_attn_f16': dict(_ATTN, pf_kv_append=('camx_q35p_kv_append16', _pf_kv_append16)),      # fp16 cache rows (python/caminus/prefill/attn.py:150-155)
+    'prefill_gdn': _GDN, 'prefill_gdn_q35': _GDN_SILU,
     'prefill_mmq_glue': {},      # its quantizers are template instances in the reference: caminus_amd.prefill.mmq binds them
     'camx': {},                  # direct access to every C entry point by its own name (Module('camx').camx_...)
 }

@@ -248,7 +248,8 @@ int camx_q3p_emb(const uint8_t * W, int rb, int vocab, const int32_t * toks, flo
 int camx_emb_gather(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, int N, int n, int fmt,
                     camx_stream_t stream);
 /* Gather + dequant + (x += d) + RMSNorm * nw with fp32 / fp16 / q8_1 copies of the normed row in one pass per row
- * (q3p_emb followed by q3p_add_rms16 and OP_RMS_MUL's q8_1 copy). xbf = bf16 of the gathered row; x = the residual row. */
+ * (q3p_emb followed by q3p_add_rms16 and OP_RMS_MUL's q8_1 copy). xbf = bf16 of the gathered row; x = the residual row. The addend d must
+ * not overlap x (up to 256 rows a row's slabs are written by four waves that each read the whole addend row). */
 int camx_emb_gather_add_rms(const uint8_t * W, long rb, int vocab, const int32_t * toks, float * x, uint16_t * xbf, const float * d,
                             const float * nw, float eps, float * h, uint16_t * h16, void * q8, int N, int n, int fmt,
                             camx_stream_t stream);

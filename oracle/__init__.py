@@ -539,11 +539,13 @@ def actq_bwd(x, g, clip=1.0, qmax=7, bf16=False):
     lib().orc_actq_bwd(_p(x), I(int(bf16)), _p(g), _p(dx), I(M), I(K), F(clip), I(qmax)); return dx
 
 
-def silu_mul_actq_bwd(gu, g, clip=1.0, qmax=7):
-    """-> dgu bf16 bits [M, 2F]"""
+def silu_mul_actq_bwd(gu, g, clip=1.0, qmax=7, table=False):
+    """-> dgu bf16 bits [M, 2F]. table: the derivative's sigmoid from the correctly rounded single-precision exponential (the definition of
+    the HIP kernel's table) instead of the C library's expf"""
     gu = _c(gu, np.uint16); M, F2 = gu.shape
     dgu = np.empty((M, F2), np.uint16); g = _c(g, np.uint16)
-    lib().orc_silu_mul_actq_bwd(_p(gu), I(F2), I(F2 // 2), _p(g), _p(dgu), I(M), F(clip), I(qmax)); return dgu
+    fn = lib().orc_silu_mul_actq_bwd_tab if table else lib().orc_silu_mul_actq_bwd
+    fn(_p(gu), I(F2), I(F2 // 2), _p(g), _p(dgu), I(M), F(clip), I(qmax)); return dgu
 
 
 def block_entry_bwd(x, nw, rstd, wab, dy, dab, clip=1.0, qmax=7):

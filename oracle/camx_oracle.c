@@ -917,8 +917,12 @@ ORC_API void orc_actq_bwd(const void * x, int is_bf16, const uint16_t * g, void 
         for (int k = 0; k < K; k++) { if (is_bf16) ((uint16_t *)dx)[(size_t)r * K + k] = orc_f2bf(out[k]); else ((float *)dx)[(size_t)r * K + k] = out[k]; }
     }
 }
-/* silu_mul_actq_bwd (actq.hip:140-153, 311-314): dgu [M][2F] = [dg | du] */
-ORC_API void orc_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, int M, float clip, int qmax) {
+/* silu_mul_actq_bwd (actq.hip:140-153, 311-314): dgu [M][2F] = [dg | du]. tab = 0: the sigmoid of silu's derivative from the C library's
+ * expf, as the reference's source reads. tab = 1: from ex = (float)exp(-(double)g), the correctly rounded single-precision exponential: the
+ * definition of the 65536-entry table the HIP kernel reads (one entry per bf16 gate), restated here so that dg can be compared bit for bit.
+ * The two differ where glibc's expf is not correctly rounded (rare; at most one bf16 step in dg). The reference holds no fixture for this
+ * gradient: parity of dg with the reference's own device expf is unpinned beyond that step. */
+static void silu_mul_actq_bwd_impl(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, int M, float clip, int qmax, int tab) {
 #pragma omp parallel for schedule(static)
     for (int r = 0; r < M; r++) {
         float src[8192], out[8192];
@@ -927,11 +931,18 @@ ORC_API void orc_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uin
         actq_bwd_row(src, g + (size_t)r * F, F, clip, qmax, out);
         for (int k = 0; k < F; k++) {
             const float dact = out[k], gg = orc_bf2f(row[k]), uu = orc_bf2f(row[F + k]);
-            const float ex = expf(-gg), sl = rbf(gg / (1.0f + ex)), sig = 1.0f / (1.0f + ex), ds = rbf(dact * uu);
+            const float ex = expf(-gg), sl = rbf(gg / (1.0f + ex)), ds = rbf(dact * uu);
+            const float sig = 1.0f / (1.0f + (tab ? (float)exp(-(double)gg) : ex));
             dgu[(size_t)r * 2 * F + k] = orc_f2bf(ds * sig * fmaf(gg, 1.0f - sig, 1.0f));
             dgu[(size_t)r * 2 * F + F + k] = orc_f2bf(dact * sl);
         }
     }
+}
+ORC_API void orc_silu_mul_actq_bwd(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, int M, float clip, int qmax) {
+    silu_mul_actq_bwd_impl(gu, ld, F, g, dgu, M, clip, qmax, 0);
+}
+ORC_API void orc_silu_mul_actq_bwd_tab(const uint16_t * gu, int ld, int F, const uint16_t * g, uint16_t * dgu, int M, float clip, int qmax) {
+    silu_mul_actq_bwd_impl(gu, ld, F, g, dgu, M, clip, qmax, 1);
 }
 /* block_entry_bwd (actq.hip:275-304): thread t = k % 256 adds dot terms in k order with fmaf; 8 x 32 tree; d <= 1024 */
 ORC_API void orc_block_entry_bwd(const float * x, const float * nw, const float * rstd_in, const uint16_t * wab, int nab, const uint16_t * dy,

@@ -147,6 +147,7 @@ def test_silu_mul_actq_bwd(M, Fh, ld):
     got = host(dgu, np.uint16)
     assert close_16(got, want, 'bf16')
     assert (got == want).mean() > 0.99
+    assert bits_equal(got, O.silu_mul_actq_bwd(gu, g, table=True))        # bit for bit against the table's own definition (every gate here is finite)
 
 
 @pytest.mark.parametrize('M,Fh', [(6, 1024), (1200, 256), (5, 2304)])

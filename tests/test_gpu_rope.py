@@ -5,6 +5,7 @@ Q8 rows: bit-exact bytes of the oracle's codec applied to the fp16 row the F16 f
 where the reference places the stage boundary (tests/engine/test_q3m_kvq8_atts.py:2-7)."""
 import numpy as np
 import pytest
+import torch
 
 import oracle as O
 from caminus_amd import rope
@@ -217,3 +218,33 @@ def test_prefill_sized_rope_equals_the_small_batch_kernel(nh, nkv, yarn):
     blocks = wide[3].reshape(rows, 2 * M // 32, 34)
     assert (blocks[pos0 + 7, 0:4] == 0xa5).all() and (blocks[pos0 + 9, M // 32 + 1] == 0xa5).all()    # the rotation spreads the infinity over its head
     assert not (blocks[pos0 + 7, 4:] == 0xa5).all(1).any() and not (blocks[pos0 + 9, M // 32] == 0xa5).all() and not (blocks[pos0 + 8] == 0xa5).all(1).any()
+
+
+@pytest.mark.parametrize('q8', [0, 1])
+def test_qk_rope_unpaged_position_array_refusals_at_chunk_size(q8):
+    """the same refusals in the kernel that takes 2048 and more rows with a position array (four tokens per workgroup): a position past
+    the cache and a negative one set bit 1 and leave their rows unwritten, q16 is written for every token, every other row carries the
+    bytes the small-batch kernel writes for it, and nothing else is touched"""
+    rng = np.random.default_rng(2100 + q8)
+    nh, nkv, n, rows = 32, 4, 2100, 2200
+    par = qk_par(rng); M = nkv * 128; rb = 2 * (M // 32) * 34
+    qkv = outliers(rng, (n, (nh + 2 * nkv) * 128))
+    pos = rng.permutation(rows)[:n].astype(np.int32)
+    pos[100] = rows; pos[1500] = -3
+    fill = np.full((rows, rb if q8 else 2 * M), 0xa5 if q8 else 0xa5a5, np.uint8 if q8 else np.uint16)
+    pd, qd, posd = dev(par), dev(qkv), dev(pos)
+    ca = dev(fill); ea = dev(np.zeros(1, np.int32)); qa = dev(np.zeros((n, nh, 128), np.uint16))
+    call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(qa), ptr(ca), ptr(ea), NULL, I(0), I(0), I(rows), I(n), I(0), I(q8))
+    cb = dev(fill); eb = dev(np.zeros(1, np.int32)); qb = dev(np.zeros((n, nh, 128), np.uint16))
+    for lo in range(0, n, 150):                                           # the same tokens through the small-batch kernel
+        m = min(150, n - lo)
+        call('camx_qk_rope_paged', ptr(qd[lo:]), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd[lo:]), ptr(qb[lo:]), ptr(cb), ptr(eb), NULL, I(0), I(0), I(rows), I(m), I(0), I(q8))
+    assert int(host(ea)[0]) == int(host(eb)[0]) == 1
+    assert torch.equal(ca, cb) and torch.equal(qa, qb)
+    got = host(ca, None if q8 else np.uint16)
+    written = np.zeros(rows, bool); written[pos[(pos >= 0) & (pos < rows)]] = True
+    assert (got[~written] == (0xa5 if q8 else 0xa5a5)).all() and not (got[written] == (0xa5 if q8 else 0xa5a5)).all(axis=1).any()
+    q = host(qa, np.uint16)
+    assert q[100].any() and q[1500].any()
+    rq, _, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos, q8=bool(q8), cache=fill, n_pages=rows)
+    assert oerr == 1 and close_16(q, rq, 'f16', floor=HADAMARD_FLOOR if q8 else None)
