@@ -436,7 +436,9 @@ __global__ void __launch_bounds__(256) qk_rope_wide_tokens(RopeArgs a) {
 // burst of reads per wave, then its arithmetic, then one burst of writes), the norm weights and the tokens' cos / sin rows in LDS.
 // The operations and their order are qk_rope_wide_tokens': same bits. F32IN: fp32 rows (two 128-bit loads per lane and step) of up to 48
 // heads, the last step possibly short (16384 tokens x 40 heads: 92 -> 86.5 us against the pipelined kernel).
-template <bool YARN, int STEPS, int TPW, bool F32IN = false, bool Q8 = false>
+// GEN: any addressing the token kernels take (a position per token or a device-resident base, a page table, a bound on the cache's rows),
+// with their refusals: a row that is refused is not written and sets its error bit; q16 is written for every token.
+template <bool YARN, int STEPS, int TPW, bool F32IN = false, bool Q8 = false, bool GEN = false>
 __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     __shared__ __attribute__((aligned(16))) float rc[TPW][64];
     __shared__ __attribute__((aligned(16))) float rs[TPW][64];
@@ -465,7 +467,8 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     }
     nrm[tid] = a.par[tid];
     if (wave < TPW) {                                                       // wave w: the cos / sin row of token t0 + w
-        const int pos = a.pos0 + (t0 + wave < a.n ? t0 + wave : a.n - 1);
+        const int tw = t0 + wave < a.n ? t0 + wave : a.n - 1;
+        const int pos = GEN ? rope_pos(a, tw) : a.pos0 + tw;
         float c, sn;
         if (YARN) { const float theta = (float)pos * a.par[258 + lane], ms = a.par[322]; c = cosf(theta) * ms; sn = sinf(theta) * ms; }
         else { const float theta = (float)pos * rope_freq(a.par[256], lane); c = cosf(theta); sn = sinf(theta); }
@@ -477,8 +480,20 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     for (int ti = 0; ti < TPW; ti++) {
         const int t = t0 + ti;
         if (t >= a.n) break;
-        const int pos = a.pos0 + t;
-        uint16_t * cw = (uint16_t *)a.cache + (size_t)pos * 2 * M;
+        const int pos = GEN ? rope_pos(a, t) : a.pos0 + t;
+        bool span = true;                                                   // (wave-uniform) the token's cache row may be written
+        size_t rowi = (size_t)pos;
+        if (GEN) {
+            span = pos >= 0 && (a.page_table ? pos / a.page < a.pt_stride : (a.rows == 0 || pos < a.rows));
+            if (!span) { if (a.err && tid == 0) atomicOr(a.err, 1); }
+            else if (a.page_table) {
+                const int pg = a.page_table[(size_t)t * a.pt_stride + pos / a.page];
+                if (pg < 0 || pg >= a.n_pages) { if (tid == 0) atomicOr(a.err, 8); span = false; }
+                else rowi = (size_t)pg * a.page + (size_t)(pos % a.page);
+            }
+            if (!span) rowi = 0;
+        }
+        uint16_t * cw = (uint16_t *)a.cache + rowi * 2 * M;
         uint16_t * qw = a.q16 + (size_t)t * a.nh * 128;
         const int j0 = 8 * (l16 & 7);
         f32x4 c4[2], s4[2];
@@ -540,7 +555,7 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
             if constexpr (Q8) {                                             // the Q8 rows, as in qk_rope_wide_tokens (a wave's four heads are of one kind)
                 const bool q_heads = h0 < a.nh, v_heads = h0 >= nqk;
                 const int h = h0 + hq;
-                uint8_t * cwb = (uint8_t *)a.cache + (size_t)pos * (2 * (M / 32) * 34);
+                uint8_t * cwb = (uint8_t *)a.cache + rowi * (2 * (M / 32) * 34);
                 float v8[8];
                 if (v_heads) {
 #pragma unroll
@@ -561,14 +576,14 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
                     RSTORE((u32x4 *)(qw + (size_t)h * 128 + 8 * l16), out);
                 } else {
                     const size_t b = v_heads ? M / 32 + (size_t)(h - nqk) * 4 + (l16 >> 2) : (size_t)(h - a.nh) * 4 + (l16 >> 2);
-                    kv_q8_emit_w8(v8, cwb + b * 34, l16 & 3, a.err, true);
+                    kv_q8_emit_w8(v8, cwb + b * 34, l16 & 3, a.err, span);
                 }
                 continue;
             }
             if (h0 >= nqk) {                                                // V heads: fp16 copy
 #pragma unroll
                 for (int p = 0; p < 4; p++) out[p] = pack_f16x2(x[2 * p], x[2 * p + 1]);
-                RSTORE((u32x4 *)(cw + M + (size_t)(h0 - nqk) * 128 + lo), out);
+                if (!GEN || span) RSTORE((u32x4 *)(cw + M + (size_t)(h0 - nqk) * 128 + lo), out);
                 continue;
             }
             const bool isq = h0 < a.nh;
@@ -582,7 +597,7 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
             }
 #pragma unroll
             for (int p = 0; p < 4; p++) out[p] = pack_f16x2(y[2 * p], y[2 * p + 1]);
-            RSTORE((u32x4 *)((isq ? qw + (size_t)h0 * 128 : cw + (size_t)(h0 - a.nh) * 128) + lo), out);
+            if (!GEN || isq || span) RSTORE((u32x4 *)((isq ? qw + (size_t)h0 * 128 : cw + (size_t)(h0 - a.nh) * 128) + lo), out);
         }
     }
 }
@@ -590,8 +605,16 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
 template <bool YARN, int TPW, bool Q8>
 static bool rope_chunk_launch_f32(const RopeArgs & a, hipStream_t st) {
     const int items = a.nh + 2 * a.nkv;
-    if (a.pos || a.posb || a.page_table || items > 48 || (a.nh & 3) || (a.nkv & 3) || (Q8 && (a.pos0 < 0 || a.rows != 0))) return false;
+    if (items > 48 || (a.nh & 3) || (a.nkv & 3)) return false;
     const dim3 grid((a.n + TPW - 1) / TPW), block(256);
+    if (a.pos || a.posb || a.page_table || a.rows != 0) {                   // a batch of sequences, each at its own position and row
+        switch ((items + 15) >> 4) {
+        case 1: qk_rope_chunk<YARN, 1, TPW, true, Q8, true><<<grid, block, 0, st>>>(a); break;
+        case 2: qk_rope_chunk<YARN, 2, TPW, true, Q8, true><<<grid, block, 0, st>>>(a); break;
+        default: qk_rope_chunk<YARN, 3, TPW, true, Q8, true><<<grid, block, 0, st>>>(a); break;
+        }
+        return true;
+    }
     switch ((items + 15) >> 4) {
     case 1: qk_rope_chunk<YARN, 1, TPW, true, Q8><<<grid, block, 0, st>>>(a); break;
     case 2: qk_rope_chunk<YARN, 2, TPW, true, Q8><<<grid, block, 0, st>>>(a); break;
@@ -1137,8 +1160,12 @@ static void rope_dispatch(const RopeArgs & a, int yarn, bool q8, hipStream_t st)
 static int rope_launch(const RopeArgs & a, int yarn, bool q8, hipStream_t st, bool bf16in = false) {
     if (rope_check(a, q8, bf16in)) return CAMX_EINVAL;
     if (a.n == 0) return CAMX_OK;
-    const bool wide = (!q8 || !bf16in) && !a.page_table && (a.ldq & (bf16in ? 7 : 3)) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 &&
-                      ((uintptr_t)a.cache & 15) == 0;
+    const bool aligned = (a.ldq & (bf16in ? 7 : 3)) == 0 && ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q16 & 15) == 0 && ((uintptr_t)a.cache & 15) == 0;
+    const bool wide = (!q8 || !bf16in) && !a.page_table && aligned;
+    // a batch of 2048 and more sequences through a page table: the chunk kernel with the token kernels' addressing and refusals
+    if (a.page_table && !bf16in && aligned && a.n >= 2048 &&
+        (q8 ? (yarn ? rope_chunk_launch_f32<true, 1, true>(a, st) : rope_chunk_launch_f32<false, 1, true>(a, st))
+            : (yarn ? rope_chunk_launch_f32<true, 1, false>(a, st) : rope_chunk_launch_f32<false, 1, false>(a, st)))) CAMX_LAUNCH_RET();
     // one token per workgroup: 29.9 us for 4096 tokens x 80 heads on cold lines (two tokens: 32.4, four: 34.9; the general kernel below: 32.3)
     if (wide && bf16in && a.n >= 2048 && (yarn ? rope_chunk_launch<true, 1>(a, st) : rope_chunk_launch<false, 1>(a, st))) {}
     else if (wide && bf16in && a.n >= 2048) {          // enough tokens to fill the chip two to a workgroup (4096 tokens, every launch on cold lines: 32.2 us; four: 34.0, one: 33.7)

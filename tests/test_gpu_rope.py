@@ -248,3 +248,37 @@ def test_qk_rope_unpaged_position_array_refusals_at_chunk_size(q8):
     assert q[100].any() and q[1500].any()
     rq, _, oerr = O.qk_rope(qkv, nh, nkv, par, n, pos=pos, q8=bool(q8), cache=fill, n_pages=rows)
     assert oerr == 1 and close_16(q, rq, 'f16', floor=HADAMARD_FLOOR if q8 else None)
+
+
+@pytest.mark.parametrize('q8,yarn', [(1, 0), (0, 0), (1, 1)])
+def test_qk_rope_paged_at_chunk_size_equals_the_small_batch_kernel(q8, yarn):
+    """2304 sequences through a page table in one launch (the chunk kernel with per-sequence addressing) against the same sequences in
+    launches of 150 (the per-token kernel): the same bytes everywhere, the same error word; a position past the table row, a negative
+    one and a page id outside the cache are refused, their rows stay untouched and their q16 is written"""
+    rng = np.random.default_rng(2304 + q8 + 2 * yarn)
+    nh, nkv, n, page, maxp = 32, 4, 2304, 16, 8
+    n_pages = n * 2
+    par = qk_par(rng, yarn_table=rope.yarn_table(128, 1e6, 4.0, 32768) if yarn else None)
+    M = nkv * 128; rb = 2 * (M // 32) * 34 if q8 else 4 * M
+    qkv = outliers(rng, (n, (nh + 2 * nkv) * 128))
+    pos = rng.integers(0, page * maxp, n).astype(np.int32)
+    table = rng.integers(0, n_pages, (n, maxp)).astype(np.int32)
+    table[np.arange(n), pos // page] = rng.permutation(n_pages)[:n]          # the pages this launch writes are distinct
+    pos[7] = page * maxp + 3; pos[900] = -1; table[1300, pos[1300] // page] = n_pages; table[2000, pos[2000] // page] = -4
+    pd, qd, posd, td = dev(par), dev(qkv), dev(pos), dev(table)
+    fill = np.full((n_pages * page, rb), 0x3c, np.uint8)
+    ca = dev(fill); ea = dev(np.zeros(1, np.int32)); qa = dev(np.zeros((n, nh, 128), np.uint16))
+    call('camx_qk_rope_paged', ptr(qd), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd), ptr(qa), ptr(ca), ptr(ea), ptr(td), I(maxp), I(page), I(n_pages), I(n), I(yarn), I(q8))
+    cb = dev(fill); eb = dev(np.zeros(1, np.int32)); qb = dev(np.zeros((n, nh, 128), np.uint16))
+    for lo in range(0, n, 150):
+        m = min(150, n - lo)
+        call('camx_qk_rope_paged', ptr(qd[lo:]), I(qkv.shape[1]), I(nh), I(nkv), ptr(pd), ptr(posd[lo:]), ptr(qb[lo:]), ptr(cb), ptr(eb), ptr(td[lo:]), I(maxp), I(page), I(n_pages),
+             I(m), I(yarn), I(q8))
+    assert int(host(ea)[0]) == int(host(eb)[0]) == 9
+    assert torch.equal(ca, cb) and torch.equal(qa, qb)
+    got = host(ca)
+    ok = np.ones(n, bool); ok[[7, 900, 1300, 2000]] = False
+    rows = table[np.arange(n), np.clip(pos, 0, page * maxp - 1) // page].astype(np.int64) * page + np.clip(pos, 0, None) % page
+    written = np.zeros(n_pages * page, bool); written[rows[ok]] = True
+    assert (got[~written] == 0x3c).all() and not (got[written] == 0x3c).all(axis=1).any()
+    assert host(qa, np.uint16)[[7, 900, 1300, 2000]].any(axis=(1, 2)).all()
