@@ -436,7 +436,12 @@ def prefill_scale_sweep(B, T=4096, only=None):
     timeit('cast_bf16 16M', Mr * Kq * 6, mk)
     ntk, Ks, neu = T, 2048, 8
     def mk(i):
-        x = B.acts((ntk, Ks), torch.float32, i); ids = torch.randperm(ntk * neu, device=dev).to(torch.int32); vy = torch.empty((Ks // 128) * ntk * neu * 144, dtype=torch.uint8, device=dev)
+        x = B.acts((ntk, Ks), torch.float32, i); vy = torch.empty((Ks // 128) * ntk * neu * 144, dtype=torch.uint8, device=dev)
+        # the compact columns as the router's sort produces them (python/caminus/prefill/glue.py: columns grouped by expert, a group's tokens in
+        # order): 128 experts, each token's 8 by the top of random scores
+        g = torch.Generator(device=dev); g.manual_seed(900 + i)
+        ex = torch.rand((ntk, 128), generator=g, device=dev).topk(neu, dim=1).indices.reshape(-1)
+        order = torch.argsort(ex, stable=True); ids = torch.empty(ntk * neu, dtype=torch.int32, device=dev); ids[order] = torch.arange(ntk * neu, dtype=torch.int32, device=dev)
         return lambda: B.call('camx_quantize_mmq_q8_1_scatter', _p(x), _p(ids), _p(vy), L64(Ks), L64(0), L64(Ks), L64(0), L64(Ks), I(ntk * neu), I(1), I(neu), I(1), I(ntk))
     timeit(f'quantize_mmq_q8_1_scatter {T}x2048 to 8 columns each', ntk * Ks * 4 + (Ks // 128) * ntk * neu * 144, mk)
     def mk(i):

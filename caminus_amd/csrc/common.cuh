@@ -197,7 +197,7 @@ CAMX_DEV void q8_1_emit(f32x4 v, uint8_t * blk, int sub) {
 // MODE 1: the values are silu(v * rs) first (OP_GG_Q8_1's mode 1).
 CAMX_DEV float silu_div(float x) { return x / (1.0f + expf(-x)); }
 template <int MODE>
-CAMX_DEV void q8_1_block_lane(const float * in, uint32_t * out, int rot, float rs) {
+CAMX_DEV void q8_1_block_lane(const float * in, uint32_t * out, int rot, float rs, bool active = true) {   // active = false: every step but the stores
     f32x4 v[8];
 #pragma unroll
     for (int k = 0; k < 8; k++) v[k] = *(const f32x4 *)(in + 4 * ((k + rot) & 7));
@@ -215,7 +215,7 @@ CAMX_DEV void q8_1_block_lane(const float * in, uint32_t * out, int rot, float r
     const float sum = w0 + w1;
     const float d = amax / 127.0f;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // (out may lie where other lanes' values were)
-    out[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
+    if (active) out[0] = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
     float r = __builtin_amdgcn_rcpf(d);
     r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
 #pragma unroll
@@ -235,7 +235,23 @@ CAMX_DEV void q8_1_block_lane(const float * in, uint32_t * out, int rot, float r
             for (int e = 0; e < 4; e++) c[e] = (int)(p[e] + __builtin_copysignf(0.49999997f, p[e]));
         }
         const uint32_t codes = ((uint32_t)c[0] & 0xffu) | (((uint32_t)c[1] & 0xffu) << 8) | (((uint32_t)c[2] & 0xffu) << 16) | ((uint32_t)c[3] << 24);
-        out[1 + ((k + rot) & 7)] = amax != 0.0f ? codes : 0u;
+        if (active) out[1 + ((k + rot) & 7)] = amax != 0.0f ? codes : 0u;
+    }
+}
+// The q8_1 blocks of a row that sits in this wave's LDS in element order (seg: nb32 * 32 floats, nb32 a multiple of 8): lane l quantizes
+// block 64 p + l of pass p whole; the 9-dword blocks of a pass are staged over the values the pass has consumed and leave as 16-byte
+// stores to dst (16-byte aligned; 36 nb32 bytes). Every lane of the wave calls it.
+CAMX_DEV void q8_1_row_from_lds(float * seg, int nb32, uint8_t * dst, int lraw) {
+    for (int p0 = 0; p0 < nb32; p0 += 64) {
+        const int nbp = nb32 - p0 < 64 ? nb32 - p0 : 64;            // blocks of this pass
+        float * in = seg + 32 * p0;
+        uint32_t * stage = (uint32_t *)in;
+        const bool on = lraw < nbp;
+        q8_1_block_lane<0>(in + 32 * (on ? lraw : 0), stage + 9 * lraw, lraw, 0.0f, on);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
+        u32x4 * d16 = (u32x4 *)(dst + (size_t)p0 * 36);
+        const int n16 = nbp * 9 / 4;                                 // 16-byte pieces of the pass (nbp % 8 == 0)
+        for (int i = lraw; i < n16; i += 64) __builtin_nontemporal_store(*(const u32x4 *)(stage + 4 * i), d16 + i);
     }
 }
 

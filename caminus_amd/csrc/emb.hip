@@ -113,8 +113,12 @@ struct EmbArgs {
 // SPLIT (batches too small to fill the chip): a workgroup per row. Every wave decodes the row and, with a tail, walks the same
 // sum of squares (the same operations on the same values: the same bits in all four), but converts, quantizes and stores only
 // the slabs j = wave (mod 4): the serial part behind the reduction, eight q8_1 slabs for a 2048-wide row, is a quarter as long.
-template <int FMT, int NI_MAX, bool TAIL, bool EXACT, bool SPLIT = false>
+// QL (wave-per-row batches with a q8_1 copy): the normed row goes to the wave's own LDS and lane l quantizes block l whole, instead of eight
+// lanes sharing a block and each repeating its divide and two butterflies (105 instructions per lane and slab; the fused Q4_K row is bound by
+// its instruction count: 1565 per wave)
+template <int FMT, int NI_MAX, bool TAIL, bool EXACT, bool SPLIT = false, bool QL = false>
 __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
+    __shared__ __attribute__((aligned(16))) float qrows[QL ? 4 : 1][QL ? NI_MAX * 256 : 4];
     const int lane = slot_of(threadIdx.x & 63), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t = SPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
     if (t >= a.n) return;
@@ -126,7 +130,7 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
     const int N = EXACT ? NI_MAX * 256 : a.N, ni = EXACT ? NI_MAX : N >> 8;
     // short rows: the addend and gamma do not depend on the token id, so they are requested before the table row is decoded
     // (one memory round trip after the id instead of three)
-    constexpr bool PRE = TAIL;
+    constexpr bool PRE = TAIL && SPLIT;      // (wave-per-row batches are bound by their waves per SIMD: 64 fewer registers without the early copies)
     f32x4 gpre[PRE ? NI_MAX : 1], dpre[PRE ? NI_MAX : 1];
     if (PRE) {
 #pragma unroll
@@ -213,8 +217,13 @@ __global__ void __launch_bounds__(256) emb_rows(EmbArgs a) {
             const size_t o = (size_t)t * N + 256 * j + 4 * lane;
             if (a.h) *(f32x4 *)(a.h + o) = v;
             if (a.h16) *(u32x2 *)(a.h16 + o) = pack_f16x4(v);
-            if (a.q8) q8_1_emit(v, a.q8 + ((size_t)t * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
+            if (QL) *(f32x4 *)(qrows[wave] + 256 * j + 4 * lane) = v;
+            else if (a.q8) q8_1_emit(v, a.q8 + ((size_t)t * (N >> 5) + 8 * j + (lane >> 3)) * 36, lane & 7);
         }
+    if (QL) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();          // the wave's row is in LDS
+        q8_1_row_from_lds(qrows[wave], N >> 5, a.q8 + (size_t)t * (N >> 5) * 36, threadIdx.x & 63);
+    }
 }
 
 template <int FMT>
@@ -235,6 +244,12 @@ static int launch_emb(const EmbArgs & a0, hipStream_t st) {
         CAMX_LAUNCH_RET();
     }
     const dim3 grid((a.n + 3) / 4);
+    if (tail && a.q8 && ((uintptr_t)a.q8 & 15) == 0 && (ni == 4 || ni == 8 || ni == 16)) {
+        if (ni == 8) emb_rows<FMT, 8, true, true, false, true><<<grid, block, 0, st>>>(a);
+        else if (ni == 16) emb_rows<FMT, 16, true, true, false, true><<<grid, block, 0, st>>>(a);
+        else emb_rows<FMT, 4, true, true, false, true><<<grid, block, 0, st>>>(a);
+        CAMX_LAUNCH_RET();
+    }
 #define CAMX_EMB(NI, EX) (tail ? emb_rows<FMT, NI, true, EX><<<grid, block, 0, st>>>(a) : emb_rows<FMT, NI, false, EX><<<grid, block, 0, st>>>(a))
     if (ni == 8) CAMX_EMB(8, true); else if (ni == 16) CAMX_EMB(16, true); else if (ni == 20) CAMX_EMB(20, true); else if (ni == 4) CAMX_EMB(4, true);
     else if (ni <= 8) CAMX_EMB(8, false); else if (ni <= 16) CAMX_EMB(16, false); else if (ni <= 24) CAMX_EMB(24, false); else CAMX_EMB(32, false);

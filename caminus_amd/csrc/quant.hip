@@ -143,12 +143,23 @@ CAMX_DEV f32x4 swiglu_bf16x4(u32x2 gw, u32x2 uw, u32x2 * packed, const uint16_t 
 template <int LAYOUT, int SRC>
 __global__ void __launch_bounds__(256) mmq_q8_1_rows(MmqArgs a) {
     const int lane = slot_of(threadIdx.x & 63);
-    const int col = blockIdx.x * 4 + (threadIdx.x >> 6);            // source row index
+    // Scattering: workgroups are dealt to the eight XCDs in turn, and each XCD has its own L2. A token's 144-byte blocks share their
+    // 128-byte lines with the blocks of the neighbouring columns, which belong to tokens a few rows away (the router groups columns by
+    // expert, a group's tokens in order); when those tokens run on another XCD the two halves of a line leave as two partial writes.
+    // So an XCD takes a contiguous range of token groups (workgroup b -> group (b % 8) * (G / 8) + b / 8), and neighbours meet in one L2.
+    int bx = blockIdx.x;
+    if (a.kexp && (gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
+    const int col = bx * 4 + (threadIdx.x >> 6);                    // source row index
     if (col >= a.nsrc) return;
     const long slab = blockIdx.y;                                   // 256 values = 2 blocks of 128
     const long i0 = slab * 256 + 4 * lane;
     if (i0 >= a.Kp) return;                                         // (Kp is a multiple of 512: never taken for half a wave)
     const long srow = a.kexp ? col : (a.ids ? a.ids[col] : col);
+    // scattering: the row's destination columns come in with the row (lane s holds column s of each batch of 64), not one dependent
+    // load per column between the stores
+    const int lraw = threadIdx.x & 63;
+    int dcols = 0;
+    if (a.kexp && lraw < a.kexp) dcols = a.ids[(long)col * a.kexp + lraw];
     f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
     if (i0 < a.K) {                                                 // K % 4 == 0: a lane's four values are in or out together
         if (SRC == SRC_F32) v = *(const f32x4 *)((const float *)a.x + srow * a.stride + i0);
@@ -174,7 +185,8 @@ __global__ void __launch_bounds__(256) mmq_q8_1_rows(MmqArgs a) {
     const uint32_t hdr = LAYOUT == MMQ_DS4 ? ((uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16)) : __builtin_bit_cast(uint32_t, d);
     const int nwrite = a.kexp ? a.kexp : 1;
     for (int slot = 0; slot < nwrite; slot++) {
-        const long dcol = a.kexp ? a.ids[(long)col * a.kexp + slot] : col;
+        if (a.kexp && slot >= 64 && (slot & 63) == 0) dcols = slot + lraw < a.kexp ? a.ids[(long)col * a.kexp + slot + lraw] : 0;
+        const long dcol = a.kexp ? __builtin_amdgcn_readlane(dcols, slot & 63) : col;
         uint8_t * blk = a.y + (kb * a.ncols + dcol) * 144;
         *(uint32_t *)(blk + 16 + 4 * l32) = q;
         if ((lane & 7) == 0) *(uint32_t *)(blk + 4 * (l32 >> 3)) = hdr;
