@@ -371,6 +371,11 @@ def prefill_scale_sweep(B, T=4096, only=None):
         k = B.acts((T, M), torch.float32, i); v = B.acts((T, M), torch.float32, i + 2); cache = torch.empty(T * 1088, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
         return lambda: B.call('camx_own_kv_q8_append', _p(k), I(M), _p(v), I(M), I(M), _p(cache), I(0), I(T), _p(err), I(T))
     timeit(f'own_kv_q8_append {T}x512', T * (M * 8 + 1088), mk)
+    TD = 65536              # the codec at depth: the rows of a long context (the reader is what a decode step walks: kernels/k3_own_atts.h:297-467)
+    def mk(i):
+        k = B.acts((TD, M), torch.float32, i); v = B.acts((TD, M), torch.float32, i + 2); cache = torch.empty(TD * 1088, dtype=torch.uint8, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_own_kv_q8_append', _p(k), I(M), _p(v), I(M), I(M), _p(cache), I(0), I(TD), _p(err), I(TD))
+    timeit('own_kv_q8_append 65536x512 (at depth)', TD * (M * 8 + 1088), mk)
     def mk(i):
         x = B.acts((T * 36, 128), torch.float32, i); y = torch.empty_like(x)
         return lambda: B.call('camx_hadamard128', _p(x), _p(y), L64(T * 36))
@@ -505,6 +510,12 @@ def prefill_scale_sweep(B, T=4096, only=None):
         k = torch.empty((T, M), dtype=torch.float16, device=dev); v = torch.empty((T, M), dtype=torch.float16, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
         return lambda: B.call('camx_own_kv_q8_read', _p(cache), NULL, I(0), I(T), I(M), _p(k), I(M), _p(v), I(M), _p(err), I(T), I(1))
     timeit(f'own_kv_q8_read {T}x512 -> f16', T * (1088 + M * 4), mk)
+    def mk(i):
+        cache = torch.randint(0, 256, (TD * 1088,), device=dev, dtype=torch.uint8)
+        cache.view(TD * 32, 34)[:, :2] = (torch.rand((TD * 32, 1), device=dev) * 9e-3 + 1e-3).to(torch.float16).view(torch.uint8).view(TD * 32, 2)
+        k = torch.empty((TD, M), dtype=torch.float16, device=dev); v = torch.empty((TD, M), dtype=torch.float16, device=dev); err = torch.zeros(1, dtype=torch.int32, device=dev)
+        return lambda: B.call('camx_own_kv_q8_read', _p(cache), NULL, I(0), I(TD), I(M), _p(k), I(M), _p(v), I(M), _p(err), I(TD), I(1))
+    timeit('own_kv_q8_read 65536x512 -> f16 (at depth)', TD * (1088 + M * 4), mk)
     page, n_pages = 256, max(64, T // 64)
     def mk(i):
         qkv = B.acts((T, ldq), torch.float32, i); q16 = torch.empty((T, nh, 128), dtype=torch.float16, device=dev)
@@ -667,6 +678,29 @@ def main():
         med, mean = B.time_launch(lambda: dst.copy_(src), reps=a.steps, warm=a.warmup)
         print(json.dumps({'kernel': 'copy_ref', 'bytes_read': src.numel(), 'bytes_written': src.numel(), 'us': round(mean, 2),
                           'GBps': round(2 * src.numel() / (mean * 1e-6) / 1e9, 1)}))
+        return
+    if a.only == 'copy_sizes':
+        # the runtime's own device copy (hipMemcpy device to device, through torch) at the sizes of the sweep's launches, timed like them (30
+        # back to back over copies in rotation, footprint >= 1.2 GB): what a launch that moves S bytes can reach at all on this machine
+        B.ramp()
+        res = {}
+        for mb in (6, 12, 24, 48, 55, 84, 126, 183, 256, 512):
+            n = mb << 20
+            nc = max(3, min(16, -(-1_200_000_000 // (2 * n))))
+            src = [torch.ones(n, dtype=torch.uint8, device=B.dev) for _ in range(nc)]; dst = [torch.empty(n, dtype=torch.uint8, device=B.dev) for _ in range(nc)]
+            for i in range(nc): dst[i].copy_(src[i])
+            torch.cuda.synchronize()
+            ts = []
+            for rep in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for k in range(30): dst[k % nc].copy_(src[k % nc])
+                e1.record(); e1.synchronize()
+                ts.append(e0.elapsed_time(e1) * 1e3 / 30)
+            ts.sort()
+            res[f'{2 * n / 1e6:.1f} MB'] = {'us': round(ts[2], 2), 'GBps': round(2 * n / ts[2] / 1e3, 1), 'frac_of_8TBps': round(2 * n / ts[2] / 1e3 / HBM_PEAK_GBPS, 4)}
+            del src, dst; torch.cuda.empty_cache()
+        print(json.dumps({'metric': 'device-to-device copy by the runtime, bytes read + written per launch', 'n_gpus': 1, 'copy_sizes': res}))
         return
     traffic = hbm_traffic()
     NC = a.copies

@@ -749,7 +749,10 @@ int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void 
     if (!x || !w || !state || !y || C < 1 || T < 1 || ldx < C || ldy < C || ((uintptr_t)w & 15)) return CAMX_EINVAL;
     const int vw = bf16 ? 8 : 4;
     if ((long)T * C >= (1L << 20) && C % vw == 0 && ldx % vw == 0 && ldy % vw == 0 && !(((uintptr_t)x | (uintptr_t)y) & 15)) {
-        const int tr = 32;       // tokens per wave: 16 and 64 measured 15 % slower (halo re-reads; too few waves) (a decode / verify batch takes the one-value-per-thread kernel below)
+        // tokens per wave: at 4096 tokens 16 and 64 measured 15 % slower than 32 (halo re-reads; too few waves); from 16384 tokens on there
+        // are waves enough for 64, and the three halo rows a wave re-reads are 5 % of its reads instead of 9 % (a decode / verify batch
+        // takes the one-value-per-thread kernel below)
+        const int tr = T >= 16384 ? 64 : 32;
         const dim3 gs((unsigned)((C / vw + 63) / 64), (unsigned)((T + tr - 1) / tr)), bs(64);
         if (bf16) gdn_conv_stream<true><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr); else gdn_conv_stream<false><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr);
         CAMX_LAUNCH_RET();
@@ -805,7 +808,7 @@ int camx_gdn_conv_l2(const void * x, const float * w, const float * state, void 
     if (!x || !w || !state || !qk || C < 128 || (C & 127) || T < 1 || ldx < C || (y && ldy < C) || heads < 1 || heads > C / 128 || (ldx % vw) || (y && ldy % vw) ||
         ((uintptr_t)w & 15) || (((uintptr_t)x | (uintptr_t)y | (uintptr_t)qk) & 15)) return CAMX_EINVAL;
     if ((long)T * C >= (1L << 20)) {
-        const int tr = 32;
+        const int tr = T >= 16384 ? 64 : 32;
         const dim3 gs((unsigned)((C / vw + 63) / 64), (unsigned)((T + tr - 1) / tr)), bs(64);
         if (bf16) gdn_conv_stream<true, true><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr, qk, heads, rs);
         else gdn_conv_stream<false, true><<<gs, bs, 0, st>>>(x, w, state, y, C, T, ldx, ldy, tr, qk, heads, rs);
