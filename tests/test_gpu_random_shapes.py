@@ -82,3 +82,47 @@ def test_random_shapes(seed):
             fn(*args)
         except Exception as e:
             raise AssertionError(f'{fn.__module__}.{fn.__name__}{args}: {type(e).__name__}: {e}') from e
+
+
+def _fused_generators(r):
+    import test_gpu_fused_tape as FT
+    ri, ch = r.randint, r.choice
+
+    def conv_l2():
+        c = 128 * ch([1, 2, 3, 8, 10, 32, 80]); t = ch([ri(1, 40), ri(1, 40), ri(260, 1200), 8192 // (c // 128) + ri(0, 50)])
+        return t, c, ri(1, c // 128), ri(0, 1)
+
+    def dense_q8():
+        nkv = ri(1, 4)
+        return ch([ri(1, 20), ri(1, 20), ri(300, 900)]), ri(1, 24), nkv, ch([16, 32, 64, 128, 256]), ri(0, 3000)
+
+    def qk2():
+        d = ch([64, 96, 128, 256, 512])
+        return ch([1, 3, 16, 70]), ri(1, 24), ri(1, 4), d, ch([x for x in (8, 16, 32, 64, 128, 256) if x <= d]), ri(0, 1)
+
+    def op_nr():
+        d = ch([64, 96, 128, 256, 512])
+        return ch([1, 3, 16, 400, 600]), ri(1, 24), d, ch([x for x in (8, 16, 32, 64, 128, 256) if x <= d]), d + 4 * ri(0, 64)
+
+    return [
+        (FT.test_gdn_conv_l2_equals_the_two_launches, conv_l2),
+        (FT.test_op_gdn_conv_l2_equals_the_two_tape_ops, lambda: (lambda g: (128 * g, ri(1, 20), ri(1, g)))(ch([1, 2, 5, 8, 80]))),
+        (FT.test_qk_nr_q8_equals_the_six_launches, dense_q8),
+        (FT.test_qk_nr_qk_equals_two_launches, qk2),
+        (FT.test_op_qk_nr_reads_its_position_on_the_device, op_nr),
+        (FT.test_op_kv_append_three_row_formats, lambda: (32 * ri(1, 40), ch([ri(1, 40), ri(1, 40), ri(1024, 1300)]))),
+        (FT.test_op_own_qk_rope_reads_its_position_on_the_device, lambda: (ch([1, 2, 7, 300, 2049, 2100]), ri(0, 1), ri(0, 1))),
+    ]
+
+
+@pytest.mark.parametrize('seed', [30260])
+def test_random_shapes_of_the_fused_and_tape_entry_points(seed):
+    r = random.Random(seed)
+    gens = _fused_generators(r)
+    for _ in range(120):
+        fn, draw = r.choice(gens)
+        args = draw()
+        try:
+            fn(*args)
+        except Exception as e:
+            raise AssertionError(f'{fn.__module__}.{fn.__name__}{args}: {type(e).__name__}: {e}') from e
