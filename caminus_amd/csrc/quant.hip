@@ -428,9 +428,13 @@ __global__ void __launch_bounds__(256) silu_small_fill() {             // after 
 }
 
 #define SWS_IPW 2                                                          // items (token groups) per wave, loaded together
-template <int LAYOUT, int SRC>
+// SCAT (quantize_mmq_q8_1's scatter form): row t is token t, and each of its blocks goes to the kexp columns sc_ids[t * kexp + slot] of a
+// block row of ncols_dst columns: the group's eight staged blocks leave as 16-byte pieces, 8 kexp block copies per item (the rows kernel
+// writes the same blocks four bytes per lane, two blocks per wave: 35 against 23 us for 4096 tokens x 2048 to 8 columns each).
+template <int LAYOUT, int SRC, bool SCAT = false>
 __global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void * __restrict__ gu, const int32_t * __restrict__ ids, long ld, long F,
-                                                                    uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T, unsigned ncolp) {
+                                                                    uint8_t * __restrict__ y, uint16_t * __restrict__ act, int T, unsigned ncolp,
+                                                                    const int32_t * __restrict__ sc_ids = nullptr, int kexp = 0, int ncols_dst = 0) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
     const int lraw = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint8_t * stage = (uint8_t *)lut + (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : 0) + wave * (SWM_TOK * 144);
@@ -444,8 +448,15 @@ __global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void 
     // the block column moves on by one every 16 workgroups (1024 tokens) of the walk: with a row stride that is a power of two (8192
     // fp32 values) the rows of one column fall on a fraction of the memory channels, and the walk would keep the whole chip on them
     // (8192 x 8192: 0.60 -> 0.72 of peak; 6144- and 17408-wide rows: unchanged)
-    const unsigned tb = blockIdx.x % ntb;
-    const long tg0 = ((long)tb * SWS_WAVES + wave) * (SWM_TOK * SWS_IPW), unit = (blockIdx.x / ntb + tb / 16) % ncolp;
+    unsigned tb = blockIdx.x % ntb, un = blockIdx.x / ntb + tb / 16;
+    if (SCAT && (ntb & 7) == 0) {
+        // Scattering: a block shares its first and last line with the blocks of the neighbouring columns, which belong to tokens a few rows
+        // away (the router groups columns by expert, a group's tokens in order). Workgroups are dealt to the eight XCDs in turn and each
+        // XCD has its own L2, so an XCD takes a contiguous eighth of the token blocks: neighbours meet in one L2 and leave as whole lines.
+        const unsigned m = blockIdx.x >> 3, per = ntb >> 3;
+        tb = (blockIdx.x & 7) * per + m % per; un = m / per;
+    }
+    const long tg0 = ((long)tb * SWS_WAVES + wave) * (SWM_TOK * SWS_IPW), unit = un % ncolp;
     SwmItem it[SWS_IPW];
     if (SRC == SRC_F32) {
         // fp32 rows: a lane's eight values are 32 bytes, so loading them into its registers takes two requests that each use half of
@@ -488,10 +499,26 @@ __global__ void __launch_bounds__(SWS_WAVES * 64) swiglu_mmq_oneshot(const void 
                 swm_compute<LAYOUT, SRC, true, LUT_FULL>(it[k], g_silu_lut, stage, F, act, T, tg, unit, lraw);
         }
         const int nunits = (int)min((long)SWM_TOK, T - tg) * 9;           // tokens of the group that exist
-        uint8_t * dst = y + ((size_t)unit * T + (size_t)tg) * 144;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();       // the wave's own LDS writes, in order
-        if (lraw < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 16 * lraw), (u32x4 *)(dst + 16 * lraw));
-        if (lraw < 8 && 64 + lraw < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 1024 + 16 * lraw), (u32x4 *)(dst + 1024 + 16 * lraw));
+        if (SCAT) {
+            const int nbc = (nunits / 9) * kexp;                          // block copies of the group: token slot b / kexp to its column number b % kexp
+            for (int b0 = 0; b0 < nbc; b0 += 64) {
+                const int dc = b0 + lraw < nbc ? sc_ids[(size_t)tg * kexp + b0 + lraw] : 0;        // (the group's columns are one contiguous run of the list)
+                const int nb = nbc - b0 < 64 ? nbc - b0 : 64;
+#pragma unroll
+                for (int i = 0; i < 9; i++) {
+                    const int p = 64 * i + lraw, b = p / 9, part = p - 9 * b;
+                    const int col = __shfl(dc, b & 63, 64);
+                    // (plain stores: a block shares its first and last line with the neighbouring columns' blocks, which other workgroups write;
+                    // the lines are completed in L2. Past the caches each block would leave as partial lines: 51 instead of 25 us)
+                    if (b < nb) *(u32x4 *)(y + ((size_t)unit * ncols_dst + col) * 144 + 16 * part) = *(const u32x4 *)(stage + ((b0 + b) / kexp) * 144 + 16 * part);
+                }
+            }
+        } else {
+            uint8_t * dst = y + ((size_t)unit * T + (size_t)tg) * 144;
+            if (lraw < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 16 * lraw), (u32x4 *)(dst + 16 * lraw));
+            if (lraw < 8 && 64 + lraw < nunits) __builtin_nontemporal_store(*(const u32x4 *)(stage + 1024 + 16 * lraw), (u32x4 *)(dst + 1024 + 16 * lraw));
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
     }
 }
@@ -502,6 +529,13 @@ static void launch_oneshot(const void * src, const int32_t * ids, long ld, long 
     const size_t lds = (SRC == SRC_SWIGLU_BF16 ? 2 * SWS_TAB : SWS_WAVES * SWS_IPW * SWM_TOK * 512) + SWS_WAVES * SWM_TOK * 144;
     if (layout == MMQ_DS4) swiglu_mmq_oneshot<MMQ_DS4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol);
     else swiglu_mmq_oneshot<MMQ_D4, SRC><<<grid, block, lds, st>>>(src, ids, ld, F, (uint8_t *)vy, act, T, (unsigned)ncol);
+}
+static void launch_oneshot_scatter(const float * x, const int32_t * sc_ids, long ld, long K, void * vy, int ntok, int kexp, int ncols_dst, long ncol, int layout, hipStream_t st) {
+    const int per = SWS_WAVES * SWM_TOK * SWS_IPW;
+    const dim3 grid((unsigned)((ntok + per - 1) / per) * (unsigned)ncol), block(SWS_WAVES * 64);
+    const size_t lds = SWS_WAVES * SWS_IPW * SWM_TOK * 512 + SWS_WAVES * SWM_TOK * 144;
+    if (layout == MMQ_DS4) swiglu_mmq_oneshot<MMQ_DS4, SRC_F32, true><<<grid, block, lds, st>>>(x, nullptr, ld, K, (uint8_t *)vy, nullptr, ntok, (unsigned)ncol, sc_ids, kexp, ncols_dst);
+    else swiglu_mmq_oneshot<MMQ_D4, SRC_F32, true><<<grid, block, lds, st>>>(x, nullptr, ld, K, (uint8_t *)vy, nullptr, ntok, (unsigned)ncol, sc_ids, kexp, ncols_dst);
 }
 
 // act = bf16(bf16(silu g) * u) of wide bf16 rows [g (H) | u (H)] with the same table: persistent workgroups, a lane takes 8
@@ -661,6 +695,10 @@ int camx_quantize_mmq_q8_1_scatter(const float * x, const int32_t * ids, void * 
     if (!x || !vy || !ids || ne00 < 4 || ne00 % 4 || s02 < ne00 || s02 % 4 || ne0 % 512 || ne0 < ne00 || ne0 >= ne00 + 512 || ne2 != 1 ||
         n_expert_used < 1 || ntok < 0 || ne1 != ntok * n_expert_used || (layout != MMQ_D4 && layout != MMQ_DS4) ||
         ((uintptr_t)x & 15) || ((uintptr_t)vy & 15)) return CAMX_EINVAL;
+    if (ntok >= 2048 && ne0 / 128 <= 65535 && (long)ntok * n_expert_used < 0x7fffffffL) {      // a prefill chunk: the one-shot form
+        launch_oneshot_scatter(x, ids, s02, ne00, vy, ntok, n_expert_used, ne1, ne0 / 128, layout, st);
+        CAMX_LAUNCH_RET();
+    }
     MmqArgs a = {x, ids, (uint8_t *)vy, nullptr, ne00, ne0, s02, ne1, ntok, n_expert_used, nullptr};
     return launch_mmq<SRC_F32>(a, layout, st);
 }

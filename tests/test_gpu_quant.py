@@ -56,7 +56,7 @@ def test_mmq_quantize(K, ncols, layout):
         assert bits_equal(host(y), ref)
 
 
-@pytest.mark.parametrize('K,ntok,k,pad', [(768, 9, 8, 0), (2048, 4, 2, 0), (264, 2051, 3, 8), (1024, 2048, 8, 0), (392, 4100, 1, 4)])
+@pytest.mark.parametrize('K,ntok,k,pad', [(768, 9, 8, 0), (2048, 4, 2, 0), (264, 2051, 3, 8), (1024, 2048, 8, 0), (392, 4100, 1, 4), (520, 2101, 11, 0), (128, 2049, 70, 4)])
 def test_mmq_quantize_scatter(K, ntok, k, pad):
     """small batches and prefill chunks: token counts that end inside a group of 8, widths that end inside a block, padded source rows"""
     rng = np.random.default_rng(K)
