@@ -1,6 +1,8 @@
 """The position-span checks and KV row geometry the launch wrappers share. Mirrors the corresponding helpers of the
 reference's python/caminus/engine/k3.py (ContextBoundsError :413-420, check_span :423-437, kv_pos_bytes :530-532,
-kv_rows :535-540); the persistent tape engine of that module is not part of this library."""
+kv_rows :535-540), and TapeOps: the tape's row ops (python/caminus/engine/k3.py:854-860, 1002-1008, 1057-1089, 1209-1257) with
+their Seg field order, each one launch of the library with the position read from a device word. The persistent tape walker of
+that module (one kernel that runs a whole layer, matrix products included) is not part of this library."""
 import numpy as np
 
 from ..errors import InvalidKVEncoding, NumericalFailure   # noqa: F401  (re-exported as in the reference module)
