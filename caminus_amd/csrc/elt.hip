@@ -181,7 +181,7 @@ __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ 
     const int cv = blockIdx.x * 64 + (L2 && !BF16 ? lane_l2 : (int)threadIdx.x);
     if (cv * VW >= C) return;
     const int c0 = cv * VW, t0 = blockIdx.y * TR, t1 = T < t0 + TR ? T : t0 + TR;
-    auto row = [&](int t) {                                            // (a row index past the range is clamped: the load is harmless and never used)
+    auto row = [&](int t) {                                            // (a row index past the batch is clamped: the load is harmless and never used)
         const int tc = t < T - 1 ? t : T - 1;
         return BF16 ? __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + (size_t)tc * ldx + c0))
                     : __builtin_nontemporal_load((const u32x4 *)((const float *)x + (size_t)tc * ldx + c0));
@@ -195,6 +195,12 @@ __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ 
             for (int p = 0; p < 4; p++) { const uint32_t b = r[p]; o[p % VW] = __builtin_bit_cast(float, b); }
         }
     };
+    u32x4 halo[3];                                                     // the three rows before the range (another wave's tokens; clamped when the state stands in)
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int tj = t0 - 3 + j < 0 ? 0 : t0 - 3 + j;
+        halo[j] = BF16 ? *(const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0) : *(const u32x4 *)((const float *)x + (size_t)tj * ldx + c0);
+    }
     u32x4 ring[P];
 #pragma unroll
     for (int u = 0; u < P; u++) ring[u] = row(t0 + u);
@@ -208,7 +214,7 @@ __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ 
         if (tj < 0) {
 #pragma unroll
             for (int k = 0; k < VW; k++) win[j][k] = st[(size_t)(c0 + k) * 3 + 3 + tj];
-        } else widen(win[j], BF16 ? *(const u32x4 *)((const uint16_t *)x + (size_t)tj * ldx + c0) : *(const u32x4 *)((const float *)x + (size_t)tj * ldx + c0));
+        } else widen(win[j], halo[j]);
     }
     auto emit = [&](int tt, int u) {                                   // token tt's output from window slots u .. u + 3 (mod 4)
         float r[VW];
@@ -242,13 +248,30 @@ __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ 
         }
     };
     int t = t0;
-    for (; t + P <= t1; t += P) {                                      // whole groups of eight tokens: no guards
+    for (; t + 2 * P <= t1; t += P) {                                  // whole groups of eight tokens whose successors are all in the range: no guards
+#pragma unroll
+        for (int u = 0; u < P; u++) {
+            // the whole row is widened before its ring slot is requested again: left to itself the compiler widens half of it later,
+            // keeps that half in a copy, and hoists the copies of all eight slots (and the waits for their loads) to the top of the loop
+            widen(win[(u + 3) & 3], ring[u]);
+#pragma unroll
+            for (int k = 0; k < VW; k++) asm volatile("" : "+v"(win[(u + 3) & 3][k]));
+            __builtin_amdgcn_sched_barrier(0);
+            ring[u] = row(t + u + P);
+            __builtin_amdgcn_sched_barrier(0);
+            emit(t + u, u);
+        }
+    }
+    // the last whole group requests only rows this wave will use: a row past the range is another wave's, and would come from HBM
+    // twice (with eight rows requested ahead regardless, 4096 x 10240 read 34 % more than its input, 16384 tokens 17 %)
+    if (t + P <= t1) {
 #pragma unroll
         for (int u = 0; u < P; u++) {
             widen(win[(u + 3) & 3], ring[u]);
-            ring[u] = row(t + u + P);
+            if (t + u + P < t1) ring[u] = row(t + u + P);
             emit(t + u, u);
         }
+        t += P;
     }
 #pragma unroll
     for (int u = 0; u < P; u++)                                        // the last, partial group
