@@ -15,6 +15,7 @@
 // order with fmaf, the 32 lanes of a half-wave combine by xor 16, 8, 4, 2, 1, the eight half-wave sums are added in order.
 #include "common.cuh"
 #include <mutex>
+#include <type_traits>
 
 #define HSCALE 0.08837890625f      // bf16(1 / sqrt(128))
 
@@ -107,6 +108,22 @@ struct RmsSrc {
     }
     CAMX_DEV f32x4 operator()(int row, int k, u32x2 &) const { return (*this)(row, k); }
 };
+// The same source for a row that one wave holds in registers (rows of at most 256 NR values): round c of the lane is elements
+// 256 c + 4 slot .. + 3, the elements the lane holds in the row's sum of squares and in the projections, so x and the norm
+// weights are read once.
+template <int NR>
+struct RmsRegSrc {
+    static constexpr bool bf16_valued = false;
+    static constexpr bool by_round = true;
+    f32x4 xk[NR], wk[NR]; float rstd;
+    CAMX_DEV f32x4 at(int c) const {
+        f32x4 a; a.x = xk[c].x * rstd * wk[c].x; a.y = xk[c].y * rstd * wk[c].y; a.z = xk[c].z * rstd * wk[c].z; a.w = xk[c].w * rstd * wk[c].w;
+        return a;
+    }
+    CAMX_DEV f32x4 operator()(int, int k, u32x2 &) const { return at(k >> 8); }
+};
+template <typename S, typename = void> struct SrcByRound : std::false_type {};
+template <typename S> struct SrcByRound<S, std::void_t<decltype(S::by_round)>> : std::true_type {};
 
 // u = bf16(H128 . bf16(source)) for the NR rounds of this half-wave; returns the lane's max |u| over its active chunks
 // NHW: the half-waves that share a row (8: a 256-thread workgroup; 2: one wave); half-wave hw takes chunks hw, hw + NHW, ...
@@ -117,7 +134,10 @@ CAMX_DEV float actq_rotate(Src src, int row, int l, int hw, int nch, f32x4 (&u)[
         const int ch = hw + NHW * c;
         f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
         u32x2 kp = {0u, 0u};
-        if (ch < nch) v = src(row, ch * 128 + 4 * l, kp);
+        if (ch < nch) {
+            if constexpr (SrcByRound<Src>::value) { static_assert(NHW == 2, "a wave per row"); v = src.at(c); }
+            else v = src(row, ch * 128 + 4 * l, kp);
+        }
         if (keep) keep[c] = kp;
         u[c] = v;
     }
@@ -422,6 +442,8 @@ struct SinkSiluMul {
 #undef S_
         dgp = pack_f2bf_x4(dg); dup = pack_f2bf_x4(du);
     }
+    // (the gates and multipliers are read a second time here: held in registers since the source fetched them they cost 48 more,
+    // two waves per SIMD instead of three, and 8192 x 2048 takes 65 us instead of 62)
     CAMX_DEV void st8(int row, int k, f32x4 a, f32x4 b, u32x4 keep) const {
         const uint16_t * r = gu + (size_t)row * ld + k;
         const u32x4 gw = *(const u32x4 *)r, uw = *(const u32x4 *)(r + F);
@@ -670,17 +692,46 @@ __global__ void __launch_bounds__(32 * NHW) block_entry_fwd_k(const float * x, c
     __shared__ float slot;
     const int row = blockIdx.x;
     const float * xr = x + (size_t)row * d;
-    const float ss = row_tree_sum(SqTerm{xr}, d, &slot);
-    const float rstd = rsqrt_exact(ss / (float)d + eps);
-    if (threadIdx.x == 0 && rstd_out) rstd_out[row] = rstd;
-    actq_fwd_row<NR, RmsSrc, NHW>(RmsSrc{x, nw, rstd, d}, row, y, s, d, clip, qmax, codes, lds);
-    if (nab == 0) return;
     constexpr int NW = NHW / 2, NA = NR * NHW / 2;       // waves per row; 256-element steps of a row
     constexpr bool KEEP = NA <= 8;
     const int lane = slot_of(threadIdx.x & 63), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const AbTerm term{xr, nw, rstd, wab};
     f32x4 hk[KEEP ? NA : 1];
-    if (KEEP) {
+    float rstd;
+    if constexpr (NHW == 2) {                            // the row and the norm weights in registers: every HBM byte of x crosses once
+        RmsRegSrc<NR> src;
+#pragma unroll
+        for (int c = 0; c < NR; c++) {
+            const int k = 256 * c + 4 * lane;
+            src.xk[c] = src.wk[c] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+            if (k < d) { src.xk[c] = __builtin_nontemporal_load((const f32x4 *)(xr + k)); src.wk[c] = *(const f32x4 *)(nw + k); }
+        }
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < NR; c++)
+            if (256 * c + 4 * lane < d) {
+                acc.x = __builtin_fmaf(src.xk[c].x, src.xk[c].x, acc.x); acc.y = __builtin_fmaf(src.xk[c].y, src.xk[c].y, acc.y);
+                acc.z = __builtin_fmaf(src.xk[c].z, src.xk[c].z, acc.z); acc.w = __builtin_fmaf(src.xk[c].w, src.xk[c].w, acc.w);
+            }
+        const float ss = wave_groups_in_order(group32_sum(acc));
+        rstd = rsqrt_exact(ss / (float)d + eps);
+        src.rstd = rstd;
+        if (threadIdx.x == 0 && rstd_out) rstd_out[row] = rstd;
+        actq_fwd_row<NR, RmsRegSrc<NR>, NHW>(src, row, y, s, d, clip, qmax, codes, lds);
+        if (nab == 0) return;
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const f32x4 a = src.at(i % NR);
+            hk[KEEP ? i : 0] = 256 * i + 4 * lane < d ? (f32x4){rbf(a.x), rbf(a.y), rbf(a.z), rbf(a.w)} : (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    } else {
+        const float ss = row_tree_sum(SqTerm{xr}, d, &slot);
+        rstd = rsqrt_exact(ss / (float)d + eps);
+        if (threadIdx.x == 0 && rstd_out) rstd_out[row] = rstd;
+        actq_fwd_row<NR, RmsSrc, NHW>(RmsSrc{x, nw, rstd, d}, row, y, s, d, clip, qmax, codes, lds);
+        if (nab == 0) return;
+    }
+    const AbTerm term{xr, nw, rstd, wab};
+    if (KEEP && NHW != 2) {
 #pragma unroll
         for (int i = 0; i < NA; i++) { const int k = 256 * i + 4 * lane; hk[KEEP ? i : 0] = k < d ? term(k) : (f32x4){0.0f, 0.0f, 0.0f, 0.0f}; }
     }
@@ -728,8 +779,16 @@ __global__ void __launch_bounds__(64) block_entry_bwd_k(const float * x, const f
     const int row = blockIdx.x, la = slot_of(threadIdx.x);
     const float rstd = rstd_in[row];
     const float * xr = x + (size_t)row * d;
+    RmsRegSrc<NR> src;                                   // x and the norm weights once, for the quantizer's source and the RMSNorm backward
+#pragma unroll
+    for (int c = 0; c < NR; c++) {
+        const int k = 256 * c + 4 * la;
+        src.xk[c] = src.wk[c] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        if (k < d) { src.xk[c] = __builtin_nontemporal_load((const f32x4 *)(xr + k)); src.wk[c] = *(const f32x4 *)(nw + k); }
+    }
+    src.rstd = rstd;
     f32x4 dh[NR];
-    actq_bwd_row<NR, RmsSrc, SinkNone, 2>(RmsSrc{x, nw, rstd, d}, row, dy, SinkNone{}, d, clip, qmax, nullptr, dh);
+    actq_bwd_row<NR, RmsRegSrc<NR>, SinkNone, 2>(src, row, dy, SinkNone{}, d, clip, qmax, nullptr, dh);
     if (nab) {                                           // the projections' part of dh
         const int half = nab / 2;
         float dabs[2][8];                                // the row's dab by group, the same in every lane: scalar registers
@@ -774,7 +833,7 @@ __global__ void __launch_bounds__(64) block_entry_bwd_k(const float * x, const f
         const int k = 256 * c + 4 * la;
         gw[c] = xh[c] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
         if (k < d) {
-            const f32x4 w = *(const f32x4 *)(nw + k), xv = *(const f32x4 *)(xr + k);
+            const f32x4 w = src.wk[c], xv = src.xk[c];
             gw[c] = (f32x4){dh[c].x * w.x, dh[c].y * w.y, dh[c].z * w.z, dh[c].w * w.w};
             xh[c] = (f32x4){xv.x * rstd, xv.y * rstd, xv.z * rstd, xv.w * rstd};
             acc.x = __builtin_fmaf(gw[c].x, xh[c].x, acc.x); acc.y = __builtin_fmaf(gw[c].y, xh[c].y, acc.y);
