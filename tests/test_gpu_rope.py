@@ -220,13 +220,14 @@ def test_prefill_sized_rope_equals_the_small_batch_kernel(nh, nkv, yarn):
     assert not (blocks[pos0 + 7, 4:] == 0xa5).all(1).any() and not (blocks[pos0 + 9, M // 32] == 0xa5).all() and not (blocks[pos0 + 8] == 0xa5).all(1).any()
 
 
-@pytest.mark.parametrize('q8', [0, 1])
-def test_qk_rope_unpaged_position_array_refusals_at_chunk_size(q8):
-    """the same refusals in the kernel that takes 2048 and more rows with a position array (four tokens per workgroup): a position past
-    the cache and a negative one set bit 1 and leave their rows unwritten, q16 is written for every token, every other row carries the
-    bytes the small-batch kernel writes for it, and nothing else is touched"""
-    rng = np.random.default_rng(2100 + q8)
-    nh, nkv, n, rows = 32, 4, 2100, 2200
+@pytest.mark.parametrize('q8,nh,nkv', [(0, 32, 4), (1, 32, 4), (0, 30, 2), (1, 30, 2)])
+def test_qk_rope_unpaged_position_array_refusals_at_chunk_size(q8, nh, nkv):
+    """the same refusals in the kernels that take 2048 and more rows with a position array (a token per workgroup when the head counts are
+    multiples of four, four tokens per workgroup otherwise): a position past the cache and a negative one set bit 1 and leave their rows
+    unwritten, q16 is written for every token, every other row carries the bytes the small-batch kernel writes for it, and nothing else
+    is touched"""
+    rng = np.random.default_rng(2100 + q8 + nh)
+    n, rows = 2100, 2200
     par = qk_par(rng); M = nkv * 128; rb = 2 * (M // 32) * 34
     qkv = outliers(rng, (n, (nh + 2 * nkv) * 128))
     pos = rng.permutation(rows)[:n].astype(np.int32)
