@@ -800,8 +800,8 @@ def main():
         # the launch-bound op-sets as they would run in a decode loop: each shape's launches captured once into a HIP graph
         # and replayed (every entry point is stream-ordered, allocates nothing and keeps no host state per call)
         graphs = {}
-        for prefix in ('c1_', 'c4_', 'c5_'):
-            fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'six_launches' not in name and not name.endswith('_k')]
+        for prefix, rep in (('c1_', 1), ('c4_', 1), ('c5_', 1), ('c1_', 8)):      # (x 8: as many launches as a few layers of a decode step queue)
+            fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'six_launches' not in name and not name.endswith('_k')] * rep
             for fn in fns: fn()
             torch.cuda.synchronize()
             gr = torch.cuda.CUDAGraph()
@@ -817,7 +817,7 @@ def main():
             for _ in range(50): gr.replay()
             g1.record(); g1.synchronize()
             us = g0.elapsed_time(g1) * 1e3 / 50
-            graphs[prefix + 'opsets_as_one_graph'] = {'launches': len(fns), 'us_per_replay': round(us, 2), 'us_per_launch': round(us / len(fns), 2)}
+            graphs[prefix + ('opsets_as_one_graph' if rep == 1 else f'opsets_x{rep}_as_one_graph')] = {'launches': len(fns), 'us_per_replay': round(us, 2), 'us_per_launch': round(us / len(fns), 2)}
         out['opset_graphs'] = graphs
     if not a.no_cpu and not a.only:
         out['cpu_baseline'] = cpu_baseline(w)
