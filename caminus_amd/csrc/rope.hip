@@ -1251,7 +1251,7 @@ int camx_op_qk_nr(const float * x, int head_stride, int heads, int dim, const fl
 int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const void * xk, int k_stride, int nkv, const float * wk, int D, int nrot,
                   float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, void * outq, void * outk, int T, int io, hipStream_t st) {
     if (!xq || !xk || !wq || !wk || !outq || !outk || T < 0 || nh < 1 || nkv < 1 || D < 1 || D > 512 || q_stride < D || k_stride < D || nrot < 0 || nrot > D ||
-        (nrot & 1) || io < 0 || io > 1 || (!pos && !pos_dev && pos0 < 0)) return CAMX_EINVAL;
+        (nrot & 1) || io < 0 || io > 1 || (!pos && !pos_dev && (pos0 < 0 || pos0 > 0x7fffffff - T))) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
     NrArgs a = {xq, q_stride, nh, wq, D, nrot, theta_scale, eps, pos0, pos, outq, T, pos_dev, xk, k_stride, nkv, wk, outk};
     const int es = io ? 2 : 4;
@@ -1269,7 +1269,7 @@ int camx_qk_nr_q8(const float * q, int q_stride, int nh, const float * k, int ld
                   int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, float * qo, uint8_t * cache, int rows,
                   int * err, int T, hipStream_t st) {
     if (!q || !k || !v || !qn || !kn || !qo || !cache || !err || T < 0 || nh < 1 || nkv < 1 || q_stride < 256 || (q_stride & 3) || ldk < nkv * 256 || ldv < nkv * 256 ||
-        ((ldk | ldv) & 3) || rows < 1 || (!pos && !pos_dev && pos0 < 0) ||
+        ((ldk | ldv) & 3) || rows < 1 || (!pos && !pos_dev && (pos0 < 0 || pos0 > 0x7fffffff - T)) ||
         (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)qn | (uintptr_t)kn | (uintptr_t)qo) & 15) || ((uintptr_t)cache & 1)) return CAMX_EINVAL;
     if (nrot != 16 && nrot != 32 && nrot != 64 && nrot != 128 && nrot != 256) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
