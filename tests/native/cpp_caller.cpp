@@ -87,6 +87,24 @@ extern "C" __attribute__((visibility("default"))) int cpp_caller_run(char * msg,
         orc_kv_q8_append(k.data(), M, v.data(), M, M, cache.data(), 2, rows, T, &werr);
         if (!rc && !(same(dc.download<uint8_t>(), cache) && derr.download<int>()[0] == werr && werr == 2)) rc = fail(msg, len, "Q8 KV rows or error word differ from the oracle");
     }
+    if (!rc) {   // the tape's form of the same append: tables filled up front, the position in a device word, advanced between two calls
+        const int T = 2, M = 256, rows = 8;
+        if (const int e = camx_init(st)) rc = fail(msg, len, "camx_init", e);
+        std::vector<float> k((size_t)T * M), v((size_t)T * M);
+        for (auto & e : k) e = normal(rng);
+        for (auto & e : v) e = normal(rng);
+        std::vector<uint8_t> cache((size_t)rows * 2 * (M / 32) * 34, 0x5a);
+        int pos = 1, werr = 0;
+        DeviceBuffer dk(k.data(), k.size() * 4), dv(v.data(), v.size() * 4), dc(cache.data(), cache.size()), derr(nullptr, 4), dpos(&pos, 4);
+        for (int call = 0; call < 2 && !rc; call++, pos += 5) {              // rows 1, 2, then 6, 7
+            if (hipMemcpyAsync(dpos.p, &pos, 4, hipMemcpyHostToDevice, st) != hipSuccess) rc = fail(msg, len, "hipMemcpyAsync");
+            const int e = camx_op_kv_append(dk.as<float>(), dv.as<float>(), dc.p, dpos.as<int32_t>(), M, 2, derr.as<int>(), rows, T, st);
+            if (e) rc = fail(msg, len, "camx_op_kv_append", e);
+            (void)hipStreamSynchronize(st);
+            orc_kv_q8_append(k.data(), M, v.data(), M, M, cache.data(), pos, rows, T, &werr);
+        }
+        if (!rc && !(same(dc.download<uint8_t>(), cache) && derr.download<int>()[0] == 0 && werr == 0)) rc = fail(msg, len, "tape-form Q8 KV rows differ from the oracle");
+    }
     if (!rc && camx_add_rms_q8_1(nullptr, nullptr, nullptr, 0, nullptr, 1e-6f, nullptr, nullptr, nullptr, 2048, 1, st) != 1) rc = fail(msg, len, "a null row pointer was not refused");
     (void)hipStreamDestroy(st);
     return rc;
