@@ -699,8 +699,18 @@ def main():
                 ts.append(e0.elapsed_time(e1) * 1e3 / 30)
             ts.sort()
             res[f'{2 * n / 1e6:.1f} MB'] = {'us': round(ts[2], 2), 'GBps': round(2 * n / ts[2] / 1e3, 1), 'frac_of_8TBps': round(2 * n / ts[2] / 1e3 / HBM_PEAK_GBPS, 4)}
+            # the library's own flat copy (camx_copy_cols_bf16 on whole rows: 16 bytes per thread, non-temporal both ways), timed the same way
+            own = []
+            for rep in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for k in range(30): B.call('camx_copy_cols_bf16', _p(src[k % nc]), I(4096), I(0), _p(dst[k % nc]), I(4096), I(0), I(4096), L64(n // 8192))
+                e1.record(); e1.synchronize()
+                own.append(e0.elapsed_time(e1) * 1e3 / 30)
+            own.sort()
+            res[f'{2 * n / 1e6:.1f} MB'].update({'own_copy_us': round(own[2], 2), 'own_copy_frac_of_8TBps': round(2 * n / own[2] / 1e3 / HBM_PEAK_GBPS, 4)})
             del src, dst; torch.cuda.empty_cache()
-        print(json.dumps({'metric': 'device-to-device copy by the runtime, bytes read + written per launch', 'n_gpus': 1, 'copy_sizes': res}))
+        print(json.dumps({'metric': 'device-to-device copy by the runtime and by the library, bytes read + written per launch', 'n_gpus': 1, 'copy_sizes': res}))
         return
     traffic = hbm_traffic()
     NC = a.copies

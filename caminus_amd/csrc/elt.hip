@@ -248,34 +248,29 @@ __global__ void __launch_bounds__(64) gdn_conv_stream(const void * __restrict__ 
         }
     };
     int t = t0;
-    for (; t + 2 * P <= t1; t += P) {                                  // whole groups of eight tokens whose successors are all in the range: no guards
+    // No row past the wave's range is requested: it is another wave's, and would come from HBM twice (with eight rows requested ahead
+    // regardless, 4096 x 10240 read 34 % more than its input, 16384 tokens 17 %). The last group asks for the range's last row again
+    // instead, which is still on its way or in L2 (+ 3 % of reads); a branch around the request would do without that, but with it the
+    // compiler keeps all eight tokens of a group live at once (fp32 rows: 404 registers instead of 92).
+    for (; t + P <= t1; t += P) {                                      // whole groups of eight tokens
 #pragma unroll
         for (int u = 0; u < P; u++) {
             // the whole row is widened before its ring slot is requested again: left to itself the compiler widens half of it later,
             // keeps that half in a copy, and hoists the copies of all eight slots (and the waits for their loads) to the top of the loop
             widen(win[(u + 3) & 3], ring[u]);
+            if constexpr (BF16) {
 #pragma unroll
-            for (int k = 0; k < VW; k++) asm volatile("" : "+v"(win[(u + 3) & 3][k]));
-            __builtin_amdgcn_sched_barrier(0);
-            ring[u] = row(t + u + P);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int k = 0; k < VW; k++) asm volatile("" : "+v"(win[(u + 3) & 3][k]));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            ring[u] = row(t + u + P < t1 ? t + u + P : t1 - 1);
+            if constexpr (BF16) __builtin_amdgcn_sched_barrier(0);
             emit(t + u, u);
         }
-    }
-    // the last whole group requests only rows this wave will use: a row past the range is another wave's, and would come from HBM
-    // twice (with eight rows requested ahead regardless, 4096 x 10240 read 34 % more than its input, 16384 tokens 17 %)
-    if (t + P <= t1) {
-#pragma unroll
-        for (int u = 0; u < P; u++) {
-            widen(win[(u + 3) & 3], ring[u]);
-            if (t + u + P < t1) ring[u] = row(t + u + P);
-            emit(t + u, u);
-        }
-        t += P;
     }
 #pragma unroll
     for (int u = 0; u < P; u++)                                        // the last, partial group
-        if (t + u < t1) { widen(win[(u + 3) & 3], ring[u]); emit(t + u, u); }
+        if (t + u < t1) { widen(win[(u + 3) & 3], ring[u]); emit(t + u, u); __builtin_amdgcn_sched_barrier(0); }
 }
 
 template <bool BF16>
@@ -664,6 +659,11 @@ __global__ void __launch_bounds__(256) copy_cols_bf16_k(const uint16_t * __restr
         out[r * ld_out + c_out + c] = in[r * ld_in + c_in + c];
     }
 }
+// whole contiguous rows (n == ld_in == ld_out): one 16-byte unit per thread, past the caches both ways
+__global__ void __launch_bounds__(256) copy_flat16(const u32x4 * __restrict__ in, u32x4 * __restrict__ out, long n16) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(in + i), out + i);
+}
 // every offset and width a multiple of 8 values: 16-byte units
 __global__ void __launch_bounds__(256) copy_cols_bf16_vec(const u32x4 * __restrict__ in, int ld_in, int c_in, u32x4 * __restrict__ out, int ld_out,
                                                           int c_out, int n, long rows) {
@@ -903,7 +903,10 @@ int camx_cast_bf16(const float * x, uint16_t * out, long n, hipStream_t st) {
 int camx_copy_cols_bf16(const uint16_t * in, int ld_in, int c_in, uint16_t * out, int ld_out, int c_out, int n, long rows, hipStream_t st) {
     if (!in || !out || n < 0 || rows < 0 || c_in < 0 || c_out < 0 || c_in + n > ld_in || c_out + n > ld_out) return CAMX_EINVAL;
     if (n == 0 || rows == 0) return CAMX_OK;
-    if (!((ld_in | c_in | ld_out | c_out | n) & 7) && !(((uintptr_t)in | (uintptr_t)out) & 15) && rows * (n / 8) < 0x7fffffffL * 256)
+    const bool vec = !((ld_in | c_in | ld_out | c_out | n) & 7) && !(((uintptr_t)in | (uintptr_t)out) & 15) && rows * (n / 8) < 0x7fffffffL * 256;
+    if (vec && n == ld_in && n == ld_out)
+        copy_flat16<<<dim3((unsigned)((rows * (n / 8) + 255) / 256)), dim3(256), 0, st>>>((const u32x4 *)in, (u32x4 *)out, rows * (n / 8));
+    else if (vec)
         copy_cols_bf16_vec<<<dim3((unsigned)((rows * (n / 8) + 255) / 256)), dim3(256), 0, st>>>((const u32x4 *)in, ld_in / 8, c_in / 8, (u32x4 *)out, ld_out / 8,
                                                                                                 c_out / 8, n / 8, rows);
     else copy_cols_bf16_k<<<GRID_1D(rows * n), dim3(256), 0, st>>>(in, ld_in, c_in, out, ld_out, c_out, n, rows);

@@ -450,17 +450,30 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     const int lo = 128 * hq + 8 * l16;                                      // this lane's element offset inside a wave step
     constexpr int NW = F32IN ? 2 : 1;
     u32x4 xin[TPW][STEPS][NW];
+    // fp32 rows: a lane's eight values are 32 bytes, so loading them straight into its registers takes two requests that each use half of
+    // every line. The wave's four heads of a step (2 KiB) go to LDS instead, 16 bytes per lane with neighbouring lanes on neighbouring
+    // addresses (whole lines per request, no registers held while they fly), and each lane reads its eight values from there.
+    // (not for the Q8 rows, whose time is their arithmetic: the 24 KiB per workgroup cost them resident waves, 94 -> 101 us at 16384 tokens)
+    constexpr bool STAGE = F32IN && !Q8;
+    __shared__ __attribute__((aligned(16))) float stg[STAGE ? TPW * STEPS * 2048 : 4];
 #pragma unroll
     for (int ti = 0; ti < TPW; ti++) {
         const int tk = t0 + ti < a.n ? t0 + ti : a.n - 1;
         const size_t e = (size_t)tk * a.ldq + 512 * wave + lo;               // heads 16 s + 4 wave .. + 3
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
-            if (F32IN) {
+            if (F32IN && !STAGE) {
                 xin[ti][s][0] = xin[ti][s][NW - 1] = (u32x4){0u, 0u, 0u, 0u};
                 if (16 * s + 4 * wave < items) {
                     const float * p = (const float *)a.qkv + e + 2048 * s;
                     xin[ti][s][0] = __builtin_nontemporal_load((const u32x4 *)p); xin[ti][s][NW - 1] = __builtin_nontemporal_load((const u32x4 *)(p + 4));
+                }
+            } else if (STAGE) {
+                if (16 * s + 4 * wave < items) {
+                    const float * p = (const float *)a.qkv + (size_t)tk * a.ldq + 2048 * s + 512 * wave + 4 * lane;
+                    float * d = stg + (ti * STEPS + s) * 2048 + 512 * wave;
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p, (__attribute__((address_space(3))) void *)d, 16, 0, 2);
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p + 256), (__attribute__((address_space(3))) void *)(d + 256), 16, 0, 2);
                 }
             } else xin[ti][s][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)a.qkv + e + 2048 * s));
         }
@@ -474,7 +487,20 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
         else { const float theta = (float)pos * rope_freq(a.par[256], lane); c = cosf(theta); sn = sinf(theta); }
         rc[wave][lane] = c; rs[wave][lane] = sn;
     }
+    if (STAGE) __builtin_amdgcn_s_waitcnt(0x0f70);                          // vmcnt(0): the wave's own heads have landed in LDS
     __syncthreads();
+    if (STAGE) {
+#pragma unroll
+        for (int ti = 0; ti < TPW; ti++)
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                xin[ti][s][0] = xin[ti][s][NW - 1] = (u32x4){0u, 0u, 0u, 0u};
+                if (16 * s + 4 * wave < items) {
+                    const float * q = stg + (ti * STEPS + s) * 2048 + 512 * wave + lo;
+                    xin[ti][s][0] = *(const u32x4 *)q; xin[ti][s][NW - 1] = *(const u32x4 *)(q + 4);
+                }
+            }
+    }
     const float eps = a.par[257];
 #pragma unroll
     for (int ti = 0; ti < TPW; ti++) {

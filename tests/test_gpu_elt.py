@@ -105,6 +105,9 @@ def test_core_and_fuse():
     dd2 = dev(dst)                                                     # offsets and width in whole 16-byte units
     call('camx_copy_cols_bf16', ptr(dev(m)), I(D), I(8), ptr(dd2), I(64), I(16), I(40), L64(T))
     assert bits_equal(host(dd2, np.uint16), O.copy_cols_bf16(m, 8, dst, 16, 40))
+    whole = rng.integers(0, 65536, (517, 64)).astype(np.uint16); dd3 = dev(np.zeros((517, 64), np.uint16))     # whole contiguous rows: the flat copy
+    call('camx_copy_cols_bf16', ptr(dev(whole)), I(64), I(0), ptr(dd3), I(64), I(0), I(64), L64(517))
+    assert bits_equal(host(dd3, np.uint16), whole)
     ys = O.f2bf(outliers(rng, (4, D))); pos = np.array([-1, 0, 3, -1, 2, 1, -1, -1, 0], np.int32)
     x2 = outliers(rng, (T, D))
     for has in (True, False):
