@@ -276,6 +276,135 @@ __global__ void __launch_bounds__(256) add_rms_rows_any(NormArgs a) {
     }
 }
 
+// The chunk form with a row divided over W waves of the workgroup (W = 4: a workgroup per row; W = 2: two rows): a wave takes the NS
+// slabs part NS .. of its row (N = 256 NS W), so a quarter or half of the row sits in a wave, W times as many waves are in flight, and each
+// stores its part of the residual as soon as its own loads are back. The sum of squares keeps its order: logical thread 4 lane + k chains
+// its elements slab by slab, so the lane's four partial sums go from wave to wave through LDS (part p continues where part p - 1 stopped)
+// and the last part forms the row's total with the same tree. Gamma comes straight into registers (a wave needs NS slabs of it).
+template <int NS, int W, int ADD, int OUT>
+__global__ void __launch_bounds__(256) add_rms_rows_div(NormArgs a) {
+    static_assert(ADD == ADD_NONE || ADD == ADD_F32_SLOTS || ADD == ADD_F32_DIRECT, "the addends of the row kernels");
+    constexpr int N = NS * W * 256, RPW = 4 / W;
+    __shared__ __attribute__((aligned(16))) float chain[RPW][256];
+    __shared__ float totsh[RPW];
+    const int lraw = threadIdx.x & 63, lane = slot_of(lraw), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = wave / W, part = wave % W;
+    const int row = a.row0 + blockIdx.x * RPW + rw;
+    const int e0 = part * (NS * 256) + 4 * lane;                        // this lane's first element of the row
+    float * xr = a.x + (size_t)row * N + e0;
+    f32x4 xv[NS];
+#pragma unroll
+    for (int j = 0; j < NS; j++) xv[j] = __builtin_nontemporal_load((const f32x4 *)(xr + 256 * j));
+    bool added = false;
+    if (ADD == ADD_F32_SLOTS && a.S > 0) {
+        const float * dr = (const float *)a.d + (size_t)row * a.S * N + e0;
+        const float * wr = a.w ? a.w + (size_t)row * a.S : nullptr;
+        f32x4 acc[NS];
+#pragma unroll
+        for (int j = 0; j < NS; j++) acc[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s = 0; s < a.S; s++) {
+            const float ws = wr ? wr[s] : 1.0f;
+            f32x4 dv[NS];
+#pragma unroll
+            for (int j = 0; j < NS; j++) dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + (size_t)s * N + 256 * j));
+#pragma unroll
+            for (int j = 0; j < NS; j++) {
+                if (wr) {
+                    acc[j].x = __builtin_fmaf(ws, dv[j].x, acc[j].x); acc[j].y = __builtin_fmaf(ws, dv[j].y, acc[j].y);
+                    acc[j].z = __builtin_fmaf(ws, dv[j].z, acc[j].z); acc[j].w = __builtin_fmaf(ws, dv[j].w, acc[j].w);
+                } else acc[j] = acc[j] + dv[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NS; j++) xv[j] = xv[j] + acc[j];
+        added = true;
+    }
+    if (ADD == ADD_F32_DIRECT && a.d) {
+        const float * dr = (const float *)a.d + (size_t)row * N + e0;
+        f32x4 dv[NS];
+#pragma unroll
+        for (int j = 0; j < NS; j++) dv[j] = __builtin_nontemporal_load((const f32x4 *)(dr + 256 * j));
+#pragma unroll
+        for (int j = 0; j < NS; j++) xv[j] = xv[j] + dv[j];
+        added = true;
+    }
+    const float * gw = a.nw + (size_t)(row % a.wr) * N + e0;
+    f32x4 g[NS];
+#pragma unroll
+    for (int j = 0; j < NS; j++) g[j] = *(const f32x4 *)(gw + 256 * j);
+    if (added) {
+#pragma unroll
+        for (int j = 0; j < NS; j++) __builtin_nontemporal_store(xv[j], (f32x4 *)(xr + 256 * j));
+    }
+#pragma unroll
+    for (int p = 0; p < W; p++) {
+        if (part == p) {
+            f32x4 ss = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (p) ss = *(const f32x4 *)(chain[rw] + 4 * lraw);
+#pragma unroll
+            for (int j = 0; j < NS; j++) {
+                ss.x = __builtin_fmaf(xv[j].x, xv[j].x, ss.x); ss.y = __builtin_fmaf(xv[j].y, xv[j].y, ss.y);
+                ss.z = __builtin_fmaf(xv[j].z, xv[j].z, ss.z); ss.w = __builtin_fmaf(xv[j].w, xv[j].w, ss.w);
+            }
+            if (p < W - 1) *(f32x4 *)(chain[rw] + 4 * lraw) = ss;
+            else { const float tot = wave_groups_in_order(group32_sum(ss)); if (lraw == 0) totsh[rw] = tot; }
+        }
+        __syncthreads();
+    }
+    const float scale = rsqrt_exact(totsh[rw] / (float)N + a.eps);
+    if ((OUT & NORM_SCL) && part == 0 && lane == 0) a.scl[row] = scale;
+    auto emit = [&](auto redo) {
+        constexpr bool REDO = decltype(redo)::value;
+        bool nan = false;
+#pragma unroll
+        for (int j = 0; j < NS; j++) {
+            const f32x4 gj = g[j];
+            f32x4 t, v;
+            t.x = xv[j].x * scale; t.y = xv[j].y * scale; t.z = xv[j].z * scale; t.w = xv[j].w * scale;
+            v.x = t.x * gj.x; v.y = t.y * gj.y; v.z = t.z * gj.z; v.w = t.w * gj.w;
+            const size_t o = (size_t)row * N + e0 + 256 * j;
+            if (REDO) { *(u32x2 *)(a.hbf + o) = pack_bf16x4_rne(v); continue; }
+            if (OUT & NORM_H) __builtin_nontemporal_store(v, (f32x4 *)(a.h + o));
+            if (OUT & NORM_H16) {
+                u32x2 * p16 = (u32x2 *)(a.h16 + (size_t)row * a.ld16 + e0 + 256 * j);
+                const u32x2 pk = ADD == ADD_F32_DIRECT ? (u32x2){mul_pack_f16x2_once(t.x, gj.x, t.y, gj.y), mul_pack_f16x2_once(t.z, gj.z, t.w, gj.w)}
+                                                       : pack_f16x4(v);
+                __builtin_nontemporal_store(pk, p16);
+            }
+            if (OUT & NORM_HBF) {
+                nan |= any_nan4(v);
+                __builtin_nontemporal_store((u32x2){hw_pk_bf16(v.x, v.y), hw_pk_bf16(v.z, v.w)}, (u32x2 *)(a.hbf + o));
+            }
+            if (OUT & NORM_Q8) q8_1_emit(v, a.q8 + ((size_t)row * (N >> 5) + 8 * (part * NS + j) + (lane >> 3)) * 36, lane & 7);
+        }
+        return nan;
+    };
+    const bool nan = emit(std::false_type{});
+    if ((OUT & NORM_HBF) && __builtin_expect(__builtin_amdgcn_ballot_w64(nan) != 0, 0)) emit(std::true_type{});
+}
+template <int ADD, int OUT>
+static int launch_norm_div(const NormArgs & a, hipStream_t st) {
+    if constexpr (ADD == ADD_NONE || ADD == ADD_F32_SLOTS || ADD == ADD_F32_DIRECT) {
+        // Measured against the wave-per-row chunk form (cold lines): with a q8_1 copy 23.1 -> 22.2 us at 4096 x 2048 (the encode behind the
+        // reduction is a quarter as long per wave), 2560-wide rows over two waves 24.3 -> 23.4 us at 8192 rows, and 1.5 - 2 % from 16384 rows on;
+        // q3p_add_rms16 at 4096 x 2048 is slower this way (26.7 -> 28.3 us) and keeps the wave per row.
+        const int ni = a.N >> 8;
+        if (!((OUT & NORM_Q8) || ni == 10 || a.rows >= 16384)) return 0;
+        const int w = ni == 10 ? 2 : 4, rpw = 4 / w, rows = a.rows - a.rows % rpw;
+        if (rows == 0) return 0;
+        NormArgs b = a; b.rows = rows;
+        const dim3 grid(rows / rpw), block(256);
+        switch (ni) {
+        case 4: add_rms_rows_div<1, 4, ADD, OUT><<<grid, block, 0, st>>>(b); return rows;
+        case 8: add_rms_rows_div<2, 4, ADD, OUT><<<grid, block, 0, st>>>(b); return rows;
+        case 10: add_rms_rows_div<5, 2, ADD, OUT><<<grid, block, 0, st>>>(b); return rows;
+        case 16: add_rms_rows_div<4, 4, ADD, OUT><<<grid, block, 0, st>>>(b); return rows;
+        case 20: add_rms_rows_div<5, 4, ADD, OUT><<<grid, block, 0, st>>>(b); return rows;
+        }
+    }
+    return 0;
+}
+
 // The chunk form of add_rms_rows for one set of copies, if the launch fits it: returns the rows it took (whole workgroups).
 template <int ADD, int OUT>
 static int launch_norm_chunk(const NormArgs & a, hipStream_t st) {
@@ -311,7 +440,7 @@ static int launch_norm(const NormArgs & a0, hipStream_t st) {
     if (vec && a.stream && a.rows >= 1024 && (ADD == ADD_NONE || ADD == ADD_HC || a.d)) {
         const int mask = (a.h ? NORM_H : 0) | (a.h16 ? NORM_H16 : 0) | (a.hbf ? NORM_HBF : 0) | (a.q8 ? NORM_Q8 : 0) | (a.scl ? NORM_SCL : 0);
         int done = 0;
-        (void)((mask == CHUNK_OUTS && ((done = launch_norm_chunk<ADD, CHUNK_OUTS>(a, st)), true)) || ...);
+        (void)((mask == CHUNK_OUTS && ((done = launch_norm_div<ADD, CHUNK_OUTS>(a, st)) || (done = launch_norm_chunk<ADD, CHUNK_OUTS>(a, st)), true)) || ...);
         if (done) {
             const hipError_t e = hipGetLastError();
             if (e != hipSuccess || done == a.rows) return (int)e;

@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize('n,N,S,weighted', [(1, 2048, 1, False), (5, 2048, 8, True), (3, 256, 0, False), (7, 1024, 3, True), (256, 2048, 1, False),
-                                                (1027, 2048, 2, True), (1024, 1024, 1, False), (1030, 2048, 8, False)])
+                                                (1027, 2048, 2, True), (1024, 1024, 1, False), (1030, 2048, 8, False), (16385, 2048, 1, False), (16384, 1024, 3, True)])
 def test_q3p_add_rms16(n, N, S, weighted):
     rng = np.random.default_rng(1001 + n + N + S)
     x = outliers(rng, (n, N)); d = outliers(rng, (n, max(S, 1), N)); w = rng.random((n, max(S, 1))).astype(np.float32)
@@ -33,7 +33,7 @@ def test_q3p_add_rms16(n, N, S, weighted):
     assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(got[:, :N], ref['h16']) and (got[:, N:] == 0x5a5a).all()
 
 
-@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096), (520, 4096), (513, 8192), (600, 3072), (1030, 2560), (1025, 5120), (1024, 4096)])
+@pytest.mark.parametrize('n,N', [(2, 5120), (3, 2560), (1, 8192), (2, 16384), (4, 4096), (520, 4096), (513, 8192), (600, 3072), (1030, 2560), (1025, 5120), (1024, 4096), (16385, 1024), (16384, 5120)])
 def test_q35p_add_rms16(n, N):
     rng = np.random.default_rng(7 + N)
     x = outliers(rng, (n, N)); d = outliers(rng, (n, N)); nw = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
@@ -75,7 +75,7 @@ def test_add_rms_bf16(n, N):
     assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(hbf, np.uint16), ref['hbf'])
 
 
-@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2), (516, 3072, 4), (512, 5120, 1), (1028, 2560, 4), (1026, 2048, 1), (1024, 5120, 4)])
+@pytest.mark.parametrize('R,K,wr', [(8, 2560, 4), (3, 2048, 1), (5, 100, 1), (2, 896, 2), (516, 3072, 4), (512, 5120, 1), (1028, 2560, 4), (1029, 2560, 1), (1026, 2048, 1), (1024, 5120, 4), (16388, 2048, 4)])
 def test_rms_mul_and_rmsnorm(R, K, wr):
     rng = np.random.default_rng(R * K)
     x = outliers(rng, (R, K)); w = (1 + 0.1 * rng.standard_normal((wr, K))).astype(np.float32)
