@@ -610,7 +610,7 @@ int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf,
 int camx_op_rms_mul(const float * x, const float * w, float * y, uint8_t * q8, int R, int wr, int K, float eps, hipStream_t st) {
     if (K < 1 || R < 0 || wr < 1 || !x || !w || (q8 && K % 32)) return CAMX_EINVAL;
     NormArgs a = {(float *)x, nullptr, nullptr, 0, w, wr, eps, y, nullptr, K, nullptr, q8, nullptr, K, R, nullptr, 1, 0.0f};
-    return launch_norm<ADD_NONE>(a, st);
+    return launch_norm<ADD_NONE, NORM_H, NORM_H | NORM_Q8>(a, st);
 }
 
 // pf_hc_post_rms: res [T * HC][N] updated in place, then its norm with w [HC][N]; xn, xnbf, scl optional
@@ -624,7 +624,7 @@ int camx_pf_hc_post_rms(const float * b, const float * inj, float * res, const f
 int camx_rmsnorm_f32(const float * x, const float * w, float * out, int D, float eps, int rows, hipStream_t st) {
     if (D < 1 || rows < 0 || !x || !w || !out) return CAMX_EINVAL;
     NormArgs a = {(float *)x, nullptr, nullptr, 0, w, 1, eps, out, nullptr, D, nullptr, nullptr, nullptr, D, rows, nullptr, 1, 0.0f};
-    return launch_norm<ADD_NONE>(a, st);
+    return launch_norm<ADD_NONE, NORM_H>(a, st);
 }
 
 }   // extern "C"
