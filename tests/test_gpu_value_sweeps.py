@@ -28,6 +28,30 @@ def same_or_nan(got, want):
     return np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan]) and bool(np.isnan(got[nan]).all())
 
 
+@pytest.mark.parametrize('N,S', [(2048, 1), (1024, 3), (4096, 0)])
+def test_norm_chunk_forms_on_extreme_values(N, S):
+    """the same value classes through the forms that take 1024 and more rows (a wave per row, and a row divided over the waves of a
+    workgroup when a q8_1 copy is asked for): every copy against the oracle, NaN for NaN"""
+    rng = np.random.default_rng(4000 + N + S)
+    rows = 1100
+    with np.errstate(all='ignore'):
+        xx = values(rng, (rows, N)); dd = values(rng, (rows, max(S, 1), N)); w = rng.standard_normal((rows, max(S, 1))).astype(f32)
+        nw = (1 + 0.1 * rng.standard_normal(N)).astype(f32)
+        ref = O.add_rms16(xx.copy(), nw, 1e-6, d=dd if S else None, w=w if S else None, S=S, want_q8=True)
+        finite_rows = ~np.isnan(ref['h']).any(1)
+        for with_q8 in (True, False):
+            xd = dev(xx.copy()); h = dev(np.zeros((rows, N), f32)); h16 = dev(np.zeros((rows, N), np.uint16)); q8 = dev(np.zeros((rows, N // 32, 36), np.uint8))
+            if with_q8:
+                call('camx_add_rms_q8_1', ptr(xd), ptr(dev(dd)) if S else NULL, ptr(dev(w)) if S else NULL, I(S), ptr(dev(nw)), F(1e-6), ptr(h), ptr(h16), ptr(q8), I(N), I(rows))
+                assert bits_equal(host(q8)[finite_rows], ref['q8'][finite_rows])
+            elif N <= 2048:
+                call('camx_q3p_add_rms16', ptr(xd), ptr(dev(dd)) if S else NULL, ptr(dev(w)) if S else NULL, I(S), ptr(dev(nw)), F(1e-6), ptr(h), ptr(h16), I(N), I(rows))
+            else:
+                continue
+            assert same_or_nan(host(xd), ref['x']) and same_or_nan(host(h), ref['h'])
+            assert bits_equal(host(h16, np.uint16)[finite_rows], ref['h16'][finite_rows])
+
+
 @pytest.mark.parametrize('seed', range(8))
 def test_quantizers_and_norms(seed):
     rng = np.random.default_rng(1000 + seed)
