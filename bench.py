@@ -810,8 +810,20 @@ def main():
         # the launch-bound op-sets as they would run in a decode loop: each shape's launches captured once into a HIP graph
         # and replayed (every entry point is stream-ordered, allocates nothing and keeps no host state per call)
         graphs = {}
-        for prefix, rep in (('c1_', 1), ('c4_', 1), ('c5_', 1), ('c1_', 8)):      # (x 8: as many launches as a few layers of a decode step queue)
-            fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'six_launches' not in name and not name.endswith('_k')] * rep
+        by_name = {name: fn for name, _, fn in sets}
+        # config 4's row ops of one layer on the dense Q8 line (linear-attention conv + L2, full-attention QK-norm + rotary + Hadamard + Q8 append,
+        # the gate), eight layers in one graph: as the separate launches of the reference's tape and as this library's fused launches
+        layer_sep = (['c4_conv4_silu', 'c4_l2norm_qk', 'c4_dense_q8_qk_nr_hadamard_append_six_launches', 'c4_sigmoid_gate'], 9)
+        layer_fused = (['c4_conv4_silu_l2_one_launch', 'c4_dense_q8_qk_nr_hadamard_append_one_launch', 'c4_sigmoid_gate'], 3)
+        for prefix, rep in (('c1_', 1), ('c4_', 1), ('c5_', 1), ('c1_', 8), (layer_sep, 8), (layer_fused, 8)):      # (x 8: as many launches as a few layers of a decode step queue)
+            if isinstance(prefix, tuple):
+                names, per = prefix
+                if not all(n in by_name for n in names): continue
+                fns = [by_name[n] for n in names] * rep; nl = per * rep
+                prefix = 'c4_layer_separate_' if per == 9 else 'c4_layer_fused_'
+            else:
+                fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'six_launches' not in name and not name.endswith('_k')] * rep
+                nl = len(fns)
             for fn in fns: fn()
             torch.cuda.synchronize()
             gr = torch.cuda.CUDAGraph()
@@ -827,7 +839,7 @@ def main():
             for _ in range(50): gr.replay()
             g1.record(); g1.synchronize()
             us = g0.elapsed_time(g1) * 1e3 / 50
-            graphs[prefix + ('opsets_as_one_graph' if rep == 1 else f'opsets_x{rep}_as_one_graph')] = {'launches': len(fns), 'us_per_replay': round(us, 2), 'us_per_launch': round(us / len(fns), 2)}
+            graphs[prefix + ('opsets_as_one_graph' if rep == 1 else f'opsets_x{rep}_as_one_graph')] = {'launches': nl, 'us_per_replay': round(us, 2), 'us_per_launch': round(us / nl, 2)}
         out['opset_graphs'] = graphs
     if not a.no_cpu and not a.only:
         out['cpu_baseline'] = cpu_baseline(w)
