@@ -239,7 +239,16 @@ def extra_opsets(B):
     out.append(('c4_dense_q8_qk_nr_hadamard_append_one_launch', by4,
                 lambda: B.call('camx_qk_nr_q8', _p(q32), I(2 * D4), I(24), _p(k32), I(M4), _p(v32), I(M4), I(4), _p(w4), _p(wk4), I(64), F(ts7), F(1e-6), I(0), _p(posw), NULL,
                                _p(qo32), _p(cache4), I(rows4), _p(err4), I(T4))))
-    out.append(('_keep4', 0, [l2f, ycf, kx, wk4, ok4, q32, k32, v32, ko32, qo32, vr32, cache4, err4, posw]))
+    # the attention output of the same line: the Hadamard in chunks of 64 and the gate multiply behind it (q35_dense.py:419-420)
+    att32 = B.acts((T4 * 24, D4), torch.float32, 74); gat16 = torch.empty((T4 * 24, D4), dtype=torch.float16, device=B.dev)
+    def att_two():
+        B.call('camx_op_hadamard', _p(att32), I(T4 * 24 * D4 // 64), I(64), I(1))
+        B.call('camx_op_gate_mul16', _p(att32), _p(q32), I(2 * D4), I(D4), _p(gat16), I(T4 * 24 * D4), I(D4))
+    bya = T4 * 24 * D4 * (4 + 4 + 2)
+    out.append(('c4_dense_q8_att_hadamard_gate_two_launches', bya, att_two))
+    out.append(('c4_dense_q8_att_hadamard_gate_one_launch', bya,
+                lambda: B.call('camx_op_hadamard_gate_mul16', _p(att32), NULL, _p(q32), I(2 * D4), I(D4), _p(gat16), I(T4 * 24 * D4), I(D4), I(64))))
+    out.append(('_keep4', 0, [l2f, ycf, kx, wk4, ok4, q32, k32, v32, ko32, qo32, vr32, cache4, err4, posw, att32, gat16]))
     # batched decode: 256 sequences, Q8 KV codec into a paged cache
     S5 = 256
     x5 = B.acts((S5, N), torch.float32, 51); d5 = B.acts((S5, 1, N), torch.float32, 52)
@@ -802,7 +811,8 @@ def main():
         # a fused launch beside the launches it replaces
         for fused, parts in (('c4_conv4_silu_l2_one_launch', ('c4_conv4_silu', 'c4_l2norm_qk')),
                              ('c4_qk_nr_partial_rotary_q_and_k_one_launch', ('c4_qk_nr_partial_rotary_q', 'c4_qk_nr_partial_rotary_k')),
-                             ('c4_dense_q8_qk_nr_hadamard_append_one_launch', ('c4_dense_q8_qk_nr_hadamard_append_six_launches',))):
+                             ('c4_dense_q8_qk_nr_hadamard_append_one_launch', ('c4_dense_q8_qk_nr_hadamard_append_six_launches',)),
+                             ('c4_dense_q8_att_hadamard_gate_one_launch', ('c4_dense_q8_att_hadamard_gate_two_launches',))):
             if fused in ops:
                 for key in ('us', 'us_cache_hot', 'us_queued'):
                     ops[fused][key + '_of_the_launches_it_replaces'] = round(sum(ops[p][key] for p in parts), 2)
@@ -813,16 +823,16 @@ def main():
         by_name = {name: fn for name, _, fn in sets}
         # config 4's row ops of one layer on the dense Q8 line (linear-attention conv + L2, full-attention QK-norm + rotary + Hadamard + Q8 append,
         # the gate), eight layers in one graph: as the separate launches of the reference's tape and as this library's fused launches
-        layer_sep = (['c4_conv4_silu', 'c4_l2norm_qk', 'c4_dense_q8_qk_nr_hadamard_append_six_launches', 'c4_sigmoid_gate'], 9)
-        layer_fused = (['c4_conv4_silu_l2_one_launch', 'c4_dense_q8_qk_nr_hadamard_append_one_launch', 'c4_sigmoid_gate'], 3)
+        layer_sep = (['c4_conv4_silu', 'c4_l2norm_qk', 'c4_dense_q8_qk_nr_hadamard_append_six_launches', 'c4_dense_q8_att_hadamard_gate_two_launches'], 10)
+        layer_fused = (['c4_conv4_silu_l2_one_launch', 'c4_dense_q8_qk_nr_hadamard_append_one_launch', 'c4_dense_q8_att_hadamard_gate_one_launch'], 3)
         for prefix, rep in (('c1_', 1), ('c4_', 1), ('c5_', 1), ('c1_', 8), (layer_sep, 8), (layer_fused, 8)):      # (x 8: as many launches as a few layers of a decode step queue)
             if isinstance(prefix, tuple):
                 names, per = prefix
                 if not all(n in by_name for n in names): continue
                 fns = [by_name[n] for n in names] * rep; nl = per * rep
-                prefix = 'c4_layer_separate_' if per == 9 else 'c4_layer_fused_'
+                prefix = 'c4_layer_separate_' if per == 10 else 'c4_layer_fused_'
             else:
-                fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'six_launches' not in name and not name.endswith('_k')] * rep
+                fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'launches' not in name and not name.endswith('_k')] * rep
                 nl = len(fns)
             for fn in fns: fn()
             torch.cuda.synchronize()

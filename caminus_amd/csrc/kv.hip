@@ -241,6 +241,54 @@ __global__ void __launch_bounds__(256) hadamard_chunks(float * __restrict__ x, l
     if (active) __builtin_nontemporal_store(v, (f32x4 *)(x + c * N + 4 * l));        // (in place and streamed: non-temporal both ways, 107 -> 94 us for 600 MB)
 }
 
+// OP_HADAMARD on the attention output followed by OP_GATE_MUL16 (python/caminus/engine/q35_dense.py:419-420: the dense Q8 line rotates the
+// attention output back in chunks of 64 and multiplies it by the sigmoid of the gate half of the q projection): hadamard_chunks' transform
+// (same pairs, same order, same scale) and gate_mul's fp32 -> fp16 form on the values as the first kernel would have stored them, in one
+// pass; xo (optional) receives the transformed values, as the in-place op would leave them.
+CAMX_DEV float kv_sigmoid_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }      // gate_mul's form for 16-bit outputs
+template <int N>
+__global__ void __launch_bounds__(256) hadamard_gate16_k(const float * __restrict__ x, float * __restrict__ xo, const float * __restrict__ gate,
+                                                         uint16_t * __restrict__ y16, long C, int D, int stride, int off) {
+    constexpr int LPC = N / 4;
+    f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    long c; int l; bool active;
+    if (N == 128) {
+        const int lane = slot_of(threadIdx.x & 63); l = lane & 31;
+        c = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+        active = c < C;
+        if (active) v = __builtin_nontemporal_load((const f32x4 *)(x + c * 128 + 4 * l));
+        v = hadamard128_l4(v, l, false);
+    } else {
+        const int lane = threadIdx.x & 63;
+        c = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / LPC) + lane / LPC;
+        l = lane % LPC;
+        active = c < C;
+        if (active) v = __builtin_nontemporal_load((const f32x4 *)(x + c * N + 4 * l));
+        float a, b;
+        a = v.x; b = v.y; v.x = a + b; v.y = a - b;
+        a = v.z; b = v.w; v.z = a + b; v.w = a - b;
+        a = v.x; b = v.z; v.x = a + b; v.z = a - b;
+        a = v.y; b = v.w; v.y = a + b; v.w = a - b;
+#pragma unroll
+        for (int m = 1; m < LPC; m <<= 1) {
+            const bool hi = (l & m) != 0;
+            const float p0 = __shfl_xor(v.x, m, 64), p1 = __shfl_xor(v.y, m, 64), p2 = __shfl_xor(v.z, m, 64), p3 = __shfl_xor(v.w, m, 64);
+            v.x = hi ? p0 - v.x : v.x + p0; v.y = hi ? p1 - v.y : v.y + p1;
+            v.z = hi ? p2 - v.z : v.z + p2; v.w = hi ? p3 - v.w : v.w + p3;
+        }
+    }
+    const float scale = 1.0f / sqrtf((float)N);
+    v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+    if (!active) return;
+    const long e = c * N + 4 * l, h = e / D;
+    const int d = (int)(e - h * D);
+    if (xo) __builtin_nontemporal_store(v, (f32x4 *)(xo + e));
+    const f32x4 g = __builtin_nontemporal_load((const f32x4 *)(gate + (size_t)h * stride + off + d));
+    f32x4 o;
+    o.x = v.x * kv_sigmoid_fast(g.x); o.y = v.y * kv_sigmoid_fast(g.y); o.z = v.z * kv_sigmoid_fast(g.z); o.w = v.w * kv_sigmoid_fast(g.w);
+    __builtin_nontemporal_store(pack_f16x4(o), (u32x2 *)(y16 + e));
+}
+
 // out-of-place 128-point transform with the literal scale 0x1.6a09e6p-4f (the Q8 KV cache's rotation)
 __global__ void __launch_bounds__(256) hadamard128_heads(const float * __restrict__ x, float * __restrict__ y, long heads) {
     const int lane = slot_of(threadIdx.x & 63);
@@ -326,6 +374,23 @@ int camx_pf_hadamard(float * x, int C, int n, int rpb, hipStream_t st) {
     if (n == 64) hadamard_chunks<64><<<dim3(blocks), dim3(256), 0, st>>>(x, C);
     else if (n == 128) hadamard_chunks<128><<<dim3(blocks), dim3(256), 0, st>>>(x, C);
     else hadamard_chunks<256><<<dim3(blocks), dim3(256), 0, st>>>(x, C);
+    CAMX_LAUNCH_RET();
+}
+
+// OP_HADAMARD (chunks of hn values of a) then OP_GATE_MUL16 in one launch: a fp32 [n] (n = heads * dim values, dim % hn == 0), gate at
+// (i / dim) * head_stride + offset + i % dim, out16 fp16 [n]; a_out (optional, may be a) = the transformed values. Equal to camx_op_hadamard
+// followed by camx_op_gate_mul16 bit for bit.
+int camx_op_hadamard_gate_mul16(const float * a, float * a_out, const float * gate, int head_stride, int offset, uint16_t * out16, int n, int dim, int hn,
+                                hipStream_t st) {
+    if (!a || !gate || !out16 || n < 0 || dim < 1 || (hn != 64 && hn != 128 && hn != 256) || dim % hn || n % dim || head_stride < dim || offset < 0 ||
+        ((head_stride | offset) & 3) || (((uintptr_t)a | (uintptr_t)a_out | (uintptr_t)gate) & 15) || ((uintptr_t)out16 & 7)) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const long C = n / hn;
+    const int cpw = 256 / hn;
+    const unsigned blocks = (unsigned)((C + 4 * cpw - 1) / (4 * cpw));
+    if (hn == 64) hadamard_gate16_k<64><<<dim3(blocks), dim3(256), 0, st>>>(a, a_out, gate, out16, C, dim, head_stride, offset);
+    else if (hn == 128) hadamard_gate16_k<128><<<dim3(blocks), dim3(256), 0, st>>>(a, a_out, gate, out16, C, dim, head_stride, offset);
+    else hadamard_gate16_k<256><<<dim3(blocks), dim3(256), 0, st>>>(a, a_out, gate, out16, C, dim, head_stride, offset);
     CAMX_LAUNCH_RET();
 }
 

@@ -133,6 +133,15 @@ class TapeOps:
         assert out16.dtype == self._torch.float16 and out16.numel() >= n
         return self._go('camx_op_gate_mul16', self._p(a), self._p(gate), I(head_stride), I(offset), self._p(out16), I(n), I(dim))
 
+    def hadamard_gate_mul16(self, a, n, gate, head_stride, offset, out16, dim, keep=True, dep=-1, team=-1):
+        """hadamard(a, n) then gate_mul16(a, gate, head_stride, offset, out16, dim) in one launch (the dense Q8 line's attention output:
+        python/caminus/engine/q35_dense.py:419-420); keep: a is left transformed, as the in-place op leaves it"""
+        I = self._C.c_int
+        ne = a.numel(); assert n in (64, 128, 256) and dim % n == 0 and ne % dim == 0
+        assert gate.numel() >= (ne // dim - 1) * head_stride + offset + dim and out16.dtype == self._torch.float16 and out16.numel() >= ne
+        return self._go('camx_op_hadamard_gate_mul16', self._p(a), self._p(a if keep else None), self._p(gate), I(head_stride), I(offset), self._p(out16),
+                        I(ne), I(dim), I(n))
+
     def gdn_l2(self, x, out, heads, dim, eps, x_stride=0, dep=-1, team=-1):
         I, F = self._C.c_int, self._C.c_float
         return self._go('camx_op_gdn_l2', self._p(x), self._p(out), I(heads), I(dim), F(np.float32(eps / dim)), I(x_stride), I(self.T))

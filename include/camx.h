@@ -105,6 +105,12 @@ int camx_op_kv_append(const float * k, const float * v, void * cache, const int3
 int camx_op_hadamard(float * x, int C, int n, int rows_per_task, camx_stream_t stream);
 /* OP_GATE_MUL16 (k3.py:1209-1219; kernels/k3_q35_ops.h:381-391): a, W = gate, y = out16 fp16, N = n, K = dim, pad1 = head_stride, pad2 = offset. */
 int camx_op_gate_mul16(const float * a, const float * gate, int head_stride, int offset, uint16_t * out16, int n, int dim, camx_stream_t stream);
+/* The dense Q8 line's OP_HADAMARD on the attention output and the OP_GATE_MUL16 behind it in one launch (python/caminus/engine/q35_dense.py:419-420):
+ * chunks of hn in {64, 128, 256} values of a are transformed, then multiplied by the gate as above; a_out (optional, may be a) receives the
+ * transformed values. dim % hn == 0, n % dim == 0, head_stride and offset multiples of 4, 16-byte aligned a / gate. Every bit equals
+ * camx_op_hadamard followed by camx_op_gate_mul16. */
+int camx_op_hadamard_gate_mul16(const float * a, float * a_out, const float * gate, int head_stride, int offset, uint16_t * out16, int n, int dim,
+                                int hn, camx_stream_t stream);
 /* OP_GDN_L2 (k3.py:1002-1008; kernels/k3_q35_ops.h:181-194): a = x, y = out, rs = eps / dim, N = T * heads, K = dim, pad1 = x_stride (0: heads * dim). */
 int camx_op_gdn_l2(const float * x, float * out, int heads, int dim, float rs, int x_stride, int T, camx_stream_t stream);
 /* OP_OWN_SWIGLU16 (k3.py:854-860; kernels/k3_own_ops.h:258-262): a = g, W = u, y = y16, N = n. */

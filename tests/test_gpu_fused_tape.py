@@ -220,6 +220,28 @@ def test_op_kv_append_three_row_formats(M, T):
     assert rerr == 0 and bits_equal(host(c).reshape(-1), rc.reshape(-1))
 
 
+@pytest.mark.parametrize('T,nh,D,n', [(16, 24, 256, 64), (1, 24, 256, 64), (3, 5, 256, 256), (7, 12, 128, 128), (300, 24, 256, 64)])
+def test_hadamard_gate_mul16_equals_the_two_tape_ops(T, nh, D, n):
+    """the attention output's Hadamard and the gate multiply behind it in one launch: out16 and the transformed values carry the bits of
+    camx_op_hadamard followed by camx_op_gate_mul16; with a_out NULL the input is left as it was"""
+    rng = np.random.default_rng(420 + T + n)
+    a = outliers(rng, (T * nh, D)); qg = outliers(rng, (T * nh, 2 * D))
+    a1 = dev(a); qgd = dev(qg); y1 = dev(np.zeros((T * nh, D), np.uint16))
+    call('camx_op_hadamard', ptr(a1), I(a.size // n), I(n), I(1))
+    call('camx_op_gate_mul16', ptr(a1), ptr(qgd), I(2 * D), I(D), ptr(y1), I(a.size), I(D))
+    a2 = dev(a); y2 = dev(np.ones((T * nh, D), np.uint16))
+    call('camx_op_hadamard_gate_mul16', ptr(a2), ptr(a2), ptr(qgd), I(2 * D), I(D), ptr(y2), I(a.size), I(D), I(n))
+    assert torch.equal(y1, y2) and torch.equal(a1, a2)
+    a3 = dev(a); y3 = dev(np.ones((T * nh, D), np.uint16))
+    call('camx_op_hadamard_gate_mul16', ptr(a3), NULL, ptr(qgd), I(2 * D), I(D), ptr(y3), I(a.size), I(D), I(n))
+    assert torch.equal(y1, y3) and bits_equal(host(a3), a)
+    ref = O.gate_mul(O.hadamard_n(a, n).reshape(a.shape), qg, D, 2 * D, D, f16=True)
+    assert close_16(host(y2, np.uint16), ref, 'f16')
+    for bad in ((I(a.size), I(D), I(32)), (I(a.size), I(D + 32), I(n)), (I(a.size - 4), I(D), I(n))):          # a chunk size, a head and a length that do not fit
+        p = lambda t: C.c_void_p(t.data_ptr())
+        assert camx().camx_op_hadamard_gate_mul16(p(a2), NULL, p(qgd), I(2 * D), I(D), p(y2), *bad, stream()) == 1
+
+
 def test_thin_tape_ops_equal_their_prefill_namesakes():
     rng = np.random.default_rng(31)
     x = outliers(rng, (64, 256)); xa, xb = dev(x), dev(x)
