@@ -176,6 +176,23 @@ def extra_opsets(B):
     n = 8 * 768
     g = B.acts((n,), torch.float32, 16); u = B.acts((n,), torch.float32, 17); y16 = torch.empty(n, dtype=torch.float16, device=B.dev)
     out.append(('c1_swiglu', n * 10, lambda: B.call('camx_q3p_swiglu', _p(g), _p(u), _p(y16), I(n))))
+    # the decode token's attention inputs as the reference's tape chains them (python/caminus/engine/q3moe_one.py:316-318): OP_QK_NR (k) ->
+    # OP_KV_APPEND (fp16 rows) and OP_QK_NR (q), three launches, and the one that replaces them
+    hd1, M1 = 128, nkv * 128
+    q1 = B.acts((nh, hd1), torch.float32, 18); k1 = B.acts((nkv, hd1), torch.float32, 19); v1 = B.acts((1, M1), torch.float32, 20)
+    wq1 = B.gamma(hd1, 21); wk1 = B.gamma(hd1, 22); qo1 = torch.empty((nh, hd1), device=B.dev); ko1 = torch.empty((nkv, hd1), device=B.dev)
+    posw1 = torch.tensor([1234], dtype=torch.int32, device=B.dev); err1 = torch.zeros(1, dtype=torch.int32, device=B.dev)
+    ts6 = float(np.float32(np.float32(1e6) ** np.float32(-2.0 / hd1))); eb1 = int(np.array([1e-6], np.float32).view(np.int32)[0])
+    def nr_kv_three():
+        B.call('camx_op_qk_nr', _p(k1), I(hd1), I(nkv), I(hd1), _p(wk1), _p(posw1), _p(ko1), I(hd1), F(ts6), I(eb1), I(1))
+        B.call('camx_op_kv_append', _p(ko1), _p(v1), _p(cache), _p(posw1), I(M1), I(0), _p(err1), I(4096), I(1))
+        B.call('camx_op_qk_nr', _p(q1), I(hd1), I(nh), I(hd1), _p(wq1), _p(posw1), _p(qo1), I(hd1), F(ts6), I(eb1), I(1))
+    by1 = (nh + 2 * nkv) * hd1 * 4 + 2 * hd1 * 4 + nh * hd1 * 4 + 2 * M1 * 2
+    out.append(('c1_qk_nr_kv_append_three_launches', by1, nr_kv_three))
+    out.append(('c1_qk_nr_kv_append_one_launch', by1,
+                lambda: B.call('camx_qk_nr_kv', _p(q1), I(hd1), I(nh), _p(wq1), _p(k1), I(hd1), _p(v1), I(M1), I(nkv), _p(wk1), I(hd1), I(hd1), F(ts6), F(1e-6), I(0),
+                               _p(posw1), NULL, _p(qo1), NULL, _p(cache), I(0), I(4096), _p(err1), I(1))))
+    out.append(('_keep1', 0, [q1, k1, v1, wq1, wk1, qo1, ko1, posw1, err1]))
     # embedding gather, 151936 x 2048, 256 ids
     V, n_tok = 151936, 256
     rng = np.random.default_rng(1002)
@@ -812,7 +829,8 @@ def main():
         for fused, parts in (('c4_conv4_silu_l2_one_launch', ('c4_conv4_silu', 'c4_l2norm_qk')),
                              ('c4_qk_nr_partial_rotary_q_and_k_one_launch', ('c4_qk_nr_partial_rotary_q', 'c4_qk_nr_partial_rotary_k')),
                              ('c4_dense_q8_qk_nr_hadamard_append_one_launch', ('c4_dense_q8_qk_nr_hadamard_append_six_launches',)),
-                             ('c4_dense_q8_att_hadamard_gate_one_launch', ('c4_dense_q8_att_hadamard_gate_two_launches',))):
+                             ('c4_dense_q8_att_hadamard_gate_one_launch', ('c4_dense_q8_att_hadamard_gate_two_launches',)),
+                             ('c1_qk_nr_kv_append_one_launch', ('c1_qk_nr_kv_append_three_launches',))):
             if fused in ops:
                 for key in ('us', 'us_cache_hot', 'us_queued'):
                     ops[fused][key + '_of_the_launches_it_replaces'] = round(sum(ops[p][key] for p in parts), 2)

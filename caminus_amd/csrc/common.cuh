@@ -186,6 +186,20 @@ CAMX_DEV void q8_1_emit(f32x4 v, uint8_t * blk, int sub) {
     if (sub == 0) *(uint32_t *)blk = (uint32_t)f2h_bits(d) | ((uint32_t)f2h_bits(sum) << 16);
 }
 
+// ---- q8_0 (ggml 34-byte block) of 32 values held by 8 lanes x 4 registers; sub = lane & 7 -------------------------------
+// d = amax / 127 stored as half, codes roundf(x * (1 / d)) (the cache writer's form: kernels/k3_gguf_ops.h:1520-1553). Every lane of
+// the group takes part in the max; active = false: no store.
+CAMX_DEV void pf_q8_0_emit(f32x4 xv, uint8_t * blk, int sub, bool active) {        // 8 lanes x 4 values: one block
+    const float amax = group8_max(absmax4(xv));
+    const float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
+    if (!active) return;
+    f32x4 t; t.x = xv.x * id; t.y = xv.y * id; t.z = xv.z * id; t.w = xv.w * id;
+    const uint32_t q = pack_round_i8x4(t);
+    uint16_t * o = (uint16_t *)(blk + 2 + 4 * sub);
+    o[0] = (uint16_t)q; o[1] = (uint16_t)(q >> 16);
+    if (sub == 0) *(uint16_t *)blk = f2h_bits(d);
+}
+
 // ---- q8_1 block of 32 consecutive floats in LDS, all of it in one lane -------------------------------------------------------
 // in: the block's 32 values; out: its 9 dwords (LDS); rot: the lane's number (the pieces are read in the order rot, rot + 1, ..
 // mod 8, so that the lanes of a request fall on different banks). The sum keeps the 32-thread butterfly's tree (xor 16, 8, 4, 2, 1

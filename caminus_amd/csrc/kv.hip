@@ -70,16 +70,6 @@ __global__ void __launch_bounds__(256) kv_q8_append_wave_rows(const float * __re
 }
 
 // pf_kv_append (q8_0 rows): no refusal rules; d stored as half, codes roundf(x * (1 / d)); err bit 1 for a row outside
-CAMX_DEV void pf_q8_0_emit(f32x4 xv, uint8_t * blk, int sub, bool active) {        // 8 lanes x 4 values: one block
-    const float amax = group8_max(absmax4(xv));
-    const float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
-    if (!active) return;
-    f32x4 t; t.x = xv.x * id; t.y = xv.y * id; t.z = xv.z * id; t.w = xv.w * id;
-    const uint32_t q = pack_round_i8x4(t);
-    uint16_t * o = (uint16_t *)(blk + 2 + 4 * sub);
-    o[0] = (uint16_t)q; o[1] = (uint16_t)(q >> 16);
-    if (sub == 0) *(uint16_t *)blk = f2h_bits(d);
-}
 __global__ void __launch_bounds__(256) pf_kv_append_rows(const float * __restrict__ k, int ldk, const float * __restrict__ v, int ldv, int M,
                                                          uint8_t * __restrict__ cache, int pos0, int rows, int * __restrict__ err,
                                                          const int32_t * __restrict__ posb = nullptr) {

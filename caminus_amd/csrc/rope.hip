@@ -668,21 +668,49 @@ struct NrArgs {
     const void * x; int head_stride, heads; const float * w; int D, nrot; float theta_scale, eps; int pos0; const int32_t * pos; void * out; int T;
     const int32_t * posb;            // the tape's device-resident position: row r sits at posb[0] + r (pos and pos0 unused)
     const void * x2; int head_stride2, heads2; const float * w2; void * out2;   // a second group of heads per token (k beside q); qk_nr_heads only
+    const float * v; int ldv; void * cache; int rows; int * err;                // qk_nr_heads<.., KV>: the token's v row and the cache that takes k and v
 };
-CAMX_DEV float nr_pos(const NrArgs & a, int tok) { return (float)(a.pos ? a.pos[tok] : (a.posb ? a.posb[0] : a.pos0) + tok); }
+CAMX_DEV int nr_posi(const NrArgs & a, int tok) { return a.pos ? a.pos[tok] : (a.posb ? a.posb[0] : a.pos0) + tok; }
+CAMX_DEV float nr_pos(const NrArgs & a, int tok) { return (float)nr_posi(a, tok); }
 // One wave per (token, head), four per workgroup, nothing shared between them: each wave issues its head's loads, computes
 // the token's cos / sin for the rotated pairs into its own LDS rows while they are in flight, normalizes, parks the normed
 // head in LDS for the partner reads of the rotation, and stores. No barrier; a verify batch of 16 tokens x 28 heads is 448
 // independent waves instead of 16 workgroups that loop over their heads.
-template <bool BF16, bool VEC>
+// KV 1 / 2 (fp32, VEC): the tape's OP_KV_APPEND behind the k heads' OP_QK_NR in the same launch. Each token has heads2 more waves, one per
+// head of its v row; the k heads' results and the v heads go to cache row position(token) as OP_KV_APPEND writes them from the fp32
+// buffers (1: fp16 [K | V], kv_append16_k; 2: ggml q8_0 blocks, K's then V's, pf_kv_append_rows: a lane's 4 values and its 8-lane group
+// are one block's), out2 only if given. A position outside [0, rows): err bit 1, the cache row is not written, the fp32 outputs are.
+template <bool BF16, bool VEC, int KV = 0>
 __global__ void __launch_bounds__(256) qk_nr_heads(NrArgs a) {
     __shared__ float rc[4][256], rs[4][256];
     __shared__ __attribute__((aligned(16))) float nrm[4][512];
     const int tid = threadIdx.x, lraw = tid & 63, lane = slot_of(lraw), wave = tid >> 6, half = a.nrot / 2;
     const long gw = (long)blockIdx.x * 4 + wave;
-    const int hpt = a.heads + a.heads2;                          // heads per token over both groups
+    const int hpt = a.heads + a.heads2 + (KV ? a.heads2 : 0);    // heads per token over the groups
     if (gw >= (long)a.T * hpt) return;
     const int tok = (int)(gw / hpt), hh = (int)(gw - (long)tok * hpt);
+    [[maybe_unused]] bool row_ok = true;
+    [[maybe_unused]] size_t M = 0;
+    if constexpr (KV != 0) {
+        const long p = nr_posi(a, tok);
+        row_ok = p >= 0 && p < a.rows;
+        M = (size_t)a.heads2 * a.D;
+        if (hh >= a.heads + a.heads2) {                           // (wave-uniform) a head of the token's v row: no arithmetic but the cache's
+            const int hv = hh - a.heads - a.heads2;
+            if (!row_ok) { if (hv == 0 && lraw == 0) atomicOr(a.err, 1); return; }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int i0 = 256 * j + 4 * lane;
+                const bool in = i0 < a.D;
+                f32x4 vv = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (in) vv = *(const f32x4 *)(a.v + (size_t)tok * a.ldv + (size_t)hv * a.D + i0);
+                const size_t e = M + (size_t)hv * a.D + i0;      // the value's index in the cache row's [K | V]
+                if (KV == 1) { if (in) *(u32x2 *)((uint16_t *)a.cache + (size_t)p * 2 * M + e) = pack_f16x4(vv); }
+                else if (256 * j < a.D) pf_q8_0_emit(vv, (uint8_t *)a.cache + ((size_t)p * (2 * M / 32) + (in ? e / 32 : 0)) * 34, lane & 7, in);
+            }
+            return;
+        }
+    }
     const bool g2 = hh >= a.heads;                               // (wave-uniform) this head belongs to the second group
     if (g2) { a.x = a.x2; a.w = a.w2; a.out = a.out2; a.head_stride = a.head_stride2; }
     const size_t hi = g2 ? (size_t)tok * a.heads2 + (hh - a.heads) : (size_t)tok * a.heads + hh;
@@ -746,6 +774,19 @@ __global__ void __launch_bounds__(256) qk_nr_heads(NrArgs a) {
             }
         }
         const int i0 = 256 * j + 4 * lane;
+        if constexpr (KV != 0) {
+            if (g2) {                                            // a k head: the cache row's K part (and the fp32 buffer only if the caller keeps one)
+                const bool in = i0 < a.D;
+                const f32x4 v = {y[0], y[1], y[2], y[3]};
+                if (in && a.out) *(f32x4 *)((float *)a.out + yo + i0) = v;
+                if (!row_ok) continue;                           // (the token's first v wave reports it)
+                const long p = nr_posi(a, tok);
+                const size_t e = (size_t)(hh - a.heads) * a.D + i0;
+                if (KV == 1) { if (in) *(u32x2 *)((uint16_t *)a.cache + (size_t)p * 2 * M + e) = pack_f16x4(v); }
+                else if (256 * j < a.D) pf_q8_0_emit(v, (uint8_t *)a.cache + ((size_t)p * (2 * M / 32) + (in ? e / 32 : 0)) * 34, lane & 7, in);
+                continue;
+            }
+        }
         if (VEC) {
             if (i0 < a.D) {
                 const f32x4 v = {y[0], y[1], y[2], y[3]};
@@ -1285,6 +1326,26 @@ int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const
     const dim3 grid((unsigned)(((long)T * (nh + nkv) + 3) / 4)), block(256);
     if (io) { if (vec) qk_nr_heads<true, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<true, false><<<grid, block, 0, st>>>(a); }
     else { if (vec) qk_nr_heads<false, true><<<grid, block, 0, st>>>(a); else qk_nr_heads<false, false><<<grid, block, 0, st>>>(a); }
+    CAMX_LAUNCH_RET();
+}
+// The fp16 / q8_0 cache lines' three tape segments in one launch: OP_QK_NR (k) -> OP_KV_APPEND and OP_QK_NR (q) (python/caminus/engine/
+// q3moe_one.py:316-318, 368-370; python/caminus/engine/q35_dense.py:414-417; kernels/k3_gguf_ops.h:1520-1553). q, k heads and positions as
+// camx_qk_nr_qk (fp32); v fp32 [T][nkv * D] at ldv; qo [T][nh][D]; ko [T][nkv][D] optional (NULL: the normed k only reaches the cache);
+// cache row position(t): work 0 fp16 [K | V] (8-byte aligned), work 1 ggml q8_0 blocks (D % 32 == 0). err bit 1: a position outside
+// [0, rows) (that cache row is not written; qo and ko are). D % 4 == 0, strides % 4 == 0, 16-byte aligned fp32 pointers.
+int camx_qk_nr_kv(const float * q, int q_stride, int nh, const float * wq, const float * k, int k_stride, const float * v, int ldv, int nkv, const float * wk,
+                  int D, int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, float * qo, float * ko, void * cache,
+                  int work, int rows, int * err, int T, hipStream_t st) {
+    if (!q || !k || !v || !wq || !wk || !qo || !cache || !err || T < 0 || nh < 1 || nkv < 1 || D < 4 || D > 512 || (D & 3) || q_stride < D || k_stride < D ||
+        ((q_stride | k_stride | ldv) & 3) || (long)nkv * D > 0x7fffffffL || ldv < nkv * D || nrot < 0 || nrot > D || (nrot & 1) || work < 0 || work > 1 ||
+        (work == 1 && (D & 31)) || rows < 1 || (!pos && !pos_dev && (pos0 < 0 || pos0 > 0x7fffffff - T)) ||
+        (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)qo | (uintptr_t)ko) & 15) || ((uintptr_t)cache & (work ? 1 : 7))) return CAMX_EINVAL;
+    if (T == 0) return CAMX_OK;
+    NrArgs a = {q, q_stride, nh, wq, D, nrot, theta_scale, eps, pos0, pos, qo, T, pos_dev, k, k_stride, nkv, wk, ko, v, ldv, cache, rows, err};
+    const long waves = (long)T * (nh + 2 * nkv);
+    if ((waves + 3) / 4 > 0x7fffffffL) return CAMX_EINVAL;
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    if (work) qk_nr_heads<false, true, 2><<<grid, block, 0, st>>>(a); else qk_nr_heads<false, true, 1><<<grid, block, 0, st>>>(a);
     CAMX_LAUNCH_RET();
 }
 // The dense Q8 line's six segments in one launch (see qk_nr_q8_k): heads of 256 dims. q [T][nh] heads at q_stride floats (the q | gate

@@ -167,3 +167,18 @@ class TapeOps:
         rows = kv_rows(cache, M, True)
         return self._go('camx_qk_nr_q8', self._p(q), I(q_head_stride), I(heads), self._p(k), I(M), self._p(v), I(M), I(kv_heads), self._p(qn), self._p(kn), I(n_rot),
                         F(theta_scale), F(eps), I(0), self._p(pos), self._p(None), self._p(qo), self._p(cache), I(rows), self._p(self.kv_error), I(self.T))
+
+    def qk_nr_kv(self, q, q_head_stride, heads, k, k_head_stride, v, kv_heads, dim, qn, kn, pos, qo, cache, n_rot, theta_scale, eps, ko=None, q8=False,
+                 dep=-1, team=-1):
+        """qk_nr(k) -> kv_append(ko, v, cache, pos, q8) and qk_nr(q) in one launch (the fp16 and q8_0 cache lines:
+        python/caminus/engine/q3moe_one.py:316-318); ko: the buffer the separate ops pass between them, written only if given"""
+        I, F = self._C.c_int, self._C.c_float
+        M = kv_heads * dim
+        if q8 and self.kv_q8_dense: raise ValueError('qk_nr_kv: the dense Q8 line has its own chain (qk_nr_q8)')
+        if v.numel() != self.T * M: raise ValueError('qk_nr_kv: V must contain a whole row per pass token')
+        rows = kv_rows(cache, M, q8)
+        if rows < self.T: raise ValueError('qk_nr_kv: fewer physical cache rows than pass tokens')
+        if self.kv_error is None: raise ValueError('qk_nr_kv: an int32 error word (kv_error) receives the span bit')
+        return self._go('camx_qk_nr_kv', self._p(q), I(q_head_stride), I(heads), self._p(qn), self._p(k), I(k_head_stride), self._p(v), I(M), I(kv_heads), self._p(kn),
+                        I(dim), I(n_rot), F(theta_scale), F(eps), I(0), self._p(pos), self._p(None), self._p(qo), self._p(ko), self._p(cache), I(1 if q8 else 0),
+                        I(rows), self._p(self.kv_error), I(self.T))

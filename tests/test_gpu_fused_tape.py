@@ -179,6 +179,78 @@ def test_qk_nr_qk_equals_two_launches(T, nh, nkv, D, nrot, io):
         assert torch.equal(oq1, oq2) and torch.equal(ok1, ok2)
 
 
+@pytest.mark.parametrize('work', [0, 1])
+@pytest.mark.parametrize('T,nh,nkv,D,nrot', [(1, 32, 4, 128, 128), (16, 24, 4, 256, 64), (3, 5, 2, 96, 32), (2, 3, 1, 512, 64), (5, 2, 3, 32, 8), (300, 8, 2, 128, 128)])
+def test_qk_nr_kv_equals_the_three_tape_ops(T, nh, nkv, D, nrot, work):
+    """q and k norm + rotary and the cache append in one launch against OP_QK_NR (k), OP_KV_APPEND, OP_QK_NR (q) one after another:
+    the fp32 outputs and every byte of the cache (fp16 rows and q8_0 rows), with the position on the device, on the host, per row,
+    and with tokens that fall outside the cache."""
+    rng = np.random.default_rng(T + nh + D + work)
+    M = nkv * D; qs, ks, ldv = 2 * D, D + 8, M + 4
+    xq = outliers(rng, (T * nh, qs)); xk = outliers(rng, (T * nkv, ks)); xv = outliers(rng, (T, ldv))
+    wq = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32); wk = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    ts = _theta(1e7, nrot); eb = int(np.array([1e-6], np.float32).view(np.int32)[0])
+    xqd, xkd, xvd, wqd, wkd = dev(xq), dev(xk), dev(xv), dev(wq), dev(wk)
+    vc = dev(np.ascontiguousarray(xv[:, :M]))                          # OP_KV_APPEND reads v at stride M
+    rows = 40 + T; rb = 2 * M * 2 if work == 0 else 2 * (M // 32) * 34
+    def three(p0):
+        pd = dev(np.array([p0], np.int32))
+        oq = dev(np.zeros((T * nh, D), np.float32)); ok = dev(np.zeros((T * nkv, D), np.float32))
+        c = dev(np.full((rows, rb), 0xa5, np.uint8)); e = dev(np.zeros(1, np.int32))
+        call('camx_op_qk_nr', ptr(xkd), I(ks), I(nkv), I(D), ptr(wkd), ptr(pd), ptr(ok), I(nrot), F(ts), I(eb), I(T))
+        call('camx_op_kv_append', ptr(ok), ptr(vc), ptr(c), ptr(pd), I(M), I(work), ptr(e), I(rows), I(T))
+        call('camx_op_qk_nr', ptr(xqd), I(qs), I(nh), I(D), ptr(wqd), ptr(pd), ptr(oq), I(nrot), F(ts), I(eb), I(T))
+        return oq, ok, c, int(host(e)[0])
+    for p0 in (0, 17, 40, 40 + T - 1 if T > 1 else 39):              # the last ones push tokens past the cache's end
+        oq1, ok1, c1, e1 = three(p0)
+        assert e1 == (1 if p0 + T > rows else 0)
+        for pd, ph, keep in ((dev(np.array([p0], np.int32)), 0, True), (None, p0, True), (None, p0, False)):
+            oq2 = dev(np.full((T * nh, D), 5, np.float32)); ok2 = dev(np.full((T * nkv, D), 5, np.float32))
+            c2 = dev(np.full((rows, rb), 0xa5, np.uint8)); e2 = dev(np.zeros(1, np.int32))
+            call('camx_qk_nr_kv', ptr(xqd), I(qs), I(nh), ptr(wqd), ptr(xkd), I(ks), ptr(xvd), I(ldv), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6),
+                 I(ph), ptr(pd), NULL, ptr(oq2), ptr(ok2) if keep else NULL, ptr(c2), I(work), I(rows), ptr(e2), I(T))
+            assert torch.equal(oq1, oq2) and torch.equal(c1, c2) and int(host(e2)[0]) == e1
+            assert torch.equal(ok1, ok2) if keep else bool((ok2 == 5).all())
+    # one position per row (a verify batch): the cache row is the token's position
+    pos = rng.permutation(rows + 3)[:T].astype(np.int32) - 1         # distinct; may hold -1 and rows .. rows + 1
+    posd = dev(pos)
+    oq1 = dev(np.zeros((T * nh, D), np.float32)); ok1 = dev(np.zeros((T * nkv, D), np.float32)); c1 = dev(np.full((rows, rb), 0xa5, np.uint8))
+    call('camx_qk_nr_pos', ptr(xqd), I(qs), I(nh), ptr(wqd), I(D), I(nrot), F(ts), F(1e-6), ptr(posd), ptr(oq1), I(T), I(0))
+    call('camx_qk_nr_pos', ptr(xkd), I(ks), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6), ptr(posd), ptr(ok1), I(T), I(0))
+    bad = False
+    for t in range(T):
+        if 0 <= pos[t] < rows:
+            e = dev(np.zeros(1, np.int32))
+            call('camx_op_kv_append', ptr(ok1[t * nkv:(t + 1) * nkv]), ptr(vc[t:t + 1]), ptr(c1), ptr(posd[t:t + 1]), I(M), I(work), ptr(e), I(rows), I(1))
+            assert int(host(e)[0]) == 0
+        else:
+            bad = True
+    oq2 = dev(np.full((T * nh, D), 5, np.float32)); ok2 = dev(np.full((T * nkv, D), 5, np.float32))
+    c2 = dev(np.full((rows, rb), 0xa5, np.uint8)); e2 = dev(np.zeros(1, np.int32))
+    call('camx_qk_nr_kv', ptr(xqd), I(qs), I(nh), ptr(wqd), ptr(xkd), I(ks), ptr(xvd), I(ldv), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6),
+         I(0), NULL, ptr(posd), ptr(oq2), ptr(ok2), ptr(c2), I(work), I(rows), ptr(e2), I(T))
+    assert torch.equal(oq1, oq2) and torch.equal(ok1, ok2) and torch.equal(c1, c2) and int(host(e2)[0]) == (1 if bad else 0)
+
+
+def test_qk_nr_kv_refusals():
+    D, nh, nkv, T = 128, 4, 2, 2; M = nkv * D
+    L = camx(); p = lambda t: C.c_void_p(t.data_ptr())
+    q = dev(np.zeros((T * nh, D), np.float32)); k = dev(np.zeros((T * nkv, D), np.float32)); v = dev(np.zeros((T, M), np.float32)); w = dev(np.ones(D, np.float32))
+    qo = dev(np.zeros((T * nh, D), np.float32)); c = dev(np.zeros((8, 4 * M), np.uint8)); e = dev(np.zeros(1, np.int32))
+    def rc(**kw):
+        a = dict(q=p(q), qs=D, k=p(k), ks=D, v=p(v), ldv=M, D=D, nrot=64, pos0=0, cache=p(c), work=0, rows=8, err=p(e), T=T)
+        a.update(kw)
+        r = L.camx_qk_nr_kv(a['q'], I(a['qs']), I(nh), p(w), a['k'], I(a['ks']), a['v'], I(a['ldv']), I(nkv), p(w), I(a['D']), I(a['nrot']), F(1e-4), F(1e-6),
+                            I(a['pos0']), NULL, NULL, p(qo), NULL, a['cache'], I(a['work']), I(a['rows']), a['err'], I(a['T']), stream())
+        torch.cuda.synchronize()
+        return r
+    assert rc() == 0 and rc(T=0) == 0 and rc(work=1) == 0
+    for kw in (dict(D=126), dict(D=80, work=1), dict(qs=D + 2), dict(ks=D - 4), dict(ldv=M - 4), dict(nrot=D + 2), dict(nrot=3), dict(work=2), dict(rows=0),
+               dict(pos0=-1), dict(pos0=0x7fffffff), dict(cache=NULL), dict(err=NULL), dict(q=C.c_void_p(q.data_ptr() + 4)), dict(cache=C.c_void_p(c.data_ptr() + 2)),
+               dict(T=-1)):
+        assert rc(**kw) == 1, kw
+
+
 # ---- tape-shaped entry points: the position is a device word --------------------------------------------------------------------------
 @pytest.mark.parametrize('T,heads,D,nrot,stride', [(1, 24, 256, 64, 512), (16, 4, 256, 64, 256), (3, 5, 128, 128, 128), (2, 3, 96, 32, 100), (600, 8, 256, 64, 256)])
 def test_op_qk_nr_reads_its_position_on_the_device(T, heads, D, nrot, stride):
@@ -375,6 +447,17 @@ def test_tape_ops_object_and_f16_module():
     assert torch.equal(qo, qo2) and torch.equal(cache, cache2) and int(host(err)[0]) == 0
     with pytest.raises(ValueError): ops.hadamard(qo, 256, rows_per_task=0)
     with pytest.raises(ValueError): TapeOps(T=1, kv_q8_dense=True)
+    # the fp16 / q8_0 cache lines: qk_nr(k) -> kv_append and qk_nr(q) against qk_nr_kv
+    po = TapeOps(T=T, kv_error=err)
+    for q8 in (False, True):
+        rb = 2 * (M // 32) * 34 if q8 else 4 * M
+        ca = torch.full((rows * rb,), 0x22, dtype=torch.uint8, device=qd.device); cb = torch.full_like(ca, 0x22)
+        po.qk_nr(kd, 256, nkv, 256, knd, pos, ko, 64, ts, 1e-6); po.kv_append(ko, vd, ca, pos, q8=q8); po.qk_nr(qd, 512, nh, 256, qnd, pos, qo, 64, ts, 1e-6)
+        ko2 = torch.zeros_like(ko); qo2.zero_()
+        po.qk_nr_kv(qd, 512, nh, kd, 256, vd, nkv, 256, qnd, knd, pos, qo2, cb, 64, ts, 1e-6, ko=ko2, q8=q8)
+        torch.cuda.synchronize()
+        assert torch.equal(qo, qo2) and torch.equal(ko, ko2) and torch.equal(ca, cb) and int(host(err)[0]) == 0
+    with pytest.raises(ValueError): ops.qk_nr_kv(qd, 512, nh, kd, 256, vd, nkv, 256, qnd, knd, pos, qo2, cb, 64, ts, 1e-6, q8=True)
     # the fp16-cache build of the prefill attention module
     m = Module('prefill_attn_f16'); assert 'prefill_attn_f16' in LOADED
     c16 = torch.zeros((rows, 2 * M), dtype=torch.float16, device=qd.device); e16 = dev(np.zeros(1, np.int32))
