@@ -841,14 +841,17 @@ def main():
         by_name = {name: fn for name, _, fn in sets}
         # config 4's row ops of one layer on the dense Q8 line (linear-attention conv + L2, full-attention QK-norm + rotary + Hadamard + Q8 append,
         # the gate), eight layers in one graph: as the separate launches of the reference's tape and as this library's fused launches
-        layer_sep = (['c4_conv4_silu', 'c4_l2norm_qk', 'c4_dense_q8_qk_nr_hadamard_append_six_launches', 'c4_dense_q8_att_hadamard_gate_two_launches'], 10)
-        layer_fused = (['c4_conv4_silu_l2_one_launch', 'c4_dense_q8_qk_nr_hadamard_append_one_launch', 'c4_dense_q8_att_hadamard_gate_one_launch'], 3)
-        for prefix, rep in (('c1_', 1), ('c4_', 1), ('c5_', 1), ('c1_', 8), (layer_sep, 8), (layer_fused, 8)):      # (x 8: as many launches as a few layers of a decode step queue)
+        layer_sep = ('c4_layer_separate_', ['c4_conv4_silu', 'c4_l2norm_qk', 'c4_dense_q8_qk_nr_hadamard_append_six_launches', 'c4_dense_q8_att_hadamard_gate_two_launches'], 10)
+        layer_fused = ('c4_layer_fused_', ['c4_conv4_silu_l2_one_launch', 'c4_dense_q8_qk_nr_hadamard_append_one_launch', 'c4_dense_q8_att_hadamard_gate_one_launch'], 3)
+        # config 1's row ops of one layer on the fp16-cache tape (python/caminus/engine/q3moe_one.py:362-377): add + norm, QK-norm + rotary of k -> append and
+        # of q, add + norm, SwiGLU
+        c1_sep = ('c1_layer_separate_', ['c1_add_rms_h_h16', 'c1_qk_nr_kv_append_three_launches', 'c1_add_rms_h_h16', 'c1_swiglu'], 6)
+        c1_fused = ('c1_layer_fused_', ['c1_add_rms_h_h16', 'c1_qk_nr_kv_append_one_launch', 'c1_add_rms_h_h16', 'c1_swiglu'], 4)
+        for prefix, rep in (('c1_', 1), ('c4_', 1), ('c5_', 1), ('c1_', 8), (layer_sep, 8), (layer_fused, 8), (c1_sep, 8), (c1_fused, 8)):      # (x 8: as many launches as a few layers of a decode step queue)
             if isinstance(prefix, tuple):
-                names, per = prefix
+                prefix, names, per = prefix
                 if not all(n in by_name for n in names): continue
                 fns = [by_name[n] for n in names] * rep; nl = per * rep
-                prefix = 'c4_layer_separate_' if per == 10 else 'c4_layer_fused_'
             else:
                 fns = [fn for name, _, fn in sets if name.startswith(prefix) and 'one_launch' not in name and 'launches' not in name and not name.endswith('_k')] * rep
                 nl = len(fns)
