@@ -389,6 +389,7 @@ def test_init_then_graph_replays_at_three_positions():
     qo = dev(np.zeros((T * nh, 256), np.float32)); cache = dev(np.zeros((rows, rb), np.uint8)); err = dev(np.zeros(1, np.int32))
     std = dev(st0); yc = dev(np.zeros((T, Cc), np.float32)); xp = dev(np.zeros((T, Cc), np.float32)); qk = dev(np.zeros((T * heads, 128), np.float32))
     act = dev(np.zeros((T, 512), np.uint16)); mmq = dev(np.zeros(4 * T * 144, np.uint8))
+    c16 = dev(np.zeros((rows, 2 * M), np.uint16)); qo2 = dev(np.zeros((T * nh, 256), np.float32)); g16 = dev(np.zeros((T * nh, 256), np.uint16))
 
     def launch_all():
         s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -396,20 +397,23 @@ def test_init_then_graph_replays_at_three_positions():
         _lib.check(L.camx_qk_nr_q8(p(qd), I(512), I(nh), p(kd), I(M), p(vd), I(M), I(nkv), p(qnd), p(knd), I(64), F(ts), F(1e-6), I(0), p(pos), NULL, p(qo), p(cache), I(rows), p(err), I(T), s))
         _lib.check(L.camx_op_gdn_conv_l2(p(wcd), p(std), p(xcd), p(par), p(yc), p(xp), p(qk), I(Cc), I(T), I(heads), F(RS), s))
         _lib.check(L.camx_swiglu_mmq_q8_1(p(gud), L64(1024), L64(512), p(mmq), p(act), I(T), I(1), s))     # a table reader: no fill, no wait after camx_init
+        _lib.check(L.camx_qk_nr_kv(p(qd), I(512), I(nh), p(qnd), p(kd), I(256), p(vd), I(M), I(nkv), p(knd), I(256), I(64), F(ts), F(1e-6), I(0), p(pos), NULL, p(qo2), NULL,
+                                   p(c16), I(0), I(rows), p(err), I(T), s))
+        _lib.check(L.camx_op_hadamard_gate_mul16(p(qo2), NULL, p(qd), I(512), I(256), p(g16), I(T * nh * 256), I(256), I(64), s))
 
     def reset():
         cache.zero_(); err.zero_(); std.copy_(dev(st0))
-        for t in (qo, yc, xp, qk, act, mmq): t.zero_()
+        for t in (qo, yc, xp, qk, act, mmq, c16, qo2, g16): t.zero_()
         torch.cuda.synchronize()
 
     def snapshot():
         torch.cuda.synchronize()
-        return [host(t).copy() for t in (qo, cache, err, std, yc, xp, qk, act, mmq)]
+        return [host(t).copy() for t in (qo, cache, err, std, yc, xp, qk, act, mmq, c16, qo2, g16)]
 
     eager = {}
     for p0 in (5, 40, 63):
         reset(); pos.fill_(p0); launch_all(); eager[p0] = snapshot()
-        assert eager[p0][1][p0].any() and not eager[p0][1][:p0].any()
+        assert eager[p0][1][p0].any() and not eager[p0][1][:p0].any() and eager[p0][9][p0].any() and not eager[p0][9][:p0].any()
     reset(); pos.fill_(5)
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
