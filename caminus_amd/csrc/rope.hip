@@ -478,6 +478,19 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
             } else xin[ti][s][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)a.qkv + e + 2048 * s));
         }
     }
+    // GEN: the tokens' positions and page ids are two dependent loads per token; they start here, behind the rows' loads, and not when
+    // the token's turn comes
+    [[maybe_unused]] int posv[TPW], pgv[TPW];
+    if constexpr (GEN) {
+#pragma unroll
+        for (int ti = 0; ti < TPW; ti++) posv[ti] = rope_pos(a, t0 + ti < a.n ? t0 + ti : a.n - 1);
+#pragma unroll
+        for (int ti = 0; ti < TPW; ti++) {
+            pgv[ti] = 0;
+            if (a.page_table && posv[ti] >= 0 && posv[ti] / a.page < a.pt_stride)
+                pgv[ti] = a.page_table[(size_t)(t0 + ti < a.n ? t0 + ti : a.n - 1) * a.pt_stride + posv[ti] / a.page];
+        }
+    }
     nrm[tid] = a.par[tid];
     if (wave < TPW) {                                                       // wave w: the cos / sin row of token t0 + w
         const int tw = t0 + wave < a.n ? t0 + wave : a.n - 1;
@@ -506,14 +519,15 @@ __global__ void __launch_bounds__(256) qk_rope_chunk(RopeArgs a) {
     for (int ti = 0; ti < TPW; ti++) {
         const int t = t0 + ti;
         if (t >= a.n) break;
-        const int pos = GEN ? rope_pos(a, t) : a.pos0 + t;
+        int pos = a.pos0 + t;
+        if constexpr (GEN) pos = posv[ti];
         bool span = true;                                                   // (wave-uniform) the token's cache row may be written
         size_t rowi = (size_t)pos;
-        if (GEN) {
+        if constexpr (GEN) {
             span = pos >= 0 && (a.page_table ? pos / a.page < a.pt_stride : (a.rows == 0 || pos < a.rows));
             if (!span) { if (a.err && tid == 0) atomicOr(a.err, 1); }
             else if (a.page_table) {
-                const int pg = a.page_table[(size_t)t * a.pt_stride + pos / a.page];
+                const int pg = pgv[ti];
                 if (pg < 0 || pg >= a.n_pages) { if (tid == 0) atomicOr(a.err, 8); span = false; }
                 else rowi = (size_t)pg * a.page + (size_t)(pos % a.page);
             }
