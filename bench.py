@@ -609,12 +609,15 @@ def batch_ladder(B, tokens=(16, 64, 256, 512, 1024, 2048, 4096), only=None):
             fns = [mk(i) for i in range(ncopy)]
             for f in fns: f()
             torch.cuda.synchronize()
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for k in range(30): fns[k % ncopy]()
-            b.record(); b.synchronize()
-            us = a.elapsed_time(b) * 1e3 / 30
-            out.setdefault(name, {})[str(T)] = {'us': round(us, 2), 'GBps': round(by / us / 1e3, 1)}
+            loops = []                                       # five loops of 30 launches: the median loop's average (the first loop after the buffers are made can run slow)
+            for _ in range(5):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for k in range(30): fns[k % ncopy]()
+                b.record(); b.synchronize()
+                loops.append(a.elapsed_time(b) * 1e3 / 30)
+            us = sorted(loops)[2]
+            out.setdefault(name, {})[str(T)] = {'us': round(us, 2), 'GBps': round(by / us / 1e3, 1), 'us_loops': [round(x, 2) for x in loops]}
             del fns
         torch.cuda.empty_cache()
     return out
