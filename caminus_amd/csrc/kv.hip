@@ -335,6 +335,11 @@ static int pf_kv_append_launch(const float * k, int ldk, const float * v, int ld
     else pf_kv_append_rows<<<dim3(T), dim3(256), 0, st>>>(k, ldk, v, ldv, M, cache, pos0, rows, err, posb);
     CAMX_LAUNCH_RET();
 }
+// (for camx_qk_nr_kv's prefill-sized batches, rope.hip: the same launcher with the position from a host integer or a device word)
+int camx_i_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, const int32_t * posb, int rows, int * err,
+                        int T, hipStream_t st) {
+    return pf_kv_append_launch(k, ldk, v, ldv, M, cache, pos0, posb, rows, err, T, st);
+}
 int camx_pf_kv_append(const float * k, int ldk, const float * v, int ldv, int M, uint8_t * cache, int pos0, int rows, int * err,
                       int T, hipStream_t st) {
     return pf_kv_append_launch(k, ldk, v, ldv, M, cache, pos0, nullptr, rows, err, T, st);

@@ -214,7 +214,8 @@ int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const
  * weights and positions as camx_qk_nr_qk, fp32; v [T][nkv * D] at ldv; qo [T][nh][D]; ko [T][nkv][D] or NULL (the normed k then reaches
  * only the cache); cache row position(t): work 0 fp16 [K | V], work 1 ggml q8_0 blocks of K then of V (D % 32 == 0). err bit 1: a position
  * outside [0, rows), that cache row is not written (qo and ko are). D % 4 == 0, strides % 4 == 0, fp32 pointers 16-byte aligned, else
- * CAMX_EINVAL. Every byte equals camx_qk_nr_qk followed by camx_op_kv_append on its k output. */
+ * CAMX_EINVAL. Every byte equals camx_qk_nr_qk followed by camx_op_kv_append on its k output. One launch of a wave per head, meant for decode
+ * and verify batches; from T * nh >= 12288 with ko given (and no position array) it runs the prefill-sized kernels of the three ops instead. */
 int camx_qk_nr_kv(const float * q, int q_stride, int nh, const float * wq, const float * k, int k_stride, const float * v, int ldv, int nkv,
                   const float * wk, int D, int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, float * qo,
                   float * ko, void * cache, int work, int rows, int * err, int T, camx_stream_t stream);

@@ -180,7 +180,7 @@ def test_qk_nr_qk_equals_two_launches(T, nh, nkv, D, nrot, io):
 
 
 @pytest.mark.parametrize('work', [0, 1])
-@pytest.mark.parametrize('T,nh,nkv,D,nrot', [(1, 32, 4, 128, 128), (16, 24, 4, 256, 64), (3, 5, 2, 96, 32), (2, 3, 1, 512, 64), (5, 2, 3, 32, 8), (300, 8, 2, 128, 128)])
+@pytest.mark.parametrize('T,nh,nkv,D,nrot', [(1, 32, 4, 128, 128), (16, 24, 4, 256, 64), (3, 5, 2, 96, 32), (2, 3, 1, 512, 64), (5, 2, 3, 32, 8), (300, 8, 2, 128, 128), (300, 16, 2, 128, 64), (520, 24, 1, 256, 64)])
 def test_qk_nr_kv_equals_the_three_tape_ops(T, nh, nkv, D, nrot, work):
     """q and k norm + rotary and the cache append in one launch against OP_QK_NR (k), OP_KV_APPEND, OP_QK_NR (q) one after another:
     the fp32 outputs and every byte of the cache (fp16 rows and q8_0 rows), with the position on the device, on the host, per row,
