@@ -1334,6 +1334,11 @@ int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const
     if (!xq || !xk || !wq || !wk || !outq || !outk || T < 0 || nh < 1 || nkv < 1 || D < 1 || D > 512 || q_stride < D || k_stride < D || nrot < 0 || nrot > D ||
         (nrot & 1) || io < 0 || io > 1 || (!pos && !pos_dev && (pos0 < 0 || pos0 > 0x7fffffff - T))) return CAMX_EINVAL;
     if (T == 0) return CAMX_OK;
+    if ((long)T * nh >= 12288) {          // a prefill-sized batch: two launches of the kernels that share a token's cos / sin among its heads (2 - 3 times faster there)
+        NrArgs aq = {xq, q_stride, nh, wq, D, nrot, theta_scale, eps, pos0, pos, outq, T, pos_dev}, ak = {xk, k_stride, nkv, wk, D, nrot, theta_scale, eps, pos0, pos, outk, T, pos_dev};
+        launch_nr(aq, io, st); launch_nr(ak, io, st);
+        CAMX_LAUNCH_RET();
+    }
     NrArgs a = {xq, q_stride, nh, wq, D, nrot, theta_scale, eps, pos0, pos, outq, T, pos_dev, xk, k_stride, nkv, wk, outk};
     const int es = io ? 2 : 4;
     const bool vec = (D & 3) == 0 && ((q_stride | k_stride) & 3) == 0 && (((uintptr_t)xq | (uintptr_t)xk | (uintptr_t)outq | (uintptr_t)outk) & (4 * es - 1)) == 0;

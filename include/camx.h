@@ -205,7 +205,7 @@ int camx_qk_nr_pos(const void * xin, int head_stride, int heads, const float * w
 /* The q heads and the k heads of a token in one launch (the two OP_QK_NR segments of a full-attention layer,
  * python/caminus/engine/q35_dense.py:408-415): nh heads at xq + (t * nh + h) * q_stride with weight wq -> outq [T][nh][D], nkv heads at
  * xk + (t * nkv + h) * k_stride with wk -> outk [T][nkv][D]. Row t sits at pos[t] (pos given), else pos_dev[0] + t (pos_dev given: a
- * device word), else pos0 + t. The same bits as two camx_pf_qk_nr / camx_qk_nr_pos calls. */
+ * device word), else pos0 + t. The same bits as two camx_pf_qk_nr / camx_qk_nr_pos calls (and, from T * nh >= 12288, their two launches). */
 int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const void * xk, int k_stride, int nkv, const float * wk, int D,
                   int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, void * outq, void * outk,
                   int T, int io, camx_stream_t stream);

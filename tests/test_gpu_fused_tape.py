@@ -152,7 +152,7 @@ def test_qk_nr_q8_refusals():
 
 
 @pytest.mark.parametrize('io', [0, 1])
-@pytest.mark.parametrize('T,nh,nkv,D,nrot', [(16, 24, 4, 256, 64), (1, 24, 4, 256, 64), (3, 5, 2, 128, 128), (2, 3, 1, 96, 32), (300, 8, 2, 256, 64)])
+@pytest.mark.parametrize('T,nh,nkv,D,nrot', [(16, 24, 4, 256, 64), (1, 24, 4, 256, 64), (3, 5, 2, 128, 128), (2, 3, 1, 96, 32), (300, 8, 2, 256, 64), (520, 24, 4, 256, 64), (400, 32, 4, 128, 128)])
 def test_qk_nr_qk_equals_two_launches(T, nh, nkv, D, nrot, io):
     rng = np.random.default_rng(T + nh + D)
     qs, ks = 2 * D, D + (8 if D % 8 == 0 else 4)
