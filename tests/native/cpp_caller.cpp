@@ -105,6 +105,31 @@ extern "C" __attribute__((visibility("default"))) int cpp_caller_run(char * msg,
         }
         if (!rc && !(same(dc.download<uint8_t>(), cache) && derr.download<int>()[0] == 0 && werr == 0)) rc = fail(msg, len, "tape-form Q8 KV rows differ from the oracle");
     }
+    if (!rc) {   // a decode token's attention inputs: the tape's three launches (k norm + rotary, append, q norm + rotary) and the one that replaces them
+        const int T = 1, nh = 32, nkv = 4, D = 128, M = nkv * D, rows = 64;
+        std::vector<float> q((size_t)T * nh * D), k((size_t)T * M), v((size_t)T * M), wq(D), wk(D);
+        for (auto & e : q) e = normal(rng);
+        for (auto & e : k) e = normal(rng);
+        for (auto & e : v) e = normal(rng);
+        for (auto & e : wq) e = 1.0f + 0.1f * normal(rng);
+        for (auto & e : wk) e = 1.0f + 0.1f * normal(rng);
+        const float eps = 1e-6f, ts = 0.80584f; int eb; std::memcpy(&eb, &eps, 4);
+        int pos = 41;
+        DeviceBuffer dq(q.data(), q.size() * 4), dk(k.data(), k.size() * 4), dv(v.data(), v.size() * 4), dwq(wq.data(), D * 4), dwk(wk.data(), D * 4), dpos(&pos, 4), derr(nullptr, 4);
+        DeviceBuffer qo1(nullptr, q.size() * 4), ko1(nullptr, k.size() * 4), c1(nullptr, (size_t)rows * 2 * M * 2), qo2(nullptr, q.size() * 4), c2(nullptr, (size_t)rows * 2 * M * 2);
+        int e = camx_op_qk_nr(dk.as<float>(), D, nkv, D, dwk.as<float>(), dpos.as<int32_t>(), ko1.as<float>(), D, ts, eb, T, st);
+        if (!e) e = camx_op_kv_append(ko1.as<float>(), dv.as<float>(), c1.p, dpos.as<int32_t>(), M, 0, derr.as<int>(), rows, T, st);
+        if (!e) e = camx_op_qk_nr(dq.as<float>(), D, nh, D, dwq.as<float>(), dpos.as<int32_t>(), qo1.as<float>(), D, ts, eb, T, st);
+        if (!e) e = camx_qk_nr_kv(dq.as<float>(), D, nh, dwq.as<float>(), dk.as<float>(), D, dv.as<float>(), M, nkv, dwk.as<float>(), D, D, ts, eps, 0, dpos.as<int32_t>(), nullptr,
+                                  qo2.as<float>(), nullptr, c2.p, 0, rows, derr.as<int>(), T, st);
+        if (e) rc = fail(msg, len, "camx_qk_nr_kv or the launches it replaces", e);
+        (void)hipStreamSynchronize(st);
+        const std::vector<uint16_t> row = c2.download<uint16_t>();
+        bool written = false;
+        for (int i = 0; i < 2 * M; i++) written |= row[(size_t)pos * 2 * M + i] != 0;
+        if (!rc && !(same(qo1.download<float>(), qo2.download<float>()) && same(c1.download<uint16_t>(), row) && written && derr.download<int>()[0] == 0))
+            rc = fail(msg, len, "camx_qk_nr_kv differs from the three launches");
+    }
     if (!rc && camx_add_rms_q8_1(nullptr, nullptr, nullptr, 0, nullptr, 1e-6f, nullptr, nullptr, nullptr, 2048, 1, st) != 1) rc = fail(msg, len, "a null row pointer was not refused");
     (void)hipStreamDestroy(st);
     return rc;

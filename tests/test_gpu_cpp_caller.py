@@ -1,6 +1,6 @@
 """The C ABI called from C++ with hipMalloc'ed buffers and a stream of the caller's own (no Python tensors, no torch): add +
 RMSNorm + q8_1, the MMQ quantizer, the Q8 KV writer with a refused block, camx_init and the tape's append with its position in a
-device word, an argument refusal; each compared bit for bit with the
+device word, the decode token's fused norm + rotary + append against the three launches it replaces, an argument refusal; each compared bit for bit with the
 oracle inside tests/native/cpp_caller.cpp. Built by __graft_entry__.build() (tests/native/build.py)."""
 import ctypes
 import os
