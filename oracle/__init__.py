@@ -303,6 +303,19 @@ def qk_nr_q8(q, q_stride, nh, k, v, nkv, qn, kn, n_rot, theta_scale, eps, pos, c
     return qo, cache, err
 
 
+def qk_nr_kv(q, q_stride, nh, wq, k, k_stride, v, nkv, wk, D, n_rot, theta_scale, eps, pos0, T, cache, q8, ko=None):
+    """the fp16 / q8_0 cache lines' chain (python/caminus/engine/q3moe_one.py:316-318): OP_QK_NR of k -> OP_KV_APPEND (rows pos0 + t) and
+    OP_QK_NR of q. ko: the normed k to append instead of this function's own (a caller that holds another implementation's fp32 result and
+    wants the cache bytes that follow from it). -> (qo [T * nh, D], ko [T * nkv, D], cache after the append, err)"""
+    M = nkv * D
+    qo = qk_nr(q, q_stride, nh, wq, D, n_rot, theta_scale, eps, pos0, T)
+    kn = qk_nr(k, k_stride, nkv, wk, D, n_rot, theta_scale, eps, pos0, T)
+    ka = _c(kn if ko is None else ko, np.float32).reshape(T, M); v = _c(v, np.float32).reshape(T, M)
+    if q8: cache, err = pf_kv_append(ka, M, v, M, M, cache, pos0, T)
+    else: cache, err = kv_append16(ka, v, M, cache, pos0)
+    return qo, kn, cache, err
+
+
 # ---- rotary ---------------------------------------------------------------------------------------------------------------
 
 

@@ -211,6 +211,14 @@ def test_qk_nr_kv_equals_the_three_tape_ops(T, nh, nkv, D, nrot, work):
                  I(ph), ptr(pd), NULL, ptr(oq2), ptr(ok2) if keep else NULL, ptr(c2), I(work), I(rows), ptr(e2), I(T))
             assert torch.equal(oq1, oq2) and torch.equal(c1, c2) and int(host(e2)[0]) == e1
             assert torch.equal(ok1, ok2) if keep else bool((ok2 == 5).all())
+    # against the oracle's composition: the fp32 outputs within the rotary's tolerance, and the cache bytes that follow from the launch's own k
+    oq2 = dev(np.zeros((T * nh, D), np.float32)); ok2 = dev(np.zeros((T * nkv, D), np.float32)); c2 = dev(np.full((rows, rb), 0xa5, np.uint8)); e2 = dev(np.zeros(1, np.int32))
+    call('camx_qk_nr_kv', ptr(xqd), I(qs), I(nh), ptr(wqd), ptr(xkd), I(ks), ptr(xvd), I(ldv), I(nkv), ptr(wkd), I(D), I(nrot), F(ts), F(1e-6),
+         I(17), NULL, NULL, ptr(oq2), ptr(ok2), ptr(c2), I(work), I(rows), ptr(e2), I(T))
+    c0 = np.full((rows, rb), 0xa5, np.uint8)
+    wq_, wk_, wc, werr = O.qk_nr_kv(xq, qs, nh, wq, xk, ks, xv[:, :M], nkv, wk, D, nrot, ts, 1e-6, 17, T, c0.view(np.uint16) if work == 0 else c0, work == 1, ko=host(ok2))
+    assert close_fp32(host(oq2), wq_) and close_fp32(host(ok2), wk_) and werr == 0 and int(host(e2)[0]) == 0
+    assert bits_equal(host(c2).reshape(-1), np.ascontiguousarray(wc).view(np.uint8).reshape(-1))
     # one position per row (a verify batch): the cache row is the token's position
     pos = rng.permutation(rows + 3)[:T].astype(np.int32) - 1         # distinct; may hold -1 and rows .. rows + 1
     posd = dev(pos)
