@@ -1348,7 +1348,7 @@ int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const
     CAMX_LAUNCH_RET();
 }
 // The fp16 / q8_0 cache lines' three tape segments in one launch: OP_QK_NR (k) -> OP_KV_APPEND and OP_QK_NR (q) (python/caminus/engine/
-// q3moe_one.py:316-318, 368-370; python/caminus/engine/q35_dense.py:414-417; kernels/k3_gguf_ops.h:1520-1553). q, k heads and positions as
+// q3moe_one.py:316-318, 368-370; python/caminus/engine/q35_dense.py:408-415; kernels/k3_gguf_ops.h:1520-1553). q, k heads and positions as
 // camx_qk_nr_qk (fp32); v fp32 [T][nkv * D] at ldv; qo [T][nh][D]; ko [T][nkv][D] optional (NULL: the normed k only reaches the cache);
 // cache row position(t): work 0 fp16 [K | V] (8-byte aligned), work 1 ggml q8_0 blocks (D % 32 == 0). err bit 1: a position outside
 // [0, rows) (that cache row is not written; qo and ko are). D % 4 == 0, strides % 4 == 0, 16-byte aligned fp32 pointers.

@@ -210,7 +210,7 @@ int camx_qk_nr_qk(const void * xq, int q_stride, int nh, const float * wq, const
                   int nrot, float theta_scale, float eps, int pos0, const int32_t * pos_dev, const int32_t * pos, void * outq, void * outk,
                   int T, int io, camx_stream_t stream);
 /* The fp16 and q8_0 cache lines' chain in one launch (python/caminus/engine/q3moe_one.py:316-318 and 368-370, the non-Q8 branch of
- * python/caminus/engine/q35_dense.py:414-417: OP_QK_NR k -> OP_KV_APPEND, and OP_QK_NR q; kernels/k3_gguf_ops.h:1520-1553): q and k heads,
+ * python/caminus/engine/q35_dense.py:408-415: OP_QK_NR k -> OP_KV_APPEND, and OP_QK_NR q; kernels/k3_gguf_ops.h:1520-1553): q and k heads,
  * weights and positions as camx_qk_nr_qk, fp32; v [T][nkv * D] at ldv; qo [T][nh][D]; ko [T][nkv][D] or NULL (the normed k then reaches
  * only the cache); cache row position(t): work 0 fp16 [K | V], work 1 ggml q8_0 blocks of K then of V (D % 32 == 0). err bit 1: a position
  * outside [0, rows), that cache row is not written (qo and ko are). D % 4 == 0, strides % 4 == 0, fp32 pointers 16-byte aligned, else
