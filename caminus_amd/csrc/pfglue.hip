@@ -134,6 +134,49 @@ __global__ void __launch_bounds__(256) add_sum_k(const float * __restrict__ a, c
     }
 }
 
+// ---- the decode tape's remaining elementwise ops -------------------------------------------------------------------------------
+// OP_OWN_F16 (kernels/k3_own_ops.h:247-252): y16 = fp16(x), round to nearest even
+__global__ void __launch_bounds__(256) own_f16_k(const float * __restrict__ x, uint16_t * __restrict__ y, long n, int vec) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        if (q * 4 >= n) return;
+        __builtin_nontemporal_store(pack_f16x4(__builtin_nontemporal_load((const f32x4 *)x + q)), (u32x2 *)y + q);
+    } else {
+        for (long i = q; i < n; i += (long)gridDim.x * 256) y[i] = f2h_bits(x[i]);
+    }
+}
+// OP_OWN_MOE_SUM (kernels/k3_own_ops.h:255-256, 263-271): x[i] += acc, acc = 0 then, slot by slot, fma(w[s], d[s][i], acc) or (w null) acc + d[s][i]
+__global__ void __launch_bounds__(256) own_moe_sum_k(const float * __restrict__ d, const float * __restrict__ w, float * __restrict__ x, long n, int S, int vec) {
+    const long q = (long)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        if (q * 4 >= n) return;
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s = 0; s < S; s++) {
+            const f32x4 dv = __builtin_nontemporal_load((const f32x4 *)(d + (size_t)s * n) + q);
+            if (w) { const float ws = w[s]; acc.x = __builtin_fmaf(ws, dv.x, acc.x); acc.y = __builtin_fmaf(ws, dv.y, acc.y); acc.z = __builtin_fmaf(ws, dv.z, acc.z); acc.w = __builtin_fmaf(ws, dv.w, acc.w); }
+            else { acc.x = acc.x + dv.x; acc.y = acc.y + dv.y; acc.z = acc.z + dv.z; acc.w = acc.w + dv.w; }
+        }
+        f32x4 xv = *((const f32x4 *)x + q);
+        xv.x += acc.x; xv.y += acc.y; xv.z += acc.z; xv.w += acc.w;
+        *((f32x4 *)x + q) = xv;
+    } else {
+        for (long i = q; i < n; i += (long)gridDim.x * 256) {
+            float acc = 0.0f;
+            for (int s = 0; s < S; s++) acc = w ? __builtin_fmaf(w[s], d[(size_t)s * n + i], acc) : acc + d[(size_t)s * n + i];
+            x[i] += acc;
+        }
+    }
+}
+// OP_SHEXP_ADD (kernels/k3_gguf_ops.h:1218-1229): out[i] = moe[i] + shexp[i] * sigmoid(logit[token of i]), each step rounded on its own
+__global__ void __launch_bounds__(256) shexp_add_k(const float * __restrict__ moe, const float * __restrict__ sh, const float * __restrict__ logit,
+                                                   float * __restrict__ out, long n, int dd) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const float s = 1.0f / (1.0f + expf(-logit[i / dd]));
+        const float g = sh[i] * s;
+        out[i] = moe[i] + g;
+    }
+}
+
 // ---- bf16 operand copies with zero rows up to Tpad: y[t][j] = bf16(SILU ? silu(fma(rs, x, 0)) : x) ---------------------------
 // eight values per thread (K % 8 == 0, aligned): two 128-bit loads, one 128-bit non-temporal store
 template <bool SILU>
@@ -378,6 +421,59 @@ int camx_pf_add_sum(const float * a, const float * b, float * y, long n, hipStre
     if (n == 0) return CAMX_OK;
     const int vec = n % 4 == 0 && !(((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15) && n / 4 < 0x7fffffffL * 256;
     add_sum_k<<<vec ? dim3((unsigned)((n / 4 + 255) / 256)) : GRID_1D(n), dim3(256), 0, st>>>(a, b, y, n, vec);
+    CAMX_LAUNCH_RET();
+}
+int camx_gg_quantize_q8_1(const float * x, void * y, long n, int mode, float rs, const float * g, hipStream_t st);                 // quant.hip
+int camx_gate_mul(const void * a, const void * gate, void * y, long N, int D, int stride, int off, int io, hipStream_t st);         // elt.hip
+// The decode tape's ops next to the ones above, by their Seg fields (python/caminus/engine/k3.py): the same arithmetic as the prefill kernels
+// of the same names, which the reference states in both places (kernels/k3_gguf_ops.h:1356-1372, 1461-1489, 1607-1619, 1683-1692;
+// kernels/k3_q35_ops.h:196-211, 314-333).
+// OP_ADD_SUM (k3.py:1237-1242): a, W = b, y in place, N = n
+int camx_op_add_sum(const float * a, const float * b, float * y, int n, hipStream_t st) { return camx_pf_add_sum(a, b, y, (long)n, st); }
+// OP_GDN_GATES (k3.py:1010-1015): a = alpha [T][H], W = beta [T][H], gs = dt [H], asum = ssm_a [H], y = out [T][2H], N = H
+int camx_op_gdn_gates(const float * alpha, const float * beta, const float * dt, const float * a, float * out, int H, int T, hipStream_t st) {
+    return camx_pf_gdn_gates(alpha, H, beta, H, dt, a, out, H, T, st);
+}
+// OP_GDN_NORM (k3.py:1037-1043): a = o [N][K], W = w [K], gs = z, y = out, asum = q8 (optional: q8_1 blocks of out, K % 32 == 0), rs = eps,
+// N = T * H heads, K = S; silu: the K3_GDN_SILU builds (silu(z) instead of sigmoid(z))
+int camx_op_gdn_norm(const float * o, const float * w, const float * z, float * out, void * q8, int N, int K, float eps, int silu, hipStream_t st) {
+    if (N < 0 || silu < 0 || silu > 1 || (q8 && (K & 31))) return CAMX_EINVAL;
+    const int rc = camx_pf_gdn_norm(o, w, z, out, K, eps, (long)N, silu, st);
+    if (rc || !q8 || N == 0) return rc;
+    return camx_gg_quantize_q8_1(out, q8, (long)N * K, 0, 0.0f, nullptr, st);      // q8_emit of every stored value (kernels/k3_gguf_ops.h:1486)
+}
+// OP_GDN_NORM16 (k3.py:1045-1055): the SiLU form, y = out16 fp16
+int camx_op_gdn_norm16(const float * o, const float * w, const float * z, uint16_t * out16, int N, int K, float eps, hipStream_t st) {
+    return N < 0 ? CAMX_EINVAL : camx_q35p_gdn_norm16(o, w, z, out16, K, eps, (long)N, st);
+}
+// OP_GATE_MUL (k3.py:1201-1207): a, W = gate, y = out fp32, asum = q8 (optional, n % 32 == 0), N = n, K = dim, pad1 = head_stride, pad2 = offset
+int camx_op_gate_mul(const float * a, const float * gate, int head_stride, int offset, float * out, void * q8, int n, int dim, hipStream_t st) {
+    if (n < 0 || (q8 && (n & 31))) return CAMX_EINVAL;
+    const int rc = camx_gate_mul(a, gate, out, (long)n, dim, head_stride, offset, 0, st);
+    if (rc || !q8 || n == 0) return rc;
+    return camx_gg_quantize_q8_1(out, q8, (long)n, 0, 0.0f, nullptr, st);
+}
+// OP_OWN_F16 (k3.py:846-852): a = x, y = out fp16, N = n
+int camx_op_own_f16(const float * x, uint16_t * out16, int n, hipStream_t st) {
+    if (!x || !out16 || n < 0) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const int vec = n % 4 == 0 && !((uintptr_t)x & 15) && !((uintptr_t)out16 & 7);
+    own_f16_k<<<vec ? dim3((unsigned)((n / 4 + 255) / 256)) : GRID_1D(n), dim3(256), 0, st>>>(x, out16, n, vec);
+    CAMX_LAUNCH_RET();
+}
+// OP_OWN_MOE_SUM (k3.py:862-868): a = d [slots][n], gs = w [slots] or null (weights 1), y = x in place, N = n, pad1 = slots (1 .. 64)
+int camx_op_own_moe_sum(const float * d, const float * w, float * x, int n, int slots, hipStream_t st) {
+    if (!d || !x || n < 0 || slots < 1 || slots > 64) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    const int vec = n % 4 == 0 && !(((uintptr_t)d | (uintptr_t)x) & 15);
+    own_moe_sum_k<<<vec ? dim3((unsigned)((n / 4 + 255) / 256)) : GRID_1D(n), dim3(256), 0, st>>>(d, w, x, n, slots, vec);
+    CAMX_LAUNCH_RET();
+}
+// OP_SHEXP_ADD (k3.py:958-963): a = moe, W = shexp, gs = gate logit [T], y = out, N = n (T tokens of n / T values)
+int camx_op_shexp_add(const float * moe, const float * shexp, const float * gate_logit, float * out, int n, int T, hipStream_t st) {
+    if (!moe || !shexp || !gate_logit || !out || n < 0 || T < 1 || n % T) return CAMX_EINVAL;
+    if (n == 0) return CAMX_OK;
+    shexp_add_k<<<GRID_1D(n), dim3(256), 0, st>>>(moe, shexp, gate_logit, out, n, n / T);
     CAMX_LAUNCH_RET();
 }
 static int to_bf16_launch(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, bool silu, hipStream_t st) {

@@ -103,6 +103,43 @@ class TapeOps:
         n = g.numel(); assert u.numel() == n and y16.dtype == self._torch.float16 and y16.numel() >= n
         return self._go('camx_op_own_swiglu16', self._p(g), self._p(u), self._p(y16), self._C.c_int(n))
 
+    def own_f16(self, x, out, rows_per_task=1024, dep=-1, team=-1):
+        n = x.numel(); assert x.dtype == self._torch.float32 and out.dtype == self._torch.float16 and out.numel() >= n
+        return self._go('camx_op_own_f16', self._p(x), self._p(out), self._C.c_int(n))
+
+    def own_moe_sum(self, d, x, slots=1, w=None, rows_per_task=1024, dep=-1, team=-1):
+        n = x.numel(); assert d.numel() >= slots * n and (w is None or w.numel() >= slots) and 1 <= slots <= 64
+        return self._go('camx_op_own_moe_sum', self._p(d), self._p(w), self._p(x), self._C.c_int(n), self._C.c_int(slots))
+
+    def shexp_add(self, moe, shexp, gate_logit, out, rows_per_task=1024, dep=-1, team=-1):
+        n = out.numel(); assert n % self.T == 0 and gate_logit.numel() >= self.T
+        return self._go('camx_op_shexp_add', self._p(moe), self._p(shexp), self._p(gate_logit), self._p(out), self._C.c_int(n), self._C.c_int(self.T))
+
+    def add_sum(self, a, b, y, rows_per_task=1024, dep=-1, team=-1):
+        return self._go('camx_op_add_sum', self._p(a), self._p(b), self._p(y), self._C.c_int(y.numel()))
+
+    def gdn_gates(self, alpha, beta, dt, a, out, dep=-1, team=-1):
+        H = alpha.numel() // self.T
+        return self._go('camx_op_gdn_gates', self._p(alpha), self._p(beta), self._p(dt), self._p(a), self._p(out), self._C.c_int(H), self._C.c_int(self.T))
+
+    def gdn_norm(self, o, w, z, out, H, S, eps, dep=-1, team=-1, q8=None, silu=False):
+        """silu: the reference's K3_GDN_SILU modules (silu(z) in place of sigmoid(z))"""
+        I, F = self._C.c_int, self._C.c_float
+        if q8 is not None: assert S % 32 == 0
+        return self._go('camx_op_gdn_norm', self._p(o), self._p(w), self._p(z), self._p(out), self._p(q8), I(self.T * H), I(S), F(eps), I(1 if silu else 0))
+
+    def gdn_norm16(self, o, w, z, out16, H, S, eps, dep=-1, team=-1):
+        I, F = self._C.c_int, self._C.c_float
+        N = self.T * H
+        assert o.numel() >= N * S and w.numel() == S and z.numel() >= N * S and out16.dtype == self._torch.float16 and out16.numel() >= N * S
+        return self._go('camx_op_gdn_norm16', self._p(o), self._p(w), self._p(z), self._p(out16), I(N), I(S), F(eps))
+
+    def gate_mul(self, a, gate, head_stride, offset, out, dim, rows_per_task=256, dep=-1, team=-1, q8=None):
+        I = self._C.c_int
+        n = a.numel()
+        if q8 is not None: assert n % 32 == 0 and rows_per_task % 32 == 0
+        return self._go('camx_op_gate_mul', self._p(a), self._p(gate), I(head_stride), I(offset), self._p(out), self._p(q8), I(n), I(dim))
+
     def qk_nr(self, x, head_stride, heads, dim, w, pos, out, n_rot, theta_scale, eps, dep=-1, team=-1):
         I, F = self._C.c_int, self._C.c_float
         eb = int(np.array([eps], dtype=np.float32).view(np.int32)[0])

@@ -115,6 +115,30 @@ int camx_op_hadamard_gate_mul16(const float * a, float * a_out, const float * ga
 int camx_op_gdn_l2(const float * x, float * out, int heads, int dim, float rs, int x_stride, int T, camx_stream_t stream);
 /* OP_OWN_SWIGLU16 (k3.py:854-860; kernels/k3_own_ops.h:258-262): a = g, W = u, y = y16, N = n. */
 int camx_op_own_swiglu16(const float * g, const float * u, uint16_t * y16, int n, camx_stream_t stream);
+/* The tape's row ops on either side of the ones above, by their Seg fields; the arithmetic is that of the prefill kernels of the same names.
+ * OP_OWN_F16 (k3.py:846-852; kernels/k3_own_ops.h:247-252): out16 = fp16(x), round to nearest even. */
+int camx_op_own_f16(const float * x, uint16_t * out16, int n, camx_stream_t stream);
+/* OP_OWN_MOE_SUM (k3.py:862-868; kernels/k3_own_ops.h:255-256, 263-271): x[i] += acc with acc = 0, then per slot fma(w[s], d[s * n + i], acc),
+ * or acc + d[s * n + i] when w is NULL (the attention's residual add with slots = 1). slots 1 .. 64. */
+int camx_op_own_moe_sum(const float * d, const float * w, float * x, int n, int slots, camx_stream_t stream);
+/* OP_SHEXP_ADD (k3.py:958-963; kernels/k3_gguf_ops.h:1218-1229): out = moe + shexp * sigmoid(gate_logit[token]), n = T * (n / T) values. */
+int camx_op_shexp_add(const float * moe, const float * shexp, const float * gate_logit, float * out, int n, int T, camx_stream_t stream);
+/* OP_ADD_SUM (k3.py:1237-1242; kernels/k3_gguf_ops.h:1683-1692): y = y + (a + b). */
+int camx_op_add_sum(const float * a, const float * b, float * y, int n, camx_stream_t stream);
+/* OP_GDN_GATES (k3.py:1010-1015; kernels/k3_gguf_ops.h:1356-1372, kernels/k3_q35_ops.h:196-211): out [T][2H] = softplus(alpha + dt) * a |
+ * sigmoid(beta); alpha, beta [T][H]. */
+int camx_op_gdn_gates(const float * alpha, const float * beta, const float * dt, const float * a, float * out, int H, int T, camx_stream_t stream);
+/* OP_GDN_NORM (k3.py:1037-1043; kernels/k3_gguf_ops.h:1461-1489): N = T * H heads of K values, out = ((o * rsqrt(mean(o^2) + eps)) * w) *
+ * sigmoid(z), or * silu(z) with silu = 1 (the reference's K3_GDN_SILU builds); q8 (optional, K % 32 == 0) receives the q8_1 blocks of out
+ * (a second launch). K % 4 == 0, K <= 1024, 16-byte aligned rows, as camx_pf_gdn_norm. */
+int camx_op_gdn_norm(const float * o, const float * w, const float * z, float * out, void * q8, int N, int K, float eps, int silu,
+                     camx_stream_t stream);
+/* OP_GDN_NORM16 (k3.py:1045-1055; kernels/k3_q35_ops.h:314-333): the SiLU form with fp16 output. */
+int camx_op_gdn_norm16(const float * o, const float * w, const float * z, uint16_t * out16, int N, int K, float eps, camx_stream_t stream);
+/* OP_GATE_MUL (k3.py:1201-1207; kernels/k3_gguf_ops.h:1607-1619): out fp32 = a * sigmoid(gate[(i / dim) * head_stride + offset + i % dim]);
+ * q8 (optional, n % 32 == 0) receives the q8_1 blocks of out (a second launch). */
+int camx_op_gate_mul(const float * a, const float * gate, int head_stride, int offset, float * out, void * q8, int n, int dim,
+                     camx_stream_t stream);
 /* The prologue of OP_OWN_ATTS (k3.py:1151-1199, Seg.asum = pos; kernels/k3_own_atts.h:183-274): camx_q3p_qk_rope / _q8 with token t at
  * pos[0] + t read on the device, checked there against the cache's `rows` (err bit 1: the row is not written, q16 is). err is required. */
 int camx_op_own_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float * par, const int32_t * pos, uint16_t * q16, void * cache,

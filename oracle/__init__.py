@@ -472,6 +472,23 @@ def kv_append16(k, v, M, cache, pos0):
     return cache, int(err[0])
 
 
+def own_moe_sum(d, w, x, slots):
+    """OP_OWN_MOE_SUM (kernels/k3_own_ops.h:263-271): x += the slot-ordered fma chain (w None: plain adds) -> x"""
+    d = _c(d, np.float32); x = _c(x, np.float32).copy(); w = None if w is None else _c(w, np.float32)
+    lib().orc_own_moe_sum(_p(d), _p(w), _p(x), C.c_long(x.size), I(slots)); return x
+
+
+def shexp_add(moe, shexp, logit, T):
+    """OP_SHEXP_ADD (kernels/k3_gguf_ops.h:1220-1229) -> out"""
+    moe = _c(moe, np.float32); shexp = _c(shexp, np.float32); logit = _c(logit, np.float32); out = np.empty_like(moe)
+    lib().orc_shexp_add(_p(moe), _p(shexp), _p(logit), _p(out), C.c_long(moe.size), I(T)); return out
+
+
+def own_f16(x):
+    """OP_OWN_F16 (kernels/k3_own_ops.h:247-252) -> fp16 bits"""
+    return f2h(x)
+
+
 def add_sum(a, b, y):
     a = _c(a, np.float32); b = _c(b, np.float32); y = _c(y, np.float32).copy()
     lib().orc_add_sum(_p(a), _p(b), _p(y), C.c_long(y.size)); return y

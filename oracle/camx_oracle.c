@@ -1010,6 +1010,23 @@ ORC_API void orc_kv_append16(const float * k, int ldk, const float * v, int ldv,
         for (int i = 0; i < M; i++) { cache[(size_t)pos * 2 * M + i] = orc_f2h(k[(size_t)tt * ldk + i]); cache[(size_t)pos * 2 * M + M + i] = orc_f2h(v[(size_t)tt * ldv + i]); }
     }
 }
+/* OP_OWN_MOE_SUM (kernels/k3_own_ops.h:263-271) */
+ORC_API void orc_own_moe_sum(const float * d, const float * w, float * x, long n, int S) {
+    for (long i = 0; i < n; i++) {
+        float acc = 0.0f;
+        for (int s = 0; s < S; s++) acc = w ? fmaf(w[s], d[(size_t)s * n + i], acc) : acc + d[(size_t)s * n + i];
+        x[i] += acc;
+    }
+}
+/* OP_SHEXP_ADD (kernels/k3_gguf_ops.h:1220-1229) */
+ORC_API void orc_shexp_add(const float * moe, const float * sh, const float * logit, float * out, long n, int T) {
+    const long dd = n / T;
+    for (long i = 0; i < n; i++) {
+        const float s = 1.0f / (1.0f + expf(-logit[i / dd]));
+        const float g = sh[i] * s;
+        out[i] = moe[i] + g;
+    }
+}
 ORC_API void orc_add_sum(const float * a, const float * b, float * y, long n) { for (long i = 0; i < n; i++) { const float ab = a[i] + b[i]; y[i] = y[i] + ab; } }
 static inline uint16_t to_bf16_plain(float v) { const uint32_t u = f2u(v); return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16); }
 ORC_API void orc_to_bf16_rows(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, int silu) {

@@ -322,6 +322,74 @@ def test_hadamard_gate_mul16_equals_the_two_tape_ops(T, nh, D, n):
         assert camx().camx_op_hadamard_gate_mul16(p(a2), NULL, p(qgd), I(2 * D), I(D), p(y2), *bad, stream()) == 1
 
 
+@pytest.mark.parametrize('n,slots,T', [(2048, 8, 1), (2048, 1, 1), (4 * 2048, 8, 4), (1000, 3, 2), (37, 64, 1), (16 * 5120, 1, 16)])
+def test_op_own_f16_moe_sum_shexp_add_against_the_oracle(n, slots, T):
+    """the tape's elementwise ops beside the row ops: OP_OWN_MOE_SUM (slot-ordered fma chain, and the plain adds without weights) and
+    OP_OWN_F16 bit for bit, OP_SHEXP_ADD within the gate's exponential"""
+    rng = np.random.default_rng(n + slots)
+    d = outliers(rng, (slots, n)); w = rng.standard_normal(slots).astype(np.float32); x = outliers(rng, (n,))
+    for wt in (w, None):
+        xd = dev(x)
+        call('camx_op_own_moe_sum', ptr(dev(d)), ptr(dev(wt)) if wt is not None else NULL, ptr(xd), I(n), I(slots))
+        assert bits_equal(host(xd), O.own_moe_sum(d, wt, x, slots))
+    base = dev(np.concatenate([x, np.zeros(4, np.float32)]))          # an unaligned view: the scalar form
+    if n % 4 == 0:
+        xu = base[1:1 + n]; xu.copy_(dev(x))
+        call('camx_op_own_moe_sum', ptr(dev(d)), ptr(dev(w)), ptr(xu), I(n), I(slots))
+        assert bits_equal(host(xu), O.own_moe_sum(d, w, x, slots))
+    v = np.concatenate([outliers(rng, (n - 8,)) * np.float32(300), np.array([65504, 65519.99, 65520, 1 + 2.0 ** -11, 2.0 ** -25, -0.0, 1e-8, np.inf], np.float32)]) if n > 8 else x
+    y = dev(np.zeros(n, np.uint16))
+    call('camx_op_own_f16', ptr(dev(v)), ptr(y), I(n))
+    assert bits_equal(host(y, np.uint16), O.own_f16(v))
+    moe = outliers(rng, (n,)); sh = outliers(rng, (n,)); lg = (4 * rng.standard_normal(T)).astype(np.float32); out = dev(np.zeros(n, np.float32))
+    if n % T == 0:
+        call('camx_op_shexp_add', ptr(dev(moe)), ptr(dev(sh)), ptr(dev(lg)), ptr(out), I(n), I(T))
+        assert close_fp32(host(out).reshape(T, -1), O.shexp_add(moe, sh, lg, T).reshape(T, -1))
+    L = camx(); p = lambda t: C.c_void_p(t.data_ptr())
+    assert L.camx_op_own_moe_sum(p(out), NULL, p(out), I(n), I(65), stream()) == 1 and L.camx_op_own_moe_sum(p(out), NULL, p(out), I(n), I(0), stream()) == 1
+    assert L.camx_op_shexp_add(p(out), p(out), p(out), p(out), I(n), I(0), stream()) == 1 and L.camx_op_own_f16(NULL, p(y), I(n), stream()) == 1
+    if n % 7: assert L.camx_op_shexp_add(p(out), p(out), p(out), p(out), I(n), I(7), stream()) == 1
+
+
+def test_tape_ops_of_the_gdn_and_gate_rows_equal_their_prefill_namesakes():
+    """OP_GDN_GATES, OP_GDN_NORM (+ its q8_1 copy), OP_GDN_NORM16, OP_GATE_MUL (+ q8_1 copy) and OP_ADD_SUM by their Seg fields: the bits of the
+    prefill entry points the reference states the same arithmetic in, and the oracle's q8_1 blocks of the stored values"""
+    rng = np.random.default_rng(55)
+    T, H, S = 3, 48, 128
+    al = outliers(rng, (T, H)); be = outliers(rng, (T, H)); dt = rng.standard_normal(H).astype(np.float32); A = -np.abs(rng.standard_normal(H)).astype(np.float32)
+    ald, bed, dtd, Ad = dev(al), dev(be), dev(dt), dev(A)
+    g1 = dev(np.zeros((T, 2 * H), np.float32)); g2 = dev(np.ones((T, 2 * H), np.float32))
+    call('camx_pf_gdn_gates', ptr(ald), I(H), ptr(bed), I(H), ptr(dtd), ptr(Ad), ptr(g1), I(H), I(T))
+    call('camx_op_gdn_gates', ptr(ald), ptr(bed), ptr(dtd), ptr(Ad), ptr(g2), I(H), I(T))
+    assert torch.equal(g1, g2)
+    o = outliers(rng, (T * H, S)); z = outliers(rng, (T * H, S)); w = (1 + 0.1 * rng.standard_normal(S)).astype(np.float32)
+    od, zd, wd = dev(o), dev(z), dev(w)
+    for silu in (0, 1):
+        y1 = dev(np.zeros((T * H, S), np.float32)); y2 = dev(np.ones((T * H, S), np.float32)); q8 = dev(np.zeros(T * H * S // 32 * 36, np.uint8))
+        call('camx_pf_gdn_norm', ptr(od), ptr(wd), ptr(zd), ptr(y1), I(S), F(1e-6), L64(T * H), I(silu))
+        call('camx_op_gdn_norm', ptr(od), ptr(wd), ptr(zd), ptr(y2), ptr(q8), I(T * H), I(S), F(1e-6), I(silu))
+        assert torch.equal(y1, y2) and bits_equal(host(q8).reshape(-1, 36), O.q8_1(host(y2).reshape(-1)))
+        y3 = dev(np.ones((T * H, S), np.float32))
+        call('camx_op_gdn_norm', ptr(od), ptr(wd), ptr(zd), ptr(y3), NULL, I(T * H), I(S), F(1e-6), I(silu))
+        assert torch.equal(y1, y3)
+    h1 = dev(np.zeros((T * H, S), np.uint16)); h2 = dev(np.ones((T * H, S), np.uint16))
+    call('camx_q35p_gdn_norm16', ptr(od), ptr(wd), ptr(zd), ptr(h1), I(S), F(1e-6), L64(T * H))
+    call('camx_op_gdn_norm16', ptr(od), ptr(wd), ptr(zd), ptr(h2), I(T * H), I(S), F(1e-6))
+    assert torch.equal(h1, h2)
+    nh, D = 24, 256
+    a = outliers(rng, (T * nh, D)); qg = outliers(rng, (T * nh, 2 * D)); ad, qgd = dev(a), dev(qg)
+    m1 = dev(np.zeros((T * nh, D), np.float32)); m2 = dev(np.ones((T * nh, D), np.float32)); q8 = dev(np.zeros(T * nh * D // 32 * 36, np.uint8))
+    call('camx_gate_mul', ptr(ad), ptr(qgd), ptr(m1), L64(a.size), I(D), I(2 * D), I(D), I(0))
+    call('camx_op_gate_mul', ptr(ad), ptr(qgd), I(2 * D), I(D), ptr(m2), ptr(q8), I(a.size), I(D))
+    assert torch.equal(m1, m2) and bits_equal(host(q8).reshape(-1, 36), O.q8_1(host(m2).reshape(-1)))
+    ya = outliers(rng, (5000,)); s1, s2 = dev(ya), dev(ya); aa, bb = dev(outliers(rng, (5000,))), dev(outliers(rng, (5000,)))
+    call('camx_pf_add_sum', ptr(aa), ptr(bb), ptr(s1), L64(5000)); call('camx_op_add_sum', ptr(aa), ptr(bb), ptr(s2), I(5000))
+    assert torch.equal(s1, s2)
+    L = camx(); p = lambda t: C.c_void_p(t.data_ptr())
+    assert L.camx_op_gdn_norm(p(od), p(wd), p(zd), p(y1), p(q8), I(T * H), I(S), F(1e-6), I(2), stream()) == 1        # a gate form that does not exist
+    assert L.camx_op_gate_mul(p(ad), p(qgd), I(2 * D), I(D), p(m2), p(q8), I(a.size - 8), I(D), stream()) == 1        # a q8_1 copy of a partial block
+
+
 def test_thin_tape_ops_equal_their_prefill_namesakes():
     rng = np.random.default_rng(31)
     x = outliers(rng, (64, 256)); xa, xb = dev(x), dev(x)
@@ -470,6 +538,16 @@ def test_tape_ops_object_and_f16_module():
         torch.cuda.synchronize()
         assert torch.equal(qo, qo2) and torch.equal(ko, ko2) and torch.equal(ca, cb) and int(host(err)[0]) == 0
     with pytest.raises(ValueError): ops.qk_nr_kv(qd, 512, nh, kd, 256, vd, nkv, 256, qnd, knd, pos, qo2, cb, 64, ts, 1e-6, q8=True)
+    # the elementwise tape ops through the host mirror
+    xs = dev(outliers(rng, (T * 512,))); ds_ = dev(outliers(rng, (3, T * 512))); ws = dev(rng.standard_normal(3).astype(np.float32)); x0 = host(xs).copy()
+    po.own_moe_sum(ds_, xs, slots=3, w=ws); h16 = torch.zeros(T * 512, dtype=torch.float16, device=qd.device); po.own_f16(xs, h16)
+    torch.cuda.synchronize()
+    want = O.own_moe_sum(host(ds_), host(ws), x0, 3)
+    assert bits_equal(host(xs), want) and bits_equal(host(h16.view(torch.int16), np.uint16), O.own_f16(want))
+    lg = dev(np.array([0.0, -200.0], np.float32)); so = torch.zeros_like(xs); po.shexp_add(xs, ds_[0], lg, so); po.add_sum(ds_[1], ds_[2], so)
+    torch.cuda.synchronize()
+    sh_ = want.reshape(T, -1) + np.stack([host(ds_[0]).reshape(T, -1)[0] * np.float32(0.5), np.zeros(512, np.float32)])
+    assert bits_equal(host(so), (sh_.reshape(-1) + (host(ds_[1]) + host(ds_[2]))).astype(np.float32))
     # the fp16-cache build of the prefill attention module
     m = Module('prefill_attn_f16'); assert 'prefill_attn_f16' in LOADED
     c16 = torch.zeros((rows, 2 * M), dtype=torch.float16, device=qd.device); e16 = dev(np.zeros(1, np.int32))

@@ -644,6 +644,50 @@ def test_core_elementwise_exact():
     assert np.array_equal(O.embedding_f32(tok, emb), emb[tok])
 
 
+def test_tape_elementwise_ops_known_answers():
+    """OP_OWN_MOE_SUM, OP_SHEXP_ADD and OP_OWN_F16 against exact rational arithmetic, a case only a fused multiply-add gets right,
+    closed forms of the gate, and numpy's fp16 rounding."""
+    from fractions import Fraction
+    rng = np.random.default_rng(77)
+    # one rounding per fma, slot order: exact rationals rounded to the nearest fp32 (ties cannot occur at these magnitudes by accident:
+    # the assert below compares with both neighbours' midpoints through the exact value)
+    def rnd(fr):                                    # Fraction -> nearest fp32 (ties to even), through the two neighbouring floats
+        a = f32(float(fr)); lo = a if Fraction(float(a)) <= fr else np.nextafter(a, f32(-np.inf), dtype=f32); hi = np.nextafter(lo, f32(np.inf), dtype=f32)
+        if Fraction(float(lo)) == fr: return lo
+        dl, dh = fr - Fraction(float(lo)), Fraction(float(hi)) - fr
+        if dl != dh: return lo if dl < dh else hi
+        return lo if (lo.view(np.uint32) & 1) == 0 else hi
+    n, S = 13, 5
+    d = rng.standard_normal((S, n)).astype(f32); w = rng.standard_normal(S).astype(f32); x = rng.standard_normal(n).astype(f32)
+    want = np.empty(n, f32)
+    for i in range(n):
+        acc = f32(0)
+        for s in range(S): acc = rnd(Fraction(float(w[s])) * Fraction(float(d[s, i])) + Fraction(float(acc)))
+        want[i] = rnd(Fraction(float(x[i])) + Fraction(float(acc)))
+    assert np.array_equal(O.own_moe_sum(d, w, x, S).view(np.uint32), want.view(np.uint32))
+    # slot 0 leaves -(1 + 2^-11) in the sum; slot 1 adds (1 + 2^-12)^2 = 1 + 2^-11 + 2^-24: the last bit survives only in a fused multiply-add
+    one = f32(1) + f32(2.0 ** -12)
+    got = O.own_moe_sum(np.array([[-(f32(1) + f32(2.0 ** -11))], [one]], f32), np.array([1, one], f32), np.zeros(1, f32), 2)
+    assert got[0] == f32(2.0 ** -24)
+    # no weights: plain adds from zero in slot order, then one add into x
+    plain = x + ((((f32(0) + d[0]) + d[1]) + d[2]) + d[3])
+    assert np.array_equal(O.own_moe_sum(d[:4], None, x, 4), plain.astype(f32))
+    assert np.array_equal(O.own_moe_sum(d[:1], None, x, 1), x + d[0])
+    # the shared expert's gate: logit 0 -> exactly one half; a very negative logit -> exactly moe; the logit is the token's
+    moe = rng.standard_normal((3, 8)).astype(f32); sh = rng.standard_normal((3, 8)).astype(f32)
+    assert np.array_equal(O.shexp_add(moe, sh, np.zeros(3, f32), 3), moe + sh * f32(0.5))
+    assert np.array_equal(O.shexp_add(moe, sh, np.full(3, -200, f32), 3), moe)
+    lg = np.array([0.0, -200.0, 3.0], f32)
+    got = O.shexp_add(moe, sh, lg, 3)
+    assert np.array_equal(got[0], moe[0] + sh[0] * f32(0.5)) and np.array_equal(got[1], moe[1])
+    s64 = 1.0 / (1.0 + np.exp(-3.0))
+    assert np.allclose(got[2], moe[2].astype(np.float64) + sh[2].astype(np.float64) * s64, rtol=1e-6, atol=1e-7) and not np.array_equal(got[2], moe[2])
+    # fp16: numpy's round-to-nearest-even conversion, ties and the overflow boundary included
+    v = np.concatenate([rng.standard_normal(4096).astype(f32) * f32(100), np.array([65504, 65519.99, 65520, 1 + 2.0 ** -11, 1 + 3 * 2.0 ** -11, 2.0 ** -25, 2.0 ** -24, -0.0, 1e-8], f32)])
+    with np.errstate(over='ignore'):               # 65520 rounds to infinity: the case under test
+        assert np.array_equal(O.own_f16(v), v.astype(np.float16).view(np.uint16))
+
+
 # ---- actq: invariants (the pins against a torch graph and autograd are in test_oracle_actq_autograd.py) --------------------------------
 
 def test_actq_invariants():
