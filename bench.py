@@ -527,6 +527,18 @@ def prefill_scale_sweep(B, T=4096, only=None):
         return lambda: B.call('camx_pf_add_sum', _p(a), _p(b), _p(y), L64(Mr * Kq))
     timeit('pf_add_sum 16M', Mr * Kq * 16, mk)
     def mk(i):
+        x = B.acts((Mr * Kq,), torch.float32, i); y = torch.empty(Mr * Kq, dtype=torch.float16, device=dev)
+        return lambda: B.call('camx_op_own_f16', _p(x), _p(y), I(Mr * Kq))
+    timeit('op_own_f16 16M', Mr * Kq * 6, mk)
+    def mk(i):
+        n = T * 2048; d = B.acts((8, n), torch.float32, i); wv = B.acts((8,), torch.float32, i + 1); x = B.acts((n,), torch.float32, i + 2)
+        return lambda: B.call('camx_op_own_moe_sum', _p(d), _p(wv), _p(x), I(n), I(8))
+    timeit(f'op_own_moe_sum {T}x2048, 8 slots', T * 2048 * 40, mk)
+    def mk(i):
+        n = T * 2048; moe = B.acts((n,), torch.float32, i); sh = B.acts((n,), torch.float32, i + 1); lg = B.acts((T,), torch.float32, i + 2); o = torch.empty(n, device=dev)
+        return lambda: B.call('camx_op_shexp_add', _p(moe), _p(sh), _p(lg), _p(o), I(n), I(T))
+    timeit(f'op_shexp_add {T}x2048', T * 2048 * 12, mk)
+    def mk(i):
         x = B.acts((4096, 5120), torch.float32, i); y = torch.empty((4096, 5120), dtype=torch.bfloat16, device=dev)
         return lambda: B.call('camx_pf_to_bf16', _p(x), I(5120), _p(y), I(4096), I(4096), I(5120))
     timeit('pf_to_bf16 4096x5120', 4096 * 5120 * 6, mk)

@@ -156,9 +156,9 @@ __global__ void __launch_bounds__(256) own_moe_sum_k(const float * __restrict__ 
             if (w) { const float ws = w[s]; acc.x = __builtin_fmaf(ws, dv.x, acc.x); acc.y = __builtin_fmaf(ws, dv.y, acc.y); acc.z = __builtin_fmaf(ws, dv.z, acc.z); acc.w = __builtin_fmaf(ws, dv.w, acc.w); }
             else { acc.x = acc.x + dv.x; acc.y = acc.y + dv.y; acc.z = acc.z + dv.z; acc.w = acc.w + dv.w; }
         }
-        f32x4 xv = *((const f32x4 *)x + q);
+        f32x4 xv = __builtin_nontemporal_load((const f32x4 *)x + q);
         xv.x += acc.x; xv.y += acc.y; xv.z += acc.z; xv.w += acc.w;
-        *((f32x4 *)x + q) = xv;
+        __builtin_nontemporal_store(xv, (f32x4 *)x + q);
     } else {
         for (long i = q; i < n; i += (long)gridDim.x * 256) {
             float acc = 0.0f;
@@ -175,6 +175,19 @@ __global__ void __launch_bounds__(256) shexp_add_k(const float * __restrict__ mo
         const float g = sh[i] * s;
         out[i] = moe[i] + g;
     }
+}
+// rows of a multiple of 4 values, 16-byte aligned: the token in blockIdx.y, four values per lane, the gate once per lane
+__global__ void __launch_bounds__(256) shexp_add_rows(const float * __restrict__ moe, const float * __restrict__ sh, const float * __restrict__ logit,
+                                                      float * __restrict__ out, int dd4) {
+    const int q = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    if (q >= dd4) return;
+    const size_t e = (size_t)t * dd4 + q;
+    const f32x4 m = __builtin_nontemporal_load((const f32x4 *)moe + e), h = __builtin_nontemporal_load((const f32x4 *)sh + e);
+    const float s = 1.0f / (1.0f + expf(-logit[t]));
+    f32x4 r;
+    { const float g = h.x * s; r.x = m.x + g; } { const float g = h.y * s; r.y = m.y + g; }
+    { const float g = h.z * s; r.z = m.z + g; } { const float g = h.w * s; r.w = m.w + g; }
+    __builtin_nontemporal_store(r, (f32x4 *)out + e);
 }
 
 // ---- bf16 operand copies with zero rows up to Tpad: y[t][j] = bf16(SILU ? silu(fma(rs, x, 0)) : x) ---------------------------
@@ -473,7 +486,10 @@ int camx_op_own_moe_sum(const float * d, const float * w, float * x, int n, int 
 int camx_op_shexp_add(const float * moe, const float * shexp, const float * gate_logit, float * out, int n, int T, hipStream_t st) {
     if (!moe || !shexp || !gate_logit || !out || n < 0 || T < 1 || n % T) return CAMX_EINVAL;
     if (n == 0) return CAMX_OK;
-    shexp_add_k<<<GRID_1D(n), dim3(256), 0, st>>>(moe, shexp, gate_logit, out, n, n / T);
+    const int dd = n / T;
+    if (dd % 4 == 0 && T <= 65535 && !(((uintptr_t)moe | (uintptr_t)shexp | (uintptr_t)out) & 15))
+        shexp_add_rows<<<dim3((unsigned)((dd / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st>>>(moe, shexp, gate_logit, out, dd / 4);
+    else shexp_add_k<<<GRID_1D(n), dim3(256), 0, st>>>(moe, shexp, gate_logit, out, n, dd);
     CAMX_LAUNCH_RET();
 }
 static int to_bf16_launch(const float * x, int ldx, uint16_t * y, int T, int Tpad, int K, float rs, bool silu, hipStream_t st) {

@@ -112,6 +112,8 @@ def _fused_generators(r):
         (FT.test_op_qk_nr_reads_its_position_on_the_device, op_nr),
         (FT.test_op_kv_append_three_row_formats, lambda: (32 * ri(1, 40), ch([ri(1, 40), ri(1, 40), ri(1024, 1300)]))),
         (FT.test_op_own_qk_rope_reads_its_position_on_the_device, lambda: (ch([1, 2, 7, 300, 2049, 2100]), ri(0, 1), ri(0, 1))),
+        (FT.test_op_own_f16_moe_sum_shexp_add_against_the_oracle,
+         lambda: (lambda t: (t * ch([9, 37, 256, 1000, 2048, 5120]), ri(1, 64), t))(ch([1, 2, 3, 16]))),
         (FT.test_qk_nr_kv_equals_the_three_tape_ops,
          lambda: (lambda d: (ch([1, 3, 16, 70]), ri(1, 24), ri(1, 4), d, ch([x for x in (8, 16, 32, 64, 128, 256) if x <= d]), ri(0, 1)))(ch([32, 64, 96, 128, 256, 512]))),
         (FT.test_hadamard_gate_mul16_equals_the_two_tape_ops,
