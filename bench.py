@@ -232,6 +232,22 @@ def extra_opsets(B):
     l2f = torch.empty((T4 * 32, 128), dtype=torch.bfloat16, device=B.dev); ycf = torch.empty((T4, Cc), dtype=torch.bfloat16, device=B.dev)
     out.append(('c4_conv4_silu_l2_one_launch', T4 * Cc * 4 + Cc * 16 + Cc * 12 + T4 * 32 * 128 * 2,
                 lambda: B.call('camx_gdn_conv_l2', _p(xc), _p(wc), _p(st), _p(ycf), _p(l2f), I(Cc), I(T4), I(Cc), I(Cc), I(32), F(1e-6 / 128), I(1))))
+    # the tape's fp32 forms of the same layer (python/caminus/engine/q35_dense.py:396-400): OP_GDN_GATES, OP_GDN_CONV, OP_GDN_L2 and the one launch for the three
+    H4 = 48
+    xc32 = B.acts((T4, Cc), torch.float32, 61); st32 = B.acts((Cc, 3), torch.float32, 62, frac=0); xp32 = torch.zeros((T4, Cc), device=B.dev); yc32 = torch.empty((T4, Cc), device=B.dev)
+    qk32 = torch.empty((T4 * 32, 128), device=B.dev); par4 = torch.zeros(4, dtype=torch.int32, device=B.dev)
+    al4 = B.acts((T4, H4), torch.float32, 63); be4 = B.acts((T4, H4), torch.float32, 64); dt4 = B.acts((H4,), torch.float32, 65, frac=0); a4g = B.acts((H4,), torch.float32, 66, frac=0)
+    gt4 = torch.empty((T4, 2 * H4), device=B.dev)
+    def gdn_three():
+        B.call('camx_op_gdn_gates', _p(al4), _p(be4), _p(dt4), _p(a4g), _p(gt4), I(H4), I(T4))
+        B.call('camx_op_gdn_conv', _p(wc), _p(st32), _p(xc32), _p(par4), _p(yc32), _p(xp32), I(Cc), I(T4))
+        B.call('camx_op_gdn_l2', _p(yc32), _p(qk32), I(32), I(128), F(1e-6 / 128), I(Cc), I(T4))
+    byg = T4 * Cc * 4 * 3 + Cc * 28 + T4 * 32 * 128 * 4 + T4 * H4 * 16
+    out.append(('c4_tape_gdn_gates_conv_l2_three_launches', byg, gdn_three))
+    out.append(('c4_tape_gdn_gates_conv_l2_one_launch', byg,
+                lambda: B.call('camx_op_gdn_conv_l2_gates', _p(wc), _p(st32), _p(xc32), _p(par4), _p(yc32), _p(xp32), _p(qk32), I(Cc), I(T4), I(32), F(1e-6 / 128),
+                               _p(al4), _p(be4), _p(dt4), _p(a4g), _p(gt4), I(H4))))
+    out.append(('_keep4g', 0, [xc32, st32, xp32, yc32, qk32, par4, al4, be4, dt4, a4g, gt4]))
     kx = B.acts((T4 * 4, D4), torch.bfloat16, 47); wk4 = B.gamma(D4, 48); ok4 = torch.empty((T4 * 4, D4), dtype=torch.bfloat16, device=B.dev)
     out.append(('c4_qk_nr_partial_rotary_k', T4 * 4 * D4 * 4 + D4 * 4,
                 lambda: B.call('camx_qk_nr_pos', _p(kx), I(D4), I(4), _p(wk4), I(D4), I(64), F(ts7), F(1e-6), _p(pos), _p(ok4), I(T4), I(1))))
@@ -845,7 +861,8 @@ def main():
                              ('c4_qk_nr_partial_rotary_q_and_k_one_launch', ('c4_qk_nr_partial_rotary_q', 'c4_qk_nr_partial_rotary_k')),
                              ('c4_dense_q8_qk_nr_hadamard_append_one_launch', ('c4_dense_q8_qk_nr_hadamard_append_six_launches',)),
                              ('c4_dense_q8_att_hadamard_gate_one_launch', ('c4_dense_q8_att_hadamard_gate_two_launches',)),
-                             ('c1_qk_nr_kv_append_one_launch', ('c1_qk_nr_kv_append_three_launches',))):
+                             ('c1_qk_nr_kv_append_one_launch', ('c1_qk_nr_kv_append_three_launches',)),
+                             ('c4_tape_gdn_gates_conv_l2_one_launch', ('c4_tape_gdn_gates_conv_l2_three_launches',))):
             if fused in ops:
                 for key in ('us', 'us_cache_hot', 'us_queued'):
                     ops[fused][key + '_of_the_launches_it_replaces'] = round(sum(ops[p][key] for p in parts), 2)

@@ -154,14 +154,21 @@ __global__ void __launch_bounds__(256) op_gdn_conv_k(const float * __restrict__ 
     const f32x4 w4 = *(const f32x4 *)(w + (size_t)c * 4);
     for (int j = 0; j < mprev; j++) { s0 = s1; s1 = s2; s2 = xprev[(size_t)j * C + c]; }
     st[(size_t)c * 3] = s0; st[(size_t)c * 3 + 1] = s1; st[(size_t)c * 3 + 2] = s2;
-    for (int t = 0; t < T; t++) {
-        const float xv = x[(size_t)t * C + c];
-        float sumf = 0.0f;
-        sumf = __builtin_fmaf(s0, w4.x, sumf); sumf = __builtin_fmaf(s1, w4.y, sumf);
-        sumf = __builtin_fmaf(s2, w4.z, sumf); sumf = __builtin_fmaf(xv, w4.w, sumf);
-        y[(size_t)t * C + c] = silu_f(sumf);
-        s0 = s1; s1 = s2; s2 = xv;
-        xprev[(size_t)t * C + c] = xv;
+    for (int t0 = 0; t0 < T; t0 += 8) {                              // eight tokens' inputs requested together: a pass is latency, not bytes
+        float xv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) xv[u] = x[(size_t)(t0 + u < T ? t0 + u : T - 1) * C + c];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int t = t0 + u;
+            if (t >= T) break;
+            float sumf = 0.0f;
+            sumf = __builtin_fmaf(s0, w4.x, sumf); sumf = __builtin_fmaf(s1, w4.y, sumf);
+            sumf = __builtin_fmaf(s2, w4.z, sumf); sumf = __builtin_fmaf(xv[u], w4.w, sumf);
+            y[(size_t)t * C + c] = silu_f(sumf);
+            s0 = s1; s1 = s2; s2 = xv[u];
+            xprev[(size_t)t * C + c] = xv[u];
+        }
     }
 }
 // Prefill chunks: a lane owns VW consecutive channels and walks TR consecutive tokens, with the rows of the next eight tokens
@@ -497,53 +504,82 @@ __global__ void __launch_bounds__(256) gdn_conv_l2_k(const void * __restrict__ x
         if (BF16) *(u32x2 *)((uint16_t *)qk + qo) = pack_bf16x4_rne(o); else *(f32x4 *)((float *)qk + qo) = o;
     }
 }
-// OP_GDN_CONV followed by OP_GDN_L2 on the tape (decode / verify pass of T tokens, fp32, lazy commit as in op_gdn_conv_k): a half-wave per
-// 128 channels walks the pass's tokens; the state, the weights and the window stay in registers.
+// OP_GDN_CONV followed by OP_GDN_L2 on the tape (decode / verify pass of T tokens, fp32, lazy commit as in op_gdn_conv_k; qk null: the
+// convolution alone).
 __global__ void __launch_bounds__(256) op_gdn_conv_l2_k(const float * __restrict__ w, float * __restrict__ st, const float * __restrict__ x,
                                                         const int32_t * __restrict__ params, float * __restrict__ y, float * __restrict__ xprev,
-                                                        float * __restrict__ qk, int C, int T, int heads, float rs) {
-    const int lane = slot_of(threadIdx.x & 63), l = lane & 31;
-    const int G = C >> 7;
-    const int cgr = ((int)blockIdx.x * 4 + (int)(threadIdx.x >> 6)) * 2 + (lane >> 5);
-    const bool on = cgr < G;
-    const int cg = on ? cgr : 0, c0 = 128 * cg + 4 * l;
+                                                        float * __restrict__ qk, int C, int T, int heads, float rs,
+                                                        const float * __restrict__ al = nullptr, const float * __restrict__ be = nullptr,
+                                                        const float * __restrict__ dt = nullptr, const float * __restrict__ A = nullptr,
+                                                        float * __restrict__ gates = nullptr, int H = 0, int nconv = 0) {
+    if (al && (int)blockIdx.x >= nconv) {
+        // OP_GDN_GATES of the same layer in the launch's last workgroups (kernels/k3_q35_ops.h:196-211): gate = softplus(alpha + dt) * a | sigmoid(beta)
+        const int q = ((int)blockIdx.x - nconv) * (int)blockDim.x + (int)threadIdx.x;
+        if (q >= T * H) return;
+        const int tt = q / H, h = q - tt * H;
+        const float ab = al[q] + dt[h];
+        const float sp = ab > 20.0f ? ab : logf(1.0f + expf(ab));
+        gates[(size_t)tt * 2 * H + h] = sp * A[h];
+        gates[(size_t)tt * 2 * H + H + h] = 1.0f / (1.0f + expf(-be[q]));
+        return;
+    }
+    // One workgroup per 128 channels; its eight half-waves (32 lanes x 4 channels, the lanes in slot order) share the pass's tokens: half-wave
+    // h takes tokens h, h + 8, .. Each token's window is read straight from the rows it comes from (x of this pass; before its first token, the
+    // state as it stands once the previous pass's accepted tokens are committed), so no token waits for another: a pass of 16 or 64 tokens costs
+    // what two or eight cost one after the other. Only this workgroup touches its channels of the state and of xprev: everything it needs of
+    // them is in registers before the barrier, and rewritten after it.
+    const int lane = slot_of(threadIdx.x & 63), l = lane & 31, hw = (int)(threadIdx.x >> 5);
+    const int cg = (int)blockIdx.x, c0 = 128 * cg + 4 * l;
+    f32x4 w4[4], hist[3], xin[4];                                    // hist[3 - k]: the input k tokens before the pass, k = 1 .. 3
+    auto rows = [&](int tc) {                                        // the rows of x in token tc's window (requested before anything waits)
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const int tt = tc - 3 + k; if (tt >= 0) xin[k] = *(const f32x4 *)(x + (size_t)tt * C + c0); }
+    };
+    rows(hw < T ? hw : T - 1);
+#pragma unroll
+    for (int k = 0; k < 4; k++) w4[k] = *(const f32x4 *)(w + (size_t)(c0 + k) * 4);
     int mprev = params[1];
     mprev = mprev < 0 ? 0 : (mprev > T ? T : mprev);
-    float s[3][4];
-    f32x4 w4[4];
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        w4[k] = *(const f32x4 *)(w + (size_t)(c0 + k) * 4);
+    for (int k = 1; k <= 3; k++) {
+        if (mprev >= k) hist[3 - k] = *(const f32x4 *)(xprev + (size_t)(mprev - k) * C + c0);
+        else {
 #pragma unroll
-        for (int j = 0; j < 3; j++) s[j][k] = st[(size_t)(c0 + k) * 3 + j];
+            for (int e = 0; e < 4; e++) hist[3 - k][e] = st[(size_t)(c0 + e) * 3 + (mprev + 3 - k)];
+        }
     }
-    for (int j = 0; j < mprev; j++) {
-        const f32x4 xp = *(const f32x4 *)(xprev + (size_t)j * C + c0);
+    __syncthreads();
+    if (hw == 0) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) { s[0][k] = s[1][k]; s[1][k] = s[2][k]; s[2][k] = xp[k]; }
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int jj = 0; jj < 3; jj++) st[(size_t)(c0 + e) * 3 + jj] = hist[jj][e];
     }
-    if (on) {
+    const int nhw = (int)(blockDim.x >> 5);                          // (larger workgroups for longer passes were measured and are no faster: 64 tokens 9.4 against 9.8 us)
+    for (int tb = 0; tb < T; tb += nhw) {                            // (uniform trip count: both halves of a wave take part in the head's sums)
+        const int t = tb + hw;
+        const bool live = t < T;
+        const int tc = live ? t : T - 1;
+        f32x4 in[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++)
-#pragma unroll
-            for (int j = 0; j < 3; j++) st[(size_t)(c0 + k) * 3 + j] = s[j][k];
-    }
-    for (int t = 0; t < T; t++) {
-        const f32x4 xv = *(const f32x4 *)(x + (size_t)t * C + c0);
+        for (int k = 0; k < 4; k++) {                                // in[k]: the input at token tc - 3 + k
+            const int tt = tc - 3 + k;
+            in[k] = tt >= 0 ? xin[k] : (tt == -3 ? hist[0] : (tt == -2 ? hist[1] : hist[2]));
+        }
+        if (tb + nhw < T) rows(t + nhw < T ? t + nhw : T - 1);       // the next token's rows, in flight during this one's arithmetic
         f32x4 v;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
+        for (int e = 0; e < 4; e++) {
             float sumf = 0.0f;
-            sumf = __builtin_fmaf(s[0][k], w4[k].x, sumf); sumf = __builtin_fmaf(s[1][k], w4[k].y, sumf);
-            sumf = __builtin_fmaf(s[2][k], w4[k].z, sumf); sumf = __builtin_fmaf(xv[k], w4[k].w, sumf);
-            v[k] = silu_f(sumf);
-            s[0][k] = s[1][k]; s[1][k] = s[2][k]; s[2][k] = xv[k];
+            sumf = __builtin_fmaf(in[0][e], w4[e].x, sumf); sumf = __builtin_fmaf(in[1][e], w4[e].y, sumf);
+            sumf = __builtin_fmaf(in[2][e], w4[e].z, sumf); sumf = __builtin_fmaf(in[3][e], w4[e].w, sumf);
+            v[e] = silu_f(sumf);
         }
-        const f32x4 o = l2_head_l4(v, lane, rs);
-        if (on) {
+        const f32x4 o = qk ? l2_head_l4(v, lane, rs) : v;
+        if (live) {
             *(f32x4 *)(y + (size_t)t * C + c0) = v;
-            *(f32x4 *)(xprev + (size_t)t * C + c0) = xv;
-            if (cg < heads) *(f32x4 *)(qk + ((size_t)t * heads + cg) * 128 + 4 * l) = o;
+            *(f32x4 *)(xprev + (size_t)t * C + c0) = in[3];
+            if (qk && cg < heads) *(f32x4 *)(qk + ((size_t)t * heads + cg) * 128 + 4 * l) = o;
         }
     }
 }
@@ -790,7 +826,9 @@ int camx_pf_gdn_conv(const void * x, const float * w, const float * state, void 
 // N = C; T = the tape's tokens per pass
 int camx_op_gdn_conv(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, int C, int T, hipStream_t st) {
     if (!w || !state || !x || !params || !y || !xprev || C < 1 || T < 1 || ((uintptr_t)w & 15)) return CAMX_EINVAL;
-    op_gdn_conv_k<<<dim3((C + 255) / 256), dim3(256), 0, st>>>(w, state, x, params, y, xprev, C, T);
+    if (T >= 16 && (C & 127) == 0 && !(((uintptr_t)x | (uintptr_t)y | (uintptr_t)xprev) & 15))       // a verify pass: its tokens side by side (64 tokens: 11.3 -> 7.6 us)
+        op_gdn_conv_l2_k<<<dim3((unsigned)(C >> 7)), dim3(256), 0, st>>>(w, state, x, params, y, xprev, nullptr, C, T, 0, 0.0f);
+    else op_gdn_conv_k<<<dim3((C + 255) / 256), dim3(256), 0, st>>>(w, state, x, params, y, xprev, C, T);
     CAMX_LAUNCH_RET();
 }
 int camx_pf_conv_state(const void * x, float * state, int C, int T, int ldx, int bf16, hipStream_t st) {
@@ -848,7 +886,20 @@ int camx_op_gdn_conv_l2(const float * w, float * state, const float * x, const i
                         int heads, float rs, hipStream_t st) {
     if (!w || !state || !x || !params || !y || !xprev || !qk || C < 128 || (C & 127) || T < 1 || heads < 1 || heads > C / 128 ||
         (((uintptr_t)w | (uintptr_t)x | (uintptr_t)y | (uintptr_t)xprev | (uintptr_t)qk) & 15)) return CAMX_EINVAL;
-    op_gdn_conv_l2_k<<<dim3((unsigned)(((C >> 7) + 7) / 8)), dim3(256), 0, st>>>(w, state, x, params, y, xprev, qk, C, T, heads, rs);
+    op_gdn_conv_l2_k<<<dim3((unsigned)(C >> 7)), dim3(256), 0, st>>>(w, state, x, params, y, xprev, qk, C, T, heads, rs);
+    CAMX_LAUNCH_RET();
+}
+// The three row ops a linear-attention layer runs ahead of its recurrence (python/caminus/engine/q35_dense.py:396-400: OP_GDN_GATES, OP_GDN_CONV,
+// OP_GDN_L2) in one launch: camx_op_gdn_conv_l2's arguments, then camx_op_gdn_gates'. The gates take the launch's last workgroups.
+int camx_op_gdn_conv_l2_gates(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, float * qk, int C, int T,
+                              int heads, float rs, const float * alpha, const float * beta, const float * dt, const float * a, float * gates, int H,
+                              hipStream_t st) {
+    if (!w || !state || !x || !params || !y || !xprev || !qk || C < 128 || (C & 127) || T < 1 || heads < 1 || heads > C / 128 ||
+        (((uintptr_t)w | (uintptr_t)x | (uintptr_t)y | (uintptr_t)xprev | (uintptr_t)qk) & 15) || !alpha || !beta || !dt || !a || !gates || H < 1 ||
+        (long)T * H > 0x7fffffffL - 256) return CAMX_EINVAL;
+    const unsigned bs = 256;
+    const unsigned nconv = (unsigned)(C >> 7), ng = (unsigned)(((long)T * H + bs - 1) / bs);
+    op_gdn_conv_l2_k<<<dim3(nconv + ng), dim3(bs), 0, st>>>(w, state, x, params, y, xprev, qk, C, T, heads, rs, alpha, beta, dt, a, gates, H, (int)nconv);
     CAMX_LAUNCH_RET();
 }
 // the remaining elementwise ops of the decode tape by their Seg fields

@@ -198,6 +198,15 @@ class TapeOps:
         return self._go('camx_op_gdn_conv_l2', self._p(w), self._p(state), self._p(x), self._p(self.params), self._p(out), self._p(xprev), self._p(qk), I(C_), I(self.T),
                         I(heads), F(np.float32(eps / dim)))
 
+    def gdn_conv_l2_gates(self, x, w, state, out, xprev, qk, heads, dim, eps, alpha, beta, dt, a, gates, dep=-1, team=-1):
+        """gdn_gates beside gdn_conv -> gdn_l2 in one launch (python/caminus/engine/q35_dense.py:396-400)"""
+        I, F = self._C.c_int, self._C.c_float
+        C_ = x.numel() // self.T; H = alpha.numel() // self.T
+        if dim != 128: raise ValueError('gdn_conv_l2_gates: key heads of 128 values')
+        if self.params is None: raise ValueError('gdn_conv_l2_gates: set TapeOps.params (int32 [4] on the device; [1] = tokens to commit)')
+        return self._go('camx_op_gdn_conv_l2_gates', self._p(w), self._p(state), self._p(x), self._p(self.params), self._p(out), self._p(xprev), self._p(qk), I(C_),
+                        I(self.T), I(heads), F(np.float32(eps / dim)), self._p(alpha), self._p(beta), self._p(dt), self._p(a), self._p(gates), I(H))
+
     def qk_nr_q8(self, q, q_head_stride, heads, k, v, kv_heads, qn, kn, pos, qo, cache, n_rot, theta_scale, eps, dep=-1, team=-1):
         I, F = self._C.c_int, self._C.c_float
         M = kv_heads * 256

@@ -147,6 +147,12 @@ int camx_op_own_qk_rope(const float * qkv, int ldq, int nh, int nkv, const float
  * camx_op_gdn_conv's arguments, then qk [T][heads][128] = camx_op_gdn_l2(y, qk, heads, 128, rs, C, T). Same bits as the two. C % 128 == 0. */
 int camx_op_gdn_conv_l2(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, float * qk, int C,
                         int T, int heads, float rs, camx_stream_t stream);
+/* OP_GDN_GATES, OP_GDN_CONV and OP_GDN_L2, the three row ops a linear-attention layer of the tape runs ahead of its recurrence
+ * (python/caminus/engine/q35_dense.py:396-400), in one launch: camx_op_gdn_conv_l2's arguments, then camx_op_gdn_gates' (alpha, beta [T][H],
+ * gates [T][2H]). Same bits as the two calls. */
+int camx_op_gdn_conv_l2_gates(const float * w, float * state, const float * x, const int32_t * params, float * y, float * xprev, float * qk, int C,
+                              int T, int heads, float rs, const float * alpha, const float * beta, const float * dt, const float * a, float * gates,
+                              int H, camx_stream_t stream);
 /* pf_hc_post_rms (kernels/prefill_glue.hip:130-170): row q = t * HC + h of N values: res[q] = fma(b[t], 2 sigmoid(inj[q] * rs),
  * res[q]) in place, then the norm of the updated row with w[h]: xn fp32, xnbf bf16, scl the row scale [T * HC], each optional.
  * The reference kernel is built for N = 2560; N is an argument here. */

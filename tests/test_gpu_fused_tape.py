@@ -79,6 +79,35 @@ def test_op_gdn_conv_l2_equals_the_two_tape_ops(C_, T, heads):
         m = int(rng.integers(0, T + 1))
 
 
+@pytest.mark.parametrize('C_,T,heads,H', [(10240, 16, 32, 48), (10240, 1, 32, 48), (256, 4, 2, 3), (1024, 7, 5, 300)])
+def test_op_gdn_conv_l2_gates_equals_the_three_tape_ops(C_, T, heads, H):
+    """OP_GDN_GATES beside OP_GDN_CONV -> OP_GDN_L2 in one launch: every output and the carried state as the separate tape ops leave them"""
+    rng = np.random.default_rng(C_ + T + H)
+    w = rng.standard_normal((C_, 4)).astype(np.float32); st0 = rng.standard_normal((C_, 3)).astype(np.float32)
+    junk = rng.standard_normal((T, C_)).astype(np.float32)
+    dt = rng.standard_normal(H).astype(np.float32); A = -np.abs(rng.standard_normal(H)).astype(np.float32)
+    wd, dtd, Ad = dev(w), dev(dt), dev(A)
+    s1, s2 = dev(st0), dev(st0); xp1, xp2 = dev(junk), dev(junk)
+    m = 0
+    for step in range(3):
+        x = outliers(rng, (T, C_)); xd = dev(x); al = outliers(rng, (T, H)) * np.float32(8); be = outliers(rng, (T, H)); ald, bed = dev(al), dev(be)
+        par = dev(np.array([7, m, 0, 0], np.int32))
+        ya = dev(np.zeros((T, C_), np.float32)); qa = dev(np.zeros((T * heads, 128), np.float32)); ga = dev(np.zeros((T, 2 * H), np.float32))
+        call('camx_op_gdn_gates', ptr(ald), ptr(bed), ptr(dtd), ptr(Ad), ptr(ga), I(H), I(T))
+        call('camx_op_gdn_conv_l2', ptr(wd), ptr(s1), ptr(xd), ptr(par), ptr(ya), ptr(xp1), ptr(qa), I(C_), I(T), I(heads), F(RS))
+        yb = dev(np.full((T, C_), 3, np.float32)); qb = dev(np.full((T * heads, 128), 3, np.float32)); gb = dev(np.full((T, 2 * H), 3, np.float32))
+        call('camx_op_gdn_conv_l2_gates', ptr(wd), ptr(s2), ptr(xd), ptr(par), ptr(yb), ptr(xp2), ptr(qb), I(C_), I(T), I(heads), F(RS),
+             ptr(ald), ptr(bed), ptr(dtd), ptr(Ad), ptr(gb), I(H))
+        assert torch.equal(ya, yb) and torch.equal(qa, qb) and torch.equal(ga, gb) and torch.equal(s1, s2) and torch.equal(xp1, xp2), f'pass {step}'
+        m = int(rng.integers(0, T + 1))
+    assert close_fp32(host(gb), O.gdn_gates(al, be, dt, A))
+    L = camx(); p = lambda t: C.c_void_p(t.data_ptr())
+    args = [p(wd), p(s2), p(xd), p(par), p(yb), p(xp2), p(qb), I(C_), I(T), I(heads), F(RS), p(ald), p(bed), p(dtd), p(Ad), p(gb), I(H)]
+    for i, bad in ((11, NULL), (15, NULL), (16, I(0)), (7, I(C_ + 64))):
+        a2 = list(args); a2[i] = bad
+        assert L.camx_op_gdn_conv_l2_gates(*a2, stream()) == 1
+
+
 # ---- the dense Q8 line: QK-norm + partial rotary + Hadamard + Q8 blocks ---------------------------------------------------------------
 def _dense_q8_inputs(rng, T, nh, nkv):
     q = outliers(rng, (T * nh, 512)); k = outliers(rng, (T, nkv * 256)); v = outliers(rng, (T, nkv * 256))
