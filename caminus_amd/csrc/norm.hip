@@ -567,9 +567,17 @@ int camx_q3p_add_rms16(float * x, const float * d, const float * w, int S, const
 
 // OP_OWN_ADD_RMS16 with its Seg fields (python/caminus/engine/k3.py:881-902): W = nw, gs = w, a = d, asum = h, y = x, rs = eps, N,
 // K = the fp16 copy's token stride (elements, >= N), pad1 = S, aux = h16, tokens = the tape's T
+// OP_OWN_ADD_RMS16 as the dense line's modules run it (kernels/k3_q35_ops.h:79-130): any row length N = 256 NI up to 65536, one addend with
+// weight 1 (S = 1) or none, h always written, the fp16 copy rounded once from the last product (camx_q35p_add_rms16's arithmetic) at token stride K
+int camx_op_q35_add_rms16(float * x, const float * d, int S, const float * nw, float eps, float * h, uint16_t * h16, int N, int K, int tokens, hipStream_t st) {
+    if (N < 256 || N % 256 || N > 65536 || K < N || S < 0 || S > 1 || tokens < 0 || !x || !nw || !h || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
+    NormArgs a = {x, S ? d : nullptr, nullptr, 0, nw, 1, eps, h, h16, K, nullptr, nullptr, nullptr, N, tokens, nullptr, 1, 0.0f};
+    return launch_norm<ADD_F32_DIRECT, NORM_H | NORM_H16>(a, st);
+}
 int camx_op_own_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h, uint16_t * h16,
                           int N, int K, int tokens, hipStream_t st) {
-    if (N < 256 || N % 256 || N > 2048 || K < N || S < 0 || S > 8 || tokens < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
+    if (N < 256 || N % 256 || N > 65536 || K < N || S < 0 || S > 8 || tokens < 0 || !x || !nw || !h16 || (S > 0 && !d)) return CAMX_EINVAL;
+    if (N > 2048) return w ? CAMX_EINVAL : camx_op_q35_add_rms16(x, d, S, nw, eps, h, h16, N, K, tokens, st);      // only the dense line's modules have rows this long
     NormArgs a = {x, d, w, d ? S : 0, nw, 1, eps, h, h16, K, nullptr, nullptr, nullptr, N, tokens, nullptr, 1, 0.0f};
     return launch_norm<ADD_F32_SLOTS, NORM_H16, NORM_H | NORM_H16>(a, st);
 }

@@ -54,13 +54,14 @@ OWN_FMT = {'Q4_K': 4, 'IQ2_S': 7}
 
 
 class TapeOps:
-    def __init__(self, T=1, kv_q8_dense=False, kv_error=None):
+    def __init__(self, T=1, kv_q8_dense=False, kv_error=None, q35=False):
         """T: tokens per pass; kv_q8_dense: kv_append(q8=True) writes the dense Q8 line's blocks with the codec's refusal rules (the
         reference's K3_Q35_KV_Q8 modules) and needs kv_error, the sticky int32 word"""
         import ctypes
         import torch
         from ..device import lib as _lib
         self.T, self.kv_q8_dense, self.kv_error = int(T), bool(kv_q8_dense), kv_error
+        self.q35 = bool(q35)            # the dense line's modules: own_add_rms16 at any row length, one unweighted addend, the fp16 copy rounded once
         if self.kv_q8_dense and kv_error is None: raise ValueError('TapeOps: the dense Q8 KV line needs its error word (kv_error)')
         self._C, self._torch, self._L, self._check = ctypes, torch, _lib.load(), _lib.check
         self.params = None              # the pass parameters of gdn_conv (int32 [4] on the device; [1] = tokens of the previous pass to commit)
@@ -89,7 +90,10 @@ class TapeOps:
     def own_add_rms16(self, x, nw, h, h16, eps, d=None, slots=0, w=None, dep=-1, team=-1, tokens=1, h16_stride=None):
         I, F = self._C.c_int, self._C.c_float
         n = x.numel() // tokens; hs = n if h16_stride is None else int(h16_stride)
-        if n % 256 or not 256 <= n <= 2048: raise ValueError(f'own_add_rms16: n {n} (a multiple of 256, at most 2048)')
+        if n % 256 or not 256 <= n <= 65536: raise ValueError(f'own_add_rms16: n {n} (a multiple of 256, at most 65536)')
+        if self.q35 or n > 2048:                                     # (the dense line's modules: kernels/k3_q35_ops.h:79-130)
+            if slots > 1 or w is not None or h is None: raise ValueError(f'own_add_rms16: the dense line takes one unweighted addend or none, and the fp32 copy')
+            return self._go('camx_op_q35_add_rms16', self._p(x), self._p(d), I(slots), self._p(nw), F(eps), self._p(h), self._p(h16), I(n), I(hs), I(tokens))
         assert 0 <= slots <= 8 and (slots == 0 or d.numel() >= tokens * slots * n) and (w is None or w.numel() >= tokens * slots)
         return self._go('camx_op_own_add_rms16', self._p(x), self._p(d), self._p(w), I(slots), self._p(nw), F(eps), self._p(h), self._p(h16), I(n), I(hs), I(tokens))
 

@@ -66,9 +66,15 @@ int camx_pf_rms_mul(const float * x, const float * w, float * y, uint16_t * ybf,
                     camx_stream_t stream);
 /* OP_OWN_ADD_RMS16 (kernels/k3_own_ops.h:326-383) with the tape's Seg fields (python/caminus/engine/k3.py:881-902): y = x, a = d,
  * gs = w, pad1 = S, W = nw, rs = eps, asum = h, aux = h16, N, K = the token stride of h16 in elements (>= N), team = tokens.
- * camx_q3p_add_rms16 is the same pass with K = N. */
+ * camx_q3p_add_rms16 is the same pass with K = N. Rows longer than 2048 values exist only on the dense line's modules and are forwarded
+ * to camx_op_q35_add_rms16 (S <= 1, w NULL, h required). */
 int camx_op_own_add_rms16(float * x, const float * d, const float * w, int S, const float * nw, float eps, float * h, uint16_t * h16,
                           int N, int K, int tokens, camx_stream_t stream);
+/* OP_OWN_ADD_RMS16 as the dense line's modules run it (kernels/k3_q35_ops.h:79-130, host python/caminus/engine/k3.py:881-902): any row length
+ * N = 256 NI up to 65536, S = 1 (x += d) or 0, h always written, the fp16 copy rounded once from the last product (camx_q35p_add_rms16's
+ * arithmetic) at token stride K. The reference selects this form by module; camx_op_own_add_rms16 forwards rows longer than 2048 here. */
+int camx_op_q35_add_rms16(float * x, const float * d, int S, const float * nw, float eps, float * h, uint16_t * h16, int N, int K, int tokens,
+                          camx_stream_t stream);
 /* OP_GG_Q8_1 (kernels/k3_gguf_ops.h:55-77) with the tape's Seg fields in their order (python/caminus/engine/k3.py:649-659):
  * a = x, y, N = n, work = 0 plain / 1 silu(x * rs) / 2 silu(x) * gs[i], rs, gs. The same blocks as camx_gg_quantize_q8_1. */
 int camx_op_gg_q8_1(const float * x, void * y, int n, int work, float rs, const float * gs, camx_stream_t stream);

@@ -3,7 +3,9 @@ import numpy as np
 import pytest
 
 import oracle as O
-from gpu_util import F, I, NULL, bits_equal, call, dev, host, outliers, ptr
+import ctypes as C
+
+from gpu_util import F, I, NULL, bits_equal, call, camx, dev, host, outliers, ptr, stream
 
 pytestmark = pytest.mark.gpu
 
@@ -43,6 +45,19 @@ def test_q35p_add_rms16(n, N):
         ddv = dev(dd_) if dd_ is not None else None
         call('camx_q35p_add_rms16', ptr(xd), ptr(ddv), ptr(nwd), F(1e-6), ptr(h), ptr(h16), I(N), I(n))
         assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16, np.uint16), ref['h16'])
+        # the tape's form of the same op (OP_OWN_ADD_RMS16 on the dense line: rows longer than 2048, one addend or none), h16 at its own stride
+        K = N + 64
+        for sym in ('camx_op_q35_add_rms16',) + (('camx_op_own_add_rms16',) if N > 2048 else ()):
+            xd = dev(x); h = dev(np.zeros((n, N), np.float32)); h16 = dev(np.full((n, K), 0x5a5a, np.uint16))
+            extra = (NULL,) if sym == 'camx_op_own_add_rms16' else ()
+            call(sym, ptr(xd), ptr(ddv), *extra, I(1 if dd_ is not None else 0), ptr(nwd), F(1e-6), ptr(h), ptr(h16), I(N), I(K), I(n))
+            got = host(h16, np.uint16)
+            assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(got[:, :N], ref['h16']) and (got[:, N:] == 0x5a5a).all(), sym
+    if N > 2048:                                                      # what the long-row form does not take: weights, more than one addend, no fp32 copy
+        L = camx(); p = lambda t: C.c_void_p(t.data_ptr()); ddv = dev(d)
+        assert L.camx_op_own_add_rms16(p(xd), p(ddv), p(nwd), I(1), p(nwd), F(1e-6), p(h), p(h16), I(N), I(K), I(1), stream()) == 1
+        assert L.camx_op_own_add_rms16(p(xd), p(ddv), NULL, I(2), p(nwd), F(1e-6), p(h), p(h16), I(N), I(K), I(1), stream()) == 1
+        assert L.camx_op_own_add_rms16(p(xd), p(ddv), NULL, I(1), p(nwd), F(1e-6), NULL, p(h16), I(N), I(K), I(1), stream()) == 1
 
 
 @pytest.mark.parametrize('n,N', [(4, 2048), (256, 2048), (2, 5120), (1026, 2048), (1024, 4096)])
