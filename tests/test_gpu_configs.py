@@ -11,7 +11,7 @@ import torch
 
 import oracle as O
 from caminus_amd import rope
-from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, dev, host, outliers, ptr
+from gpu_util import F, I, L64, NULL, bits_equal, call, close_16, close_fp32, dev, host, outliers, ptr
 from vectors import q4k_table, q80_table, qk_par
 
 pytestmark = pytest.mark.gpu
@@ -184,6 +184,64 @@ def test_config4_hybrid_verify_batch():
         yl = dev(np.zeros((T * heads, 128), np.uint16))
         call('camx_pf_gdn_l2', ptr(dev(xl)), ptr(yl), I(heads), I(128), I(heads * 128), F(np.float32(1e-6 / 128)), I(T), I(1))
         assert bits_equal(host(yl, np.uint16), O.f2bf(O.gdn_l2(O.bf2f(xl), T, heads, 128, 1e-6)))
+
+
+@pytest.mark.parametrize('T', [1, 16])
+def test_config4_decode_tape_row_ops_of_both_layer_kinds(T):
+    """The dense line's decode / verify tape at config 4's shapes, fp32 as the tape runs it (python/caminus/engine/q35_dense.py:389-425), through the
+    host mirror's TapeOps(q35=True) with the fused launches: per layer the add + norm of 5120-wide rows, then either the linear-attention
+    row ops (gates | conv4 + SiLU with the lazy commit | L2 norm of 32 key heads; the gated norm of 48 value heads to fp16) or the
+    full-attention ones (QK-norm + partial rotary of 4 k heads into the fp16 cache beside v, and of 24 q heads; the sigmoid gate to fp16),
+    and the SwiGLU of the 17408-wide FFN. Two passes, the second committing part of the first."""
+    from caminus_amd.engine.k3 import TapeOps
+    rng = np.random.default_rng(1004 + T)
+    D, CH, NK, NV, S, nh, nkv, hd, nrot, FF, rows = 5120, 10240, 16, 48, 128, 24, 4, 256, 64, 17408, 64
+    M = nkv * hd; eps = 1e-6
+    ts = float(np.float32(np.float32(1e7) ** np.float32(-2.0 / nrot)))
+    err = dev(np.zeros(1, np.int32)); pos = dev(np.array([0], np.int32)); par = dev(np.zeros(4, np.int32))
+    E = TapeOps(T=T, kv_error=err, q35=True); E.params = par
+    nw = _gamma(rng, D); wc = rng.standard_normal((CH, 4)).astype(np.float32); st = rng.standard_normal((CH, 3)).astype(np.float32)
+    dt = rng.standard_normal(NV).astype(np.float32); A = -np.abs(rng.standard_normal(NV)).astype(np.float32); gw = _gamma(rng, S)
+    qn = _gamma(rng, hd); kn = _gamma(rng, hd)
+    nwd, wcd, std, dtd, Ad, gwd, qnd, knd = (dev(a) for a in (nw, wc, st, dt, A, gw, qn, kn))
+    xprev_ref = np.zeros((T, CH), np.float32); xpd = dev(xprev_ref); st_ref = st
+    cache = dev(np.zeros((rows, 2 * M), np.uint16)); cache_ref = np.zeros((rows, 2 * M), np.uint16)
+    mprev = 0
+    for step, p0 in enumerate((7, 7 + T)):
+        pos.fill_(p0); par.copy_(dev(np.array([0, mprev, 0, 0], np.int32)))
+        # the layer's entry: x += blk, h = rms_norm(x) * w, h16 (rounded once)
+        x = outliers(rng, (T, D)); blk = outliers(rng, (T, D))
+        xd = dev(x); h = dev(np.zeros((T, D), np.float32)); h16 = torch.zeros((T, D), dtype=torch.float16, device=xd.device)
+        E.own_add_rms16(xd, nwd, h, h16, eps, d=dev(blk), slots=1, tokens=T)
+        ref = O.add_rms16_q35(x, nw, eps, d=blk)
+        assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16.view(torch.int16), np.uint16), ref['h16'])
+        # a linear-attention layer
+        qkv = outliers(rng, (T, CH)); al = outliers(rng, (T, NV)) * np.float32(6); be = outliers(rng, (T, NV))
+        conv = dev(np.zeros((T, CH), np.float32)); qk = dev(np.zeros((T * 2 * NK, S), np.float32)); gates = dev(np.zeros((T, 2 * NV), np.float32))
+        E.gdn_conv_l2_gates(dev(qkv), wcd, std, conv, xpd, qk, 2 * NK, S, eps, dev(al), dev(be), dtd, Ad, gates)
+        ry, st_ref, xprev_ref = O.op_gdn_conv(wc, st_ref, qkv, mprev, xprev_ref)
+        got_y = host(conv)
+        assert close_fp32(got_y, ry) and bits_equal(host(std), st_ref) and bits_equal(host(xpd), xprev_ref)
+        assert bits_equal(host(qk), O.gdn_l2(got_y, T, 2 * NK, S, eps, ldx=CH)) and close_fp32(host(gates), O.gdn_gates(al, be, dt, A))
+        o = outliers(rng, (T * NV, S)); z = outliers(rng, (T * NV, S)); fin16 = torch.zeros((T * NV, S), dtype=torch.float16, device=xd.device)
+        E.gdn_norm16(dev(o), gwd, dev(z), fin16, NV, S, eps)
+        assert close_16(host(fin16.view(torch.int16), np.uint16), O.gdn_norm(o, gw, z, eps, silu=True)[1], 'f16')
+        # a full-attention layer
+        kr = outliers(rng, (T, M)); vr = outliers(rng, (T, M)); qf = outliers(rng, (T * nh, 2 * hd))
+        qo = dev(np.zeros((T * nh, hd), np.float32)); ko = dev(np.zeros((T * nkv, hd), np.float32))
+        E.qk_nr_kv(dev(qf), 2 * hd, nh, dev(kr), hd, dev(vr), nkv, hd, qnd, knd, pos, qo, cache, nrot, ts, eps, ko=ko)
+        wq_, wk_, cache_ref, werr = O.qk_nr_kv(qf, 2 * hd, nh, qn, kr.reshape(T * nkv, hd), hd, vr, nkv, kn, hd, nrot, ts, eps, p0, T, cache_ref, False, ko=host(ko))
+        assert close_fp32(host(qo), wq_) and close_fp32(host(ko), wk_) and werr == 0 and bits_equal(host(cache.view(torch.int16), np.uint16), cache_ref)
+        att = outliers(rng, (T * nh, hd)); gat16 = torch.zeros((T * nh, hd), dtype=torch.float16, device=xd.device)
+        E.gate_mul16(dev(att), dev(qf), 2 * hd, hd, gat16, hd)
+        assert close_16(host(gat16.view(torch.int16), np.uint16), O.gate_mul(att, qf, hd, 2 * hd, hd, f16=True), 'f16')
+        # the FFN's activation
+        g = outliers(rng, (T * FF,)); u = outliers(rng, (T * FF,)); y16 = torch.zeros(T * FF, dtype=torch.float16, device=xd.device)
+        E.own_swiglu16(dev(g), dev(u), y16)
+        assert close_16(host(y16.view(torch.int16), np.uint16), O.swiglu16(g, u), 'f16')
+        mprev = int(rng.integers(0, T + 1))
+    torch.cuda.synchronize()
+    assert int(host(err)[0]) == 0 and E.n == 2 * 6
 
 
 def test_config5_batched_decode_paged_q8():
