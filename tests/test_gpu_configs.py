@@ -57,6 +57,58 @@ def test_config1_decode_token():
     assert close_16(host(y16, np.uint16), O.swiglu16(g, u), 'f16')
 
 
+@pytest.mark.parametrize('T', [1, 4])
+def test_config1_decode_tape_row_ops(T):
+    """The qwen3moe decode tape at config 1's shapes through the host mirror's TapeOps (python/caminus/engine/q3moe_one.py:308-334, 352-377): the
+    three-stage entry (expert sum -> RMS norm -> fp16) and its one-launch form, the fp16-cache attention inputs as one launch (QK-norm + NeoX
+    rotary of 4 k heads into the cache beside v, and of 32 q heads), the own line's norm + rotary + append behind OP_OWN_ATTS, the
+    attention output's fp16 copy, and SwiGLU over 8 experts x 768. T = 4: the verify module's pass."""
+    from caminus_amd.engine.k3 import TapeOps
+    rng = np.random.default_rng(1001 + T)
+    D, hd, nh, nkv, KU, FF, rows = 2048, 128, 32, 4, 8, 768, 4096
+    M = nkv * hd; eps = 1e-6; ts = float(np.float32(np.float32(1e6) ** np.float32(-2.0 / hd)))
+    p0 = int(rng.integers(0, rows - T))
+    err = dev(np.zeros(1, np.int32)); pos = dev(np.array([p0], np.int32))
+    E = TapeOps(T=T, kv_error=err)
+    nw = _gamma(rng, D); nwd = dev(nw)
+    # experts' sum -> norm -> fp16 as three segments, token by token as the one-token statements have it
+    x = outliers(rng, (T, D)); dexp = outliers(rng, (T, KU, D)); wts = rng.random((T, KU)).astype(np.float32)
+    xs = x.copy(); hs = np.zeros((T, D), np.float32)
+    for t in range(T):
+        xt = dev(x[t]); ht = dev(np.zeros((1, D), np.float32)); h16t = torch.zeros(D, dtype=torch.float16, device=xt.device)
+        one = TapeOps(T=1, kv_error=err)
+        one.own_moe_sum(dev(dexp[t]), xt, slots=KU, w=dev(wts[t])); one.rms_mul(xt.view(1, D), nwd.view(1, D), ht, eps); one.own_f16(ht, h16t)
+        xs[t] = O.own_moe_sum(dexp[t], wts[t], x[t], KU); hs[t] = O.rms_mul(xs[t].reshape(1, D), nw.reshape(1, D), eps)['y'][0]
+        assert bits_equal(host(xt), xs[t]) and bits_equal(host(ht)[0], hs[t]) and bits_equal(host(h16t.view(torch.int16), np.uint16), O.own_f16(hs[t]))
+    # the same as one segment (equal to the three to rounding: its own statements, the oracle's add_rms16)
+    xd = dev(x); h = dev(np.zeros((T, D), np.float32)); h16 = torch.zeros((T, D), dtype=torch.float16, device=xd.device)
+    E.own_add_rms16(xd, nwd, h, h16, eps, d=dev(dexp), slots=KU, w=dev(wts), tokens=T)
+    ref = O.add_rms16(x, nw, eps, d=dexp, w=wts, S=KU)
+    assert bits_equal(host(xd), ref['x']) and bits_equal(host(h), ref['h']) and bits_equal(host(h16.view(torch.int16), np.uint16), ref['h16'])
+    assert close_fp32(ref['h'], hs)
+    # the fp16-cache attention inputs in one launch
+    q = outliers(rng, (T * nh, hd)); k = outliers(rng, (T * nkv, hd)); v = outliers(rng, (T, M)); qn = _gamma(rng, hd); kn = _gamma(rng, hd)
+    qo = dev(np.zeros((T * nh, hd), np.float32)); ko = dev(np.zeros((T * nkv, hd), np.float32)); cache = dev(np.zeros((rows, 2 * M), np.uint16))
+    E.qk_nr_kv(dev(q), hd, nh, dev(k), hd, dev(v), nkv, hd, dev(qn), dev(kn), pos, qo, cache, hd, ts, eps, ko=ko)
+    wq_, wk_, cref, werr = O.qk_nr_kv(q, hd, nh, qn, k, hd, v, nkv, kn, hd, hd, ts, eps, p0, T, np.zeros((rows, 2 * M), np.uint16), False, ko=host(ko))
+    assert close_fp32(host(qo), wq_) and close_fp32(host(ko), wk_) and werr == 0 and bits_equal(host(cache.view(torch.int16), np.uint16), cref)
+    # the own line: norm + rotary + append of the token's q | k | v row at the device position
+    par = qk_par(rng, theta_base=1e6); ldq = (nh + 2 * nkv) * hd
+    qkv = outliers(rng, (T, ldq)); q16 = dev(np.zeros((T, nh, hd), np.uint16)); c16 = dev(np.zeros((rows, 2 * M), np.uint16))
+    call('camx_op_own_qk_rope', ptr(dev(qkv)), I(ldq), I(nh), I(nkv), ptr(dev(par)), ptr(pos), ptr(q16), ptr(c16), I(rows), ptr(err), I(T), I(0), I(0))
+    rq, rc, _ = O.qk_rope(qkv, nh, nkv, par, T, pos0=p0, rows=rows)
+    gc = host(c16, np.uint16)
+    assert close_16(host(q16, np.uint16), rq, 'f16') and close_16(gc[p0:p0 + T, :M], rc[p0:p0 + T, :M], 'f16') and bits_equal(gc[p0:p0 + T, M:], rc[p0:p0 + T, M:])
+    # the attention output's fp16 copy and the experts' activation
+    att = outliers(rng, (T * nh * hd,)); a16 = torch.zeros(T * nh * hd, dtype=torch.float16, device=xd.device)
+    E.own_f16(dev(att), a16)
+    assert bits_equal(host(a16.view(torch.int16), np.uint16), O.own_f16(att))
+    g = outliers(rng, (T * KU * FF,)); u = outliers(rng, (T * KU * FF,)); y16 = torch.zeros(T * KU * FF, dtype=torch.float16, device=xd.device)
+    E.own_swiglu16(dev(g), dev(u), y16)
+    assert close_16(host(y16.view(torch.int16), np.uint16), O.swiglu16(g, u), 'f16')
+    assert int(host(err)[0]) == 0
+
+
 @pytest.mark.parametrize('fmt', [0, 1])
 def test_config2_embedding_gather_full_table(fmt):
     """151936 x 2048 table, Q4_K (175 MB) or Q8_0 (331 MB): 256 uniformly drawn ids to fp32 and bf16, then add + RMSNorm +
