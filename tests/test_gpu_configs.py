@@ -296,6 +296,59 @@ def test_config4_decode_tape_row_ops_of_both_layer_kinds(T):
     assert int(host(err)[0]) == 0 and E.n == 2 * 6
 
 
+def test_config4_prefill_chunk_through_the_host_wrappers():
+    """A 2048-token prefill chunk of the dense line's own prefill (python/caminus/prefill/q35own.py:352-389), fp32 as it runs there, through
+    the host mirror's wrapper classes with the reference's call sequence: add + norm of 5120-wide rows; gates, conv4 + SiLU with its carried
+    state, L2 norm of the 32 key heads, gated norm of the 48 value heads; QK-norm + partial rotary of the 4 k heads, the fp16 append, the
+    24 q heads, the sigmoid gate. The first and last 8 tokens of every output against the oracle."""
+    from caminus_amd.prefill import attn, gdn, glue, q35_ops
+    rng = np.random.default_rng(1044)
+    n, D, CH, NK, NV, S, nh, nkv, hd, nrot, p0, rows = 2048, 5120, 10240, 16, 48, 128, 24, 4, 256, 64, 100, 4096
+    M = nkv * hd; eps = 1e-6; ts = float(np.float32(np.float32(1e7) ** np.float32(-2.0 / nrot)))
+    devname = 'cuda:0'
+    Oq = q35_ops.Ops(devname); A = attn.Attn(devname); Gd = gdn.Gdn(devname, 'prefill_gdn_q35'); Gl = glue.Glue(devname)
+    ends = np.r_[0:8, n - 8:n]
+    zeros16 = lambda *sh: torch.zeros(sh, dtype=torch.float16, device=devname)
+    f16 = lambda t: host(t.view(torch.int16), np.uint16)
+    x = outliers(rng, (n, D)); blk = outliers(rng, (n, D)); nw = _gamma(rng, D)
+    xd = dev(x); h = dev(np.zeros((n, D), np.float32)); h16 = zeros16(n, D)
+    Oq.add_rms16(xd, dev(nw), eps, h16, n, D, d=dev(blk), h=h)
+    ref = O.add_rms16_q35(x[ends], nw, eps, d=blk[ends])
+    assert bits_equal(host(xd)[ends], ref['x']) and bits_equal(host(h)[ends], ref['h']) and bits_equal(f16(h16)[ends], ref['h16'])
+    al = outliers(rng, (n, NV)) * np.float32(6); be = outliers(rng, (n, NV)); dt = rng.standard_normal(NV).astype(np.float32); Aa = -np.abs(rng.standard_normal(NV)).astype(np.float32)
+    gt = dev(np.zeros((n, 2 * NV), np.float32))
+    Gd.gates(dev(al), dev(be), dev(dt), dev(Aa), gt, n, NV)
+    assert close_fp32(host(gt)[ends], O.gdn_gates(al[ends], be[ends], dt, Aa))
+    qkv = outliers(rng, (n, CH)); wc = rng.standard_normal((CH, 4)).astype(np.float32); st = rng.standard_normal((CH, 3)).astype(np.float32)
+    conv = dev(np.zeros((n, CH), np.float32)); std = dev(st); qk = dev(np.zeros((n * 2 * NK, S), np.float32))
+    Gl.gdn_conv(dev(qkv), dev(wc), std, conv, CH, n)
+    Gd.l2(conv, qk, n, 2 * NK, eps, ldx=CH)
+    ry, rst = O.gdn_conv(qkv, wc, st)
+    gy = host(conv)
+    assert close_fp32(gy[ends], ry[ends]) and bits_equal(host(std), rst)
+    assert bits_equal(host(qk).reshape(n, -1)[ends], O.gdn_l2(gy[ends], len(ends), 2 * NK, S, eps, ldx=CH).reshape(len(ends), -1))
+    o = outliers(rng, (n * NV, S)); z = outliers(rng, (n * NV, S)); gw = _gamma(rng, S); fin16 = zeros16(n * NV, S)
+    Oq.gdn_norm16(dev(o), dev(gw), dev(z), fin16, n, NV, S, eps)
+    rows_ = np.r_[0:8 * NV, (n - 8) * NV:n * NV]
+    assert close_16(f16(fin16)[rows_], O.gdn_norm(o[rows_], gw, z[rows_], eps, silu=True)[1], 'f16')
+    kr = outliers(rng, (n, M)); vr = outliers(rng, (n, M)); qf = outliers(rng, (n * nh, 2 * hd)); kn = _gamma(rng, hd); qn = _gamma(rng, hd)
+    ko = dev(np.zeros((n * nkv, hd), np.float32)); qo = dev(np.zeros((n * nh, hd), np.float32))
+    cache = zeros16(rows, 2 * M); err = dev(np.zeros(1, np.int32))
+    A.qk_nr(dev(kr), hd, nkv, hd, dev(kn), nrot, ts, eps, p0, ko, n)
+    Oq.kv_append16(ko, M, dev(vr), M, cache, M, p0, n, rows, err)
+    A.qk_nr(dev(qf), 2 * hd, nh, hd, dev(qn), nrot, ts, eps, p0, qo, n)
+    gko = host(ko).reshape(n, M)
+    for t in (0, 5, n - 1):
+        assert close_fp32(gko[t].reshape(nkv, hd), O.qk_nr(kr[t].reshape(nkv, hd), hd, nkv, kn, hd, nrot, ts, eps, p0 + t, 1))
+        assert close_fp32(host(qo)[t * nh:(t + 1) * nh], O.qk_nr(qf[t * nh:(t + 1) * nh], 2 * hd, nh, qn, hd, nrot, ts, eps, p0 + t, 1))
+    want, werr = O.kv_append16(gko, vr, M, np.zeros((rows, 2 * M), np.uint16), p0)
+    assert werr == 0 and int(host(err)[0]) == 0 and bits_equal(f16(cache), want)
+    att = outliers(rng, (n * nh, hd)); x16 = zeros16(n * nh, hd)
+    Oq.gate_mul16(dev(att), dev(qf), x16, n * nh * hd, hd, 2 * hd, hd)
+    r2 = np.r_[0:8 * nh, (n - 8) * nh:n * nh]
+    assert close_16(f16(x16)[r2], O.gate_mul(att, qf, hd, 2 * hd, hd, f16=True)[r2], 'f16')
+
+
 def test_config5_batched_decode_paged_q8():
     """256 sequences at the Qwen3-30B-A3B shape: add + RMSNorm, then QK-norm -> rotary at each sequence's own position below
     131072 -> fp16 -> Hadamard-128 -> Q8 blocks into a paged cache (page 256 tokens, random table over 65536 pages, 18 GB).
