@@ -296,6 +296,47 @@ def test_config4_decode_tape_row_ops_of_both_layer_kinds(T):
     assert int(host(err)[0]) == 0 and E.n == 2 * 6
 
 
+def test_q3m_prefill_chunk_through_the_host_wrappers():
+    """A 4096-token prefill chunk of the qwen3moe own prefill (python/caminus/prefill/q3m.py's layer loop: the call stack of the 2048-wide
+    configurations) through the host mirror's wrapper classes: Q4_K embedding rows of a 32768-row table, the layer entry with the 8 weighted
+    expert rows added, QK-norm + rotary into the fp16 cache, the router's scatter of the normed rows into the MMQ layout, SwiGLU of 8 x 768 per
+    token. The first and last 8 tokens against the oracle; the scatter block for block."""
+    from caminus_amd.prefill import mmq, q3m_ops
+    rng = np.random.default_rng(1033)
+    n, N, nh, nkv, KU, FF, vocab, rows, p0 = 4096, 2048, 32, 4, 8, 768, 32768, 8192, 1000
+    M = nkv * 128; eps = 1e-6; devname = 'cuda:0'
+    Oq = q3m_ops.Ops(devname); Q = mmq.MMQ(devname)
+    ends = np.r_[0:8, n - 8:n]
+    f16 = lambda t: host(t.view(torch.int16), np.uint16)
+    tab = q4k_table(rng, vocab, N); toks = rng.integers(-3, vocab + 3, n).astype(np.int32)
+    x = dev(np.zeros((n, N), np.float32))
+    Oq.emb(dev(tab), tab.shape[1], vocab, dev(toks), x, n, N)
+    assert bits_equal(host(x)[ends], O.emb_q4k(tab, vocab, toks[ends], N)[0])
+    x0 = host(x).copy()
+    dexp = outliers(rng, (n, KU, N)); wts = rng.random((n, KU)).astype(np.float32); nw = _gamma(rng, N)
+    h = dev(np.zeros((n, N), np.float32)); h16 = torch.zeros((n, N), dtype=torch.float16, device=devname)
+    Oq.add_rms16(x, dev(nw), eps, h16, n, N, d=dev(dexp), w=dev(wts), S=KU, h=h)
+    ref = O.add_rms16(x0[ends], nw, eps, d=dexp[ends], w=wts[ends], S=KU)
+    assert bits_equal(host(x)[ends], ref['x']) and bits_equal(host(h)[ends], ref['h']) and bits_equal(f16(h16)[ends], ref['h16'])
+    par = qk_par(rng, theta_base=1e6); ldq = (nh + 2 * nkv) * 128
+    qkv = outliers(rng, (n, ldq)); q16 = torch.zeros((n, nh, 128), dtype=torch.float16, device=devname); cache = torch.zeros((rows, 2 * M), dtype=torch.float16, device=devname)
+    Oq.qk_rope(dev(qkv), ldq, nh, nkv, dev(par), p0, q16, cache, n)
+    rq, rc, _ = O.qk_rope(qkv[ends[:8]], nh, nkv, par, 8, pos0=p0, rows=rows)
+    gc = f16(cache)
+    assert close_16(f16(q16).reshape(n, -1)[:8], rq.reshape(8, -1), 'f16') and close_16(gc[p0:p0 + 8, :M], rc[p0:p0 + 8, :M], 'f16') and bits_equal(gc[p0:p0 + 8, M:], rc[p0:p0 + 8, M:])
+    assert not gc[:p0].any() and not gc[p0 + n:].any() and gc[p0 + n - 1].any()
+    # the router's compact columns: grouped by expert, a group's tokens in order
+    ex = np.argsort(-rng.random((n, 128)), axis=1)[:, :KU].reshape(-1)
+    order = np.argsort(ex, kind='stable'); ids_inv = np.empty(n * KU, np.int32); ids_inv[order] = np.arange(n * KU, dtype=np.int32)
+    y = torch.zeros(mmq.y_bytes(N, n * KU), dtype=torch.uint8, device=devname)
+    Q.quantize_scatter(h, N, n, dev(ids_inv), KU, y, 1)
+    assert bits_equal(host(y)[:(N // 128) * n * KU * 144].reshape(N // 128, n * KU, 144), O.mmq_q8_1_scatter(host(h), N, n, ids_inv, KU, 1))
+    g = outliers(rng, (n * KU * FF,)); u = outliers(rng, (n * KU * FF,)); a16 = torch.zeros(n * KU * FF, dtype=torch.float16, device=devname)
+    Oq.swiglu(dev(g), dev(u), a16, n * KU * FF)
+    e = np.r_[0:8 * KU * FF, (n - 8) * KU * FF:n * KU * FF]
+    assert close_16(f16(a16)[e], O.swiglu16(g[e], u[e]), 'f16')
+
+
 def test_config4_prefill_chunk_through_the_host_wrappers():
     """A 2048-token prefill chunk of the dense line's own prefill (python/caminus/prefill/q35own.py:352-389), fp32 as it runs there, through
     the host mirror's wrapper classes with the reference's call sequence: add + norm of 5120-wide rows; gates, conv4 + SiLU with its carried
