@@ -337,6 +337,39 @@ def test_q3m_prefill_chunk_through_the_host_wrappers():
     assert close_16(f16(a16)[e], O.swiglu16(g[e], u[e]), 'f16')
 
 
+def test_coder_glue_chunk_through_the_host_wrappers():
+    """A 2048-token chunk of the hyper-connection model's prefill glue at the shape the reference publishes its times on (4 streams of
+    2560: SURVEY's perf table), through the host mirror's Glue wrappers in the layer's order (python/caminus/prefill/glue.py): the block's
+    output into the four residual streams + their norms (fp32, bf16 and the row scale), the gated mean of the streams from the norm and
+    again from the residual with the scale, the norm alone with a per-stream gamma, the bf16 operand copies. First and last 8 tokens."""
+    from caminus_amd.prefill import glue
+    rng = np.random.default_rng(1055)
+    T, HC, D, eps = 2048, 4, 2560, 1e-6
+    G = glue.Glue('cuda:0')
+    ends = np.r_[0:8, T - 8:T]
+    b = outliers(rng, (T, D)); inj = outliers(rng, (T, HC)); res = outliers(rng, (T, HC, D)); w = (1 + 0.1 * rng.standard_normal((HC, D))).astype(np.float32)
+    resd = dev(res); xn = dev(np.zeros((T, HC, D), np.float32)); xnbf = torch.zeros((T, HC, D), dtype=torch.bfloat16, device='cuda:0'); scl = dev(np.zeros(T * HC, np.float32))
+    G.hc_post_rms(dev(b), dev(inj), resd, dev(w), T, HC, eps, xn=xn, xnbf=xnbf, scale=scl)
+    ref = O.hc_post_rms(b[ends], inj[ends], res[ends], w, eps)
+    bfb = lambda t: host(t.view(torch.int16), np.uint16)
+    assert close_fp32(host(resd)[ends], ref['res']) and close_fp32(host(xn)[ends], ref['xn']) and close_16(bfb(xnbf)[ends], ref['xnbf'], 'bf16')
+    assert close_fp32(host(scl).reshape(T, HC)[ends], ref['scale'].reshape(len(ends), HC))
+    gate = outliers(rng, (T, HC, D)); out1 = dev(np.zeros((T, D), np.float32)); out2 = dev(np.zeros((T, D), np.float32))
+    G.hc_mean(xn, dev(gate), out1, T, HC)
+    G.hc_mean(resd, dev(gate), out2, T, HC, scale=scl, w=dev(w))
+    gxn = host(xn)
+    assert close_fp32(host(out1)[ends], O.hc_mean(gxn[ends], gate[ends])) and close_fp32(host(out2)[ends], host(out1)[ends])
+    y = dev(np.zeros((T * HC, D), np.float32)); ybf = torch.zeros((T * HC, D), dtype=torch.bfloat16, device='cuda:0')
+    G.rms_mul(resd.view(T * HC, D), dev(w), y, T * HC, eps, ybf=ybf)
+    gres = host(resd).reshape(T * HC, D); r2 = np.r_[0:8 * HC, (T - 8) * HC:T * HC]
+    rr = O.rms_mul(gres[r2], w, eps)
+    assert bits_equal(host(y)[r2], rr['y']) and bits_equal(bfb(ybf)[r2], rr['ybf'])
+    xb = torch.zeros((T, D), dtype=torch.bfloat16, device='cuda:0'); sb = torch.zeros((T, D), dtype=torch.bfloat16, device='cuda:0')
+    G.to_bf16(out1, xb, T, D); G.silu_bf16(out1, sb, T, D, 0.5)
+    g1 = host(out1)
+    assert bits_equal(bfb(xb)[ends], O.to_bf16_rows(g1[ends], len(ends), len(ends), D)) and close_16(bfb(sb)[ends], O.to_bf16_rows(g1[ends], len(ends), len(ends), D, rs=0.5, silu=True), 'bf16')
+
+
 def test_config4_prefill_chunk_through_the_host_wrappers():
     """A 2048-token prefill chunk of the dense line's own prefill (python/caminus/prefill/q35own.py:352-389), fp32 as it runs there, through
     the host mirror's wrapper classes with the reference's call sequence: add + norm of 5120-wide rows; gates, conv4 + SiLU with its carried
